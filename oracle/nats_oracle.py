@@ -1,0 +1,477 @@
+"""CPU oracle for the NAtS sparse-attention inference path.  TEST INFRASTRUCTURE ONLY.
+
+This module restates, in plain per-(batch, kv-head) loops over numpy / CPU torch tensors, what the
+reference computes on its PyTorch masked-attention path.  Nothing in the shipped package imports it;
+it is used by the tests, by the smoke check and by the CPU-baseline leg of the benchmark as the
+checker the HIP kernels are compared against.
+
+Every function cites the reference lines it follows (paths relative to the reference checkout).
+
+How each function is pinned (see tests/test_oracle_*.py):
+
+* roles_from_logits ............ brute force over all orderings of 3 logits + closed form
+                                 (attention/nats_attention.py:96-109, nats_chunk_attention.py:64-95)
+* next_global_index ............ docstring vector `[0,2,2,5,5,5,6]`-style closed form, brute force
+                                 (components/masks/utils.py:85-87)
+* chunk_visibility / prefill_mask  7x7 docstring mask of components/masks/utils_simple.py:94-107,
+                                 all-global == tril, all-sw == band, golden masks written by the
+                                 reference cache (tests/golden/chunk_cache_golden.npz)
+* masked_attention ............. torch SDPA with a bool mask is the library routine itself
+* ChunkCacheOracle.update / generate_mask / post_update
+                                 golden vectors written by the reference's NAtSChunkLayerCache on CPU
+                                 (tests/golden/make_golden.py), 21 scenarios / 228 calls, compared on
+                                 every byte of cache_k, cache_v, valid_tokens, sizes and scalars
+* decode_attention ............. equals masked_attention restricted to the valid rows (gather, then dense
+                                 softmax); checked against torch SDPA
+
+Functions with parity unpinned: none of the above; the per-token cache (chunk_size == 1,
+components/cache/nats_layer_cache.py) is not restated here.
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass, field
+
+import numpy as np
+import torch
+
+ROLE_GLOBAL = 0
+ROLE_LOCAL = 1
+ROLE_SW = 2
+
+
+# ----------------------------------------------------------------------------------------------
+# roles
+# ----------------------------------------------------------------------------------------------
+def roles_from_logits(logits: torch.Tensor, global_bias: float = 0.1, force_first_global: bool = False,
+                      force_last_global: bool = False) -> np.ndarray:
+    """logits [B, S, H_kv, 3] -> roles uint8 [B, H_kv, S].
+
+    attention/nats_attention.py:96-109: the bias is added to option 0 in the logits' own dtype, the role
+    is the first maximal option, slot 0 becomes global when the segment starts inside the sink chunk;
+    attention/nats_chunk_attention.py:92-94: an open last chunk is marked global."""
+    lg = logits.clone()
+    lg[..., 0] = lg[..., 0] + torch.tensor(global_bias, dtype=lg.dtype)
+    x = lg.float().numpy()
+    B, S, H, _ = x.shape
+    roles = np.zeros((B, H, S), dtype=np.uint8)
+    for b in range(B):
+        for s in range(S):
+            for h in range(H):
+                best, arg = x[b, s, h, 0], 0
+                for o in (1, 2):
+                    if x[b, s, h, o] > best:  # strict: the first maximum wins
+                        best, arg = x[b, s, h, o], o
+                roles[b, h, s] = arg
+    if force_first_global:
+        roles[:, :, 0] = ROLE_GLOBAL
+    if force_last_global:
+        roles[:, :, -1] = ROLE_GLOBAL
+    return roles
+
+
+def one_hot_roles(roles: np.ndarray, dtype=torch.float32) -> torch.Tensor:
+    """roles [B, H, S] -> token_states_info [B, H, S, 3] (cache/nats_chunk_layer_cache.py:188-190)."""
+    t = torch.zeros(*roles.shape, 3, dtype=dtype)
+    t.scatter_(-1, torch.from_numpy(roles.astype(np.int64)).unsqueeze(-1), 1.0)
+    return t
+
+
+def roles_from_one_hot(tsi: torch.Tensor) -> np.ndarray:
+    return tsi.float().argmax(-1).numpy().astype(np.uint8)
+
+
+def next_global_index(is_global: np.ndarray) -> np.ndarray:
+    """For every slot n: the first slot g >= n that is global, the last slot counting as global.
+
+    components/masks/utils.py:85-87 (flip / cummax / flip with the last flag forced to 1)."""
+    flags = np.asarray(is_global).astype(bool)
+    S = flags.shape[-1]
+    out = np.empty(flags.shape, dtype=np.int64)
+    flat_f = flags.reshape(-1, S)
+    flat_o = out.reshape(-1, S)
+    for r in range(flat_f.shape[0]):
+        nxt = S - 1
+        for n in range(S - 1, -1, -1):
+            if flat_f[r, n] or n == S - 1:
+                nxt = n
+            flat_o[r, n] = nxt
+    return out
+
+
+# ----------------------------------------------------------------------------------------------
+# masks
+# ----------------------------------------------------------------------------------------------
+def chunk_visibility(roles: np.ndarray, window_chunks: int) -> np.ndarray:
+    """roles [B, H, S] -> bool [B, H, S(query slot m), S(key slot n)], no causal cut.
+
+    components/masks/utils.py:89-94 gives (g(n) >= m) | global-or-last(n);
+    cache/nats_chunk_layer_cache.py:603-611 replaces the columns of sliding-window slots by
+    (m - n) <= W / C, only if at least one slot anywhere is sliding-window."""
+    B, H, S = roles.shape
+    g = next_global_index(roles == ROLE_GLOBAL)
+    vis = np.zeros((B, H, S, S), dtype=bool)
+    any_sw = bool((roles == ROLE_SW).any())
+    for b in range(B):
+        for h in range(H):
+            for n in range(S):
+                is_g = roles[b, h, n] == ROLE_GLOBAL or n == S - 1
+                for m in range(S):
+                    if any_sw and roles[b, h, n] == ROLE_SW:
+                        vis[b, h, m, n] = (m - n) <= window_chunks
+                    else:
+                        vis[b, h, m, n] = (g[b, h, n] >= m) or is_g
+    return vis
+
+
+def expand_chunk_mask(vis: np.ndarray, C: int) -> np.ndarray:
+    return np.repeat(np.repeat(vis, C, axis=-1), C, axis=-2)
+
+
+def prefill_mask(roles: np.ndarray, L: int, C: int, W: int) -> np.ndarray:
+    """Token-level bool mask [B, H, L, L] of a prefill from an empty cache.
+
+    cache/nats_chunk_layer_cache.py:589-620 with chunk_fill_size == x_len == L."""
+    vis = expand_chunk_mask(chunk_visibility(roles, W // C), C)[..., :L, :L]
+    return np.tril(vis)
+
+
+def repeat_for_gqa(x: torch.Tensor, n_rep: int) -> torch.Tensor:
+    """[B, H_kv, ...] -> [B, H_kv * n_rep, ...] (models/transformer/utils.py:23-46)."""
+    if n_rep == 1:
+        return x
+    return x.repeat_interleave(n_rep, dim=1)
+
+
+def masked_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask, sm_scale: float | None = None,
+                     explicit: bool = False) -> torch.Tensor:
+    """q [B, H_q, Lq, D], k / v [B, H_kv, N, D], mask bool [B, H_kv, Lq, N] -> [B, H_q, Lq, D].
+
+    attention/nats_chunk_attention.py:130-149: repeat k, v and the mask to H_q heads, then SDPA with a bool
+    mask (`explicit=False`) or matmul / fp32 softmax cast back to q's dtype / matmul (`explicit=True`)."""
+    n_rep = q.shape[1] // k.shape[1]
+    mask_t = torch.as_tensor(mask)
+    k_r, v_r, m_r = repeat_for_gqa(k, n_rep), repeat_for_gqa(v, n_rep), repeat_for_gqa(mask_t, n_rep)
+    D = q.shape[-1]
+    scale = (1.0 / math.sqrt(D)) if sm_scale is None else sm_scale
+    if not explicit:
+        return torch.nn.functional.scaled_dot_product_attention(q, k_r, v_r, attn_mask=m_r, is_causal=False,
+                                                                scale=scale)
+    scores = torch.matmul(q, k_r.transpose(2, 3)) * scale
+    scores = scores.float().masked_fill(~m_r, float("-inf"))
+    p = torch.softmax(scores, dim=-1).type_as(q)
+    return torch.matmul(p, v_r)
+
+
+def decode_attention(q: torch.Tensor, cache_k: torch.Tensor, cache_v: torch.Tensor, valid: torch.Tensor,
+                     n_rows: int, sm_scale: float | None = None) -> torch.Tensor:
+    """One query token per sequence over the evicted cache: softmax over the rows flagged valid.
+
+    cache/nats_chunk_layer_cache.py:622-632 (mask = valid_tokens[:, :, :n_ctx_data + 1]) followed by SDPA;
+    restated as gather-valid-rows-then-dense-softmax per (b, kv-head) in fp32."""
+    B, Hq, one, D = q.shape
+    Hkv = cache_k.shape[1]
+    n_rep = Hq // Hkv
+    scale = (1.0 / math.sqrt(D)) if sm_scale is None else sm_scale
+    out = torch.zeros(B, Hq, 1, D, dtype=torch.float32)
+    for b in range(B):
+        for h in range(Hkv):
+            idx = torch.nonzero(valid[b, h, :n_rows]).flatten()
+            kk = cache_k[b, h, idx].float()
+            vv = cache_v[b, h, idx].float()
+            qq = q[b, h * n_rep:(h + 1) * n_rep, 0].float()
+            s = (qq @ kk.T) * scale
+            p = torch.softmax(s, dim=-1)
+            out[b, h * n_rep:(h + 1) * n_rep, 0] = p @ vv
+    return out.to(q.dtype)
+
+
+# ----------------------------------------------------------------------------------------------
+# tile-level accounting used by the benchmark and the tile-map tests
+# ----------------------------------------------------------------------------------------------
+def visited_tiles(roles: np.ndarray, window_chunks: int) -> np.ndarray:
+    """bool [B, H, S, S]: (q-chunk m, k-chunk n) pairs that hold at least one unmasked score."""
+    vis = chunk_visibility(roles, window_chunks)
+    S = roles.shape[-1]
+    return vis & np.tril(np.ones((S, S), dtype=bool))
+
+
+# ----------------------------------------------------------------------------------------------
+# the chunked layer cache as an explicit state machine
+# ----------------------------------------------------------------------------------------------
+@dataclass
+class ChunkCacheOracle:
+    """State of one layer (cache/nats_chunk_layer_cache.py:16-77).
+
+    `pos_k` shadows cache_k with the stream position of the token each row holds (-1 = no token); it is
+    the surviving-token index map the reference does not keep."""
+    B: int
+    H: int
+    W: int
+    C: int
+    size_global: np.ndarray = field(init=False)
+    size_local: np.ndarray = field(init=False)
+    n_ctx_data: int = field(init=False)
+    gmin: int = field(init=False)
+    tail: int = 0
+    fill: int = 0
+    fill_last: int = 0
+    seen: int = 0
+    cache_k: torch.Tensor | None = None
+    cache_v: torch.Tensor | None = None
+    pos_k: np.ndarray | None = None
+    valid: np.ndarray | None = None
+    roles: np.ndarray | None = None  # roles handed over by the last update
+
+    def __post_init__(self):
+        assert self.W % self.C == 0  # :47
+        self.size_global = np.full((self.B, self.H), self.W, dtype=np.int64)
+        self.size_local = np.zeros((self.B, self.H), dtype=np.int64)
+        self.n_ctx_data = self.W
+        self.gmin = self.W
+
+    # -- append ---------------------------------------------------------------------------------
+    def update(self, k: torch.Tensor, v: torch.Tensor, roles: np.ndarray | None):
+        """:171-256.  Returns the K, V the attention of this call runs over."""
+        B, H, x_len, D = k.shape
+        self.fill += x_len
+        if x_len == 0:
+            return self.cache_k[:, :, :self.n_ctx_data], self.cache_v[:, :, :self.n_ctx_data]
+        self.roles = None if roles is None else np.array(roles, dtype=np.uint8)
+        if self.cache_k is None:
+            pad = (-x_len) % self.C
+            rows = self.W + x_len + pad
+            self.cache_k = torch.zeros(B, H, rows, D, dtype=k.dtype)
+            self.cache_v = torch.zeros(B, H, rows, D, dtype=v.dtype)
+            self.cache_k[:, :, self.W:self.W + x_len] = k
+            self.cache_v[:, :, self.W:self.W + x_len] = v
+            self.valid = np.zeros((B, H, rows), dtype=bool)
+            self.valid[:, :, self.W:self.W + x_len] = True
+            self.pos_k = np.full((B, H, rows), -1, dtype=np.int64)
+            self.pos_k[:, :, self.W:self.W + x_len] = np.arange(self.seen, self.seen + x_len)
+            return k, v
+        start = self.n_ctx_data
+        end = start + x_len
+        need = math.ceil(end / self.C) * self.C
+        have = self.cache_k.shape[2]
+        if need > have:
+            grow = need - have
+            self.cache_k = torch.cat([self.cache_k, torch.zeros(B, H, grow, D, dtype=self.cache_k.dtype)], 2)
+            self.cache_v = torch.cat([self.cache_v, torch.zeros(B, H, grow, D, dtype=self.cache_v.dtype)], 2)
+            self.valid = np.concatenate([self.valid, np.zeros((B, H, grow), dtype=bool)], 2)
+            self.pos_k = np.concatenate([self.pos_k, np.full((B, H, grow), -1, dtype=np.int64)], 2)
+        self.cache_k[:, :, start:end] = k.to(self.cache_k.dtype)
+        self.cache_v[:, :, start:end] = v.to(self.cache_v.dtype)
+        self.valid[:, :, start:end] = True
+        self.pos_k[:, :, start:end] = np.arange(self.seen, self.seen + x_len)
+        return self.cache_k[:, :, :end], self.cache_v[:, :, :end]
+
+    # -- masks ----------------------------------------------------------------------------------
+    def _new_token_mask(self, x_len: int):
+        """:589-620.  Rows = the x_len new tokens, columns = the open chunk region [base, base + fill)."""
+        fill = self.fill
+        if self.roles is None:
+            roles = np.zeros((self.B, self.H, 1), dtype=np.uint8)
+        else:
+            roles = self.roles
+        vis = chunk_visibility(roles, self.W // self.C)
+        g = next_global_index(roles == ROLE_GLOBAL)
+        tok = expand_chunk_mask(vis, self.C)[:, :, fill - x_len:fill, :fill]
+        rows = np.arange(fill - x_len, fill)[:, None]
+        cols = np.arange(tok.shape[-1])[None, :]
+        return tok & (cols <= rows), g
+
+    def generate_mask(self, x_len: int) -> np.ndarray:
+        """:156-163, :444-511.  Bool [B, H, x_len, n_ctx_data + x_len] (or [.., x_len, x_len] from empty)."""
+        if x_len == 1:
+            if self.seen == 0:  # :628-629
+                return np.ones((1, 1, 1, 1), dtype=bool)
+            return self.valid[:, :, None, :self.n_ctx_data + 1].copy()  # :631
+        new_mask, g = self._new_token_mask(x_len)
+        if self.seen == 0 or self.valid.shape[-1] == 0:
+            return new_mask
+        C, W = self.C, self.W
+        wc = W // C
+        old_fill = self.fill - x_len
+        base = self.n_ctx_data - self.fill + x_len  # :466, first row of the open chunk region
+        cached = np.repeat(self.valid[:, :, None, :base], x_len, axis=2).copy()
+        # ring columns age with the query position (:658-713)
+        q_chunk = (np.arange(old_fill, self.fill) + self.fill_last) // C  # :666-667 (fill_last added again)
+        seen_chunks = self.seen // C
+        if self.seen < W:
+            ncol = seen_chunks * C
+            j = np.arange(ncol) // C  # ring slot counted from slot 0
+            ok = (q_chunk[:, None] + j[None, :]) < wc  # :676
+            cached[:, :, :, :ncol] &= ok[None, None]
+        else:
+            slot = np.arange(W) // C
+            newest_row = ((slot + 1) * C + W - 1 - self.tail) % W  # queue offset of each slot's last row
+            ok = np.zeros((x_len, W), dtype=bool)
+            for i in range(x_len):
+                r = old_fill + i  # offset of the query inside the open chunk region
+                if r < W:  # :687-707, rows beyond the window see no ring slot
+                    ok[i] = newest_row >= r
+            cached[:, :, :, :W] &= ok[None, None]
+        # cached local chunks are visible up to the first new global slot (:480-494, :510)
+        gmin = self.gmin
+        ncc = (base - gmin) // C
+        q_slot = np.arange(old_fill, self.fill) // C
+        for b in range(self.B):
+            for h in range(self.H):
+                lo = (self.size_global[b, h] - gmin) // C
+                hi = (self.size_global[b, h] + self.size_local[b, h] - gmin) // C
+                for cc in range(ncc):
+                    if cc >= hi:
+                        col = np.zeros(x_len, dtype=bool)
+                    elif cc < lo:
+                        col = np.ones(x_len, dtype=bool)
+                    else:
+                        col = q_slot <= g[b, h, 0]
+                    cached[b, h, :, gmin + cc * C:gmin + (cc + 1) * C] = col[:, None]
+        return np.concatenate([cached, new_mask], axis=-1)
+
+    # -- evict + compact ------------------------------------------------------------------------
+    def post_update(self, x_len: int):
+        """:262-389."""
+        C, W, B, H = self.C, self.W, self.B, self.H
+        self.seen += x_len
+        if x_len == 0 or self.fill < C:  # chunk still open (:264-268)
+            self.fill_last = self.fill
+            self.n_ctx_data += x_len
+            return
+        partial = self.fill % C
+        n_done = self.fill // C
+        off = self.n_ctx_data // C  # cache chunk that holds role slot 0
+        roles = self.roles
+        S = roles.shape[-1]
+        assert S == n_done + (1 if partial else 0), "one role slot per (possibly open) chunk"
+        first = self.seen == x_len
+
+        # 1. ring insert (:391-437): the last min(n_done, W/C) completed chunks enter the ring
+        n_ring = min(n_done, W // C)
+        start = 0 if first else self.tail
+        for i in range(n_ring * C):
+            slot = n_done - n_ring + i // C
+            src = (off + n_done - n_ring) * C + i
+            dst = (start + i) % W
+            is_sw = roles[:, :, slot] == ROLE_SW  # [B, H]
+            for b in range(B):
+                for h in range(H):
+                    if is_sw[b, h]:
+                        self.cache_k[b, h, dst] = self.cache_k[b, h, src]
+                        self.cache_v[b, h, dst] = self.cache_v[b, h, src]
+                        self.pos_k[b, h, dst] = self.pos_k[b, h, src]
+                    else:
+                        self.cache_k[b, h, dst] = 0
+                        self.cache_v[b, h, dst] = 0
+                        self.pos_k[b, h, dst] = -1
+                    self.valid[b, h, dst] = is_sw[b, h]
+        self.tail = (start + n_ring * C) % W
+        self.fill = partial
+        self.fill_last = partial
+
+        # 2. every new slot sliding-window: only the live length changes (:283-288)
+        if (roles == ROLE_SW).all():
+            self.n_ctx_data = int((self.size_global + self.size_local).max()) + self.fill
+            return
+
+        if x_len == 1:
+            # 3a. one completed chunk, scattered for every head (:289-330)
+            snap_k = self.cache_k[:, :, off * C:(off + 1) * C].clone()
+            snap_v = self.cache_v[:, :, off * C:(off + 1) * C].clone()
+            snap_p = self.pos_k[:, :, off * C:(off + 1) * C].copy()
+            for b in range(B):
+                for h in range(H):
+                    r0 = roles[b, h, 0]
+                    r_last = roles[b, h, -1]
+                    sg, sl = int(self.size_global[b, h]), int(self.size_local[b, h])
+                    dst = sg if r0 == ROLE_GLOBAL else sg + sl
+                    self.cache_k[b, h, dst:dst + C] = snap_k[b, h]
+                    self.cache_v[b, h, dst:dst + C] = snap_v[b, h]
+                    self.pos_k[b, h, dst:dst + C] = snap_p[b, h]
+                    dec = (sl // C + 1) if r0 == ROLE_GLOBAL else 0
+                    dec += 1 if r_last == ROLE_SW else 0
+                    if r0 == ROLE_GLOBAL:
+                        self.size_global[b, h] += C
+                    self.size_local[b, h] -= dec * C
+        elif not (roles == ROLE_LOCAL).all():
+            # 3b. general path (:715-868 + cache_update.py:25-76)
+            last_excluded = partial != 0
+            plans = {}
+            max_keep = 0
+            max_end = None
+            for b in range(B):
+                for h in range(H):
+                    sg, sl = int(self.size_global[b, h]), int(self.size_local[b, h])
+                    r = roles[b, h]
+                    n_glob = int((r == ROLE_GLOBAL).sum())
+                    glob_slots = [s for s in range(S) if r[s] == ROLE_GLOBAL]
+                    if last_excluded:  # :782-786
+                        n_glob -= 1
+                        glob_slots = [s for s in glob_slots if s != S - 1]
+                    last_g = glob_slots[-1] if glob_slots else -1
+                    later_local = [s for s in range(S) if s > last_g and r[s] == ROLE_LOCAL]
+                    n_other = S - max(last_g, 0) - len(later_local) - (1 if last_excluded else 0)  # :797-800
+                    dec_local = (last_g * C + sl if last_g > -1 else 0) + n_other * C
+                    keep = sorted(set(glob_slots) | set(later_local))
+                    if last_excluded:  # :809-811
+                        keep = [s for s in keep if s != S - 1]
+                    dst_base = (sg + sl) // C if last_g == -1 else sg // C  # :827-828
+                    plans[(b, h)] = (keep, dst_base, n_glob * C, dec_local)
+                    max_keep = max(max_keep, len(keep))
+                    end = len(keep) + dst_base
+                    max_end = end if max_end is None else max(max_end, end)
+            moves = []  # (b, h, src_chunk, dst_chunk), all gathered before any is written
+            for (b, h), (keep, dst_base, _, _) in plans.items():
+                for rank, s in enumerate(keep):
+                    moves.append((b, h, s + off, dst_base + rank))
+            if last_excluded and max_keep < S - 1:  # :840-857, the open chunk follows the longest head
+                for b in range(B):
+                    for h in range(H):
+                        moves.append((b, h, S - 1 + off, max_end))
+            if moves:  # cache_update.py:51-52 returns untouched when nothing is kept
+                stash = [(self.cache_k[b, h, s * C:(s + 1) * C].clone(),
+                          self.cache_v[b, h, s * C:(s + 1) * C].clone(),
+                          self.pos_k[b, h, s * C:(s + 1) * C].copy()) for (b, h, s, _) in moves]
+                for (b, h, _, d), (kk, vv, pp) in zip(moves, stash):
+                    self.cache_k[b, h, d * C:(d + 1) * C] = kk
+                    self.cache_v[b, h, d * C:(d + 1) * C] = vv
+                    self.pos_k[b, h, d * C:(d + 1) * C] = pp
+            for (b, h), (_, _, inc_g, dec_l) in plans.items():
+                self.size_global[b, h] += inc_g
+                self.size_local[b, h] -= dec_l
+
+        # 4. bookkeeping shared by both paths (:356-385)
+        self.size_local += n_done * C
+        assert not (self.size_local < 0).any()
+        self.n_ctx_data = int((self.size_global + self.size_local).max()) + self.fill
+        self.cache_k[:, :, self.n_ctx_data:] = 0
+        self.cache_v[:, :, self.n_ctx_data:] = 0
+        self.pos_k[:, :, self.n_ctx_data:] = -1
+        old_gmin = self.gmin  # :644 uses the minimum from before this call
+        if self.n_ctx_data != old_gmin:
+            last_chunk = self.n_ctx_data // C * C
+            idx = np.arange(old_gmin, last_chunk)
+            end = (self.size_global + self.size_local)[:, :, None]
+            self.valid[:, :, old_gmin:last_chunk] = idx[None, None, :] < end
+            self.valid[:, :, last_chunk:last_chunk + self.fill] = True
+        self.gmin = int(self.size_global.min())
+        if first:  # :373-380
+            keep_rows = math.ceil(self.n_ctx_data / C) * C
+            self.cache_k = self.cache_k[:, :, :keep_rows]
+            self.cache_v = self.cache_v[:, :, :keep_rows]
+            self.valid = self.valid[:, :, :keep_rows]
+            self.pos_k = self.pos_k[:, :, :keep_rows]
+
+    # -- derived observables --------------------------------------------------------------------
+    def surviving_positions(self, b: int, h: int) -> np.ndarray:
+        """Stream positions of the rows a decode step would attend to, in cache order."""
+        n = self.n_ctx_data
+        return self.pos_k[b, h, :n][self.valid[b, h, :n]]
+
+
+def kept_token_fraction(cache: ChunkCacheOracle) -> float:
+    """Mean retained-KV fraction as the reference's benchmark reports it
+    (experiments/efficiency/eval_efficiency.py:349-355)."""
+    kept = cache.size_global + cache.size_local + cache.fill
+    return float(kept.mean()) / max(cache.seen, 1)
