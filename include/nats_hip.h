@@ -1,0 +1,193 @@
+/*
+ * C ABI of the MI355X (gfx950) NAtS sparse-attention inference path.
+ *
+ * Every entry point takes raw device pointers (as produced by hipMalloc or tensor.data_ptr()), plain
+ * integer sizes / strides counted in ELEMENTS, and a HIP stream handle passed as void* (NULL = the
+ * default stream).  All work is enqueued on that stream; nothing synchronises with the host, nothing
+ * allocates or frees device memory and no pointer is kept after the call returns.
+ *
+ * Return value: 0 on success, a negative nats_status otherwise; nats_last_error() then returns a
+ * thread-local, human readable description.
+ *
+ * Citations name the reference interface each entry point stands in for (paths relative to the
+ * reference checkout, src/nats/...).
+ */
+#ifndef NATS_HIP_H
+#define NATS_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NATS_ABI_VERSION 1
+
+typedef enum {
+  NATS_OK = 0,
+  NATS_ERR_NULL_POINTER = -1,
+  NATS_ERR_BAD_SHAPE = -2,
+  NATS_ERR_BAD_DTYPE = -3,
+  NATS_ERR_UNSUPPORTED = -4,
+  NATS_ERR_WORKSPACE = -5,
+  NATS_ERR_LAUNCH = -6
+} nats_status;
+
+typedef enum { NATS_DTYPE_BF16 = 0, NATS_DTYPE_F32 = 1 } nats_dtype;
+
+/* role codes, the option order of token_states_info (components/cache/nats_chunk_layer_cache.py:188-190) */
+enum { NATS_ROLE_GLOBAL = 0, NATS_ROLE_LOCAL = 1, NATS_ROLE_SW = 2 };
+
+int nats_abi_version(void);
+const char* nats_last_error(void);
+
+/* ------------------------------------------------------------------------------------------------
+ * (a-1) role assignment.  Replaces BaseNAtSAttentionLayer._sample_for_token_info_values_inference
+ * (models/transformer/attention/nats_attention.py:96-109) and the open-chunk rule of
+ * models/transformer/attention/nats_chunk_attention.py:92-94.
+ *   logits  [B, S, H_kv, 3] contiguous, dtype bf16 or f32
+ *   roles   [B, H_kv, S] uint8 out (0 global, 1 local, 2 sliding window)
+ *   one_hot [B, H_kv, S, 3] out, same dtype as logits, may be NULL
+ * global_bias is added to option 0 in the logits' dtype (0.1 in the reference module, 0 in the HF
+ * twins); the first maximal option wins; slot 0 / the last slot are forced global on request.
+ */
+int nats_roles_from_logits(const void* logits, int dtype, int64_t B, int64_t S, int64_t H_kv, float global_bias,
+                           int force_first_global, int force_last_global, uint8_t* roles, void* one_hot,
+                           void* stream);
+
+/* (a-2) next-global index and the per-slot visibility limit derived from it.
+ * Replaces the first half of generate_hard_seq_masks (components/masks/utils.py:85-87).
+ *   roles    [B, H_kv, S] uint8
+ *   end_idx  [B, H_kv, S] int64 out, may be NULL: first global slot >= n, the last slot counting as global
+ *   vis_lim  [B, H_kv, S] int32 out, may be NULL: the last query slot that still sees key slot n
+ *            (global: INT32_MAX, local: end_idx[n], sliding window: n + W / C)
+ */
+int nats_role_scan(const uint8_t* roles, int64_t B, int64_t H_kv, int64_t S, int64_t W, int64_t C, int64_t* end_idx,
+                   int32_t* vis_lim, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * (a-3) debug / parity output: the token-level bool mask of a prefill from an empty cache, as
+ * NAtSChunkLayerCache.generate_mask builds it (components/cache/nats_chunk_layer_cache.py:589-620),
+ * evaluated with the same predicate the prefill kernels use.
+ *   vis_lim [B, H_kv, S] int32 from nats_role_scan, S = ceil(L / C)
+ *   mask    [B, H_kv, L, L] uint8 out (1 = attend)
+ */
+int nats_prefill_mask(const int32_t* vis_lim, int64_t B, int64_t H_kv, int64_t L, int64_t C, uint8_t* mask,
+                      void* stream);
+
+/* (a-3) debug / parity output: the block-sparse tile-skip map the prefill kernel walks.
+ *   tile_lim_ws  B * H_kv * T * 8 bytes of scratch, T = ceil(L / 64)
+ *   tiles        [B, H_kv, T, T] uint8 out: 1 = the 64x64 tile (query tile, key tile) is loaded
+ */
+int nats_prefill_tile_map(const int32_t* vis_lim, int64_t B, int64_t H_kv, int64_t L, int64_t C, void* tile_lim_ws,
+                          uint8_t* tiles, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * (a-4, a-5) role-masked chunked flash-attention prefill from an empty cache.
+ * Replaces nats_prefill(...) with global_kv_size=None (models/transformer/triton/nats_flashattn_fwd.py:617-692)
+ * and the generate_mask + SDPA branch of multi_head_attention
+ * (models/transformer/attention/nats_chunk_attention.py:130-149).
+ *   q [B, H_q, L, D], k / v [B, H_kv, L, D], o [B, H_q, L, D]; the last dimension is contiguous, the other
+ *   three strides are given in elements (stride_b, stride_h, stride_l)
+ *   roles [B, H_kv, S] uint8, S = ceil(L / C)
+ *   workspace: nats_prefill_workspace_bytes(...) bytes of device memory (contents need not be kept)
+ * D in {64, 128}; C a power of two in [1, 64] or a multiple of 64; W % C == 0; H_q % H_kv == 0.
+ * dtype bf16 runs QK^T and PV on bf16 MFMA with fp32 softmax state; dtype f32 runs an fp32 FMA kernel.
+ */
+size_t nats_prefill_workspace_bytes(int64_t B, int64_t H_q, int64_t H_kv, int64_t L, int64_t D, int64_t C);
+
+int nats_prefill_fwd(const void* q, const void* k, const void* v, const uint8_t* roles, void* o, int64_t B,
+                     int64_t H_q, int64_t H_kv, int64_t L, int64_t D, int64_t C, int64_t W, const int64_t* q_strides,
+                     const int64_t* k_strides, const int64_t* v_strides, const int64_t* o_strides, float sm_scale,
+                     int dtype, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * (a-8) one-token decode attention over the evicted, ragged cache.
+ * Replaces _generate_mask_one_step + SDPA (components/cache/nats_chunk_layer_cache.py:622-632,
+ * models/transformer/attention/nats_chunk_attention.py:131-142) and the flattened varlen call of
+ * models/transformer/hf/llama.py:274-295.
+ *   q [B, H_q, D] contiguous (one query token), o [B, H_q, D] contiguous
+ *   cache_k / cache_v [B, H_kv, >= n_rows, D], last dimension contiguous, strides (stride_b, stride_h, stride_row)
+ *   valid [B, H_kv, >= n_rows] uint8 (the cache's valid_tokens), strides (stride_b, stride_h), rows contiguous
+ *   n_rows = n_ctx_data + 1: rows [0, n_rows) with valid != 0 take part; rows with valid == 0 are never loaded
+ *   workspace: nats_decode_workspace_bytes(...) bytes
+ * D in {64, 128}; dtype bf16 or f32 (f32 converts on load).
+ */
+size_t nats_decode_workspace_bytes(int64_t B, int64_t H_q, int64_t H_kv, int64_t D, int64_t n_rows);
+
+int nats_decode_fwd(const void* q, const void* cache_k, const void* cache_v, const uint8_t* valid, void* o, int64_t B,
+                    int64_t H_q, int64_t H_kv, int64_t D, int64_t n_rows, const int64_t* kv_strides,
+                    const int64_t* valid_strides, float sm_scale, int dtype, void* workspace, size_t workspace_bytes,
+                    void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * (a-7) KV eviction + compaction: NAtSChunkLayerCache._post_update from its ring insert to its
+ * valid_tokens rewrite (components/cache/nats_chunk_layer_cache.py:270-371, 391-437, 634-656, 715-868)
+ * with merge_local_to_global_caches (components/cache/cache_update.py:25-76).
+ *
+ * Host-side facts travel in nats_evict_params, device-side results come back in nats_evict_result
+ * (device memory, 64 bytes, written by the call; copy it to the host when the numbers are needed).
+ */
+typedef struct {
+  int64_t B, H_kv, D;
+  int64_t C, W;
+  int64_t S;           /* role slots handed to the last update (one per chunk touched, open chunk included) */
+  int64_t x_len;       /* tokens appended by the last update */
+  int64_t fill;        /* chunk_fill_size after that update (old open-chunk tokens + x_len), >= C */
+  int64_t n_ctx_data;  /* before this call */
+  int64_t gmin;        /* _n_global_min before this call */
+  int64_t tail;        /* sliding_queue_tail before this call */
+  int64_t first;       /* 1 if these are the first tokens the layer has seen (_seen_tokens == x_len) */
+  int64_t n_alloc;     /* rows allocated in cache_k / cache_v / valid (in place) or in the new cache (out of place) */
+} nats_evict_params;
+
+typedef struct {
+  int64_t n_ctx_data;  /* after the call */
+  int64_t gmin;        /* min over (b, h) of size_global after the call */
+  int64_t all_sw;      /* 1: every slot was sliding-window, only n_ctx_data and the ring changed */
+  int64_t all_local;   /* 1: every slot was local, nothing was moved */
+  int64_t max_keep;    /* largest number of kept chunks over (b, h) */
+  int64_t max_end;     /* largest (kept + destination base) over (b, h), in chunks */
+  int64_t moved_rows;  /* rows copied by the compaction (both tensors counted once), for bandwidth accounting */
+  int64_t reserved;
+} nats_evict_result;
+
+size_t nats_evict_workspace_bytes(int64_t B, int64_t H_kv, int64_t S);
+
+/* Step 1, always: roles -> per-head plan in `workspace`, new sizes and the scalars in `result`.
+ *   size_global / size_local [B, H_kv] int64, read here, rewritten by the apply step
+ */
+int nats_evict_plan(const uint8_t* roles, const int64_t* size_global, const int64_t* size_local,
+                    const nats_evict_params* params, void* workspace, size_t workspace_bytes, nats_evict_result* result,
+                    void* stream);
+
+/* Step 2a, in place: ring insert, ordered chunk moves (all sources of a batch are read before any of its
+ * destinations is written, which equals the reference's gather-clone-then-scatter), zero fill of rows
+ * >= n_ctx_data, valid_tokens rewrite, size update.
+ *   cache_k / cache_v [B, H_kv, n_alloc, D] same dtype (element size elem_bytes in {2, 4}), strides (b, h, row)
+ *   valid [B, H_kv, n_alloc] uint8 contiguous rows, strides (b, h)
+ *   pos   [B, H_kv, n_alloc] int32 optional shadow carrying the stream position of every row (-1 = none);
+ *         moved exactly like the rows, it is the surviving-token index map.  May be NULL.
+ */
+int nats_evict_apply_inplace(void* cache_k, void* cache_v, uint8_t* valid, int32_t* pos, const uint8_t* roles,
+                             int64_t* size_global, int64_t* size_local, const nats_evict_params* params,
+                             const int64_t* kv_strides, const int64_t* valid_strides, int elem_bytes,
+                             const void* workspace, const nats_evict_result* result, void* stream);
+
+/* Step 2b, first prefill, out of place: gathers straight from the raw K / V of the prefill
+ * ([B, H_kv, x_len, D], strides (b, h, row)) into a fresh cache of n_alloc rows, producing the same
+ * bytes the in-place sequence would leave in rows [0, n_alloc) of [W zeros | K | pad].
+ * Requires params->first == 1 and the cache to have been empty; n_alloc = ceil(result.n_ctx_data / C) * C
+ * reproduces the reference's truncation (components/cache/nats_chunk_layer_cache.py:373-380).
+ */
+int nats_evict_apply_first(const void* src_k, const void* src_v, void* cache_k, void* cache_v, uint8_t* valid,
+                           int32_t* pos, const uint8_t* roles, int64_t* size_global, int64_t* size_local,
+                           const nats_evict_params* params, const int64_t* src_strides, const int64_t* kv_strides,
+                           const int64_t* valid_strides, int elem_bytes, const void* workspace,
+                           const nats_evict_result* result, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NATS_HIP_H */

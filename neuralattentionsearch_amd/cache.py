@@ -1,0 +1,358 @@
+"""KV-cache objects of the NAtS inference path, backed by the HIP eviction / compaction kernels.
+
+Same class names, constructor arguments, methods and observable attributes as the reference's
+``NAtSCache`` (src/nats/components/cache/dyn_cache.py:66-195) and ``NAtSChunkLayerCache``
+(src/nats/components/cache/nats_chunk_layer_cache.py:15-906), so the attention modules and the HF
+monkey-patches can use them unchanged.  What differs is how the state is kept:
+
+* rows live in a capacity buffer that grows geometrically; ``cache_k`` / ``cache_v`` / ``valid_tokens`` are
+  views of the logical rows, whose number equals the reference's ``cache_k.shape[2]`` at every step;
+* the first prefill is not copied into ``[W zeros | K | pad]``: the raw K / V handed to ``update`` are kept
+  until ``post_update`` gathers the surviving rows straight into a right-sized cache;
+* ``post_update`` issues two kernels (plan, apply) and reads one 64-byte struct back, instead of the
+  reference's gather / scatter ops with six device-to-host synchronisations.
+"""
+from __future__ import annotations
+
+import math
+from enum import Enum
+from typing import Any
+
+import torch
+
+from . import ops
+
+
+class ChunkMergeType(Enum):
+    """src/nats/chunk_utils.py:65-67"""
+    MEAN = 0
+    MAX = 1
+
+
+def get_pad_size(x_len: int, chunk_size: int) -> int:
+    """src/nats/chunk_utils.py:9-10"""
+    return (-x_len) % chunk_size
+
+
+def pool_chunks(x: torch.Tensor, chunk_size: int, pad_size: int, method: ChunkMergeType) -> torch.Tensor:
+    """[B, L, dim] -> [B, ceil(L / C), dim]: per-chunk mean (zero padded, divided by C) or max
+    (src/nats/chunk_utils.py:13-62)."""
+    if pad_size:
+        x = torch.nn.functional.pad(x, (0, 0, 0, pad_size))
+    x = x.unflatten(-2, (-1, chunk_size))
+    return x.mean(-2) if method == ChunkMergeType.MEAN else x.max(-2)[0]
+
+
+class NAtSChunkLayerCache:
+    """One layer's cache with chunk-granular roles.  Row layout of cache_k[b, h] between forward calls:
+
+        [0, W)                        ring of the last W tokens of completed chunks (zero rows unless sliding window)
+        [W, size_global)              global chunks, stream order
+        [size_global, +size_local)    local chunks newer than the last global chunk
+        [.., max over heads)          stale rows of shorter heads (valid_tokens == False)
+        [base, base + chunk_fill)     the open chunk, same offset for every head
+        [n_ctx_data, ..)              zeros
+    """
+
+    def __init__(self, bsz: int, n_msks: int, sliding_window_size: int, layer_id: int = 0, chunk_size: int = 16,
+                 device: torch.device | str = "cuda", track_positions: bool = False):
+        device = torch.device(device)
+        if device.type != "cuda":
+            raise ValueError("NAtSChunkLayerCache keeps its state on the GPU; pass a cuda device")
+        if sliding_window_size % chunk_size != 0:  # nats_chunk_layer_cache.py:47
+            raise ValueError("sliding_window_size must be a multiple of chunk_size")
+        self.layer_id = layer_id
+        self.bsz = bsz
+        self.n_msks = n_msks
+        self.chunk_size = chunk_size
+        self.sliding_window_size = sliding_window_size
+        self.n_chunks_per_sw = sliding_window_size // chunk_size
+        self.device = device
+        self.track_positions = track_positions
+        self.size_local_kv = torch.zeros(bsz, n_msks, device=device, dtype=torch.long)
+        self.size_global_kv = torch.full([bsz, n_msks], sliding_window_size, device=device, dtype=torch.long)
+        self.reset_cache()
+
+    # -- state ----------------------------------------------------------------------------------
+    def reset_cache(self):
+        self.size_local_kv.zero_()
+        self.size_global_kv.fill_(self.sliding_window_size)
+        self.sliding_queue_tail = 0
+        self.chunk_fill_size = 0
+        self.chunk_fill_size_last = 0
+        self.n_ctx_data = self.sliding_window_size
+        self._n_global_min = self.sliding_window_size
+        self._seen_tokens = 0
+        self._tokens_info = None
+        self._roles = None
+        self._buf_k = self._buf_v = self._buf_valid = self._buf_pos = None
+        self._rows = 0
+        self._pending = None  # raw (K, V) of a first prefill not yet compacted
+        self.last_evict_result = None
+
+    def get_seq_length(self):
+        return self._seen_tokens
+
+    def get_chunk_fill_size(self):
+        return self.chunk_fill_size
+
+    @property
+    def cache_k(self):
+        self._materialize_pending()
+        return None if self._buf_k is None else self._buf_k[:, :, :self._rows]
+
+    @property
+    def cache_v(self):
+        self._materialize_pending()
+        return None if self._buf_v is None else self._buf_v[:, :, :self._rows]
+
+    @property
+    def valid_tokens(self):
+        self._materialize_pending()
+        return None if self._buf_valid is None else self._buf_valid[:, :, :self._rows].view(torch.bool)
+
+    @property
+    def token_positions(self):
+        """int32 [B, H, rows]: stream position of the token each row holds (-1 = none); needs track_positions."""
+        self._materialize_pending()
+        return None if self._buf_pos is None else self._buf_pos[:, :, :self._rows]
+
+    # -- storage --------------------------------------------------------------------------------
+    def _allocate(self, rows: int, like: torch.Tensor, capacity: int | None = None):
+        B, H, D = like.shape[0], like.shape[1], like.shape[3]
+        cap = max(rows, capacity or 0)
+        self._buf_k = torch.zeros(B, H, cap, D, dtype=like.dtype, device=like.device)
+        self._buf_v = torch.zeros(B, H, cap, D, dtype=like.dtype, device=like.device)
+        self._buf_valid = torch.zeros(B, H, cap, dtype=torch.uint8, device=like.device)
+        self._buf_pos = (torch.full((B, H, cap), -1, dtype=torch.int32, device=like.device)
+                         if self.track_positions else None)
+        self._rows = rows
+
+    def _grow(self, rows: int):
+        cap = self._buf_k.shape[2]
+        if rows > cap:
+            new_cap = max(rows, cap + max(cap // 2, 4 * self.chunk_size))
+            new_cap = math.ceil(new_cap / self.chunk_size) * self.chunk_size
+
+            def widen(t, fill):
+                shape = list(t.shape)
+                shape[2] = new_cap
+                n = torch.full(shape, fill, dtype=t.dtype, device=t.device)
+                n[:, :, :cap] = t
+                return n
+
+            self._buf_k = widen(self._buf_k, 0)
+            self._buf_v = widen(self._buf_v, 0)
+            self._buf_valid = widen(self._buf_valid, 0)
+            if self._buf_pos is not None:
+                self._buf_pos = widen(self._buf_pos, -1)
+        self._rows = max(self._rows, rows)
+
+    def _materialize_pending(self):
+        """Writes [W zeros | K | pad] (nats_chunk_layer_cache.py:215-236) if the first prefill is still raw."""
+        if self._pending is None:
+            return
+        k, v = self._pending
+        self._pending = None
+        W, x_len = self.sliding_window_size, k.shape[2]
+        rows = W + x_len + get_pad_size(x_len, self.chunk_size)
+        self._allocate(rows, k)
+        self._buf_k[:, :, W:W + x_len] = k
+        self._buf_v[:, :, W:W + x_len] = v
+        self._buf_valid[:, :, W:W + x_len] = 1
+        if self._buf_pos is not None:
+            self._buf_pos[:, :, W:W + x_len] = torch.arange(x_len, dtype=torch.int32, device=k.device)
+
+    # -- append (nats_chunk_layer_cache.py:171-256) ----------------------------------------------
+    def update(self, key_states: torch.Tensor, value_states: torch.Tensor, token_states_info: torch.Tensor | None):
+        if not key_states.is_cuda:
+            raise ValueError("NAtSChunkLayerCache.update takes GPU tensors")
+        x_len = key_states.shape[2]
+        self.chunk_fill_size += x_len
+        if token_states_info is None:
+            assert self.chunk_fill_size < self.chunk_size, \
+                "a new token_states_info must be generated once the open chunk is full"
+        if x_len == 0:
+            return self.cache_k[:, :, :self.n_ctx_data], self.cache_v[:, :, :self.n_ctx_data]
+        self._tokens_info = token_states_info
+        self._roles = None if token_states_info is None else ops.roles_from_one_hot(token_states_info).contiguous()
+        if self._buf_k is None and self._pending is None:
+            self._pending = (key_states, value_states)
+            if self.chunk_fill_size < self.chunk_size:
+                self._materialize_pending()  # nothing will be evicted by the coming post_update
+            return key_states, value_states
+        self._materialize_pending()
+        start = self.n_ctx_data
+        end = start + x_len
+        self._grow(math.ceil(end / self.chunk_size) * self.chunk_size)
+        self._buf_k[:, :, start:end] = key_states.to(self._buf_k.dtype)
+        self._buf_v[:, :, start:end] = value_states.to(self._buf_v.dtype)
+        self._buf_valid[:, :, start:end] = 1
+        if self._buf_pos is not None:
+            self._buf_pos[:, :, start:end] = torch.arange(self._seen_tokens, self._seen_tokens + x_len,
+                                                          dtype=torch.int32, device=self.device)
+        return self._buf_k[:, :, :end], self._buf_v[:, :, :end]
+
+    # -- masks (nats_chunk_layer_cache.py:156-163, 444-460, 622-632) ------------------------------
+    def generate_mask(self, x_len: int):
+        """Debug / parity output; the attention kernels never call it."""
+        if x_len == 1:
+            if self._seen_tokens == 0:
+                return torch.ones(1, 1, 1, 1, dtype=torch.bool, device=self.device)
+            return self.valid_tokens[:, :, :self.n_ctx_data + 1].unsqueeze(-2)
+        if self._seen_tokens == 0:
+            if self._roles is None:
+                raise ValueError("generate_mask needs the roles handed to update")
+            return ops.prefill_mask(self._roles, x_len, self.chunk_size, self.sliding_window_size)
+        raise NotImplementedError("masks of a multi-token segment over an existing cache are not built yet")
+
+    # -- evict + compact (nats_chunk_layer_cache.py:258-389) -------------------------------------
+    def post_update(self, x_len: int):
+        C, W = self.chunk_size, self.sliding_window_size
+        self._seen_tokens += x_len
+        if x_len == 0 or self.chunk_fill_size < C:
+            self.chunk_fill_size_last = self.chunk_fill_size
+            self.n_ctx_data += x_len
+            return
+        fill = self.chunk_fill_size
+        partial, n_done = fill % C, fill // C
+        first = self._seen_tokens == x_len
+        roles = self._roles
+        if roles is None:
+            raise ValueError("post_update needs the roles handed to the update that completed a chunk")
+        S = roles.shape[-1]
+        src = self._pending
+        like = src[0] if src is not None else self._buf_k
+        D = like.shape[3]
+        params = ops.evict_params(self.bsz, self.n_msks, D, C, W, S, x_len, fill, self.n_ctx_data, self._n_global_min,
+                                  self.sliding_queue_tail, first, max(self._rows, C))
+        ws, result = ops.evict_plan(roles, self.size_global_kv, self.size_local_kv, params)
+        if src is not None:
+            res = ops.read_result(result)
+            if res.all_sw:  # the reference keeps the untruncated cache here (:283-288)
+                self._materialize_pending()
+                src = None
+            else:
+                rows = math.ceil(res.n_ctx_data / C) * C
+                self._pending = None
+                self._allocate(rows, like)
+                params.n_alloc = rows
+                k_raw, v_raw = src
+                if k_raw.stride(-1) != 1 or k_raw.stride() != v_raw.stride():
+                    k_raw, v_raw = k_raw.contiguous(), v_raw.contiguous()
+                ops.evict_apply_first(k_raw, v_raw, self._buf_k, self._buf_v, self._buf_valid, self._buf_pos, roles,
+                                      self.size_global_kv, self.size_local_kv, params, ws, result)
+        if src is None:
+            params.n_alloc = self._rows
+            ops.evict_apply_inplace(self._buf_k, self._buf_v, self._buf_valid, self._buf_pos, roles, self.size_global_kv,
+                                    self.size_local_kv, params, ws, result)
+            res = ops.read_result(result)
+        # host-side bookkeeping (nats_chunk_layer_cache.py:400-413, 280-288, 358, 371-380)
+        n_ring = min(n_done, self.n_chunks_per_sw)
+        start = 0 if first else self.sliding_queue_tail
+        self.sliding_queue_tail = (start + n_ring * C) % W
+        self.chunk_fill_size = partial
+        self.chunk_fill_size_last = partial
+        self.n_ctx_data = int(res.n_ctx_data)
+        self.last_evict_result = res
+        if res.all_sw:
+            return
+        self._n_global_min = int(res.gmin)
+        if first:
+            self._rows = math.ceil(self.n_ctx_data / C) * C
+
+
+class NAtSCache:
+    """Container of per-layer caches (src/nats/components/cache/dyn_cache.py:66-195)."""
+
+    def __init__(self, sliding_window_size: int, chunk_size: int = 1, track_positions: bool = False):
+        if chunk_size == 1:
+            raise NotImplementedError("the per-token cache (chunk_size == 1) is not built; use chunk_size > 1")
+        self.cache_model: list[NAtSChunkLayerCache] = []
+        self.sliding_window_size = sliding_window_size
+        self.chunk_size = chunk_size
+        self.cached_x: list[torch.Tensor | None] = []
+        self.track_positions = track_positions
+
+    def reset_cache(self):
+        self.cache_model = []
+        self.cached_x = []
+
+    def get_seq_length(self, layer_idx: int = 0) -> int:
+        if len(self.cache_model) <= layer_idx:
+            return 0
+        return self.cache_model[layer_idx]._seen_tokens
+
+    def generate_mask(self, layer_idx: int, x_len: int):
+        return self.cache_model[layer_idx].generate_mask(x_len)
+
+    def get_nats_chunk_fill_size(self, layer_idx: int = 0):
+        if len(self.cache_model) <= layer_idx or self.chunk_size == 1:
+            return 0
+        return self.cache_model[layer_idx].chunk_fill_size
+
+    def get_nats_cached_x_in_chunk(self, layer_idx: int = 0):
+        if len(self.cached_x) <= layer_idx:
+            return None
+        return self.cached_x[layer_idx]
+
+    @staticmethod
+    def merge_new_x_values_in_chunk(x_cache, x_new, chunk_size: int, chunk_merge_method=ChunkMergeType.MEAN):
+        """Running chunk statistic of the hidden states (dyn_cache.py:98-115): sum of x / C, or max."""
+        if chunk_merge_method == ChunkMergeType.MEAN:
+            add = (x_new / chunk_size).sum(1, keepdim=True)
+            return add if x_cache is None else x_cache + add
+        if x_cache is None:
+            return x_new
+        return torch.max(torch.cat([x_cache, x_new], dim=1), dim=1, keepdim=True)[0]
+
+    def _update_cache_x(self, x_update, layer_idx: int):
+        if len(self.cached_x) <= layer_idx:
+            self.cached_x.append(x_update)
+        else:
+            self.cached_x[layer_idx] = x_update
+
+    def update_nats_cached_x_in_chunk(self, x, layer_idx: int = 0, chunk_merge_method=ChunkMergeType.MEAN):
+        """dyn_cache.py:117-124"""
+        x_cache = self.get_nats_cached_x_in_chunk(layer_idx)
+        self._update_cache_x(self.merge_new_x_values_in_chunk(x_cache, x, self.chunk_size, chunk_merge_method), layer_idx)
+
+    def update_nats_cached_x_across_chunk(self, x, pre_fill_chunk_size: int, layer_idx: int = 0,
+                                          chunk_merge_method=ChunkMergeType.MEAN):
+        """Pooled hidden states of every chunk the new tokens touch, and the pad of the last one
+        (dyn_cache.py:130-171)."""
+        C = self.chunk_size
+        pre = self.get_nats_chunk_fill_size(layer_idx)
+        x_len = x.shape[1]
+        if pre != 0:
+            head_len = C - pre
+            head = self.merge_new_x_values_in_chunk(self.get_nats_cached_x_in_chunk(layer_idx), x[:, :head_len], C,
+                                                    chunk_merge_method)
+            rest = x_len - head_len
+            if rest == 0:
+                pad, pooled = 0, head
+            else:
+                pad = get_pad_size(rest, C)
+                pooled = torch.cat([head, pool_chunks(x[:, head_len:], C, pad, chunk_merge_method)], dim=1)
+        else:
+            pad = get_pad_size(x_len, C)
+            pooled = pool_chunks(x, C, pad, chunk_merge_method)
+        if pad == 0:
+            carry = None
+        else:
+            tail = x[:, pad - C:]
+            carry = (tail / C).sum(1, keepdim=True) if chunk_merge_method == ChunkMergeType.MEAN \
+                else tail.max(1, keepdim=True)[0]
+        self._update_cache_x(carry, layer_idx)
+        return pooled, pad
+
+    def update(self, key_states, value_states, layer_idx: int, cache_kwargs: dict[str, Any] | None = None):
+        if len(self.cache_model) <= layer_idx:
+            bsz, n_kv_heads = key_states.shape[:2]
+            self.cache_model.append(NAtSChunkLayerCache(bsz, n_kv_heads, self.sliding_window_size, layer_id=layer_idx,
+                                                        chunk_size=self.chunk_size, device=key_states.device,
+                                                        track_positions=self.track_positions))
+        return self.cache_model[layer_idx].update(key_states, value_states, **(cache_kwargs or {}))
+
+    def post_update(self, layer_idx: int, x_len=1, **kwargs):
+        self.cache_model[layer_idx].post_update(x_len=x_len)

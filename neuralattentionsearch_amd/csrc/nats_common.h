@@ -1,0 +1,61 @@
+// Shared helpers of the gfx950 NAtS kernels: error reporting, argument checks, small device utilities.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "nats_hip.h"
+
+namespace nats {
+
+// thread-local text behind nats_last_error()
+char* error_buffer();
+int fail(int code, const char* fmt, ...);
+
+#define NATS_REQUIRE(cond, code, ...)           \
+  do {                                          \
+    if (!(cond)) return ::nats::fail((code), __VA_ARGS__); \
+  } while (0)
+
+#define NATS_CHECK_LAUNCH(what)                                                              \
+  do {                                                                                       \
+    hipError_t e__ = hipGetLastError();                                                      \
+    if (e__ != hipSuccess) return ::nats::fail(NATS_ERR_LAUNCH, "%s: %s", (what), hipGetErrorString(e__)); \
+  } while (0)
+
+inline bool is_pow2(int64_t x) { return x > 0 && (x & (x - 1)) == 0; }
+inline int ilog2(int64_t x) {
+  int r = 0;
+  while ((int64_t(1) << r) < x) ++r;
+  return r;
+}
+
+constexpr int kWave = 64;
+constexpr int kTile = 64;  // prefill tile edge (queries and keys)
+constexpr int32_t kLimGlobal = 0x7fffffff;
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ int lane_id() { return threadIdx.x & (kWave - 1); }
+
+// bf16 <-> f32 with round-to-nearest-even, bit exact with torch's conversion for finite values
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) { return __uint_as_float(uint32_t(b) << 16); }
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return uint16_t((u >> 16) | 0x40u);  // quiet NaN
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return uint16_t(u >> 16);
+}
+
+// Orders LDS traffic between the lanes of one wavefront (no workgroup barrier needed for wave-private LDS).
+__device__ __forceinline__ void wave_lds_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+}
+
+}  // namespace nats

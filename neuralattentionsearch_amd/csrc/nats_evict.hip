@@ -1,0 +1,581 @@
+// KV eviction + compaction of the chunked NAtS layer cache (HBM-bound byte moves, bit exact).
+//
+// Follows NAtSChunkLayerCache._post_update (components/cache/nats_chunk_layer_cache.py:270-371), its
+// helpers move_sliding_window_tokens_to_head (:391-437), get_updated_cache_info (:715-868),
+// mask_invalid_tokens (:634-656) and merge_local_to_global_caches (components/cache/cache_update.py:25-76).
+//
+// plan kernel  : one workgroup; a wavefront per (b, kv head) walks the role slots 64 at a time, a ballot
+//                marks the kept slots (globals + locals after the last global) and a prefix popcount gives
+//                each kept slot its destination rank (stream compaction of slot ids).
+// apply kernels: move chunk-granular row blocks.  In place, a workgroup owns one row slice of every chunk
+//                of one (b, kv head, tensor) and processes the ordered move list in batches, reading a
+//                whole batch before writing it; because destinations never pass sources this equals
+//                gather-everything-then-scatter.  Out of place (first prefill) every destination chunk is
+//                produced independently straight from the raw K / V of the prefill.
+#include "nats_common.h"
+
+namespace nats {
+
+struct HeadPlan {
+  int32_t count;     // kept chunks (general path) or 1 (single completed chunk)
+  int32_t dst_base;  // destination of the first kept chunk, in chunks
+  int64_t sg_new;
+  int64_t sl_new;
+  int64_t pad;
+};
+
+constexpr size_t kPlanHeaderBytes = 256;
+
+__host__ __device__ inline size_t plan_lists_offset(int64_t n_heads) {
+  return (kPlanHeaderBytes + (size_t)n_heads * sizeof(HeadPlan) + 255) & ~size_t(255);
+}
+
+// ---------------------------------------------------------------------------------------------------
+// plan
+// ---------------------------------------------------------------------------------------------------
+struct WaveAgg {
+  int all_sw, all_local;
+  int max_keep, max_end;
+  long long max_tot_new, max_tot_old, max_tot_alllocal, min_sg_new, sum_keep;
+};
+
+__global__ __launch_bounds__(1024) void evict_plan_kernel(const uint8_t* __restrict__ roles,
+                                                          const int64_t* __restrict__ size_global,
+                                                          const int64_t* __restrict__ size_local, nats_evict_params p,
+                                                          char* __restrict__ ws, nats_evict_result* __restrict__ result) {
+  __shared__ WaveAgg agg[16];
+  __shared__ int all_local_flag;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int n_heads = (int)(p.B * p.H_kv);
+  const int S = (int)p.S;
+  const int C = (int)p.C;
+  const int partial = (int)(p.fill % p.C);
+  const int n_done = (int)(p.fill / p.C);
+  const int S_eff = S - (partial ? 1 : 0);
+  HeadPlan* plans = reinterpret_cast<HeadPlan*>(ws + kPlanHeaderBytes);
+  int32_t* lists = reinterpret_cast<int32_t*>(ws + plan_lists_offset(n_heads));
+
+  WaveAgg w;
+  w.all_sw = 1; w.all_local = 1; w.max_keep = 0; w.max_end = 0;
+  w.max_tot_new = 0; w.max_tot_old = 0; w.max_tot_alllocal = 0; w.min_sg_new = 0x7fffffffffffffffLL; w.sum_keep = 0;
+
+  for (int head = wave; head < n_heads; head += 16) {
+    const uint8_t* r = roles + (int64_t)head * S;
+    const long long sg = size_global[head], sl = size_local[head];
+    int32_t* keep = lists + (int64_t)head * S;
+    HeadPlan hp;
+    int head_all_sw, head_all_local;
+    if (p.x_len == 1) {
+      // one completed chunk is scattered for every head (:289-330)
+      int r0 = r[0], rl = r[S - 1];
+      bool is_g = r0 == NATS_ROLE_GLOBAL;
+      long long dst = is_g ? sg : sg + sl;
+      long long dec = (is_g ? sl / C + 1 : 0) + (rl == NATS_ROLE_SW ? 1 : 0);
+      hp.count = 1;
+      hp.dst_base = (int32_t)(dst / C);
+      hp.sg_new = sg + (is_g ? C : 0);
+      hp.sl_new = sl - dec * C + (long long)n_done * C;
+      if (lane == 0) keep[0] = 0;
+      int n_sw = 0;
+      for (int s = 0; s < S; ++s) n_sw += r[s] == NATS_ROLE_SW;
+      head_all_sw = n_sw == S;
+      head_all_local = 0;
+    } else {
+      // pass 1: counts and the last complete global slot
+      int n_glob_all = 0, n_sw = 0, n_loc = 0, last_g = -1;
+      for (int base = 0; base < S; base += kWave) {
+        int s = base + lane;
+        int role = s < S ? r[s] : 255;
+        uint64_t bg = __ballot(role == NATS_ROLE_GLOBAL);
+        uint64_t bge = __ballot(role == NATS_ROLE_GLOBAL && s < S_eff);
+        n_glob_all += __builtin_popcountll(bg);
+        n_sw += __builtin_popcountll(__ballot(role == NATS_ROLE_SW));
+        n_loc += __builtin_popcountll(__ballot(role == NATS_ROLE_LOCAL));
+        if (bge) last_g = base + 63 - __builtin_clzll(bge);
+      }
+      // pass 2: kept slots in order, destination rank by prefix popcount
+      int count = 0, later_local = 0;
+      for (int base = 0; base < S; base += kWave) {
+        int s = base + lane;
+        int role = s < S ? r[s] : 255;
+        bool loc_after = role == NATS_ROLE_LOCAL && s > last_g;
+        bool kept = s < S_eff && (role == NATS_ROLE_GLOBAL || loc_after);
+        uint64_t bk = __ballot(kept);
+        later_local += __builtin_popcountll(__ballot(loc_after));
+        if (kept) {
+          int rank = count + __builtin_popcountll(bk & ((uint64_t(1) << lane) - 1));
+          keep[rank] = s;
+        }
+        count += __builtin_popcountll(bk);
+      }
+      int n_glob = n_glob_all - (partial ? 1 : 0);                                     // :782-786
+      long long n_other = (long long)S - (last_g > 0 ? last_g : 0) - later_local - (partial ? 1 : 0);  // :797-800
+      long long dec_l = (last_g > -1 ? (long long)last_g * C + sl : 0) + n_other * C;  // :793, :802
+      hp.count = count;
+      hp.dst_base = (int32_t)((last_g == -1 ? sg + sl : sg) / C);                      // :827-828
+      hp.sg_new = sg + (long long)n_glob * C;
+      hp.sl_new = sl - dec_l + (long long)n_done * C;
+      head_all_sw = n_sw == S;
+      head_all_local = n_loc == S;
+    }
+    hp.pad = 0;
+    if (lane == 0) plans[head] = hp;
+    w.all_sw &= head_all_sw;
+    w.all_local &= head_all_local;
+    w.max_keep = max(w.max_keep, hp.count);
+    w.max_end = max(w.max_end, hp.count + hp.dst_base);
+    w.max_tot_new = max(w.max_tot_new, (long long)(hp.sg_new + hp.sl_new));
+    w.max_tot_old = max(w.max_tot_old, sg + sl);
+    w.max_tot_alllocal = max(w.max_tot_alllocal, sg + sl + (long long)n_done * C);
+    w.min_sg_new = min(w.min_sg_new, (long long)hp.sg_new);
+    w.sum_keep += hp.count;
+  }
+  if (lane == 0) agg[wave] = w;
+  __syncthreads();
+  if (tid == 0) {
+    WaveAgg t = agg[0];
+    for (int i = 1; i < 16; ++i) {
+      t.all_sw &= agg[i].all_sw;
+      t.all_local &= agg[i].all_local;
+      t.max_keep = max(t.max_keep, agg[i].max_keep);
+      t.max_end = max(t.max_end, agg[i].max_end);
+      t.max_tot_new = max(t.max_tot_new, agg[i].max_tot_new);
+      t.max_tot_old = max(t.max_tot_old, agg[i].max_tot_old);
+      t.max_tot_alllocal = max(t.max_tot_alllocal, agg[i].max_tot_alllocal);
+      t.min_sg_new = min(t.min_sg_new, agg[i].min_sg_new);
+      t.sum_keep += agg[i].sum_keep;
+    }
+    nats_evict_result res;
+    res.all_sw = t.all_sw;
+    res.all_local = (p.x_len != 1) && t.all_local && !t.all_sw;
+    res.max_keep = t.max_keep;
+    res.max_end = t.max_end;
+    res.reserved = 0;
+    if (res.all_sw) {  // :283-288
+      res.n_ctx_data = t.max_tot_old + partial;
+      res.gmin = p.gmin;
+      res.moved_rows = 0;
+    } else if (res.all_local) {  // :747-749, then :356-358
+      res.n_ctx_data = t.max_tot_alllocal + partial;
+      res.gmin = p.gmin;
+      res.moved_rows = 0;
+    } else {
+      res.n_ctx_data = t.max_tot_new + partial;
+      res.gmin = t.min_sg_new;
+      bool tail_move = p.x_len != 1 && partial && t.max_keep < S - 1;  // :840
+      res.moved_rows = (t.sum_keep + (tail_move ? n_heads : 0)) * (long long)C;
+    }
+    if (res.all_local) {
+      long long mn = 0x7fffffffffffffffLL;
+      for (int h = 0; h < n_heads; ++h) mn = min(mn, (long long)size_global[h]);
+      res.gmin = mn;
+    }
+    *result = res;
+    all_local_flag = (int)res.all_local;
+  }
+  __syncthreads();
+  if (all_local_flag) {
+    // every slot local: nothing moves and only the local size grows (:747-749, :356)
+    for (int h = tid; h < n_heads; h += 1024) {
+      plans[h].sg_new = size_global[h];
+      plans[h].sl_new = size_local[h] + (long long)n_done * C;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// movers
+// ---------------------------------------------------------------------------------------------------
+struct ApplyArgs {
+  void* tensor[3];       // cache_k, cache_v, pos (pos may be NULL)
+  const void* src[2];    // raw K, V of the prefill (out-of-place only)
+  uint8_t* valid;
+  const uint8_t* roles;
+  int64_t* size_global;
+  int64_t* size_local;
+  const char* ws;
+  const nats_evict_result* result;
+  nats_evict_params p;
+  int64_t ks_b, ks_h, ks_r;  // cache strides in elements
+  int64_t ss_b, ss_h, ss_r;  // raw K / V strides in elements (out-of-place only)
+  int64_t vs_b, vs_h;        // valid strides; pos uses the same (contiguous rows)
+  int elem_bytes;
+  int rs;                    // rows per slice
+  int n_slices;
+};
+
+// A tensor seen as units of type U: row `r` of head `head` starts at base + r * row_stride, holds upr units.
+template <typename U>
+struct TensorView {
+  U* base;
+  int64_t row_stride;
+  int upr;
+};
+
+constexpr int kUnr = 4;  // moves per wavefront and batch
+constexpr int kNu = 2;   // units per lane and chunk slice (a slice holds at most 128 units)
+
+template <typename U>
+__device__ __forceinline__ U zero_unit();
+template <>
+__device__ __forceinline__ uint4 zero_unit<uint4>() { return make_uint4(0, 0, 0, 0); }
+template <>
+__device__ __forceinline__ int32_t zero_unit<int32_t>() { return -1; }  // "no token" in the position shadow
+
+template <typename U>
+__device__ void apply_inplace_body(const ApplyArgs& a, TensorView<U> t, int head, int slice, bool owns_valid) {
+  const nats_evict_params& p = a.p;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int C = (int)p.C, S = (int)p.S;
+  const int partial = (int)(p.fill % p.C);
+  const int n_done = (int)(p.fill / p.C);
+  const int wc = (int)(p.W / p.C);
+  const int64_t off = p.n_ctx_data / p.C;
+  const int n_heads = (int)(p.B * p.H_kv);
+  const nats_evict_result res = *a.result;
+  const HeadPlan hp = reinterpret_cast<const HeadPlan*>(a.ws + kPlanHeaderBytes)[head];
+  const int32_t* keep = reinterpret_cast<const int32_t*>(a.ws + plan_lists_offset(n_heads)) + (int64_t)head * S;
+  const uint8_t* r = a.roles + (int64_t)head * S;
+  const int units = a.rs * t.upr;  // per chunk slice
+  const int row0 = slice * a.rs;
+
+  auto unit_ptr = [&](int64_t chunk, int u) -> U* {
+    return t.base + (chunk * C + row0 + u / t.upr) * t.row_stride + (u % t.upr);
+  };
+
+  // 1. ring insert (:391-437)
+  const int n_ring = n_done < wc ? n_done : wc;
+  const int start_chunk = p.first ? 0 : (int)(p.tail / p.C);
+  for (int j = wave; j < n_ring; j += 4) {
+    int slot = n_done - n_ring + j;
+    bool is_sw = r[slot] == NATS_ROLE_SW;
+    int rc = (start_chunk + j) % wc;
+    for (int u = lane; u < units; u += kWave) {
+      U val = is_sw ? *unit_ptr(off + slot, u) : zero_unit<U>();
+      *unit_ptr(rc, u) = val;
+    }
+    if (owns_valid && lane < a.rs) {
+      a.valid[(int64_t)(head / p.H_kv) * a.vs_b + (int64_t)(head % p.H_kv) * a.vs_h + (int64_t)rc * C + row0 + lane] = is_sw;
+    }
+  }
+  if (res.all_sw) return;
+  __syncthreads();
+
+  // 2. ordered chunk moves, each batch read completely before it is written
+  int n_moves;
+  bool tail_move = false;
+  if (p.x_len == 1) {
+    n_moves = 1;
+  } else if (res.all_local) {
+    n_moves = 0;
+  } else {
+    tail_move = partial && res.max_keep < S - 1;
+    n_moves = hp.count + (tail_move ? 1 : 0);
+  }
+  for (int b0 = 0; b0 < n_moves; b0 += 4 * kUnr) {
+    U regs[kUnr][kNu];
+    int64_t dsts[kUnr];
+#pragma unroll
+    for (int k = 0; k < kUnr; ++k) {
+      int mv = b0 + wave * kUnr + k;
+      dsts[k] = -1;
+      if (mv < n_moves) {
+        int64_t src, dst;
+        if (mv < hp.count) {
+          src = off + keep[mv];
+          dst = hp.dst_base + mv;
+        } else {
+          src = off + S - 1;
+          dst = res.max_end;
+        }
+        if (src != dst) {
+          dsts[k] = dst;
+#pragma unroll
+          for (int e = 0; e < kNu; ++e) {
+            int u = lane + e * kWave;
+            if (u < units) regs[k][e] = *unit_ptr(src, u);
+          }
+        }
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < kUnr; ++k) {
+      if (dsts[k] >= 0) {
+#pragma unroll
+        for (int e = 0; e < kNu; ++e) {
+          int u = lane + e * kWave;
+          if (u < units) *unit_ptr(dsts[k], u) = regs[k][e];
+        }
+      }
+    }
+  }
+  __syncthreads();
+
+  // 3. rows >= n_ctx_data are zeroed (:360-362)
+  const int64_t n_chunks_alloc = p.n_alloc / C;
+  for (int64_t ci = res.n_ctx_data / C + wave; ci < n_chunks_alloc; ci += 4) {
+    for (int u = lane; u < units; u += kWave) {
+      int64_t row = ci * C + row0 + u / t.upr;
+      if (row >= res.n_ctx_data) *unit_ptr(ci, u) = zero_unit<U>();
+    }
+  }
+
+  if (owns_valid) {
+    // 4. valid_tokens rewrite with the minimum global size from before this call (:634-656)
+    const long long sg_new = hp.sg_new, sl_new = hp.sl_new;
+    if (res.n_ctx_data != p.gmin) {
+      uint8_t* vrow = a.valid + (int64_t)(head / p.H_kv) * a.vs_b + (int64_t)(head % p.H_kv) * a.vs_h;
+      const int64_t last_chunk = res.n_ctx_data / C * C;
+      const int64_t hi = last_chunk + partial;
+      for (int64_t i = p.gmin + slice * 256 + tid; i < hi; i += (int64_t)a.n_slices * 256) {
+        vrow[i] = i < last_chunk ? (i < sg_new + sl_new) : 1;
+      }
+    }
+    if (slice == 0 && tid == 0) {
+      a.size_global[head] = sg_new;
+      a.size_local[head] = sl_new;
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void evict_apply_inplace_kernel(ApplyArgs a) {
+  const int slice = blockIdx.x;
+  const int head = blockIdx.y;
+  const int which = blockIdx.z;
+  const int b = head / (int)a.p.H_kv, h = head % (int)a.p.H_kv;
+  if (which < 2) {
+    TensorView<uint4> t;
+    int row_units = (int)(a.p.D * a.elem_bytes / 16);
+    t.base = reinterpret_cast<uint4*>(static_cast<char*>(a.tensor[which]) + (b * a.ks_b + h * a.ks_h) * a.elem_bytes);
+    t.row_stride = a.ks_r * a.elem_bytes / 16;
+    t.upr = row_units;
+    apply_inplace_body<uint4>(a, t, head, slice, which == 0);
+  } else {
+    TensorView<int32_t> t;
+    t.base = static_cast<int32_t*>(a.tensor[2]) + b * a.vs_b + h * a.vs_h;
+    t.row_stride = 1;
+    t.upr = 1;
+    apply_inplace_body<int32_t>(a, t, head, slice, false);
+  }
+}
+
+// Out of place, first prefill: destination chunk blockIdx.x of head blockIdx.y.
+__global__ __launch_bounds__(256) void evict_apply_first_kernel(ApplyArgs a) {
+  const nats_evict_params& p = a.p;
+  const int tid = threadIdx.x;
+  const int64_t ci = blockIdx.x;
+  const int head = blockIdx.y;
+  const int which = blockIdx.z;
+  const int b = head / (int)p.H_kv, h = head % (int)p.H_kv;
+  const int C = (int)p.C, S = (int)p.S;
+  const int partial = (int)(p.fill % p.C);
+  const int n_done = (int)(p.fill / p.C);
+  const int wc = (int)(p.W / p.C);
+  const int64_t L = p.x_len;
+  const int n_heads = (int)(p.B * p.H_kv);
+  const nats_evict_result res = *a.result;
+  if (res.all_sw) return;  // the reference leaves the untruncated cache in this case; not handled out of place
+  const HeadPlan hp = reinterpret_cast<const HeadPlan*>(a.ws + kPlanHeaderBytes)[head];
+  const int32_t* keep = reinterpret_cast<const int32_t*>(a.ws + plan_lists_offset(n_heads)) + (int64_t)head * S;
+  const uint8_t* r = a.roles + (int64_t)head * S;
+  const int n_ring = n_done < wc ? n_done : wc;
+  const int count = res.all_local ? 0 : hp.count;
+  const bool tail_move = !res.all_local && partial && res.max_keep < S - 1;
+
+  // where the rows of this destination chunk come from: a source chunk of the raw prefill tensor
+  // (-1 = zeros); the untouched part of [W zeros | K | pad] keeps its own rows
+  int64_t src_chunk;
+  if (ci < wc) {
+    src_chunk = -1;
+    if (ci < n_ring) {
+      int slot = n_done - n_ring + (int)ci;
+      if (r[slot] == NATS_ROLE_SW) src_chunk = slot;
+    }
+  } else {
+    int64_t rel = ci - hp.dst_base;
+    if (rel >= 0 && rel < count) {
+      src_chunk = keep[rel];
+    } else if (tail_move && ci == res.max_end) {
+      src_chunk = S - 1;
+    } else {
+      src_chunk = ci - wc;
+    }
+  }
+
+  const long long sg_new = hp.sg_new, sl_new = hp.sl_new;
+
+  if (which < 2) {
+    const int upr = (int)(p.D * a.elem_bytes / 16);
+    uint4* dst = reinterpret_cast<uint4*>(static_cast<char*>(a.tensor[which]) + (b * a.ks_b + h * a.ks_h) * a.elem_bytes);
+    const uint4* src =
+        reinterpret_cast<const uint4*>(static_cast<const char*>(a.src[which]) + (b * a.ss_b + h * a.ss_h) * a.elem_bytes);
+    const int64_t d_stride = a.ks_r * a.elem_bytes / 16, s_stride = a.ss_r * a.elem_bytes / 16;
+    for (int u = tid; u < C * upr; u += 256) {
+      int row = u / upr, col = u % upr;
+      int64_t drow = ci * C + row;
+      int64_t tok = src_chunk < 0 ? -1 : src_chunk * C + row;
+      uint4 val = make_uint4(0, 0, 0, 0);
+      if (tok >= 0 && tok < L && drow < res.n_ctx_data) val = src[tok * s_stride + col];
+      dst[drow * d_stride + col] = val;
+    }
+  } else {
+    int32_t* dst = static_cast<int32_t*>(a.tensor[2]) + b * a.vs_b + h * a.vs_h;
+    for (int row = tid; row < C; row += 256) {
+      int64_t drow = ci * C + row;
+      int64_t tok = src_chunk < 0 ? -1 : src_chunk * C + row;
+      dst[drow] = (tok >= 0 && tok < L && drow < res.n_ctx_data) ? (int32_t)tok : -1;
+    }
+  }
+
+  if (which == 0) {
+    uint8_t* vrow = a.valid + (int64_t)b * a.vs_b + (int64_t)h * a.vs_h;
+    const int64_t last_chunk = res.n_ctx_data / C * C;
+    for (int row = tid; row < C; row += 256) {
+      int64_t i = ci * C + row;
+      uint8_t v;
+      if (i < p.W) {
+        v = (ci < n_ring && src_chunk >= 0) ? 1 : 0;
+      } else {
+        v = (i - p.W) < L ? 1 : 0;  // what update() left behind (:229-236)
+        if (res.n_ctx_data != p.gmin && i >= p.gmin) {
+          if (i < last_chunk) {
+            v = i < sg_new + sl_new;
+          } else if (i < last_chunk + partial) {
+            v = 1;
+          }
+        }
+      }
+      vrow[i] = v;
+    }
+    if (ci == 0 && tid == 0) {
+      a.size_global[head] = sg_new;
+      a.size_local[head] = sl_new;
+    }
+  }
+}
+
+static int check_params(const char* who, const nats_evict_params* p) {
+  NATS_REQUIRE(p, NATS_ERR_NULL_POINTER, "%s: params must not be NULL", who);
+  NATS_REQUIRE(p->B > 0 && p->H_kv > 0 && p->D > 0 && p->S > 0, NATS_ERR_BAD_SHAPE, "%s: B=%lld H_kv=%lld D=%lld S=%lld", who,
+               (long long)p->B, (long long)p->H_kv, (long long)p->D, (long long)p->S);
+  NATS_REQUIRE(p->C > 0 && p->W > 0 && p->W % p->C == 0, NATS_ERR_BAD_SHAPE,
+               "%s: window %lld is not a positive multiple of chunk size %lld", who, (long long)p->W, (long long)p->C);
+  NATS_REQUIRE(p->x_len > 0 && p->fill >= p->C && p->fill >= p->x_len, NATS_ERR_BAD_SHAPE,
+               "%s: x_len=%lld fill=%lld: no chunk completed, nothing to evict", who, (long long)p->x_len, (long long)p->fill);
+  int64_t n_done = p->fill / p->C, partial = p->fill % p->C;
+  NATS_REQUIRE(p->S == n_done + (partial ? 1 : 0), NATS_ERR_BAD_SHAPE, "%s: S=%lld role slots for fill=%lld, chunk %lld", who,
+               (long long)p->S, (long long)p->fill, (long long)p->C);
+  NATS_REQUIRE(p->x_len != 1 || p->S == 1, NATS_ERR_BAD_SHAPE, "%s: a one-token step completes exactly one chunk", who);
+  NATS_REQUIRE(p->n_ctx_data >= p->W && p->gmin >= p->W && p->tail >= 0 && p->tail < p->W && p->tail % p->C == 0,
+               NATS_ERR_BAD_SHAPE, "%s: n_ctx_data=%lld gmin=%lld tail=%lld", who, (long long)p->n_ctx_data,
+               (long long)p->gmin, (long long)p->tail);
+  NATS_REQUIRE(p->B * p->H_kv <= 65535, NATS_ERR_BAD_SHAPE, "%s: too many (b, head) streams", who);
+  return NATS_OK;
+}
+
+}  // namespace nats
+
+using namespace nats;
+
+extern "C" size_t nats_evict_workspace_bytes(int64_t B, int64_t H_kv, int64_t S) {
+  if (B <= 0 || H_kv <= 0 || S <= 0) return 0;
+  return plan_lists_offset(B * H_kv) + (size_t)(B * H_kv * S) * sizeof(int32_t);
+}
+
+extern "C" int nats_evict_plan(const uint8_t* roles, const int64_t* size_global, const int64_t* size_local,
+                               const nats_evict_params* params, void* workspace, size_t workspace_bytes,
+                               nats_evict_result* result, void* stream) {
+  NATS_REQUIRE(roles && size_global && size_local && workspace && result, NATS_ERR_NULL_POINTER,
+               "nats_evict_plan: NULL pointer argument");
+  if (int rc = check_params("nats_evict_plan", params)) return rc;
+  size_t need = nats_evict_workspace_bytes(params->B, params->H_kv, params->S);
+  NATS_REQUIRE(workspace_bytes >= need, NATS_ERR_WORKSPACE, "nats_evict_plan: workspace %zu bytes < %zu", workspace_bytes, need);
+  hipLaunchKernelGGL(evict_plan_kernel, dim3(1), dim3(1024), 0, static_cast<hipStream_t>(stream), roles, size_global,
+                     size_local, *params, static_cast<char*>(workspace), result);
+  NATS_CHECK_LAUNCH("evict_plan_kernel");
+  return NATS_OK;
+}
+
+static int slice_geometry(const char* who, const nats_evict_params* p, int elem_bytes, int* rs, int* n_slices) {
+  NATS_REQUIRE(elem_bytes == 2 || elem_bytes == 4, NATS_ERR_BAD_DTYPE, "%s: element size %d", who, elem_bytes);
+  int64_t row_bytes = p->D * elem_bytes;
+  NATS_REQUIRE(row_bytes % 16 == 0 && row_bytes <= 2048, NATS_ERR_UNSUPPORTED, "%s: row of %lld bytes", who,
+               (long long)row_bytes);
+  int64_t r = 1;
+  while (r * 2 <= p->C && r * 2 * row_bytes <= 2048 && p->C % (r * 2) == 0) r *= 2;
+  NATS_REQUIRE(p->C % r == 0, NATS_ERR_UNSUPPORTED, "%s: chunk size %lld", who, (long long)p->C);
+  if (r > 128) r = 128;  // the position shadow moves one 4-byte unit per row
+  *rs = (int)r;
+  *n_slices = (int)(p->C / r);
+  return NATS_OK;
+}
+
+extern "C" int nats_evict_apply_inplace(void* cache_k, void* cache_v, uint8_t* valid, int32_t* pos, const uint8_t* roles,
+                                        int64_t* size_global, int64_t* size_local, const nats_evict_params* params,
+                                        const int64_t* kv_strides, const int64_t* valid_strides, int elem_bytes,
+                                        const void* workspace, const nats_evict_result* result, void* stream) {
+  NATS_REQUIRE(cache_k && cache_v && valid && roles && size_global && size_local && workspace && result,
+               NATS_ERR_NULL_POINTER, "nats_evict_apply_inplace: NULL pointer argument");
+  NATS_REQUIRE(kv_strides && valid_strides, NATS_ERR_NULL_POINTER, "nats_evict_apply_inplace: NULL stride array");
+  if (int rc = check_params("nats_evict_apply_inplace", params)) return rc;
+  NATS_REQUIRE(params->n_alloc % params->C == 0 && params->n_alloc >= params->n_ctx_data - (params->fill - params->x_len) + params->fill,
+               NATS_ERR_BAD_SHAPE, "nats_evict_apply_inplace: n_alloc=%lld", (long long)params->n_alloc);
+  ApplyArgs a;
+  if (int rc = slice_geometry("nats_evict_apply_inplace", params, elem_bytes, &a.rs, &a.n_slices)) return rc;
+  NATS_REQUIRE((kv_strides[0] * elem_bytes) % 16 == 0 && (kv_strides[1] * elem_bytes) % 16 == 0 &&
+                   (kv_strides[2] * elem_bytes) % 16 == 0 &&
+                   (reinterpret_cast<uintptr_t>(cache_k) | reinterpret_cast<uintptr_t>(cache_v)) % 16 == 0,
+               NATS_ERR_BAD_SHAPE, "nats_evict_apply_inplace: cache rows must be 16-byte aligned");
+  a.tensor[0] = cache_k; a.tensor[1] = cache_v; a.tensor[2] = pos;
+  a.src[0] = a.src[1] = nullptr;
+  a.valid = valid; a.roles = roles; a.size_global = size_global; a.size_local = size_local;
+  a.ws = static_cast<const char*>(workspace); a.result = result; a.p = *params;
+  a.ks_b = kv_strides[0]; a.ks_h = kv_strides[1]; a.ks_r = kv_strides[2];
+  a.ss_b = a.ss_h = a.ss_r = 0;
+  a.vs_b = valid_strides[0]; a.vs_h = valid_strides[1];
+  a.elem_bytes = elem_bytes;
+  dim3 grid((unsigned)a.n_slices, (unsigned)(params->B * params->H_kv), pos ? 3u : 2u);
+  hipLaunchKernelGGL(evict_apply_inplace_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream), a);
+  NATS_CHECK_LAUNCH("evict_apply_inplace_kernel");
+  return NATS_OK;
+}
+
+extern "C" int nats_evict_apply_first(const void* src_k, const void* src_v, void* cache_k, void* cache_v, uint8_t* valid,
+                                      int32_t* pos, const uint8_t* roles, int64_t* size_global, int64_t* size_local,
+                                      const nats_evict_params* params, const int64_t* src_strides, const int64_t* kv_strides,
+                                      const int64_t* valid_strides, int elem_bytes, const void* workspace,
+                                      const nats_evict_result* result, void* stream) {
+  NATS_REQUIRE(src_k && src_v && cache_k && cache_v && valid && roles && size_global && size_local && workspace && result,
+               NATS_ERR_NULL_POINTER, "nats_evict_apply_first: NULL pointer argument");
+  NATS_REQUIRE(src_strides && kv_strides && valid_strides, NATS_ERR_NULL_POINTER, "nats_evict_apply_first: NULL stride array");
+  if (int rc = check_params("nats_evict_apply_first", params)) return rc;
+  NATS_REQUIRE(params->first == 1 && params->x_len > 1 && params->fill == params->x_len && params->n_ctx_data == params->W &&
+                   params->gmin == params->W,
+               NATS_ERR_BAD_SHAPE, "nats_evict_apply_first: only the first update of an empty cache can be applied out of place");
+  NATS_REQUIRE(params->n_alloc % params->C == 0 && params->n_alloc > 0 && params->n_alloc / params->C <= 0x7fffffff,
+               NATS_ERR_BAD_SHAPE, "nats_evict_apply_first: n_alloc=%lld", (long long)params->n_alloc);
+  NATS_REQUIRE(elem_bytes == 2 || elem_bytes == 4, NATS_ERR_BAD_DTYPE, "nats_evict_apply_first: element size %d", elem_bytes);
+  NATS_REQUIRE((params->D * elem_bytes) % 16 == 0, NATS_ERR_UNSUPPORTED, "nats_evict_apply_first: row of %lld bytes",
+               (long long)(params->D * elem_bytes));
+  for (int i = 0; i < 3; ++i) {
+    NATS_REQUIRE((src_strides[i] * elem_bytes) % 16 == 0 && (kv_strides[i] * elem_bytes) % 16 == 0, NATS_ERR_BAD_SHAPE,
+                 "nats_evict_apply_first: rows must be 16-byte aligned");
+  }
+  NATS_REQUIRE((reinterpret_cast<uintptr_t>(cache_k) | reinterpret_cast<uintptr_t>(cache_v) |
+                reinterpret_cast<uintptr_t>(src_k) | reinterpret_cast<uintptr_t>(src_v)) % 16 == 0,
+               NATS_ERR_BAD_SHAPE, "nats_evict_apply_first: tensors must be 16-byte aligned");
+  ApplyArgs a;
+  a.tensor[0] = cache_k; a.tensor[1] = cache_v; a.tensor[2] = pos;
+  a.src[0] = src_k; a.src[1] = src_v;
+  a.valid = valid; a.roles = roles; a.size_global = size_global; a.size_local = size_local;
+  a.ws = static_cast<const char*>(workspace); a.result = result; a.p = *params;
+  a.ks_b = kv_strides[0]; a.ks_h = kv_strides[1]; a.ks_r = kv_strides[2];
+  a.ss_b = src_strides[0]; a.ss_h = src_strides[1]; a.ss_r = src_strides[2];
+  a.vs_b = valid_strides[0]; a.vs_h = valid_strides[1];
+  a.elem_bytes = elem_bytes; a.rs = 0; a.n_slices = 0;
+  dim3 grid((unsigned)(params->n_alloc / params->C), (unsigned)(params->B * params->H_kv), pos ? 3u : 2u);
+  hipLaunchKernelGGL(evict_apply_first_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream), a);
+  NATS_CHECK_LAUNCH("evict_apply_first_kernel");
+  return NATS_OK;
+}

@@ -1,0 +1,268 @@
+"""Torch-tensor front end of the C ABI: the operator level of the NAtS inference path.
+
+Every function takes CUDA (ROCm) tensors, passes raw pointers / strides / the current stream to
+libnats_hip.so and returns tensors.  Nothing here computes on the CPU and nothing falls back to PyTorch
+ops: CPU tensors are rejected.
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+
+import torch
+
+from . import _lib
+from ._lib import NATS_DTYPE_BF16, NATS_DTYPE_F32, EvictParams, EvictResult, check, i64_array
+
+ROLE_GLOBAL, ROLE_LOCAL, ROLE_SW = 0, 1, 2
+TILE = 64
+
+_workspaces: dict = {}
+
+
+def _stream(t: torch.Tensor):
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _ptr(t: torch.Tensor | None):
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _dtype_code(t: torch.Tensor) -> int:
+    if t.dtype == torch.bfloat16:
+        return NATS_DTYPE_BF16
+    if t.dtype == torch.float32:
+        return NATS_DTYPE_F32
+    raise ValueError(f"unsupported dtype {t.dtype}: the kernels take bfloat16 or float32")
+
+
+def _require_cuda(*ts):
+    for t in ts:
+        if t is not None and not t.is_cuda:
+            raise ValueError("the NAtS kernels run on the GPU only: got a CPU tensor")
+
+
+def workspace(device, key: str, nbytes: int) -> torch.Tensor:
+    """A per-(device, purpose) scratch buffer that only ever grows."""
+    k = (str(device), key)
+    buf = _workspaces.get(k)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+        _workspaces[k] = buf
+    return buf
+
+
+# ------------------------------------------------------------------------------------------------
+# roles
+# ------------------------------------------------------------------------------------------------
+def roles_from_logits(logits: torch.Tensor, global_bias: float = 0.1, force_first_global: bool = False,
+                      force_last_global: bool = False, with_one_hot: bool = True):
+    """logits [B, S, H_kv, 3] -> (roles uint8 [B, H_kv, S], token_states_info [B, H_kv, S, 3] or None).
+
+    models/transformer/attention/nats_attention.py:96-109."""
+    _require_cuda(logits)
+    lib = _lib.load()
+    if logits.dim() != 4 or logits.shape[-1] != 3:
+        raise ValueError(f"logits must be [B, S, H_kv, 3], got {tuple(logits.shape)}")
+    logits = logits.contiguous()
+    B, S, H, _ = logits.shape
+    roles = torch.empty(B, H, S, dtype=torch.uint8, device=logits.device)
+    one_hot = torch.empty(B, H, S, 3, dtype=logits.dtype, device=logits.device) if with_one_hot else None
+    check(lib.nats_roles_from_logits(_ptr(logits), _dtype_code(logits), B, S, H, float(global_bias),
+                                     int(force_first_global), int(force_last_global), _ptr(roles), _ptr(one_hot),
+                                     _stream(logits)))
+    return roles, one_hot
+
+
+def roles_from_one_hot(token_states_info: torch.Tensor) -> torch.Tensor:
+    """[B, H_kv, S, 3] one-hot float -> uint8 roles (index of the 1)."""
+    t = token_states_info
+    return (t[..., 1] > 0).to(torch.uint8) + 2 * (t[..., 2] > 0).to(torch.uint8)
+
+
+def role_scan(roles: torch.Tensor, W: int, C: int):
+    """roles [B, H_kv, S] -> (end_idx int64, vis_lim int32), both [B, H_kv, S].
+
+    components/masks/utils.py:85-87."""
+    _require_cuda(roles)
+    lib = _lib.load()
+    roles = roles.contiguous()
+    B, H, S = roles.shape
+    end_idx = torch.empty(B, H, S, dtype=torch.int64, device=roles.device)
+    vis_lim = torch.empty(B, H, S, dtype=torch.int32, device=roles.device)
+    check(lib.nats_role_scan(_ptr(roles), B, H, S, W, C, _ptr(end_idx), _ptr(vis_lim), _stream(roles)))
+    return end_idx, vis_lim
+
+
+def prefill_mask(roles: torch.Tensor, L: int, C: int, W: int) -> torch.Tensor:
+    """Bool [B, H_kv, L, L]: the mask NAtSChunkLayerCache.generate_mask returns for a prefill from empty."""
+    lib = _lib.load()
+    _, vis_lim = role_scan(roles, W, C)
+    B, H, _ = roles.shape
+    mask = torch.empty(B, H, L, L, dtype=torch.uint8, device=roles.device)
+    check(lib.nats_prefill_mask(_ptr(vis_lim), B, H, L, C, _ptr(mask), _stream(roles)))
+    return mask.bool()
+
+
+def prefill_tile_map(roles: torch.Tensor, L: int, C: int, W: int) -> torch.Tensor:
+    """Bool [B, H_kv, T, T], T = ceil(L / 64): the 64x64 tiles the prefill kernel loads."""
+    lib = _lib.load()
+    _, vis_lim = role_scan(roles, W, C)
+    B, H, _ = roles.shape
+    T = (L + TILE - 1) // TILE
+    scratch = torch.empty(B * H * T * 8, dtype=torch.uint8, device=roles.device)
+    tiles = torch.empty(B, H, T, T, dtype=torch.uint8, device=roles.device)
+    check(lib.nats_prefill_tile_map(_ptr(vis_lim), B, H, L, C, _ptr(scratch), _ptr(tiles), _stream(roles)))
+    return tiles.bool()
+
+
+# ------------------------------------------------------------------------------------------------
+# prefill
+# ------------------------------------------------------------------------------------------------
+def prefill_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, roles: torch.Tensor, chunk_size: int,
+                      window: int, sm_scale: float | None = None, out: torch.Tensor | None = None) -> torch.Tensor:
+    """Role-masked causal attention of a prefill from an empty cache.
+
+    q [B, H_q, L, D], k / v [B, H_kv, L, D] (any strides with a contiguous last dimension), roles uint8
+    [B, H_kv, ceil(L / chunk_size)].  Returns [B, H_q, L, D] (or fills `out`, which may be strided)."""
+    _require_cuda(q, k, v, roles)
+    lib = _lib.load()
+    if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
+        raise ValueError("q, k, v must be [B, H, L, D]")
+    B, Hq, L, D = q.shape
+    Hkv = k.shape[1]
+    if k.shape != (B, Hkv, L, D) or v.shape != (B, Hkv, L, D):
+        raise ValueError(f"shape mismatch: q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)}")
+    if not (q.dtype == k.dtype == v.dtype):
+        raise ValueError("q, k, v must share one dtype")
+    S = math.ceil(L / chunk_size)
+    if tuple(roles.shape) != (B, Hkv, S) or roles.dtype != torch.uint8:
+        raise ValueError(f"roles must be uint8 [B, H_kv, {S}], got {roles.dtype} {tuple(roles.shape)}")
+    q, k, v = (t if t.stride(-1) == 1 else t.contiguous() for t in (q, k, v))
+    roles = roles.contiguous()
+    if out is None:
+        out = torch.empty(B, Hq, L, D, dtype=q.dtype, device=q.device)
+    elif out.shape != q.shape or out.dtype != q.dtype or out.stride(-1) != 1:
+        raise ValueError("out must match q in shape and dtype and have a contiguous last dimension")
+    scale = (1.0 / math.sqrt(D)) if sm_scale is None else float(sm_scale)
+    nbytes = lib.nats_prefill_workspace_bytes(B, Hq, Hkv, L, D, chunk_size)
+    ws = workspace(q.device, "prefill", nbytes)
+    check(lib.nats_prefill_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(roles), _ptr(out), B, Hq, Hkv, L, D, chunk_size, window,
+                               i64_array(q.stride()[:3]), i64_array(k.stride()[:3]), i64_array(v.stride()[:3]),
+                               i64_array(out.stride()[:3]), scale, _dtype_code(q), _ptr(ws), ws.numel(), _stream(q)))
+    return out
+
+
+def nats_prefill(q, k, v, end_seqs_idx, sliding_tokens, sm_scale, nats_chunk_size: int = 1, global_kv_size=None,
+                 local_kv_size=None, valid_sw_tokens=None, n_ctx_data=None, sw_token_tails=None, n_rep: int = 1,
+                 n_tokens_in_first_chunk: int = 0, local_seq_max_length: int = 4, return_masks: bool = False,
+                 block_n: int = 32):
+    """Drop-in for nats_prefill of models/transformer/triton/nats_flashattn_fwd.py:617-725 (same argument
+    names and meaning, returns (o, mask or None)).
+
+    end_seqs_idx [B, H_kv, S] int64 is the next-global index computed with the last slot forced global;
+    sliding_tokens [B, H_kv, S] is option 2 of token_states_info.  A slot is global iff
+    end_seqs_idx[n] == n (nats_flashattn_fwd.py:110)."""
+    if global_kv_size is not None:
+        raise NotImplementedError("prefill over an existing evicted cache (HAS_PAST_INFO) is not built yet")
+    if q.shape[1] // k.shape[1] != n_rep:
+        raise ValueError(f"n_rep={n_rep} does not match {q.shape[1]} q heads / {k.shape[1]} kv heads")
+    S = end_seqs_idx.shape[-1]
+    slots = torch.arange(S, device=end_seqs_idx.device)
+    is_global = end_seqs_idx == slots
+    is_sw = sliding_tokens > 0
+    roles = torch.where(is_global, ROLE_GLOBAL, torch.where(is_sw, ROLE_SW, ROLE_LOCAL)).to(torch.uint8)
+    o = prefill_attention(q, k, v, roles, nats_chunk_size, local_seq_max_length, sm_scale)
+    mask = prefill_mask(roles, q.shape[2], nats_chunk_size, local_seq_max_length) if return_masks else None
+    return o, mask
+
+
+# ------------------------------------------------------------------------------------------------
+# decode
+# ------------------------------------------------------------------------------------------------
+def decode_attention(q: torch.Tensor, cache_k: torch.Tensor, cache_v: torch.Tensor, valid: torch.Tensor, n_rows: int,
+                     sm_scale: float | None = None) -> torch.Tensor:
+    """One query token per sequence over the evicted cache.
+
+    q [B, H_q, 1, D]; cache_k / cache_v [B, H_kv, >= n_rows, D]; valid bool / uint8 [B, H_kv, >= n_rows].
+    Attends to rows i < n_rows with valid[b, h, i]; returns [B, H_q, 1, D]."""
+    _require_cuda(q, cache_k, cache_v, valid)
+    lib = _lib.load()
+    B, Hq, one, D = q.shape
+    if one != 1:
+        raise ValueError("decode_attention takes exactly one query token per sequence")
+    Hkv = cache_k.shape[1]
+    if cache_k.shape != cache_v.shape or cache_k.stride() != cache_v.stride():
+        raise ValueError("cache_k and cache_v must share shape and strides")
+    if cache_k.shape[2] < n_rows or valid.shape[2] < n_rows:
+        raise ValueError(f"n_rows={n_rows} exceeds the cache ({cache_k.shape[2]} rows) or valid ({valid.shape[2]})")
+    if cache_k.stride(-1) != 1 or valid.stride(-1) != 1:
+        raise ValueError("cache rows and valid rows must be contiguous")
+    if not (q.dtype == cache_k.dtype == cache_v.dtype):
+        raise ValueError("q and the cache must share one dtype")
+    if valid.dtype == torch.bool:
+        valid = valid.view(torch.uint8)
+    qc = q.reshape(B, Hq, D).contiguous()
+    out = torch.empty(B, Hq, D, dtype=q.dtype, device=q.device)
+    scale = (1.0 / math.sqrt(D)) if sm_scale is None else float(sm_scale)
+    nbytes = lib.nats_decode_workspace_bytes(B, Hq, Hkv, D, n_rows)
+    ws = workspace(q.device, "decode", nbytes)
+    check(lib.nats_decode_fwd(_ptr(qc), _ptr(cache_k), _ptr(cache_v), _ptr(valid), _ptr(out), B, Hq, Hkv, D, n_rows,
+                              i64_array(cache_k.stride()[:3]), i64_array(valid.stride()[:2]), scale, _dtype_code(q),
+                              _ptr(ws), ws.numel(), _stream(q)))
+    return out.view(B, Hq, 1, D)
+
+
+# ------------------------------------------------------------------------------------------------
+# eviction + compaction
+# ------------------------------------------------------------------------------------------------
+def evict_params(B, H_kv, D, C, W, S, x_len, fill, n_ctx_data, gmin, tail, first, n_alloc) -> EvictParams:
+    return EvictParams(B, H_kv, D, C, W, S, x_len, fill, n_ctx_data, gmin, tail, int(first), n_alloc)
+
+
+def evict_plan(roles: torch.Tensor, size_global: torch.Tensor, size_local: torch.Tensor, params: EvictParams):
+    """Returns (workspace, result): the per-head plan (device) and the 64-byte result struct (device int64[8])."""
+    _require_cuda(roles, size_global, size_local)
+    lib = _lib.load()
+    nbytes = lib.nats_evict_workspace_bytes(params.B, params.H_kv, params.S)
+    ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=roles.device)
+    result = torch.empty(8, dtype=torch.int64, device=roles.device)
+    check(lib.nats_evict_plan(_ptr(roles), _ptr(size_global), _ptr(size_local), ctypes.byref(params), _ptr(ws), ws.numel(),
+                              _ptr(result), _stream(roles)))
+    return ws, result
+
+
+def read_result(result: torch.Tensor) -> EvictResult:
+    """Copies the device result struct to the host (synchronises with the stream)."""
+    host = result.cpu().tolist()
+    return EvictResult(*host)
+
+
+def evict_apply_inplace(cache_k, cache_v, valid, pos, roles, size_global, size_local, params: EvictParams, ws, result):
+    _require_cuda(cache_k, cache_v, valid, roles)
+    lib = _lib.load()
+    if cache_k.stride() != cache_v.stride() or cache_k.dtype != cache_v.dtype:
+        raise ValueError("cache_k and cache_v must share dtype and strides")
+    v8 = valid.view(torch.uint8) if valid.dtype == torch.bool else valid
+    if pos is not None and (pos.dtype != torch.int32 or pos.stride()[:2] != v8.stride()[:2]):
+        raise ValueError("pos must be int32 with the strides of valid")
+    check(lib.nats_evict_apply_inplace(_ptr(cache_k), _ptr(cache_v), _ptr(v8), _ptr(pos), _ptr(roles), _ptr(size_global),
+                                       _ptr(size_local), ctypes.byref(params), i64_array(cache_k.stride()[:3]),
+                                       i64_array(v8.stride()[:2]), cache_k.element_size(), _ptr(ws), _ptr(result),
+                                       _stream(cache_k)))
+
+
+def evict_apply_first(src_k, src_v, cache_k, cache_v, valid, pos, roles, size_global, size_local, params: EvictParams,
+                      ws, result):
+    _require_cuda(src_k, src_v, cache_k, cache_v, valid, roles)
+    lib = _lib.load()
+    if src_k.stride() != src_v.stride() or cache_k.stride() != cache_v.stride():
+        raise ValueError("K and V must share strides")
+    v8 = valid.view(torch.uint8) if valid.dtype == torch.bool else valid
+    if pos is not None and (pos.dtype != torch.int32 or pos.stride()[:2] != v8.stride()[:2]):
+        raise ValueError("pos must be int32 with the strides of valid")
+    check(lib.nats_evict_apply_first(_ptr(src_k), _ptr(src_v), _ptr(cache_k), _ptr(cache_v), _ptr(v8), _ptr(pos),
+                                     _ptr(roles), _ptr(size_global), _ptr(size_local), ctypes.byref(params),
+                                     i64_array(src_k.stride()[:3]), i64_array(cache_k.stride()[:3]),
+                                     i64_array(v8.stride()[:2]), cache_k.element_size(), _ptr(ws), _ptr(result),
+                                     _stream(cache_k)))

@@ -51,7 +51,7 @@ def roles_from_logits(logits: torch.Tensor, global_bias: float = 0.1, force_firs
     is the first maximal option, slot 0 becomes global when the segment starts inside the sink chunk;
     attention/nats_chunk_attention.py:92-94: an open last chunk is marked global."""
     lg = logits.clone()
-    lg[..., 0] = lg[..., 0] + torch.tensor(global_bias, dtype=lg.dtype)
+    lg[..., 0] += global_bias  # python scalar: fp32 add, rounded back to the logits' dtype
     x = lg.float().numpy()
     B, S, H, _ = x.shape
     roles = np.zeros((B, H, S), dtype=np.uint8)

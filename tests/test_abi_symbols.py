@@ -1,0 +1,85 @@
+"""CPU checks of the C-ABI library: it loads, exports every symbol include/nats_hip.h declares, and its
+argument validation rejects bad calls before anything touches a GPU."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from neuralattentionsearch_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "nats_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(nats_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_and_binding_agree():
+    assert declared_symbols() == sorted(_lib.SIGNATURES)
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    for name in declared_symbols():
+        assert hasattr(lib, name), name
+    assert lib.nats_abi_version() == _lib.ABI_VERSION
+
+
+def test_struct_sizes_match_header():
+    assert ctypes.sizeof(_lib.EvictParams) == 13 * 8
+    assert ctypes.sizeof(_lib.EvictResult) == 64
+
+
+def test_null_pointer_is_rejected_without_a_gpu():
+    lib = _lib.load()
+    rc = lib.nats_role_scan(None, 1, 1, 4, 4, 2, None, None, None)
+    assert rc == -1
+    assert b"NULL" in lib.nats_last_error()
+    with pytest.raises(ValueError):
+        _lib.check(rc)
+
+
+def test_window_not_multiple_of_chunk_is_rejected():
+    lib = _lib.load()
+    fake = ctypes.c_void_p(16)  # never dereferenced: validation fails first
+    rc = lib.nats_role_scan(fake, 1, 1, 4, 6, 4, None, None, None)
+    assert rc == -2
+    rc = lib.nats_role_scan(fake, 1, 1, 4, 6, 3, None, None, None)
+    assert rc == -4  # chunk size must be a power of two
+    with pytest.raises(NotImplementedError):
+        _lib.check(rc)
+
+
+def test_prefill_rejects_bad_head_dim_and_small_workspace():
+    lib = _lib.load()
+    fake = ctypes.c_void_p(256)
+    st = _lib.i64_array([1, 1, 1])
+    rc = lib.nats_prefill_fwd(fake, fake, fake, fake, fake, 1, 4, 2, 128, 96, 64, 128, st, st, st, st, 1.0, 0, fake, 1 << 20,
+                              None)
+    assert rc == -4
+    rc = lib.nats_prefill_fwd(fake, fake, fake, fake, fake, 1, 4, 2, 128, 128, 64, 128, st, st, st, st, 1.0, 0, fake, 8, None)
+    assert rc == -5
+    rc = lib.nats_prefill_fwd(fake, fake, fake, fake, fake, 1, 5, 2, 128, 128, 64, 128, st, st, st, st, 1.0, 0, fake, 1 << 20,
+                              None)
+    assert rc == -2
+
+
+def test_evict_params_are_validated():
+    lib = _lib.load()
+    fake = ctypes.c_void_p(256)
+    p = _lib.EvictParams(1, 2, 128, 64, 96, 1, 64, 64, 96, 96, 0, 1, 256)  # W % C != 0
+    rc = lib.nats_evict_plan(fake, fake, fake, ctypes.byref(p), fake, 1 << 20, fake, None)
+    assert rc == -2
+    p = _lib.EvictParams(1, 2, 128, 64, 128, 3, 64, 64, 128, 128, 0, 1, 256)  # S inconsistent with fill
+    rc = lib.nats_evict_plan(fake, fake, fake, ctypes.byref(p), fake, 1 << 20, fake, None)
+    assert rc == -2
+
+
+def test_ops_reject_cpu_tensors():
+    import torch
+    from neuralattentionsearch_amd import ops
+    with pytest.raises(ValueError):
+        ops.role_scan(torch.zeros(1, 1, 4, dtype=torch.uint8), 4, 2)

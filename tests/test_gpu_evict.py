@@ -1,0 +1,171 @@
+"""GPU parity, bit exact: the HIP-backed NAtSChunkLayerCache against the oracle state machine
+(which tests/test_oracle_golden.py pins to vectors written by the reference cache)."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle.nats_oracle import ChunkCacheOracle, one_hot_roles
+from tests.golden_io import Golden
+from tests.gpu_util import say
+
+pytestmark = pytest.mark.gpu
+
+GOLD = Golden()
+
+
+def compare(hip, st, where):
+    assert hip.n_ctx_data == st.n_ctx_data, (where, "n_ctx_data", hip.n_ctx_data, st.n_ctx_data)
+    scal = [hip._n_global_min, hip.sliding_queue_tail, hip.chunk_fill_size, hip.chunk_fill_size_last, hip._seen_tokens]
+    assert scal == [st.gmin, st.tail, st.fill, st.fill_last, st.seen], (where, scal)
+    assert np.array_equal(hip.size_global_kv.cpu().numpy(), st.size_global), (where, "size_global")
+    assert np.array_equal(hip.size_local_kv.cpu().numpy(), st.size_local), (where, "size_local")
+    assert tuple(hip.valid_tokens.shape) == st.valid.shape, (where, "rows", tuple(hip.valid_tokens.shape), st.valid.shape)
+    assert np.array_equal(hip.valid_tokens.cpu().numpy(), st.valid), (where, "valid_tokens")
+    # every byte of the cache, stale rows and zero tail included
+    assert torch.equal(hip.cache_k.cpu().view(torch.int16 if hip.cache_k.element_size() == 2 else torch.int32),
+                       st.cache_k.view(torch.int16 if st.cache_k.element_size() == 2 else torch.int32)), (where, "cache_k")
+    assert torch.equal(hip.cache_v.cpu().view(torch.int16 if hip.cache_v.element_size() == 2 else torch.int32),
+                       st.cache_v.view(torch.int16 if st.cache_v.element_size() == 2 else torch.int32)), (where, "cache_v")
+    if hip.token_positions is not None:
+        assert np.array_equal(hip.token_positions.cpu().numpy().astype(np.int64), st.pos_k), (where, "index map")
+
+
+def drive(name, B, H, D, C, W, segs, dtype, seed, check_masks=True):
+    """segs: list of (x_len, roles uint8 [B, H, S])."""
+    from neuralattentionsearch_amd.cache import NAtSChunkLayerCache
+    hip = NAtSChunkLayerCache(B, H, W, chunk_size=C, device="cuda", track_positions=True)
+    st = ChunkCacheOracle(B=B, H=H, W=W, C=C)
+    g = torch.Generator().manual_seed(seed)
+    t_seen = 0
+    for oi, (x_len, roles) in enumerate(segs):
+        say("evict", name, "op", oi, "x_len", x_len, "S", roles.shape[-1])
+        k = torch.randn(B, H, x_len, D, generator=g).to(dtype)
+        v = torch.randn(B, H, x_len, D, generator=g).to(dtype)
+        tsi = one_hot_roles(roles, dtype=dtype)
+        ko, vo = st.update(k, v, roles)
+        kh, vh = hip.update(k.cuda(), v.cuda(), tsi.cuda())
+        assert torch.equal(kh.cpu().view(torch.int16 if dtype == torch.bfloat16 else torch.int32),
+                           ko.contiguous().view(torch.int16 if dtype == torch.bfloat16 else torch.int32)), (name, oi, "update K")
+        if check_masks and (x_len == 1 or t_seen == 0):
+            assert np.array_equal(hip.generate_mask(x_len).cpu().numpy(), st.generate_mask(x_len)), (name, oi, "mask")
+        st.post_update(x_len)
+        hip.post_update(x_len)
+        compare(hip, st, (name, oi, x_len))
+        t_seen += x_len
+    return hip, st
+
+
+@pytest.mark.parametrize("name", GOLD.scenario_names())
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_replay_reference_scenarios(name, dtype):
+    si, sc = GOLD.scenario(name)
+    segs = [(op["x_len"], GOLD.op(si, oi)["roles"]) for oi, op in enumerate(sc["ops"])]
+    drive(name, sc["B"], sc["H"], 8, sc["C"], sc["W"], segs, dtype, seed=si)
+
+
+def role_stream(rng, B, H, C, lens, p):
+    """Roles as the attention module would hand them over for a list of segment lengths."""
+    segs, fill, seen = [], 0, 0
+    for x_len in lens:
+        total = fill + x_len
+        if total < C:
+            roles = np.zeros((B, H, 1), dtype=np.uint8)
+            fill = total
+        else:
+            S = math.ceil(total / C)
+            roles = rng.choice(3, size=(B, H, S), p=p).astype(np.uint8)
+            if seen == 0:
+                roles[:, :, 0] = 0
+            if total % C:
+                roles[:, :, -1] = 0
+            fill = total % C
+        segs.append((x_len, roles))
+        seen += x_len
+    return segs
+
+
+@pytest.mark.parametrize("C,W,D,dtype", [(64, 256, 128, torch.bfloat16), (64, 128, 64, torch.float32),
+                                         (32, 256, 128, torch.bfloat16), (8, 16, 64, torch.bfloat16),
+                                         (16, 64, 128, torch.float32)])
+def test_prefill_then_decode_random(C, W, D, dtype):
+    rng = np.random.default_rng(C + W)
+    lens = [20 * C + 5] + [1] * (3 * C + 3)
+    drive(f"prefill_decode_C{C}", 2, 4, D, C, W, role_stream(rng, 2, 4, C, lens, (0.1, 0.2, 0.7)), dtype, seed=C)
+
+
+@pytest.mark.parametrize("C,W", [(64, 256), (16, 32)])
+def test_multi_segment_and_streaming_random(C, W):
+    rng = np.random.default_rng(C)
+    lens = [10 * C, 4 * C, C, C, 3 * C + 7, 2 * C - 7, 1, 1, 5 * C] + [C] * 6
+    drive(f"multiseg_C{C}", 2, 3, 128, C, W, role_stream(rng, 2, 3, C, lens, (0.15, 0.25, 0.6)), torch.bfloat16, seed=C,
+          check_masks=True)
+
+
+def test_surviving_index_map_semantics():
+    """Kept rows = globals in stream order, then locals newer than the last global; ring = sliding-window
+    chunks among the last W tokens (definition of the compacted layout, independent of the oracle)."""
+    C, W, B, H, D = 64, 256, 1, 2, 128
+    rng = np.random.default_rng(3)
+    S = 40
+    roles = rng.choice(3, size=(B, H, S), p=(0.1, 0.3, 0.6)).astype(np.uint8)
+    roles[:, :, 0] = 0
+    hip, st = drive("index_map", B, H, D, C, W, [(S * C, roles)], torch.bfloat16, seed=1)
+    pos = hip.token_positions.cpu().numpy()
+    valid = hip.valid_tokens.cpu().numpy()
+    for h in range(H):
+        r = roles[0, h]
+        glob = [s for s in range(S) if r[s] == 0]
+        last_g = glob[-1]
+        keep = glob + [s for s in range(S) if r[s] == 1 and s > last_g]
+        want = np.concatenate([np.arange(s * C, (s + 1) * C) for s in sorted(keep)])
+        got = pos[0, h, W:][valid[0, h, W:]]
+        assert np.array_equal(got, want)
+        ring_want = np.concatenate([np.arange(s * C, (s + 1) * C) if r[s] == 2 else np.full(C, -1)
+                                    for s in range(S - W // C, S)])
+        assert np.array_equal(pos[0, h, :W], ring_want)
+
+
+def test_cfg4_bulk_eviction_properties():
+    """B=16 x 8 kv heads x 65536 tokens x 128, bf16, window 512: too large for the oracle's loops, checked
+    through size-independent properties of the compacted layout."""
+    from neuralattentionsearch_amd.cache import NAtSChunkLayerCache
+    say("evict cfg4 bulk")
+    B, H, L, D, C, W = 16, 8, 65536, 128, 64, 512
+    S = L // C
+    rng = np.random.default_rng(0)
+    roles = rng.choice(3, size=(B, H, S), p=(0.10, 0.15, 0.75)).astype(np.uint8)
+    roles[:, :, 0] = 0
+    g = torch.Generator(device="cuda").manual_seed(0)
+    k = torch.randn(B, H, L, D, generator=g, device="cuda", dtype=torch.bfloat16)
+    v = torch.randn(B, H, L, D, generator=g, device="cuda", dtype=torch.bfloat16)
+    hip = NAtSChunkLayerCache(B, H, W, chunk_size=C, device="cuda", track_positions=True)
+    tsi = one_hot_roles(roles, dtype=torch.bfloat16).cuda()
+    hip.update(k, v, tsi)
+    hip.post_update(L)
+    is_g = roles == 0
+    n_glob = is_g.sum(-1)
+    last_g = S - 1 - np.argmax(is_g[:, :, ::-1], axis=-1)
+    later_loc = np.array([[(roles[b, h, last_g[b, h] + 1:] == 1).sum() for h in range(H)] for b in range(B)])
+    sg = hip.size_global_kv.cpu().numpy()
+    sl = hip.size_local_kv.cpu().numpy()
+    assert np.array_equal(sg, W + n_glob * C)
+    assert np.array_equal(sl, later_loc * C)
+    assert hip.n_ctx_data == int((sg + sl).max())
+    assert hip.cache_k.shape[2] == math.ceil(hip.n_ctx_data / C) * C
+    pos = hip.token_positions
+    valid = hip.valid_tokens
+    # every valid row holds exactly the K / V row of the token the index map names
+    for b in (0, 7, 15):
+        for h in (0, 3, 7):
+            idx = torch.nonzero(valid[b, h]).flatten()
+            p = pos[b, h, idx].long()
+            assert (p >= 0).all()
+            assert torch.equal(hip.cache_k[b, h, idx], k[b, h, p])
+            assert torch.equal(hip.cache_v[b, h, idx], v[b, h, p])
+            body = p[idx >= W]
+            assert (body[1:] > body[:-1]).all(), "kept rows must stay in stream order"
+            assert int(valid[b, h, W:].sum()) == int(sg[b, h] - W + sl[b, h])
+    assert int(valid.sum()) == int((sg - W + sl).sum() + (roles[:, :, S - W // C:] == 2).sum() * C)
+    assert not hip.cache_k[:, :, hip.n_ctx_data:].any()
