@@ -50,8 +50,10 @@ def roles_from_logits(logits: torch.Tensor, global_bias: float = 0.1, force_firs
     attention/nats_attention.py:96-109: the bias is added to option 0 in the logits' own dtype, the role
     is the first maximal option, slot 0 becomes global when the segment starts inside the sink chunk;
     attention/nats_chunk_attention.py:92-94: an open last chunk is marked global."""
+    # `logit[..., 0] += 0.1` on the device the module runs on: torch's GPU kernels add the Python scalar in
+    # fp32 and round the sum to the logits' dtype (its CPU kernel would round the scalar to bf16 first).
     lg = logits.clone()
-    lg[..., 0] += global_bias  # python scalar: fp32 add, rounded back to the logits' dtype
+    lg[..., 0] = (lg[..., 0].float() + torch.tensor(global_bias, dtype=torch.float32)).to(lg.dtype)
     x = lg.float().numpy()
     B, S, H, _ = x.shape
     roles = np.zeros((B, H, S), dtype=np.uint8)

@@ -28,6 +28,23 @@ def test_roles_from_logits_bit_exact(dtype, bias, first, last):
     assert np.array_equal(ops.roles_from_one_hot(one_hot).cpu().numpy(), want)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_roles_match_torch_ops_on_the_device(dtype):
+    """The reference's own statement, run by torch on the GPU: logit[..., 0] += 0.1; logit.max(-1)[1]."""
+    from neuralattentionsearch_amd import ops
+    say("roles vs torch on device", dtype)
+    g = torch.Generator().manual_seed(1)
+    logits = (torch.randn(4, 512, 8, 3, generator=g) * 0.2).to(dtype)
+    logits[0, :, :, 1] = logits[0, :, :, 0] + 0.1
+    dev = logits.cuda()
+    ref = dev.clone()
+    ref[..., 0] += 0.1
+    index = ref.max(-1, keepdim=True)[1]
+    want = index.squeeze(-1).transpose(1, 2).contiguous().to(torch.uint8)
+    roles, _ = ops.roles_from_logits(dev, 0.1, False, False)
+    assert torch.equal(roles, want)
+
+
 @pytest.mark.parametrize("S", [1, 7, 64, 65, 200, 1024])
 def test_role_scan_matches_next_global_index(S):
     from neuralattentionsearch_amd import ops
