@@ -254,7 +254,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--prefill-len", type=int, default=32768)
     ap.add_argument("--skip-cpu", action="store_true")
-    ap.add_argument("--only", choices=["prefill", "decode", "evict"], default=None)
+    ap.add_argument("--only", choices=["prefill", "decode", "evict", "copy"], default=None)
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures the one-GPU hot path; it does not run on more than one GPU (--gpus 1 only)",
@@ -263,6 +263,15 @@ def main():
     from neuralattentionsearch_amd import ops  # raises if the HIP library has not been built
 
     torch.cuda.set_device(0)
+    if args.only == "copy":
+        # a plain 1 GiB device copy: the known-size dispatch the FETCH_SIZE / WRITE_SIZE counters are scaled by
+        src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_bytes": 1 << 30}))
+        return
     res = {}
     if args.only in (None, "prefill"):
         res["prefill"] = bench_prefill(args, ops)

@@ -1,0 +1,82 @@
+"""GPU: the attention module + NAtSCache end to end (prefill, then decode steps with live eviction)
+against the oracle driven with the module's own projections and role logits."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import nats_oracle as orc
+from tests.gpu_util import say
+
+pytestmark = pytest.mark.gpu
+
+
+def rope_tables(B, start, n, D, device):
+    inv = 1.0 / (10000.0 ** (torch.arange(0, D, 2, device=device).float() / D))
+    t = torch.arange(start, start + n, device=device).float()
+    f = torch.outer(t, inv)
+    emb = torch.cat([f, f], dim=-1)
+    return emb.cos()[None].expand(B, -1, -1), emb.sin()[None].expand(B, -1, -1)
+
+
+@pytest.mark.parametrize("L,C,W,steps", [(100, 16, 32, 40), (64, 16, 32, 20), (5, 8, 16, 30)])
+def test_module_prefill_and_decode(L, C, W, steps):
+    from neuralattentionsearch_amd.attention import LlamaNAtSChunkAttentionLayer, apply_rotary_pos_emb
+    from neuralattentionsearch_amd.cache import NAtSCache
+    say("attention module", L, C, W, steps)
+    torch.manual_seed(0)
+    B, dim, Hq, Hkv = 2, 512, 8, 2
+    D = dim // Hq
+    mod = LlamaNAtSChunkAttentionLayer(dim=dim, n_heads=Hq, n_kv_heads=Hkv, layer_id=0, local_seq_max_length=W,
+                                       chunk_size=C).cuda().eval()
+    with torch.no_grad():
+        mod.proj_layer.weight.mul_(8.0)  # spread the role logits
+    logits_seen = []
+    mod.proj_layer.register_forward_hook(lambda m, i, o: logits_seen.append(o.detach().float().cpu()))
+    cache = NAtSCache(sliding_window_size=W, chunk_size=C)
+    st = orc.ChunkCacheOracle(B=B, H=Hkv, W=W, C=C)
+
+    def qkv(x, start):
+        n = x.shape[1]
+        q = mod.wq(x).view(B, n, Hq, D).transpose(1, 2)
+        k = mod.wk(x).view(B, n, Hkv, D).transpose(1, 2)
+        v = mod.wv(x).view(B, n, Hkv, D).transpose(1, 2)
+        cos, sin = rope_tables(B, start, n, D, x.device)
+        q, k = apply_rotary_pos_emb(q, k, cos, sin)
+        return q, k, v, (cos, sin)
+
+    fill, seen = 0, 0
+    with torch.no_grad():
+        for step in range(steps + 1):
+            n = L if step == 0 else 1
+            x = torch.randn(B, n, dim, device="cuda")
+            q, k, v, pos = qkv(x, seen)
+            logits_seen.clear()
+            out = mod(x, pos, None, start_pos=seen, cache=cache)
+            # oracle side, fed with the module's own logits
+            total = fill + n
+            if total < C:
+                roles = np.zeros((B, Hkv, 1), dtype=np.uint8)
+                assert not logits_seen
+                fill = total
+            else:
+                lg = logits_seen[0].unflatten(-1, (Hkv, 3))
+                roles = orc.roles_from_logits(lg, 0.1, force_first_global=seen < C, force_last_global=total % C != 0)
+                assert roles.shape[-1] == math.ceil(total / C)
+                fill = total % C
+            ko, vo = st.update(k.cpu(), v.cpu(), roles)
+            if seen == 0:
+                mask = orc.prefill_mask(roles, n, C, W)
+                att = orc.masked_attention(q.cpu(), ko, vo, mask)
+            else:
+                att = orc.decode_attention(q.cpu(), ko, vo, torch.from_numpy(st.valid), st.n_ctx_data + 1)
+            st.post_update(n)
+            want = mod.wo(att.cuda().transpose(1, 2).reshape(B, n, -1))
+            err = (out - want).abs().max().item()
+            assert err < 2e-4, (step, err)
+            layer = cache.cache_model[0]
+            assert layer.n_ctx_data == st.n_ctx_data, step
+            assert np.array_equal(layer.valid_tokens.cpu().numpy(), st.valid), step
+            assert np.array_equal(layer.size_global_kv.cpu().numpy(), st.size_global), step
+            seen += n
