@@ -118,14 +118,19 @@ class NAtSChunkLayerCache:
         return None if self._buf_pos is None else self._buf_pos[:, :, :self._rows]
 
     # -- storage --------------------------------------------------------------------------------
-    def _allocate(self, rows: int, like: torch.Tensor, capacity: int | None = None):
+    def _allocate(self, rows: int, like: torch.Tensor, zero: bool = True):
+        """`zero=False` when the caller's kernel writes every row of every tensor itself."""
         B, H, D = like.shape[0], like.shape[1], like.shape[3]
-        cap = max(rows, capacity or 0)
-        self._buf_k = torch.zeros(B, H, cap, D, dtype=like.dtype, device=like.device)
-        self._buf_v = torch.zeros(B, H, cap, D, dtype=like.dtype, device=like.device)
-        self._buf_valid = torch.zeros(B, H, cap, dtype=torch.uint8, device=like.device)
-        self._buf_pos = (torch.full((B, H, cap), -1, dtype=torch.int32, device=like.device)
-                         if self.track_positions else None)
+        new = torch.zeros if zero else torch.empty
+        self._buf_k = new(B, H, rows, D, dtype=like.dtype, device=like.device)
+        self._buf_v = new(B, H, rows, D, dtype=like.dtype, device=like.device)
+        self._buf_valid = new(B, H, rows, dtype=torch.uint8, device=like.device)
+        if not self.track_positions:
+            self._buf_pos = None
+        elif zero:
+            self._buf_pos = torch.full((B, H, rows), -1, dtype=torch.int32, device=like.device)
+        else:
+            self._buf_pos = torch.empty(B, H, rows, dtype=torch.int32, device=like.device)
         self._rows = rows
 
     def _grow(self, rows: int):
@@ -235,7 +240,7 @@ class NAtSChunkLayerCache:
             else:
                 rows = math.ceil(res.n_ctx_data / C) * C
                 self._pending = None
-                self._allocate(rows, like)
+                self._allocate(rows, like, zero=False)  # the apply kernel writes all rows
                 params.n_alloc = rows
                 k_raw, v_raw = src
                 if k_raw.stride(-1) != 1 or k_raw.stride() != v_raw.stride():

@@ -4,9 +4,10 @@
 // helpers move_sliding_window_tokens_to_head (:391-437), get_updated_cache_info (:715-868),
 // mask_invalid_tokens (:634-656) and merge_local_to_global_caches (components/cache/cache_update.py:25-76).
 //
-// plan kernel  : one workgroup; a wavefront per (b, kv head) walks the role slots 64 at a time, a ballot
-//                marks the kept slots (globals + locals after the last global) and a prefix popcount gives
-//                each kept slot its destination rank (stream compaction of slot ids).
+// plan kernels : a wavefront per (b, kv head) pulls the role slots into registers, marks the kept slots
+//                (globals + locals after the last global) and gives each one its destination rank by a
+//                wave-wide prefix sum (stream compaction of slot ids); one more workgroup folds the heads
+//                into the global decisions and scalars.
 // apply kernels: move chunk-granular row blocks.  In place, a workgroup owns one row slice of every chunk
 //                of one (b, kv head, tensor) and processes the ordered move list in batches, reading a
 //                whole batch before writing it; because destinations never pass sources this equals
@@ -21,7 +22,8 @@ struct HeadPlan {
   int32_t dst_base;  // destination of the first kept chunk, in chunks
   int64_t sg_new;
   int64_t sl_new;
-  int64_t pad;
+  int32_t all_sw;    // every slot of this head is sliding-window
+  int32_t all_local; // every slot of this head is local
 };
 
 constexpr size_t kPlanHeaderBytes = 256;
@@ -31,120 +33,183 @@ __host__ __device__ inline size_t plan_lists_offset(int64_t n_heads) {
 }
 
 // ---------------------------------------------------------------------------------------------------
-// plan
+// plan, step 1: one wavefront per (b, kv head).  The head's role bytes are pulled into registers 1024
+// slots at a time (16 per lane), so the scan costs one memory latency per block; ballots are replaced by
+// per-lane bit masks plus wave-wide prefix sums, which give every kept slot its destination rank.
 // ---------------------------------------------------------------------------------------------------
-struct WaveAgg {
-  int all_sw, all_local;
-  int max_keep, max_end;
-  long long max_tot_new, max_tot_old, max_tot_alllocal, min_sg_new, sum_keep;
-};
+__device__ __forceinline__ int wave_sum(int x) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o);
+  return x;
+}
+__device__ __forceinline__ int wave_max(int x) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) x = max(x, __shfl_xor(x, o));
+  return x;
+}
+__device__ __forceinline__ int wave_excl_scan(int x, int lane) {
+  int incl = x;
+#pragma unroll
+  for (int o = 1; o < kWave; o <<= 1) {
+    int y = __shfl_up(incl, o);
+    if (lane >= o) incl += y;
+  }
+  return incl - x;
+}
 
-__global__ __launch_bounds__(1024) void evict_plan_kernel(const uint8_t* __restrict__ roles,
-                                                          const int64_t* __restrict__ size_global,
-                                                          const int64_t* __restrict__ size_local, nats_evict_params p,
-                                                          char* __restrict__ ws, nats_evict_result* __restrict__ result) {
-  __shared__ WaveAgg agg[16];
-  __shared__ int all_local_flag;
+constexpr int kSlotsPerLane = 16;
+constexpr int kSlotsPerBlock = kSlotsPerLane * kWave;
+
+__device__ __forceinline__ void load_roles(const uint8_t* __restrict__ r, int S, int base, int lane, int* rb) {
+#pragma unroll
+  for (int j = 0; j < kSlotsPerLane; ++j) {
+    int s = base + lane * kSlotsPerLane + j;
+    rb[j] = s < S ? r[s] : 255;
+  }
+}
+
+__global__ __launch_bounds__(256) void evict_plan_heads_kernel(const uint8_t* __restrict__ roles,
+                                                               const int64_t* __restrict__ size_global,
+                                                               const int64_t* __restrict__ size_local,
+                                                               nats_evict_params p, char* __restrict__ ws) {
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int n_heads = (int)(p.B * p.H_kv);
+  const int head = blockIdx.x * 4 + wave;
+  if (head >= n_heads) return;
   const int S = (int)p.S;
   const int C = (int)p.C;
   const int partial = (int)(p.fill % p.C);
   const int n_done = (int)(p.fill / p.C);
   const int S_eff = S - (partial ? 1 : 0);
   HeadPlan* plans = reinterpret_cast<HeadPlan*>(ws + kPlanHeaderBytes);
-  int32_t* lists = reinterpret_cast<int32_t*>(ws + plan_lists_offset(n_heads));
-
-  WaveAgg w;
-  w.all_sw = 1; w.all_local = 1; w.max_keep = 0; w.max_end = 0;
-  w.max_tot_new = 0; w.max_tot_old = 0; w.max_tot_alllocal = 0; w.min_sg_new = 0x7fffffffffffffffLL; w.sum_keep = 0;
-
-  for (int head = wave; head < n_heads; head += 16) {
-    const uint8_t* r = roles + (int64_t)head * S;
-    const long long sg = size_global[head], sl = size_local[head];
-    int32_t* keep = lists + (int64_t)head * S;
-    HeadPlan hp;
-    int head_all_sw, head_all_local;
-    if (p.x_len == 1) {
-      // one completed chunk is scattered for every head (:289-330)
-      int r0 = r[0], rl = r[S - 1];
-      bool is_g = r0 == NATS_ROLE_GLOBAL;
-      long long dst = is_g ? sg : sg + sl;
-      long long dec = (is_g ? sl / C + 1 : 0) + (rl == NATS_ROLE_SW ? 1 : 0);
-      hp.count = 1;
-      hp.dst_base = (int32_t)(dst / C);
-      hp.sg_new = sg + (is_g ? C : 0);
-      hp.sl_new = sl - dec * C + (long long)n_done * C;
-      if (lane == 0) keep[0] = 0;
-      int n_sw = 0;
-      for (int s = 0; s < S; ++s) n_sw += r[s] == NATS_ROLE_SW;
-      head_all_sw = n_sw == S;
-      head_all_local = 0;
-    } else {
-      // pass 1: counts and the last complete global slot
-      int n_glob_all = 0, n_sw = 0, n_loc = 0, last_g = -1;
-      for (int base = 0; base < S; base += kWave) {
-        int s = base + lane;
-        int role = s < S ? r[s] : 255;
-        uint64_t bg = __ballot(role == NATS_ROLE_GLOBAL);
-        uint64_t bge = __ballot(role == NATS_ROLE_GLOBAL && s < S_eff);
-        n_glob_all += __builtin_popcountll(bg);
-        n_sw += __builtin_popcountll(__ballot(role == NATS_ROLE_SW));
-        n_loc += __builtin_popcountll(__ballot(role == NATS_ROLE_LOCAL));
-        if (bge) last_g = base + 63 - __builtin_clzll(bge);
+  int32_t* keep = reinterpret_cast<int32_t*>(ws + plan_lists_offset(n_heads)) + (int64_t)head * S;
+  const uint8_t* r = roles + (int64_t)head * S;
+  const long long sg = size_global[head], sl = size_local[head];
+  HeadPlan hp;
+  if (p.x_len == 1) {
+    // one completed chunk is scattered for every head (:289-330)
+    int r0 = r[0], rl = r[S - 1];
+    bool is_g = r0 == NATS_ROLE_GLOBAL;
+    long long dst = is_g ? sg : sg + sl;
+    long long dec = (is_g ? sl / C + 1 : 0) + (rl == NATS_ROLE_SW ? 1 : 0);
+    hp.count = 1;
+    hp.dst_base = (int32_t)(dst / C);
+    hp.sg_new = sg + (is_g ? C : 0);
+    hp.sl_new = sl - dec * C + (long long)n_done * C;
+    hp.all_sw = r0 == NATS_ROLE_SW;
+    hp.all_local = 0;
+    if (lane == 0) keep[0] = 0;
+  } else {
+    // pass 1: counts and the last complete global slot
+    int n_glob_all = 0, n_sw = 0, n_loc = 0, last_g = -1;
+    for (int base = 0; base < S; base += kSlotsPerBlock) {
+      int rb[kSlotsPerLane];
+      load_roles(r, S, base, lane, rb);
+#pragma unroll
+      for (int j = 0; j < kSlotsPerLane; ++j) {
+        int s = base + lane * kSlotsPerLane + j;
+        n_glob_all += rb[j] == NATS_ROLE_GLOBAL;
+        n_sw += rb[j] == NATS_ROLE_SW;
+        n_loc += rb[j] == NATS_ROLE_LOCAL;
+        if (rb[j] == NATS_ROLE_GLOBAL && s < S_eff) last_g = s;
       }
-      // pass 2: kept slots in order, destination rank by prefix popcount
-      int count = 0, later_local = 0;
-      for (int base = 0; base < S; base += kWave) {
-        int s = base + lane;
-        int role = s < S ? r[s] : 255;
-        bool loc_after = role == NATS_ROLE_LOCAL && s > last_g;
-        bool kept = s < S_eff && (role == NATS_ROLE_GLOBAL || loc_after);
-        uint64_t bk = __ballot(kept);
-        later_local += __builtin_popcountll(__ballot(loc_after));
-        if (kept) {
-          int rank = count + __builtin_popcountll(bk & ((uint64_t(1) << lane) - 1));
-          keep[rank] = s;
-        }
-        count += __builtin_popcountll(bk);
-      }
-      int n_glob = n_glob_all - (partial ? 1 : 0);                                     // :782-786
-      long long n_other = (long long)S - (last_g > 0 ? last_g : 0) - later_local - (partial ? 1 : 0);  // :797-800
-      long long dec_l = (last_g > -1 ? (long long)last_g * C + sl : 0) + n_other * C;  // :793, :802
-      hp.count = count;
-      hp.dst_base = (int32_t)((last_g == -1 ? sg + sl : sg) / C);                      // :827-828
-      hp.sg_new = sg + (long long)n_glob * C;
-      hp.sl_new = sl - dec_l + (long long)n_done * C;
-      head_all_sw = n_sw == S;
-      head_all_local = n_loc == S;
     }
-    hp.pad = 0;
-    if (lane == 0) plans[head] = hp;
-    w.all_sw &= head_all_sw;
-    w.all_local &= head_all_local;
-    w.max_keep = max(w.max_keep, hp.count);
-    w.max_end = max(w.max_end, hp.count + hp.dst_base);
-    w.max_tot_new = max(w.max_tot_new, (long long)(hp.sg_new + hp.sl_new));
-    w.max_tot_old = max(w.max_tot_old, sg + sl);
-    w.max_tot_alllocal = max(w.max_tot_alllocal, sg + sl + (long long)n_done * C);
-    w.min_sg_new = min(w.min_sg_new, (long long)hp.sg_new);
-    w.sum_keep += hp.count;
+    n_glob_all = wave_sum(n_glob_all);
+    n_sw = wave_sum(n_sw);
+    n_loc = wave_sum(n_loc);
+    last_g = wave_max(last_g);
+    // pass 2: kept slots in order, destination rank by prefix sum (stream compaction of slot ids)
+    int count = 0, later_local = 0;
+    for (int base = 0; base < S; base += kSlotsPerBlock) {
+      int rb[kSlotsPerLane];
+      load_roles(r, S, base, lane, rb);
+      unsigned kept_bits = 0;
+      int loc_after = 0;
+#pragma unroll
+      for (int j = 0; j < kSlotsPerLane; ++j) {
+        int s = base + lane * kSlotsPerLane + j;
+        bool la = rb[j] == NATS_ROLE_LOCAL && s > last_g;
+        loc_after += la;
+        if (s < S_eff && (rb[j] == NATS_ROLE_GLOBAL || la)) kept_bits |= 1u << j;
+      }
+      int mine = __builtin_popcount(kept_bits);
+      int rank = count + wave_excl_scan(mine, lane);
+#pragma unroll
+      for (int j = 0; j < kSlotsPerLane; ++j) {
+        if (kept_bits & (1u << j)) keep[rank++] = base + lane * kSlotsPerLane + j;
+      }
+      count += wave_sum(mine);
+      later_local += wave_sum(loc_after);
+    }
+    int n_glob = n_glob_all - (partial ? 1 : 0);                                                      // :782-786
+    long long n_other = (long long)S - (last_g > 0 ? last_g : 0) - later_local - (partial ? 1 : 0);  // :797-800
+    long long dec_l = (last_g > -1 ? (long long)last_g * C + sl : 0) + n_other * C;                  // :793, :802
+    hp.count = count;
+    hp.dst_base = (int32_t)((last_g == -1 ? sg + sl : sg) / C);                                      // :827-828
+    hp.sg_new = sg + (long long)n_glob * C;
+    hp.sl_new = sl - dec_l + (long long)n_done * C;
+    hp.all_sw = n_sw == S;
+    hp.all_local = n_loc == S;
   }
-  if (lane == 0) agg[wave] = w;
+  if (lane == 0) plans[head] = hp;
+}
+
+// plan, step 2: one workgroup folds the per-head plans into the global decisions and scalars.
+struct PlanAgg {
+  int all_sw, all_local;
+  int max_keep, max_end;
+  long long max_tot_new, max_tot_old, max_tot_alllocal, min_sg_new, min_sg_old, sum_keep;
+};
+
+__device__ __forceinline__ void fold(PlanAgg& a, const PlanAgg& b) {
+  a.all_sw &= b.all_sw;
+  a.all_local &= b.all_local;
+  a.max_keep = max(a.max_keep, b.max_keep);
+  a.max_end = max(a.max_end, b.max_end);
+  a.max_tot_new = max(a.max_tot_new, b.max_tot_new);
+  a.max_tot_old = max(a.max_tot_old, b.max_tot_old);
+  a.max_tot_alllocal = max(a.max_tot_alllocal, b.max_tot_alllocal);
+  a.min_sg_new = min(a.min_sg_new, b.min_sg_new);
+  a.min_sg_old = min(a.min_sg_old, b.min_sg_old);
+  a.sum_keep += b.sum_keep;
+}
+
+__global__ __launch_bounds__(256) void evict_plan_finalize_kernel(const int64_t* __restrict__ size_global,
+                                                                  const int64_t* __restrict__ size_local,
+                                                                  nats_evict_params p, char* __restrict__ ws,
+                                                                  nats_evict_result* __restrict__ result) {
+  __shared__ PlanAgg agg[256];
+  __shared__ int all_local_flag;
+  const int tid = threadIdx.x;
+  const int n_heads = (int)(p.B * p.H_kv);
+  const int S = (int)p.S;
+  const int C = (int)p.C;
+  const int partial = (int)(p.fill % p.C);
+  const int n_done = (int)(p.fill / p.C);
+  HeadPlan* plans = reinterpret_cast<HeadPlan*>(ws + kPlanHeaderBytes);
+  PlanAgg w;
+  w.all_sw = 1; w.all_local = 1; w.max_keep = 0; w.max_end = 0;
+  w.max_tot_new = 0; w.max_tot_old = 0; w.max_tot_alllocal = 0;
+  w.min_sg_new = 0x7fffffffffffffffLL; w.min_sg_old = 0x7fffffffffffffffLL; w.sum_keep = 0;
+  for (int h = tid; h < n_heads; h += 256) {
+    const HeadPlan hp = plans[h];
+    const long long sg = size_global[h], sl = size_local[h];
+    PlanAgg x;
+    x.all_sw = hp.all_sw; x.all_local = hp.all_local;
+    x.max_keep = hp.count; x.max_end = hp.count + hp.dst_base;
+    x.max_tot_new = hp.sg_new + hp.sl_new; x.max_tot_old = sg + sl;
+    x.max_tot_alllocal = sg + sl + (long long)n_done * C;
+    x.min_sg_new = hp.sg_new; x.min_sg_old = sg; x.sum_keep = hp.count;
+    fold(w, x);
+  }
+  agg[tid] = w;
   __syncthreads();
+  for (int o = 128; o > 0; o >>= 1) {
+    if (tid < o) fold(agg[tid], agg[tid + o]);
+    __syncthreads();
+  }
   if (tid == 0) {
-    WaveAgg t = agg[0];
-    for (int i = 1; i < 16; ++i) {
-      t.all_sw &= agg[i].all_sw;
-      t.all_local &= agg[i].all_local;
-      t.max_keep = max(t.max_keep, agg[i].max_keep);
-      t.max_end = max(t.max_end, agg[i].max_end);
-      t.max_tot_new = max(t.max_tot_new, agg[i].max_tot_new);
-      t.max_tot_old = max(t.max_tot_old, agg[i].max_tot_old);
-      t.max_tot_alllocal = max(t.max_tot_alllocal, agg[i].max_tot_alllocal);
-      t.min_sg_new = min(t.min_sg_new, agg[i].min_sg_new);
-      t.sum_keep += agg[i].sum_keep;
-    }
+    const PlanAgg t = agg[0];
     nats_evict_result res;
     res.all_sw = t.all_sw;
     res.all_local = (p.x_len != 1) && t.all_local && !t.all_sw;
@@ -155,9 +220,9 @@ __global__ __launch_bounds__(1024) void evict_plan_kernel(const uint8_t* __restr
       res.n_ctx_data = t.max_tot_old + partial;
       res.gmin = p.gmin;
       res.moved_rows = 0;
-    } else if (res.all_local) {  // :747-749, then :356-358
+    } else if (res.all_local) {  // :747-749, then :356-358, :371
       res.n_ctx_data = t.max_tot_alllocal + partial;
-      res.gmin = p.gmin;
+      res.gmin = t.min_sg_old;
       res.moved_rows = 0;
     } else {
       res.n_ctx_data = t.max_tot_new + partial;
@@ -165,18 +230,13 @@ __global__ __launch_bounds__(1024) void evict_plan_kernel(const uint8_t* __restr
       bool tail_move = p.x_len != 1 && partial && t.max_keep < S - 1;  // :840
       res.moved_rows = (t.sum_keep + (tail_move ? n_heads : 0)) * (long long)C;
     }
-    if (res.all_local) {
-      long long mn = 0x7fffffffffffffffLL;
-      for (int h = 0; h < n_heads; ++h) mn = min(mn, (long long)size_global[h]);
-      res.gmin = mn;
-    }
     *result = res;
     all_local_flag = (int)res.all_local;
   }
   __syncthreads();
   if (all_local_flag) {
     // every slot local: nothing moves and only the local size grows (:747-749, :356)
-    for (int h = tid; h < n_heads; h += 1024) {
+    for (int h = tid; h < n_heads; h += 256) {
       plans[h].sg_new = size_global[h];
       plans[h].sl_new = size_local[h] + (long long)n_done * C;
     }
@@ -491,9 +551,14 @@ extern "C" int nats_evict_plan(const uint8_t* roles, const int64_t* size_global,
   if (int rc = check_params("nats_evict_plan", params)) return rc;
   size_t need = nats_evict_workspace_bytes(params->B, params->H_kv, params->S);
   NATS_REQUIRE(workspace_bytes >= need, NATS_ERR_WORKSPACE, "nats_evict_plan: workspace %zu bytes < %zu", workspace_bytes, need);
-  hipLaunchKernelGGL(evict_plan_kernel, dim3(1), dim3(1024), 0, static_cast<hipStream_t>(stream), roles, size_global,
-                     size_local, *params, static_cast<char*>(workspace), result);
-  NATS_CHECK_LAUNCH("evict_plan_kernel");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const unsigned n_wg = (unsigned)((params->B * params->H_kv + 3) / 4);
+  hipLaunchKernelGGL(evict_plan_heads_kernel, dim3(n_wg), dim3(256), 0, st, roles, size_global, size_local, *params,
+                     static_cast<char*>(workspace));
+  NATS_CHECK_LAUNCH("evict_plan_heads_kernel");
+  hipLaunchKernelGGL(evict_plan_finalize_kernel, dim3(1), dim3(256), 0, st, size_global, size_local, *params,
+                     static_cast<char*>(workspace), result);
+  NATS_CHECK_LAUNCH("evict_plan_finalize_kernel");
   return NATS_OK;
 }
 

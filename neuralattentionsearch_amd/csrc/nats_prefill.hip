@@ -153,30 +153,38 @@ __global__ __launch_bounds__(64) void prefill_simple_kernel(PrefillArgs a) {
 // Workgroup = 4 wavefronts = (hpw q heads of one kv head) x (qpw query tiles of 64 rows); every wavefront
 // owns 64 query rows of one q head and all wavefronts share each 64-key K / V tile through LDS.
 //
+// K / V tiles travel global -> LDS without passing through registers (global_load_lds, 16 bytes per lane),
+// double buffered, row major with 256-byte rows whose 16-byte chunks are XOR-swizzled (the lane supplies
+// the global address, so the permutation costs nothing) to keep the operand reads free of bank conflicts.
+//
 // Scores are computed transposed, S^T = K Q^T (A operand = K rows from LDS, B operand = Q from registers),
 // so a lane holds 16 keys of ONE query per accumulator and the softmax row reductions stay inside the
 // lane (one cross-lane exchange with lane ^ 32).  The exponentials leave the accumulators already in the
-// B-operand layout of O^T = V^T P^T, provided V^T is stored in LDS with the keys of every 16-key group
-// permuted by pos(o) = ((o >> 2) & 1) * 8 + (o >> 3) * 4 + (o & 3); the permutation is applied while the
-// tile is written to LDS, two keys (one dword) at a time.
+// B-operand layout of O^T = V^T P^T; its A operand V^T comes from the row-major V tile through
+// ds_read_b64_tr_b16, which hands every lane 4 consecutive keys of one head dimension.
+//
+// The running maximum is only raised when a row maximum exceeds it by more than kRescaleSlack (base-2
+// exponent); until then probabilities may exceed 1 (at most 2^kRescaleSlack), which fp32 sums and bf16
+// operands hold without loss, and O is not touched.
 // ---------------------------------------------------------------------------------------------------
-__device__ __forceinline__ int vt_pos(int key_in_tile) {
-  int o = key_in_tile & 15;
-  return (key_in_tile & ~15) | (((o >> 2) & 1) << 3) | ((o >> 3) << 2) | (o & 3);
-}
+constexpr float kRescaleSlack = 8.0f;
+
+template <int D>
+struct PrefillSmem {
+  uint16_t k[2][kTile * D];
+  uint16_t v[2][kTile * D];
+  int limk[2][kTile];
+};
 
 template <int D>
 __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
-  constexpr int KPAD = 8, VPAD = 8;
-  constexpr int OCT = D / 8;        // 16-byte units per row
-  constexpr int KU = kTile * OCT / 256;       // K units per thread (4 for D=128)
-  constexpr int VU = (kTile / 2) * OCT / 256;  // V row-pair units per thread (2 for D=128)
+  constexpr int OCT = D / 8;              // 16-byte chunks per row
+  constexpr int DMA_PER_WAVE = OCT / 4;   // 1 KiB global->LDS transfers per wavefront and tensor
   constexpr int DSTEPS = D / 16;
   constexpr int DT = D / 32;
 
-  __shared__ __attribute__((aligned(16))) uint16_t Ks[kTile][D + KPAD];
-  __shared__ __attribute__((aligned(16))) uint16_t Vt[D][kTile + VPAD];
-  __shared__ __attribute__((aligned(16))) int limk[kTile];
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  PrefillSmem<D>& sm = *reinterpret_cast<PrefillSmem<D>*>(smem_raw);
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
@@ -228,11 +236,9 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
     for (int qb = 0; qb < 2; ++qb) {
       int row = min(q0 + qb * 32 + l32, a.L - 1);
       if (!wave_live) row = 0;
-      const uint16_t* rp = qp + (int64_t)row * a.qs_l;
+      const uint4* rp = reinterpret_cast<const uint4*>(qp + (int64_t)row * a.qs_l + hl * 8);
 #pragma unroll
-      for (int s = 0; s < DSTEPS; ++s) {
-        qreg[qb][s] = *reinterpret_cast<const bf16x8*>(rp + s * 16 + hl * 8);
-      }
+      for (int s = 0; s < DSTEPS; ++s) qreg[qb][s] = __builtin_bit_cast(bf16x8, rp[s * 2]);
     }
   }
 
@@ -247,85 +253,61 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
   float l_run[2] = {0.f, 0.f};
   const float c = a.scale * 1.4426950408889634f;
 
-  uint4 kreg[KU];
-  uint4 vreg[VU][2];
-
-  auto issue_loads = [&](int kt) {
+  // global -> LDS, one 64-key tile of K and of V; rows beyond L repeat row L-1 (their scores are masked,
+  // so their probabilities are exactly 0 and a finite V row contributes nothing)
+  auto issue_tile = [&](int kt, int buf) {
 #pragma unroll
-    for (int i = 0; i < KU; ++i) {
-      int u = tid + 256 * i;
-      int row = u / OCT, oct = u % OCT;
-      int n = kt * kTile + row;
-      kreg[i] = n < a.L ? *reinterpret_cast<const uint4*>(kp + (int64_t)n * a.ks_l + oct * 8) : make_uint4(0, 0, 0, 0);
-    }
-#pragma unroll
-    for (int i = 0; i < VU; ++i) {
-      int u = tid + 256 * i;
-      int pair = u / OCT, oct = u % OCT;
-      int n = kt * kTile + pair * 2;
-      vreg[i][0] = n < a.L ? *reinterpret_cast<const uint4*>(vp + (int64_t)n * a.vs_l + oct * 8) : make_uint4(0, 0, 0, 0);
-      vreg[i][1] =
-          n + 1 < a.L ? *reinterpret_cast<const uint4*>(vp + (int64_t)(n + 1) * a.vs_l + oct * 8) : make_uint4(0, 0, 0, 0);
-    }
-  };
-  auto stage_to_lds = [&](int kt) {
-#pragma unroll
-    for (int i = 0; i < KU; ++i) {
-      int u = tid + 256 * i;
-      int row = u / OCT, oct = u % OCT;
-      *reinterpret_cast<uint4*>(&Ks[row][oct * 8]) = kreg[i];
-    }
-#pragma unroll
-    for (int i = 0; i < VU; ++i) {
-      int u = tid + 256 * i;
-      int pair = u / OCT, oct = u % OCT;
-      int col = vt_pos(pair * 2);
-      const uint32_t ra[4] = {vreg[i][0].x, vreg[i][0].y, vreg[i][0].z, vreg[i][0].w};
-      const uint32_t rb[4] = {vreg[i][1].x, vreg[i][1].y, vreg[i][1].z, vreg[i][1].w};
-#pragma unroll
-      for (int w = 0; w < 4; ++w) {
-        uint32_t even = (ra[w] & 0xffffu) | (rb[w] << 16);
-        uint32_t odd = (ra[w] >> 16) | (rb[w] & 0xffff0000u);
-        *reinterpret_cast<uint32_t*>(&Vt[oct * 8 + 2 * w][col]) = even;
-        *reinterpret_cast<uint32_t*>(&Vt[oct * 8 + 2 * w + 1][col]) = odd;
-      }
+    for (int j = 0; j < DMA_PER_WAVE; ++j) {
+      const int inst = wave * DMA_PER_WAVE + j;  // uniform
+      const int q = inst * kWave + lane;         // chunk slot in the LDS tile
+      const int row = q / OCT, pos = q % OCT;
+      const int n = min(kt * kTile + row, a.L - 1);
+      const int kchunk = pos ^ (row % OCT);
+      const int vchunk = pos ^ ((row & 3) << 1);
+      __builtin_amdgcn_global_load_lds(kp + (int64_t)n * a.ks_l + kchunk * 8,
+                                       (uint32_t __attribute__((address_space(3)))*)(&sm.k[buf][inst * kWave * 8]), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(vp + (int64_t)n * a.vs_l + vchunk * 8,
+                                       (uint32_t __attribute__((address_space(3)))*)(&sm.v[buf][inst * kWave * 8]), 16, 0, 0);
     }
     if (tid < kTile) {
       int n = kt * kTile + tid;
-      limk[tid] = n < a.L ? lim[n >> a.c_shift] : -1;
+      sm.limk[buf][tid] = n < a.L ? lim[n >> a.c_shift] : -1;
     }
   };
 
   int kt = next_visited(tl, 0, qt_hi, m0_group, lane);
-  if (kt >= 0) {
-    issue_loads(kt);
-    stage_to_lds(kt);
-  }
+  int cur = 0;
+  if (kt >= 0) issue_tile(kt, 0);
+  __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
 
   while (kt >= 0) {
     const int nxt = next_visited(tl, kt + 1, qt_hi, m0_group, lane);
-    if (nxt >= 0) issue_loads(nxt);
+    if (nxt >= 0) issue_tile(nxt, cur ^ 1);
 
     const int2 tlk = tl[kt];
     const bool visit = wave_live && kt <= my_qt && tlk.x >= my_m0;
     if (visit) {
       const bool full = kt < my_qt && tlk.y >= my_mlast;
+      const uint16_t* Kt = sm.k[cur];
+      const uint16_t* Vt = sm.v[cur];
       // ---- S^T = K Q^T ---------------------------------------------------------------------------
       f32x16 sacc[2][2];
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int qb = 0; qb < 2; ++qb)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) sacc[kb][qb][i] = 0.f;
-#pragma unroll
       for (int kb = 0; kb < 2; ++kb) {
+        const int row = kb * 32 + l32;
 #pragma unroll
         for (int s = 0; s < DSTEPS; ++s) {
-          bf16x8 ka = *reinterpret_cast<const bf16x8*>(&Ks[kb * 32 + l32][s * 16 + hl * 8]);
-          sacc[kb][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qreg[0][s], sacc[kb][0], 0, 0, 0);
-          sacc[kb][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qreg[1][s], sacc[kb][1], 0, 0, 0);
+          const int chunk = (s * 2 + hl) ^ (row % OCT);
+          bf16x8 ka = *reinterpret_cast<const bf16x8*>(Kt + row * D + chunk * 8);
+          if (s == 0) {
+            const f32x16 z = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            sacc[kb][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qreg[0][s], z, 0, 0, 0);
+            sacc[kb][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qreg[1][s], z, 0, 0, 0);
+          } else {
+            sacc[kb][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qreg[0][s], sacc[kb][0], 0, 0, 0);
+            sacc[kb][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qreg[1][s], sacc[kb][1], 0, 0, 0);
+          }
         }
       }
       // ---- mask (diagonal tile, or a tile whose slots are not uniformly visible) -----------------
@@ -335,7 +317,7 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
 #pragma unroll
           for (int g4 = 0; g4 < 4; ++g4) {
             int kk = kb * 32 + g4 * 8 + hl * 4;  // key offset in tile of accumulator 4*g4
-            int4 lm = *reinterpret_cast<const int4*>(&limk[kk]);
+            int4 lm = *reinterpret_cast<const int4*>(&sm.limk[cur][kk]);
             const int lv[4] = {lm.x, lm.y, lm.z, lm.w};
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -359,10 +341,18 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
           for (int i = 0; i < 16; ++i) mx = fmaxf(mx, sacc[kb][qb][i]);
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
-        float m_new = fmaxf(m_run[qb], mx * c);
-        float m_use = m_new == -INFINITY ? 0.f : m_new;
-        float alpha = __builtin_amdgcn_exp2f(m_run[qb] - m_use);
+        mx = fmaxf(mx, __shfl_xor(mx, 32)) * c;
+        if (__ballot(mx > m_run[qb] + kRescaleSlack)) {
+          float m_new = fmaxf(m_run[qb], mx);
+          float alpha = m_run[qb] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_run[qb] - m_new);
+          l_run[qb] *= alpha;
+          m_run[qb] = m_new;
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) oacc[dt][qb][i] *= alpha;
+        }
+        const float m_use = m_run[qb] == -INFINITY ? 0.f : m_run[qb];
         float rs = 0.f;
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
@@ -373,31 +363,39 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
             pb[qb][kb * 2 + (i >> 3)][i & 7] = (__bf16)p;
           }
         }
-        l_run[qb] = l_run[qb] * alpha + rs;
-        m_run[qb] = m_new;
-        if (__ballot(alpha != 1.f)) {
-#pragma unroll
-          for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) oacc[dt][qb][i] *= alpha;
-        }
+        l_run[qb] += rs;
       }
       // ---- O^T += V^T P^T ------------------------------------------------------------------------
+      // ds_read_b64_tr_b16: within 16 lanes, lane r reads 4 dims of key (K0 + r / 4) starting at dim
+      // D0 + 4 * (r % 4) and receives keys K0 .. K0 + 3 of dim D0 + r.
+      const int r16 = lane & 15;
+      const int dsel = (lane >> 4) & 1;
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) {
+        const int chunk0 = dt * 4 + dsel * 2 + ((r16 & 3) >> 1);
+        const int half = r16 & 1;
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-          bf16x8 va = *reinterpret_cast<const bf16x8*>(&Vt[dt * 32 + l32][t * 16 + hl * 8]);
+          bf16x4 lo, hi;
+          {
+            const int row = t * 16 + hl * 4 + (r16 >> 2);
+            const uint16_t* pa = Vt + row * D + ((chunk0 ^ ((row & 3) << 1)) * 8) + half * 4;
+            lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((bf16x4 __attribute__((address_space(3)))*)pa);
+          }
+          {
+            const int row = t * 16 + 8 + hl * 4 + (r16 >> 2);
+            const uint16_t* pa = Vt + row * D + ((chunk0 ^ ((row & 3) << 1)) * 8) + half * 4;
+            hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((bf16x4 __attribute__((address_space(3)))*)pa);
+          }
+          bf16x8 va = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
           oacc[dt][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb[0][t], oacc[dt][0], 0, 0, 0);
           oacc[dt][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb[1][t], oacc[dt][1], 0, 0, 0);
         }
       }
     }
-    __syncthreads();  // every wavefront is done reading this tile
-    if (nxt >= 0) {
-      stage_to_lds(nxt);
-      __syncthreads();
-    }
+    __builtin_amdgcn_s_waitcnt(0);  // the next tile has landed in LDS
+    __syncthreads();                // ... for every wavefront, and this tile is no longer read
+    cur ^= 1;
     kt = nxt;
   }
 
@@ -426,6 +424,21 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
       }
     }
   }
+}
+
+template <int D>
+static int launch_prefill_mfma(const PrefillArgs& a, int64_t n_wg, hipStream_t st) {
+  static bool configured = false;  // per process and head size; the attribute is a property of the kernel
+  const size_t smem = sizeof(PrefillSmem<D>);
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_mfma_kernel<D>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) return fail(NATS_ERR_LAUNCH, "hipFuncSetAttribute(%zu bytes of LDS): %s", smem, hipGetErrorString(e));
+    configured = true;
+  }
+  hipLaunchKernelGGL((prefill_mfma_kernel<D>), dim3((unsigned)n_wg), dim3(256), smem, st, a);
+  NATS_CHECK_LAUNCH("prefill_mfma_kernel");
+  return NATS_OK;
 }
 
 }  // namespace nats
@@ -522,11 +535,5 @@ extern "C" int nats_prefill_fwd(const void* q, const void* k, const void* v, con
   a.xcd_mode = ((B * H_kv) % 8 == 0) ? 1 : 0;
   int64_t n_wg = B * H_kv * a.n_hg * a.n_qg;
   NATS_REQUIRE(n_wg < (int64_t(1) << 31), NATS_ERR_BAD_SHAPE, "nats_prefill_fwd: grid too large");
-  if (D == 64) {
-    hipLaunchKernelGGL((prefill_mfma_kernel<64>), dim3((unsigned)n_wg), dim3(256), 0, st, a);
-  } else {
-    hipLaunchKernelGGL((prefill_mfma_kernel<128>), dim3((unsigned)n_wg), dim3(256), 0, st, a);
-  }
-  NATS_CHECK_LAUNCH("prefill_mfma_kernel");
-  return NATS_OK;
+  return D == 64 ? launch_prefill_mfma<64>(a, n_wg, st) : launch_prefill_mfma<128>(a, n_wg, st);
 }
