@@ -105,6 +105,9 @@ def bench_prefill(args, ops):
         "tflops_visited": flops / (ev_mean * 1e-3) / 1e12,
         "tokens_per_s": L / (ev_mean * 1e-3),
     }
+    res["shape"] = dict(B=B, Hq=Hq, Hkv=Hkv, L=L, D=D, C=C, W=W, roles="5% global / 15% local / 80% sliding")
+    if args.no_compare:
+        return res
     # the same kernel on all-global roles = dense causal attention
     roles_dense = torch.zeros_like(roles)
     _, dm, _ = time_gpu(lambda: ops.prefill_attention(q, k, v, roles_dense, C, W, out=out), max(2, args.steps // 4), 1)
@@ -120,7 +123,6 @@ def bench_prefill(args, ops):
         res["frac_of_dense_flash_throughput"] = res["tflops_visited"] / res["torch_sdpa_dense_causal_tflops"]
     except Exception as e:  # library path unavailable on this build
         res["torch_sdpa_error"] = repr(e)[:200]
-    res["shape"] = dict(B=B, Hq=Hq, Hkv=Hkv, L=L, D=D, C=C, W=W, roles="5% global / 15% local / 80% sliding")
     return res
 
 
@@ -141,15 +143,18 @@ def decode_inputs(B, Hq, Hkv, D, C, W, ctx, seed, dev):
             valid[b, h, W:W + n[b, h]] = True
     valid[:, :, base:n_rows] = True
     q = torch.randn(B, Hq, 1, D, generator=g, device=dev).bfloat16()
-    return q, k, v, torch.from_numpy(valid).to(dev), n_rows
+    hint = (torch.from_numpy(W + n).to(dev), base)  # what the cache object knows: size_global + size_local, open chunk
+    return q, k, v, torch.from_numpy(valid).to(dev), n_rows, hint
 
 
 def bench_decode(args, ops):
     B, Hq, Hkv, D, C, W, ctx = 32, 32, 8, 128, 64, 256, 65536
-    q, k, v, valid, n_rows = decode_inputs(B, Hq, Hkv, D, C, W, ctx, 0, "cuda")
+    q, k, v, valid, n_rows, (row_end, tail_start) = decode_inputs(B, Hq, Hkv, D, C, W, ctx, 0, "cuda")
     n_valid = int(valid[:, :, :n_rows].sum().item())
     bytes_alg = n_valid * D * 2 * 2 + 2 * q.numel() * 2
-    wall, ev_mean, ev_min = time_gpu(lambda: ops.decode_attention(q, k, v, valid, n_rows), args.steps * 5, args.warmup)
+    wall, ev_mean, ev_min = time_gpu(
+        lambda: ops.decode_attention(q, k, v, valid, n_rows, row_end=row_end, tail_start=tail_start),
+        args.steps * 5, args.warmup)
     return {
         "ms": ev_mean, "ms_min": ev_min, "ms_wall": wall,
         "tokens_per_s_per_layer": B / (ev_mean * 1e-3),
@@ -224,7 +229,7 @@ def cpu_baseline(args):
     }
     # decode: a 2-sequence slice of the batch, scaled linearly to batch 32
     Bs = 2
-    q, k, v, valid, n_rows = decode_inputs(Bs, 32, 8, D, C, W, 65536, 0, "cpu")
+    q, k, v, valid, n_rows, _ = decode_inputs(Bs, 32, 8, D, C, W, 65536, 0, "cpu")
     t0 = time.perf_counter()
     mask = valid[:, :, None, :n_rows]
     orc.masked_attention(q, k[:, :, :n_rows], v[:, :, :n_rows], mask)
@@ -254,6 +259,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--prefill-len", type=int, default=32768)
     ap.add_argument("--skip-cpu", action="store_true")
+    ap.add_argument("--no-compare", action="store_true", help="skip the dense comparators of the prefill leg")
     ap.add_argument("--only", choices=["prefill", "decode", "evict", "copy"], default=None)
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:

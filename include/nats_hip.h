@@ -111,15 +111,18 @@ int nats_prefill_fwd(const void* q, const void* k, const void* v, const uint8_t*
  *   cache_k / cache_v [B, H_kv, >= n_rows, D], last dimension contiguous, strides (stride_b, stride_h, stride_row)
  *   valid [B, H_kv, >= n_rows] uint8 (the cache's valid_tokens), strides (stride_b, stride_h), rows contiguous
  *   n_rows = n_ctx_data + 1: rows [0, n_rows) with valid != 0 take part; rows with valid == 0 are never loaded
+ *   row_end [B, H_kv] int64, optional (NULL = no hint): per head, rows [row_end, tail_start) are known to
+ *           hold nothing valid (the cache's size_global_kv + size_local_kv and the start of the open chunk,
+ *           components/cache/nats_chunk_layer_cache.py:644-656) and are skipped without reading valid
  *   workspace: nats_decode_workspace_bytes(...) bytes
- * D in {64, 128}; dtype bf16 or f32 (f32 converts on load).
+ * D in {64, 128}; dtype bf16 (MFMA) or f32 (fp32 FMA kernel, ignores the hint).
  */
 size_t nats_decode_workspace_bytes(int64_t B, int64_t H_q, int64_t H_kv, int64_t D, int64_t n_rows);
 
-int nats_decode_fwd(const void* q, const void* cache_k, const void* cache_v, const uint8_t* valid, void* o, int64_t B,
-                    int64_t H_q, int64_t H_kv, int64_t D, int64_t n_rows, const int64_t* kv_strides,
-                    const int64_t* valid_strides, float sm_scale, int dtype, void* workspace, size_t workspace_bytes,
-                    void* stream);
+int nats_decode_fwd(const void* q, const void* cache_k, const void* cache_v, const uint8_t* valid,
+                    const int64_t* row_end, int64_t tail_start, void* o, int64_t B, int64_t H_q, int64_t H_kv, int64_t D,
+                    int64_t n_rows, const int64_t* kv_strides, const int64_t* valid_strides, float sm_scale, int dtype,
+                    void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
  * (a-7) KV eviction + compaction: NAtSChunkLayerCache._post_update from its ring insert to its

@@ -5,9 +5,12 @@
 // Rows whose valid byte is 0 are never loaded, so whatever sits between a head's own end and the
 // batch-wide n_ctx_data costs no bandwidth.
 //
-// Split-K: grid = (splits of the row range) x (b, kv head) x (groups of q heads).  Inside a workgroup the
-// four wavefronts take interleaved 64-row tiles, keep (m, l, acc) per q head and are merged through LDS;
-// one partial per workgroup goes to the workspace and a second small kernel merges the splits.
+// Split-K: the rows of all (b, kv head) streams are cut into equal shares of 32-row tiles, one share per
+// workgroup; inside a workgroup the four wavefronts take interleaved tiles, keep (m, l, acc) per q head and
+// are merged through LDS; one partial per (workgroup, head touched) goes to the workspace and a second
+// small kernel merges the partials of every q head.
+#include <stdlib.h>
+
 #include "nats_common.h"
 
 namespace nats {
@@ -17,6 +20,7 @@ struct DecodeArgs {
   const void* k;
   const void* v;
   const uint8_t* valid;
+  const int64_t* row_end;  // optional [B*Hkv]: rows [row_end, tail_start) hold nothing valid and are skipped unseen
   void* o;
   float* ws_acc;  // [B*Hq, nsplit, D]
   float* ws_ml;   // [B*Hq, nsplit, 2]
@@ -24,202 +28,355 @@ struct DecodeArgs {
   int64_t vs_b, vs_h;
   int B, Hq, Hkv, n_rep;
   int n_rows, rows_per_split, nsplit;
+  int tail_start;
   float scale;
+  // balanced schedule of the bf16 kernel
+  int2* head_table;  // [B*Hkv] {first partial slot, number of partials}
+  int n_wg;          // workgroups along x; every one takes the same number of 32-row tiles
 };
 
 __device__ __forceinline__ float exp2_guard(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // ---------------------------------------------------------------------------------------------------
-// bf16: S^T = K Q^T on v_mfma_f32_16x16x32_bf16 (A = 16 key rows straight from global memory, B = the q
-// heads of the group padded to 16 columns), softmax per q head, probabilities broadcast through
-// wave-private LDS, PV on the vector ALU with fully coalesced 16-byte V loads.
+// bf16 kernel.  A wavefront walks 32-row tiles:
+//   K rows go straight from global memory into the A operand of v_mfma_f32_16x16x32_bf16 (S^T = K Q^T, the
+//   q heads of the group are the B columns, zero padded to 16);
+//   V rows go global -> LDS without touching registers (global_load_lds, wave-private double buffer, 16-byte
+//   chunks XOR-swizzled) and come back transposed through ds_read_b64_tr_b16 as the A operand of
+//   O^T = V^T P^T; the probabilities are already in B-operand layout when they leave the softmax.
+// Next tile's K (registers) and V (LDS) are requested before this tile's softmax and PV, so every
+// wavefront keeps about 16 KiB in flight.  A row that is not valid is never read: its lane fetches the
+// tile's first valid row instead (a cache hit), whose score is masked and whose probability is exactly 0.
 // ---------------------------------------------------------------------------------------------------
+constexpr float kDecodeRescaleSlack = 8.0f;
+constexpr int kDecTile = 32;
+
+constexpr int kMaxBalancedHeads = 2048;  // (b, kv head) streams whose tile prefix sums fit in LDS
+
+template <int D, int NREP>
+struct DecodeSmem {
+  uint16_t v[4][2][kDecTile * D];  // [wave][buffer]
+  float wacc[4][NREP][D];
+  float wm[4][NREP];
+  float wl[4][NREP];
+  int tile_prefix[kMaxBalancedHeads + 1];  // exclusive prefix of 32-row tiles per (b, kv head)
+  int slot_prefix[kMaxBalancedHeads + 1];  // exclusive prefix of partial results per (b, kv head)
+  int scan_tmp[256];
+  int first_head;
+};
+
+// exclusive prefix sum over n <= kMaxBalancedHeads values held in `dst` (dst[n] receives the total)
+__device__ __forceinline__ void block_exclusive_scan(int* dst, int n, int* tmp) {
+  const int tid = threadIdx.x;
+  const int per = (n + 255) / 256;
+  const int lo = min(tid * per, n), hi = min(lo + per, n);
+  int sum = 0;
+  for (int i = lo; i < hi; ++i) sum += dst[i];
+  tmp[tid] = sum;
+  __syncthreads();
+  if (tid == 0) {
+    int run = 0;
+    for (int i = 0; i < 256; ++i) {
+      int x = tmp[i];
+      tmp[i] = run;
+      run += x;
+    }
+    dst[n] = run;
+  }
+  __syncthreads();
+  int run = tmp[tid];
+  for (int i = lo; i < hi; ++i) {
+    int x = dst[i];
+    dst[i] = run;
+    run += x;
+  }
+  __syncthreads();
+}
+
+// Balanced schedule: all 32-row tiles of all (b, kv head) streams form one list, cut into n_wg equal
+// ranges; a workgroup works through its range head by head and emits one partial (m, l, acc) per head it
+// touches.  No workgroup is empty and all finish together, whatever the per-head lengths are.
 template <int D, int NREP>
 __global__ __launch_bounds__(256) void decode_split_mfma_kernel(DecodeArgs a) {
-  constexpr int STEPS = D / 32;
-  constexpr int LPR = D / 8;    // lanes per V row
-  constexpr int RPI = 64 / LPR; // V rows per load instruction
-  constexpr int NVL = 64 / RPI; // V loads per tile
+  constexpr int STEPS = D / 32;      // k-steps of the score MFMA
+  constexpr int OCT = D / 8;         // 16-byte chunks per row
+  constexpr int NDMA = kDecTile * OCT / kWave;  // 1 KiB transfers per V tile
+  constexpr int DB = D / 16;         // 16-dim blocks of O^T
 
-  __shared__ float p_lds[4][64][NREP];
-  __shared__ float al_lds[4][NREP];
-  __shared__ float wacc[4][NREP][D];
-  __shared__ float wm[4][NREP];
-  __shared__ float wl[4][NREP];
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  DecodeSmem<D, NREP>& sm = *reinterpret_cast<DecodeSmem<D, NREP>*>(smem_raw);
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
   const int lane = tid & 63;
   const int l16 = lane & 15;
   const int lg = lane >> 4;
-
-  const int split = blockIdx.x;
-  const int ks = blockIdx.y;  // b * Hkv + hkv
+  const int wg = blockIdx.x;
   const int grp = blockIdx.z;
-  const int b = ks / a.Hkv, hkv = ks % a.Hkv;
-  const int hq0 = hkv * a.n_rep + grp * NREP;
+  const int n_heads = a.B * a.Hkv;
+  const int ts = a.row_end ? a.tail_start : a.n_rows;
+  const int tail_tiles = (a.n_rows - ts + kDecTile - 1) / kDecTile;
 
-  const uint16_t* kp = static_cast<const uint16_t*>(a.k) + b * a.ks_b + hkv * a.ks_h;
-  const uint16_t* vp = static_cast<const uint16_t*>(a.v) + b * a.ks_b + hkv * a.ks_h;
-  const uint8_t* valp = a.valid + b * a.vs_b + hkv * a.vs_h;
-
-  // Q as the B operand: column = q head of the group (zero beyond NREP), k = 8 dims per lane group
-  bf16x8 qreg[STEPS];
-  {
-    const uint16_t* qp = static_cast<const uint16_t*>(a.q) + ((int64_t)b * a.Hq + hq0 + (l16 < NREP ? l16 : 0)) * D;
-#pragma unroll
-    for (int s = 0; s < STEPS; ++s) {
-      uint4 raw = *reinterpret_cast<const uint4*>(qp + s * 32 + lg * 8);
-      if (l16 >= NREP) raw = make_uint4(0, 0, 0, 0);
-      qreg[s] = __builtin_bit_cast(bf16x8, raw);
-    }
-  }
-
-  float acc[NREP][8];
-#pragma unroll
-  for (int h = 0; h < NREP; ++h)
-#pragma unroll
-    for (int e = 0; e < 8; ++e) acc[h][e] = 0.f;
-  float m_run = -INFINITY, l_run = 0.f;  // of q head l16 (meaningful for l16 < NREP)
-  const float c = a.scale * 1.4426950408889634f;
-
-  const int r_begin = split * a.rows_per_split;
-  const int r_end = min(r_begin + a.rows_per_split, a.n_rows);
-
-  for (int row0 = r_begin + wave * 64; row0 < r_end; row0 += 256) {
-    bool vb = (row0 + lane < r_end) && valp[row0 + lane] != 0;
-    const uint64_t vmask = __ballot(vb);
-    if (vmask == 0) continue;
-
-    uint4 kreg[4][STEPS];
-    uint4 vreg[NVL];
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      int kl = g * 16 + l16;
-      bool ok = (vmask >> kl) & 1;
-      const uint16_t* rp = kp + (int64_t)(row0 + kl) * a.ks_r + lg * 8;
-#pragma unroll
-      for (int s = 0; s < STEPS; ++s) {
-        kreg[g][s] = ok ? *reinterpret_cast<const uint4*>(rp + s * 32) : make_uint4(0, 0, 0, 0);
-      }
-    }
-#pragma unroll
-    for (int j = 0; j < NVL; ++j) {
-      int kl = j * RPI + lane / LPR;
-      bool ok = (vmask >> kl) & 1;
-      vreg[j] = ok ? *reinterpret_cast<const uint4*>(vp + (int64_t)(row0 + kl) * a.ks_r + (lane % LPR) * 8)
-                   : make_uint4(0, 0, 0, 0);
-    }
-
-    // scores: sc[g][i] belongs to key g*16 + lg*4 + i and q head l16
-    float sc[4][4];
-    float mx = -INFINITY;
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      f32x4 s4 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int s = 0; s < STEPS; ++s) {
-        s4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kreg[g][s]), qreg[s], s4, 0, 0, 0);
-      }
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        int kl = g * 16 + lg * 4 + i;
-        float sv = ((vmask >> kl) & 1) ? s4[i] : -INFINITY;
-        sc[g][i] = sv;
-        mx = fmaxf(mx, sv);
-      }
-    }
-    mx = fmaxf(mx, __shfl_xor(mx, 16));
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
-    float m_new = fmaxf(m_run, mx * c);  // vmask != 0, so mx is finite
-    float alpha = exp2_guard(m_run - m_new);
-    float rs = 0.f;
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        float p = exp2_guard(fmaf(sc[g][i], c, -m_new));
-        rs += p;
-        if (l16 < NREP) p_lds[wave][g * 16 + lg * 4 + i][l16] = p;
-      }
-    }
-    l_run = l_run * alpha + rs;
-    m_run = m_new;
-    if (lane < NREP) al_lds[wave][lane] = alpha;
-    wave_lds_sync();
-
-    float al[NREP];
-#pragma unroll
-    for (int h = 0; h < NREP; ++h) al[h] = al_lds[wave][h];
-#pragma unroll
-    for (int h = 0; h < NREP; ++h)
-#pragma unroll
-      for (int e = 0; e < 8; ++e) acc[h][e] *= al[h];
-#pragma unroll
-    for (int j = 0; j < NVL; ++j) {
-      int kl = j * RPI + lane / LPR;
-      float ph[NREP];
-#pragma unroll
-      for (int h = 0; h < NREP; ++h) ph[h] = p_lds[wave][kl][h];
-      const uint32_t w[4] = {vreg[j].x, vreg[j].y, vreg[j].z, vreg[j].w};
-#pragma unroll
-      for (int e2 = 0; e2 < 4; ++e2) {
-        float v0 = __uint_as_float(w[e2] << 16);
-        float v1 = __uint_as_float(w[e2] & 0xffff0000u);
-#pragma unroll
-        for (int h = 0; h < NREP; ++h) {
-          acc[h][2 * e2] = fmaf(ph[h], v0, acc[h][2 * e2]);
-          acc[h][2 * e2 + 1] = fmaf(ph[h], v1, acc[h][2 * e2 + 1]);
-        }
-      }
-    }
-    wave_lds_sync();
-  }
-
-  // ---- merge the lane groups of a wavefront, then the wavefronts of the workgroup --------------------
-#pragma unroll
-  for (int h = 0; h < NREP; ++h) {
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      float x = acc[h][e];
-      if (LPR < 16) x += __shfl_xor(x, 8);
-      x += __shfl_xor(x, 16);
-      x += __shfl_xor(x, 32);
-      acc[h][e] = x;
-    }
-  }
-  l_run += __shfl_xor(l_run, 16);
-  l_run += __shfl_xor(l_run, 32);
-  if (lane < LPR) {
-#pragma unroll
-    for (int h = 0; h < NREP; ++h)
-#pragma unroll
-      for (int e = 0; e < 8; ++e) wacc[wave][h][lane * 8 + e] = acc[h][e];
-  }
-  if (lane < NREP) {
-    wm[wave][lane] = m_run;
-    wl[wave][lane] = l_run;
+  // ---- schedule: tiles per head, their prefix sums, this workgroup's range ----------------------------
+  for (int h = tid; h < n_heads; h += 256) {
+    int e = a.row_end ? (int)min((long long)a.row_end[h], (long long)ts) : a.n_rows;
+    sm.tile_prefix[h] = (e + kDecTile - 1) / kDecTile + tail_tiles;
   }
   __syncthreads();
-  for (int idx = tid; idx < NREP * D; idx += 256) {
-    int h = idx / D, d = idx % D;
-    float M = fmaxf(fmaxf(wm[0][h], wm[1][h]), fmaxf(wm[2][h], wm[3][h]));
-    float sum = 0.f, lsum = 0.f;
-    if (M != -INFINITY) {
-#pragma unroll
-      for (int w = 0; w < 4; ++w) {
-        float f = exp2_guard(wm[w][h] - M);
-        sum += wacc[w][h][d] * f;
-        lsum += wl[w][h] * f;
-      }
-    }
-    int64_t head = (int64_t)b * a.Hq + hq0 + h;
-    a.ws_acc[(head * a.nsplit + split) * D + d] = sum;
-    if (d == 0) {
-      a.ws_ml[(head * a.nsplit + split) * 2 + 0] = M;
-      a.ws_ml[(head * a.nsplit + split) * 2 + 1] = lsum;
+  block_exclusive_scan(sm.tile_prefix, n_heads, sm.scan_tmp);
+  const int total = sm.tile_prefix[n_heads];
+  const int tpw = (total + a.n_wg - 1) / a.n_wg;  // tiles per workgroup
+  for (int h = tid; h < n_heads; h += 256) {
+    int p0 = sm.tile_prefix[h], p1 = sm.tile_prefix[h + 1];
+    sm.slot_prefix[h] = p1 > p0 ? (p1 - 1) / tpw - p0 / tpw + 1 : 0;
+  }
+  __syncthreads();
+  block_exclusive_scan(sm.slot_prefix, n_heads, sm.scan_tmp);
+  if (wg == 0 && grp == 0) {
+    for (int h = tid; h < n_heads; h += 256) {
+      a.head_table[h] = make_int2(sm.slot_prefix[h], sm.slot_prefix[h + 1] - sm.slot_prefix[h]);
     }
   }
+  int pos = wg * tpw;
+  const int pos_end = min(pos + tpw, total);
+  if (pos >= pos_end) return;
+  for (int h = tid; h < n_heads; h += 256) {
+    if (sm.tile_prefix[h] <= pos && pos < sm.tile_prefix[h + 1]) sm.first_head = h;
+  }
+  __syncthreads();
+  int ks = sm.first_head;  // b * Hkv + hkv
+  const float c = a.scale * 1.4426950408889634f;
+
+  while (pos < pos_end) {
+    const int p0 = sm.tile_prefix[ks], p1 = sm.tile_prefix[ks + 1];
+    if (p1 == p0) {  // a head without tiles
+      ++ks;
+      continue;
+    }
+    const int seg_end = min(pos_end, p1);
+    const int t_begin = pos - p0, t_end = seg_end - p0;  // tiles of this head
+    const int slot = sm.slot_prefix[ks] + (wg - p0 / tpw);
+
+    const int b = ks / a.Hkv, hkv = ks % a.Hkv;
+    const int hq0 = hkv * a.n_rep + grp * NREP;
+    const uint16_t* kp = static_cast<const uint16_t*>(a.k) + b * a.ks_b + hkv * a.ks_h;
+    const uint16_t* vp = static_cast<const uint16_t*>(a.v) + b * a.ks_b + hkv * a.ks_h;
+    const uint8_t* valp = a.valid + b * a.vs_b + hkv * a.vs_h;
+    // Rows are walked in 32-row tiles over [0, e) and [ts, n_rows); [e, ts) is the dead region between this
+    // head's own end and the open chunk (nothing there is valid), skipped without a look when hinted.
+    const int e = a.row_end ? (int)min((long long)a.row_end[ks], (long long)ts) : a.n_rows;
+    const int nA = (e + kDecTile - 1) / kDecTile;
+
+    // Q as the B operand: column = q head of the group (zero beyond NREP), k = 8 dims per lane group
+    bf16x8 qreg[STEPS];
+    {
+      const uint16_t* qp = static_cast<const uint16_t*>(a.q) + ((int64_t)b * a.Hq + hq0 + (l16 < NREP ? l16 : 0)) * D;
+#pragma unroll
+      for (int s = 0; s < STEPS; ++s) {
+        uint4 raw = *reinterpret_cast<const uint4*>(qp + s * 32 + lg * 8);
+        if (l16 >= NREP) raw = make_uint4(0, 0, 0, 0);
+        qreg[s] = __builtin_bit_cast(bf16x8, raw);
+      }
+    }
+
+    f32x4 oacc[DB];  // O^T block db: lane holds dims db*16 + lg*4 + i of q head l16
+#pragma unroll
+    for (int db = 0; db < DB; ++db) oacc[db] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.f;  // of q head l16 (meaningful for l16 < NREP)
+
+    uint4 kreg[2][STEPS];
+
+    auto tile_row0 = [&](int t) -> int { return t < nA ? t * kDecTile : ts + (t - nA) * kDecTile; };
+    auto tile_row1 = [&](int t) -> int {
+      return t < nA ? min(t * kDecTile + kDecTile, e) : min(ts + (t - nA + 1) * kDecTile, a.n_rows);
+    };
+    auto load_valid = [&](int t) -> uint32_t {
+      uint32_t vb = 0;
+      if (t < t_end) {
+        int r0 = tile_row0(t), r1 = tile_row1(t);
+        if (lane < kDecTile && r0 + lane < r1) vb = valp[r0 + lane];
+      }
+      return vb;
+    };
+    auto issue_k = [&](int r0, uint32_t vm) {
+      const int fv = __builtin_ctz(vm);
+#pragma unroll
+      for (int g = 0; g < 2; ++g) {
+        int kl = g * 16 + l16;
+        int row = ((vm >> kl) & 1) ? kl : fv;
+        const uint16_t* rp = kp + (int64_t)(r0 + row) * a.ks_r + lg * 8;
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) kreg[g][s] = *reinterpret_cast<const uint4*>(rp + s * 32);
+      }
+    };
+    auto issue_v = [&](int r0, uint32_t vm, int buf) {
+      const int fv = __builtin_ctz(vm);
+#pragma unroll
+      for (int j = 0; j < NDMA; ++j) {
+        const int q = j * kWave + lane;  // chunk slot in the LDS tile
+        const int row = q / OCT, cpos = q % OCT;
+        const int src_row = ((vm >> row) & 1) ? row : fv;
+        const int chunk = cpos ^ ((row & 3) << 1);
+        __builtin_amdgcn_global_load_lds(vp + (int64_t)(r0 + src_row) * a.ks_r + chunk * 8,
+                                         (uint32_t __attribute__((address_space(3)))*)(&sm.v[wave][buf][j * kWave * 8]), 16, 0,
+                                         0);
+      }
+    };
+
+    int t = t_begin + wave;
+    int cur = 0;
+    uint32_t vm = (uint32_t)__ballot(load_valid(t) != 0);
+    if (vm) {
+      issue_k(tile_row0(t), vm);
+      issue_v(tile_row0(t), vm, cur);
+    }
+    uint32_t vb_next = load_valid(t + 4);
+
+    while (t < t_end) {
+      __builtin_amdgcn_s_waitcnt(0);  // K(t) in registers, V(t) in LDS, valid bytes of the next tile loaded
+      const uint32_t vmn = (uint32_t)__ballot(vb_next != 0);
+      float sc[2][4];
+      float mx = -INFINITY;
+      if (vm) {
+        // scores: sc[g][i] belongs to key g*16 + lg*4 + i and q head l16
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+          f32x4 s4 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int s = 0; s < STEPS; ++s) {
+            s4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kreg[g][s]), qreg[s], s4, 0, 0, 0);
+          }
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            int kl = g * 16 + lg * 4 + i;
+            float sv = ((vm >> kl) & 1) ? s4[i] : -INFINITY;
+            sc[g][i] = sv;
+            mx = fmaxf(mx, sv);
+          }
+        }
+      }
+      // requests for the next tile go out before this tile's softmax and PV
+      if (vmn) {
+        issue_k(tile_row0(t + 4), vmn);
+        issue_v(tile_row0(t + 4), vmn, cur ^ 1);
+      }
+      vb_next = load_valid(t + 8);
+
+      if (vm) {
+        mx = fmaxf(mx, __shfl_xor(mx, 16));
+        mx = fmaxf(mx, __shfl_xor(mx, 32)) * c;  // vm != 0, so the maximum is finite
+        // raise the running maximum only when it is exceeded by more than the slack (probabilities stay
+        // below 2^slack otherwise); the accumulators are rescaled only then
+        if (__ballot(l16 < NREP && mx > m_run + kDecodeRescaleSlack)) {
+          float m_new = fmaxf(m_run, mx);
+          float alpha = m_run == -INFINITY ? 0.f : exp2_guard(m_run - m_new);
+          l_run *= alpha;
+          m_run = m_new;
+#pragma unroll
+          for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) oacc[db][i] *= alpha;
+        }
+        // P^T as the B operand: slot j < 4 is key lg*4 + j, slot j >= 4 is key 16 + lg*4 + (j - 4)
+        bf16x8 pfrag;
+        float rs = 0.f;
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            float p = exp2_guard(fmaf(sc[g][i], c, -m_run));
+            rs += p;
+            pfrag[g * 4 + i] = (__bf16)p;
+          }
+        }
+        l_run += rs;
+        // V^T fragments: within 16 lanes, lane r reads 4 dims of key (K0 + r / 4) starting at dim
+        // D0 + 4 * (r % 4) and receives keys K0 .. K0 + 3 of dim D0 + r (ds_read_b64_tr_b16)
+        const uint16_t* Vt = sm.v[wave][cur];
+        const int row_lo = lg * 4 + (l16 >> 2);
+        const int row_hi = 16 + row_lo;
+        const int half = l16 & 1;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          const int chunk0 = db * 2 + ((l16 & 3) >> 1);
+          const uint16_t* plo = Vt + row_lo * D + ((chunk0 ^ ((row_lo & 3) << 1)) * 8) + half * 4;
+          const uint16_t* phi = Vt + row_hi * D + ((chunk0 ^ ((row_hi & 3) << 1)) * 8) + half * 4;
+          bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((bf16x4 __attribute__((address_space(3)))*)plo);
+          bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((bf16x4 __attribute__((address_space(3)))*)phi);
+          bf16x8 va = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+          oacc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pfrag, oacc[db], 0, 0, 0);
+        }
+      }
+      t += 4;
+      vm = vmn;
+      cur ^= 1;
+    }
+    __builtin_amdgcn_s_waitcnt(0);
+
+    // ---- merge the wavefronts of the workgroup, emit this head's partial ------------------------------
+    l_run += __shfl_xor(l_run, 16);
+    l_run += __shfl_xor(l_run, 32);
+    if (l16 < NREP) {
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) sm.wacc[wave][l16][db * 16 + lg * 4 + i] = oacc[db][i];
+    }
+    if (lane < NREP) {
+      sm.wm[wave][lane] = m_run;
+      sm.wl[wave][lane] = l_run;
+    }
+    __syncthreads();
+    for (int idx = tid; idx < NREP * D; idx += 256) {
+      int h = idx / D, d = idx % D;
+      float M = fmaxf(fmaxf(sm.wm[0][h], sm.wm[1][h]), fmaxf(sm.wm[2][h], sm.wm[3][h]));
+      float sum = 0.f, lsum = 0.f;
+      if (M != -INFINITY) {
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          float f = exp2_guard(sm.wm[w][h] - M);
+          sum += sm.wacc[w][h][d] * f;
+          lsum += sm.wl[w][h] * f;
+        }
+      }
+      const int64_t prt = (int64_t)slot * a.n_rep + grp * NREP + h;  // partial of (slot, q head in the kv group)
+      a.ws_acc[prt * D + d] = sum;
+      if (d == 0) {
+        a.ws_ml[prt * 2 + 0] = M;
+        a.ws_ml[prt * 2 + 1] = lsum;
+      }
+    }
+    __syncthreads();  // wacc / wm / wl are reused by the next head
+    pos = seg_end;
+    ++ks;
+  }
+}
+
+// merge the partials of one q head (balanced schedule): grid = B*Hq, block = D threads
+__global__ void decode_merge_balanced_kernel(const float* __restrict__ ws_acc, const float* __restrict__ ws_ml,
+                                             const int2* __restrict__ head_table, uint16_t* __restrict__ o, int Hq, int Hkv,
+                                             int D) {
+  const int head = blockIdx.x;  // b * Hq + hq
+  const int d = threadIdx.x;
+  if (d >= D) return;
+  const int n_rep = Hq / Hkv;
+  const int b = head / Hq, hq = head % Hq;
+  const int2 tab = head_table[b * Hkv + hq / n_rep];
+  const int r = hq % n_rep;
+  float M = -INFINITY;
+  for (int s = 0; s < tab.y; ++s) M = fmaxf(M, ws_ml[((int64_t)(tab.x + s) * n_rep + r) * 2]);
+  float sum = 0.f, lsum = 0.f;
+  if (M != -INFINITY) {
+    for (int s = 0; s < tab.y; ++s) {
+      const int64_t prt = (int64_t)(tab.x + s) * n_rep + r;
+      float ms = ws_ml[prt * 2];
+      if (ms == -INFINITY) continue;
+      float f = exp2_guard(ms - M);
+      sum += ws_acc[prt * D + d] * f;
+      lsum += ws_ml[prt * 2 + 1] * f;
+    }
+  }
+  o[(int64_t)head * D + d] = f32_to_bf16_bits(lsum > 0.f ? sum / lsum : 0.f);
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -330,13 +487,43 @@ static void decode_split_geometry(int64_t B, int64_t H_kv, int64_t n_rows, int* 
   if (r < 256) r = 256;
   if (r > 8192) r = 8192;
   *rows_per_split = (int)r;
-  *nsplit = (int)((n_rows + r - 1) / r);
+  // the walk over [0, row_end) and [tail_start, n_rows) can take one 32-row tile more than ceil(n_rows / 32)
+  *nsplit = (int)((n_rows + 32 + r - 1) / r);
 }
 
+// workgroups of the balanced bf16 schedule: two per compute unit, fewer when there is little to do
+static int decode_balanced_workgroups(int64_t B, int64_t H_kv, int64_t n_rows) {
+  static int n_cu = 0;
+  if (n_cu == 0) {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) {
+      n_cu = v;
+    } else {
+      n_cu = 256;
+    }
+  }
+  int64_t upper = B * H_kv * ((n_rows + kDecTile - 1) / kDecTile + 1);  // tiles, at most
+  int64_t want = (upper + 7) / 8;                                        // at least 8 tiles per workgroup
+  int64_t cap = 2 * (int64_t)n_cu;
+  return (int)(want < 1 ? 1 : (want > cap ? cap : want));
+}
+
+static size_t align256(size_t x) { return (x + 255) & ~size_t(255); }
+
 template <int D, int NREP>
-static void launch_mfma(const DecodeArgs& a, int groups, hipStream_t st) {
-  dim3 grid((unsigned)a.nsplit, (unsigned)(a.B * a.Hkv), (unsigned)groups);
-  hipLaunchKernelGGL((decode_split_mfma_kernel<D, NREP>), grid, dim3(256), 0, st, a);
+static int launch_mfma(const DecodeArgs& a, int groups, hipStream_t st) {
+  static bool configured = false;  // the LDS attribute is a property of the kernel
+  const size_t smem = sizeof(DecodeSmem<D, NREP>);
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&decode_split_mfma_kernel<D, NREP>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) return fail(NATS_ERR_LAUNCH, "hipFuncSetAttribute(%zu bytes of LDS): %s", smem, hipGetErrorString(e));
+    configured = true;
+  }
+  dim3 grid((unsigned)a.n_wg, 1u, (unsigned)groups);
+  hipLaunchKernelGGL((decode_split_mfma_kernel<D, NREP>), grid, dim3(256), smem, st, a);
+  return NATS_OK;
 }
 
 }  // namespace nats
@@ -347,13 +534,16 @@ extern "C" size_t nats_decode_workspace_bytes(int64_t B, int64_t H_q, int64_t H_
   if (B <= 0 || H_q <= 0 || H_kv <= 0 || D <= 0 || n_rows <= 0) return 0;
   int rps, ns;
   decode_split_geometry(B, H_kv, n_rows, &rps, &ns);
-  return (size_t)B * H_q * ns * (D + 2) * sizeof(float);
+  size_t split_layout = (size_t)B * H_q * ns * (D + 2) * sizeof(float);  // fp32 kernel: [q head][split]
+  size_t slots = (size_t)decode_balanced_workgroups(B, H_kv, n_rows) + (size_t)(B * H_kv);
+  size_t balanced_layout = align256((size_t)(B * H_kv) * sizeof(int2)) + slots * (H_q / H_kv) * (D + 2) * sizeof(float);
+  return split_layout > balanced_layout ? split_layout : balanced_layout;
 }
 
-extern "C" int nats_decode_fwd(const void* q, const void* cache_k, const void* cache_v, const uint8_t* valid, void* o,
-                               int64_t B, int64_t H_q, int64_t H_kv, int64_t D, int64_t n_rows, const int64_t* kv_strides,
-                               const int64_t* valid_strides, float sm_scale, int dtype, void* workspace,
-                               size_t workspace_bytes, void* stream) {
+extern "C" int nats_decode_fwd(const void* q, const void* cache_k, const void* cache_v, const uint8_t* valid,
+                               const int64_t* row_end, int64_t tail_start, void* o, int64_t B, int64_t H_q, int64_t H_kv,
+                               int64_t D, int64_t n_rows, const int64_t* kv_strides, const int64_t* valid_strides,
+                               float sm_scale, int dtype, void* workspace, size_t workspace_bytes, void* stream) {
   NATS_REQUIRE(q && cache_k && cache_v && valid && o && workspace, NATS_ERR_NULL_POINTER,
                "nats_decode_fwd: NULL pointer argument");
   NATS_REQUIRE(kv_strides && valid_strides, NATS_ERR_NULL_POINTER, "nats_decode_fwd: NULL stride array");
@@ -368,6 +558,8 @@ extern "C" int nats_decode_fwd(const void* q, const void* cache_k, const void* c
   NATS_REQUIRE(n_rows < (int64_t(1) << 30) && B * H_q <= (int64_t(1) << 30), NATS_ERR_BAD_SHAPE,
                "nats_decode_fwd: problem too large");
   NATS_REQUIRE(B * H_kv <= 65535 && B * H_q <= 65535 * 16, NATS_ERR_BAD_SHAPE, "nats_decode_fwd: too many (b, head) streams");
+  NATS_REQUIRE(row_end == nullptr || (tail_start >= 0 && tail_start <= n_rows), NATS_ERR_BAD_SHAPE,
+               "nats_decode_fwd: tail_start=%lld outside [0, n_rows=%lld]", (long long)tail_start, (long long)n_rows);
   size_t need = nats_decode_workspace_bytes(B, H_q, H_kv, D, n_rows);
   NATS_REQUIRE(workspace_bytes >= need, NATS_ERR_WORKSPACE, "nats_decode_fwd: workspace %zu bytes < %zu", workspace_bytes,
                need);
@@ -381,12 +573,16 @@ extern "C" int nats_decode_fwd(const void* q, const void* cache_k, const void* c
   hipStream_t st = static_cast<hipStream_t>(stream);
   DecodeArgs a;
   a.q = q; a.k = cache_k; a.v = cache_v; a.valid = valid; a.o = o;
+  a.row_end = dtype == NATS_DTYPE_BF16 ? row_end : nullptr;
+  a.tail_start = (int)tail_start;
   a.ks_b = kv_strides[0]; a.ks_h = kv_strides[1]; a.ks_r = kv_strides[2];
   a.vs_b = valid_strides[0]; a.vs_h = valid_strides[1];
   a.B = (int)B; a.Hq = (int)H_q; a.Hkv = (int)H_kv; a.n_rep = (int)(H_q / H_kv);
   a.n_rows = (int)n_rows;
   decode_split_geometry(B, H_kv, n_rows, &a.rows_per_split, &a.nsplit);
   a.scale = sm_scale;
+  a.head_table = nullptr;
+  a.n_wg = 0;
   a.ws_acc = static_cast<float*>(workspace);
   a.ws_ml = a.ws_acc + (size_t)B * H_q * a.nsplit * D;
 
@@ -404,27 +600,36 @@ extern "C" int nats_decode_fwd(const void* q, const void* cache_k, const void* c
     return NATS_OK;
   }
 
+  NATS_REQUIRE(B * H_kv <= kMaxBalancedHeads, NATS_ERR_UNSUPPORTED,
+               "nats_decode_fwd: %lld (batch, kv head) streams, the bf16 kernel schedules at most %d", (long long)(B * H_kv),
+               kMaxBalancedHeads);
+  a.n_wg = decode_balanced_workgroups(B, H_kv, n_rows);
+  a.head_table = static_cast<int2*>(workspace);
+  a.ws_acc = reinterpret_cast<float*>(static_cast<char*>(workspace) + align256((size_t)(B * H_kv) * sizeof(int2)));
+  a.ws_ml = a.ws_acc + ((size_t)a.n_wg + (size_t)(B * H_kv)) * (size_t)a.n_rep * D;
   int n_rep = a.n_rep;
   int nrep_k = (n_rep % 8 == 0) ? 8 : (n_rep % 4 == 0) ? 4 : (n_rep % 2 == 0) ? 2 : 1;
   int groups = n_rep / nrep_k;
+  int rc;
   if (D == 128) {
     switch (nrep_k) {
-      case 8: launch_mfma<128, 8>(a, groups, st); break;
-      case 4: launch_mfma<128, 4>(a, groups, st); break;
-      case 2: launch_mfma<128, 2>(a, groups, st); break;
-      default: launch_mfma<128, 1>(a, groups, st); break;
+      case 8: rc = launch_mfma<128, 8>(a, groups, st); break;
+      case 4: rc = launch_mfma<128, 4>(a, groups, st); break;
+      case 2: rc = launch_mfma<128, 2>(a, groups, st); break;
+      default: rc = launch_mfma<128, 1>(a, groups, st); break;
     }
   } else {
     switch (nrep_k) {
-      case 8: launch_mfma<64, 8>(a, groups, st); break;
-      case 4: launch_mfma<64, 4>(a, groups, st); break;
-      case 2: launch_mfma<64, 2>(a, groups, st); break;
-      default: launch_mfma<64, 1>(a, groups, st); break;
+      case 8: rc = launch_mfma<64, 8>(a, groups, st); break;
+      case 4: rc = launch_mfma<64, 4>(a, groups, st); break;
+      case 2: rc = launch_mfma<64, 2>(a, groups, st); break;
+      default: rc = launch_mfma<64, 1>(a, groups, st); break;
     }
   }
+  if (rc) return rc;
   NATS_CHECK_LAUNCH("decode_split_mfma_kernel");
-  hipLaunchKernelGGL((decode_merge_kernel<true>), dim3((unsigned)(B * H_q)), dim3((unsigned)D), 0, st, a.ws_acc, a.ws_ml, o,
-                     a.nsplit, (int)D);
-  NATS_CHECK_LAUNCH("decode_merge_kernel");
+  hipLaunchKernelGGL(decode_merge_balanced_kernel, dim3((unsigned)(B * H_q)), dim3((unsigned)D), 0, st, a.ws_acc, a.ws_ml,
+                     a.head_table, static_cast<uint16_t*>(o), (int)H_q, (int)H_kv, (int)D);
+  NATS_CHECK_LAUNCH("decode_merge_balanced_kernel");
   return NATS_OK;
 }

@@ -37,17 +37,6 @@ struct PrefillArgs {
   float scale;   // softmax scale
 };
 
-// first visited key tile in [from, last] for a query tile whose first role slot is m0, or -1
-__device__ __forceinline__ int next_visited(const int2* __restrict__ tl, int from, int last, int m0, int lane) {
-  for (int base = from; base <= last; base += kWave) {
-    int kt = base + lane;
-    bool v = kt <= last && tl[kt].x >= m0;
-    uint64_t bits = __ballot(v);
-    if (bits) return __builtin_amdgcn_readfirstlane(base + (int)__builtin_ctzll(bits));
-  }
-  return -1;
-}
-
 // ---------------------------------------------------------------------------------------------------
 // fp32 / generic kernel: 64 lanes = 64 query rows, key sub-tiles of 32 rows staged in LDS as fp32.
 // ---------------------------------------------------------------------------------------------------
@@ -169,11 +158,15 @@ __global__ __launch_bounds__(64) void prefill_simple_kernel(PrefillArgs a) {
 // ---------------------------------------------------------------------------------------------------
 constexpr float kRescaleSlack = 8.0f;
 
+constexpr int kWin = 1024;  // key tiles whose visit list is built at once
+
 template <int D>
 struct PrefillSmem {
   uint16_t k[2][kTile * D];
   uint16_t v[2][kTile * D];
   int limk[2][kTile];
+  int4 vlist[kWin];  // visited key tiles of the current window: {tile, max vis_lim, min vis_lim, -}
+  int vcount;
 };
 
 template <int D>
@@ -255,7 +248,7 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
 
   // global -> LDS, one 64-key tile of K and of V; rows beyond L repeat row L-1 (their scores are masked,
   // so their probabilities are exactly 0 and a finite V row contributes nothing)
-  auto issue_tile = [&](int kt, int buf) {
+  auto issue_tile = [&](int kt, int buf, bool need_lim) {
 #pragma unroll
     for (int j = 0; j < DMA_PER_WAVE; ++j) {
       const int inst = wave * DMA_PER_WAVE + j;  // uniform
@@ -269,134 +262,164 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
       __builtin_amdgcn_global_load_lds(vp + (int64_t)n * a.vs_l + vchunk * 8,
                                        (uint32_t __attribute__((address_space(3)))*)(&sm.v[buf][inst * kWave * 8]), 16, 0, 0);
     }
-    if (tid < kTile) {
+    if (need_lim && tid < kTile) {
       int n = kt * kTile + tid;
       sm.limk[buf][tid] = n < a.L ? lim[n >> a.c_shift] : -1;
     }
   };
 
-  int kt = next_visited(tl, 0, qt_hi, m0_group, lane);
-  int cur = 0;
-  if (kt >= 0) issue_tile(kt, 0);
-  __builtin_amdgcn_s_waitcnt(0);
-  __syncthreads();
-
-  while (kt >= 0) {
-    const int nxt = next_visited(tl, kt + 1, qt_hi, m0_group, lane);
-    if (nxt >= 0) issue_tile(nxt, cur ^ 1);
-
-    const int2 tlk = tl[kt];
-    const bool visit = wave_live && kt <= my_qt && tlk.x >= my_m0;
-    if (visit) {
-      const bool full = kt < my_qt && tlk.y >= my_mlast;
-      const uint16_t* Kt = sm.k[cur];
-      const uint16_t* Vt = sm.v[cur];
-      // ---- S^T = K Q^T ---------------------------------------------------------------------------
-      f32x16 sacc[2][2];
+  auto compute_tile = [&](int kt, int cur, bool full) {
+    const uint16_t* Kt = sm.k[cur];
+    const uint16_t* Vt = sm.v[cur];
+    // ---- S^T = K Q^T ---------------------------------------------------------------------------
+    f32x16 sacc[2][2];
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb) {
-        const int row = kb * 32 + l32;
+    for (int kb = 0; kb < 2; ++kb) {
+      const int row = kb * 32 + l32;
 #pragma unroll
-        for (int s = 0; s < DSTEPS; ++s) {
-          const int chunk = (s * 2 + hl) ^ (row % OCT);
-          bf16x8 ka = *reinterpret_cast<const bf16x8*>(Kt + row * D + chunk * 8);
-          if (s == 0) {
-            const f32x16 z = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-            sacc[kb][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qreg[0][s], z, 0, 0, 0);
-            sacc[kb][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qreg[1][s], z, 0, 0, 0);
-          } else {
-            sacc[kb][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qreg[0][s], sacc[kb][0], 0, 0, 0);
-            sacc[kb][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qreg[1][s], sacc[kb][1], 0, 0, 0);
-          }
+      for (int s = 0; s < DSTEPS; ++s) {
+        const int chunk = (s * 2 + hl) ^ (row % OCT);
+        bf16x8 ka = *reinterpret_cast<const bf16x8*>(Kt + row * D + chunk * 8);
+        if (s == 0) {
+          const f32x16 z = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+          sacc[kb][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qreg[0][s], z, 0, 0, 0);
+          sacc[kb][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qreg[1][s], z, 0, 0, 0);
+        } else {
+          sacc[kb][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qreg[0][s], sacc[kb][0], 0, 0, 0);
+          sacc[kb][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qreg[1][s], sacc[kb][1], 0, 0, 0);
         }
       }
-      // ---- mask (diagonal tile, or a tile whose slots are not uniformly visible) -----------------
-      if (!full) {
+    }
+    // ---- mask (diagonal tile, or a tile whose slots are not uniformly visible) -----------------
+    if (!full) {
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
+      for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
-          for (int g4 = 0; g4 < 4; ++g4) {
-            int kk = kb * 32 + g4 * 8 + hl * 4;  // key offset in tile of accumulator 4*g4
-            int4 lm = *reinterpret_cast<const int4*>(&sm.limk[cur][kk]);
-            const int lv[4] = {lm.x, lm.y, lm.z, lm.w};
+        for (int g4 = 0; g4 < 4; ++g4) {
+          int kk = kb * 32 + g4 * 8 + hl * 4;  // key offset in tile of accumulator 4*g4
+          int4 lm = *reinterpret_cast<const int4*>(&sm.limk[cur][kk]);
+          const int lv[4] = {lm.x, lm.y, lm.z, lm.w};
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              int key = kt * kTile + kk + e;
+          for (int e = 0; e < 4; ++e) {
+            int key = kt * kTile + kk + e;
 #pragma unroll
-              for (int qb = 0; qb < 2; ++qb) {
-                int qtok = q0 + qb * 32 + l32;
-                bool vis = key <= qtok && (qtok >> a.c_shift) <= lv[e];
-                if (!vis) sacc[kb][qb][g4 * 4 + e] = -INFINITY;
-              }
+            for (int qb = 0; qb < 2; ++qb) {
+              int qtok = q0 + qb * 32 + l32;
+              bool vis = key <= qtok && (qtok >> a.c_shift) <= lv[e];
+              if (!vis) sacc[kb][qb][g4 * 4 + e] = -INFINITY;
             }
           }
         }
       }
-      // ---- online softmax, one query per lane and q block ----------------------------------------
-      bf16x8 pb[2][4];
+    }
+    // ---- online softmax, one query per lane and q block ----------------------------------------
+    bf16x8 pb[2][4];
 #pragma unroll
-      for (int qb = 0; qb < 2; ++qb) {
-        float mx = -INFINITY;
+    for (int qb = 0; qb < 2; ++qb) {
+      float mx = -INFINITY;
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
+      for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-          for (int i = 0; i < 16; ++i) mx = fmaxf(mx, sacc[kb][qb][i]);
-        mx = fmaxf(mx, __shfl_xor(mx, 32)) * c;
-        if (__ballot(mx > m_run[qb] + kRescaleSlack)) {
-          float m_new = fmaxf(m_run[qb], mx);
-          float alpha = m_run[qb] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_run[qb] - m_new);
-          l_run[qb] *= alpha;
-          m_run[qb] = m_new;
+        for (int i = 0; i < 16; ++i) mx = fmaxf(mx, sacc[kb][qb][i]);
+      mx = fmaxf(mx, __shfl_xor(mx, 32)) * c;
+      if (__ballot(mx > m_run[qb] + kRescaleSlack)) {
+        float m_new = fmaxf(m_run[qb], mx);
+        float alpha = m_run[qb] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_run[qb] - m_new);
+        l_run[qb] *= alpha;
+        m_run[qb] = m_new;
 #pragma unroll
-          for (int dt = 0; dt < DT; ++dt)
+        for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) oacc[dt][qb][i] *= alpha;
-        }
-        const float m_use = m_run[qb] == -INFINITY ? 0.f : m_run[qb];
-        float rs = 0.f;
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
-#pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            float p = __builtin_amdgcn_exp2f(fmaf(sacc[kb][qb][i], c, -m_use));
-            rs += p;
-            pb[qb][kb * 2 + (i >> 3)][i & 7] = (__bf16)p;
-          }
-        }
-        l_run[qb] += rs;
+          for (int i = 0; i < 16; ++i) oacc[dt][qb][i] *= alpha;
       }
-      // ---- O^T += V^T P^T ------------------------------------------------------------------------
-      // ds_read_b64_tr_b16: within 16 lanes, lane r reads 4 dims of key (K0 + r / 4) starting at dim
-      // D0 + 4 * (r % 4) and receives keys K0 .. K0 + 3 of dim D0 + r.
-      const int r16 = lane & 15;
-      const int dsel = (lane >> 4) & 1;
+      const float m_use = m_run[qb] == -INFINITY ? 0.f : m_run[qb];
+      float rs = 0.f;
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        const int chunk0 = dt * 4 + dsel * 2 + ((r16 & 3) >> 1);
-        const int half = r16 & 1;
+      for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          bf16x4 lo, hi;
-          {
-            const int row = t * 16 + hl * 4 + (r16 >> 2);
-            const uint16_t* pa = Vt + row * D + ((chunk0 ^ ((row & 3) << 1)) * 8) + half * 4;
-            lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((bf16x4 __attribute__((address_space(3)))*)pa);
-          }
-          {
-            const int row = t * 16 + 8 + hl * 4 + (r16 >> 2);
-            const uint16_t* pa = Vt + row * D + ((chunk0 ^ ((row & 3) << 1)) * 8) + half * 4;
-            hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((bf16x4 __attribute__((address_space(3)))*)pa);
-          }
-          bf16x8 va = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-          oacc[dt][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb[0][t], oacc[dt][0], 0, 0, 0);
-          oacc[dt][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb[1][t], oacc[dt][1], 0, 0, 0);
+        for (int i = 0; i < 16; ++i) {
+          float p = __builtin_amdgcn_exp2f(fmaf(sacc[kb][qb][i], c, -m_use));
+          rs += p;
+          pb[qb][kb * 2 + (i >> 3)][i & 7] = (__bf16)p;
         }
+      }
+      l_run[qb] += rs;
+    }
+    // ---- O^T += V^T P^T ------------------------------------------------------------------------
+    // ds_read_b64_tr_b16: within 16 lanes, lane r reads 4 dims of key (K0 + r / 4) starting at dim
+    // D0 + 4 * (r % 4) and receives keys K0 .. K0 + 3 of dim D0 + r.
+    const int r16 = lane & 15;
+    const int dsel = (lane >> 4) & 1;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      const int chunk0 = dt * 4 + dsel * 2 + ((r16 & 3) >> 1);
+      const int half = r16 & 1;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        bf16x4 lo, hi;
+        {
+          const int row = t * 16 + hl * 4 + (r16 >> 2);
+          const uint16_t* pa = Vt + row * D + ((chunk0 ^ ((row & 3) << 1)) * 8) + half * 4;
+          lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((bf16x4 __attribute__((address_space(3)))*)pa);
+        }
+        {
+          const int row = t * 16 + 8 + hl * 4 + (r16 >> 2);
+          const uint16_t* pa = Vt + row * D + ((chunk0 ^ ((row & 3) << 1)) * 8) + half * 4;
+          hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((bf16x4 __attribute__((address_space(3)))*)pa);
+        }
+        bf16x8 va = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        oacc[dt][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb[0][t], oacc[dt][0], 0, 0, 0);
+        oacc[dt][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb[1][t], oacc[dt][1], 0, 0, 0);
       }
     }
-    __builtin_amdgcn_s_waitcnt(0);  // the next tile has landed in LDS
-    __syncthreads();                // ... for every wavefront, and this tile is no longer read
-    cur ^= 1;
-    kt = nxt;
+  };
+
+  const int mlast_group = (min(qt_hi * kTile + kTile - 1, a.L - 1)) >> a.c_shift;
+  int cur = 0;
+  for (int w0 = 0; w0 <= qt_hi; w0 += kWin) {
+    // ---- visit list of this window: wavefront 0 compacts the tiles some query tile of the group sees ----
+    if (wave == 0) {
+      int2 vals[kWin / kWave];
+#pragma unroll
+      for (int j = 0; j < kWin / kWave; ++j) {
+        int t = w0 + j * kWave + lane;
+        vals[j] = t <= qt_hi ? tl[t] : make_int2(-1, -1);
+      }
+      int count = 0;
+#pragma unroll
+      for (int j = 0; j < kWin / kWave; ++j) {
+        int t = w0 + j * kWave + lane;
+        bool v = t <= qt_hi && vals[j].x >= m0_group;
+        uint64_t bits = __ballot(v);
+        if (v) sm.vlist[count + __builtin_popcountll(bits & ((uint64_t(1) << lane) - 1))] = make_int4(t, vals[j].x, vals[j].y, 0);
+        count += __builtin_popcountll(bits);
+      }
+      if (lane == 0) sm.vcount = count;
+    }
+    __syncthreads();
+    const int n_vis = sm.vcount;
+    if (n_vis > 0) {
+      issue_tile(sm.vlist[0].x, cur, true);
+      __builtin_amdgcn_s_waitcnt(0);
+      __syncthreads();
+    }
+    for (int idx = 0; idx < n_vis; ++idx) {
+      const int4 ent = sm.vlist[idx];
+      const int kt = ent.x;
+      if (idx + 1 < n_vis) {
+        const int4 en = sm.vlist[idx + 1];
+        // the element mask is only evaluated on diagonal tiles and on tiles with mixed visibility
+        issue_tile(en.x, cur ^ 1, en.x >= qt_lo || en.z < mlast_group);
+      }
+      const bool visit = wave_live && kt <= my_qt && ent.y >= my_m0;
+      if (visit) {
+        const bool full = kt < my_qt && ent.z >= my_mlast;
+        compute_tile(kt, cur, full);
+      }
+      __builtin_amdgcn_s_waitcnt(0);  // the next tile has landed in LDS
+      __syncthreads();                // ... for every wavefront, and this tile is no longer read
+      cur ^= 1;
+    }
   }
 
   // ---- epilogue -----------------------------------------------------------------------------------

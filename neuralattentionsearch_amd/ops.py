@@ -181,11 +181,14 @@ def nats_prefill(q, k, v, end_seqs_idx, sliding_tokens, sm_scale, nats_chunk_siz
 # decode
 # ------------------------------------------------------------------------------------------------
 def decode_attention(q: torch.Tensor, cache_k: torch.Tensor, cache_v: torch.Tensor, valid: torch.Tensor, n_rows: int,
-                     sm_scale: float | None = None) -> torch.Tensor:
+                     sm_scale: float | None = None, row_end: torch.Tensor | None = None,
+                     tail_start: int | None = None) -> torch.Tensor:
     """One query token per sequence over the evicted cache.
 
     q [B, H_q, 1, D]; cache_k / cache_v [B, H_kv, >= n_rows, D]; valid bool / uint8 [B, H_kv, >= n_rows].
-    Attends to rows i < n_rows with valid[b, h, i]; returns [B, H_q, 1, D]."""
+    Attends to rows i < n_rows with valid[b, h, i]; returns [B, H_q, 1, D].
+    Optional hint: `row_end` int64 [B, H_kv] and `tail_start` state that rows [row_end, tail_start) of a head
+    hold nothing valid (size_global_kv + size_local_kv and the start of the open chunk); they are skipped."""
     _require_cuda(q, cache_k, cache_v, valid)
     lib = _lib.load()
     B, Hq, one, D = q.shape
@@ -207,7 +210,12 @@ def decode_attention(q: torch.Tensor, cache_k: torch.Tensor, cache_v: torch.Tens
     scale = (1.0 / math.sqrt(D)) if sm_scale is None else float(sm_scale)
     nbytes = lib.nats_decode_workspace_bytes(B, Hq, Hkv, D, n_rows)
     ws = workspace(q.device, "decode", nbytes)
-    check(lib.nats_decode_fwd(_ptr(qc), _ptr(cache_k), _ptr(cache_v), _ptr(valid), _ptr(out), B, Hq, Hkv, D, n_rows,
+    if row_end is not None:
+        if tail_start is None or tuple(row_end.shape) != (B, Hkv) or row_end.dtype != torch.int64:
+            raise ValueError("row_end must be int64 [B, H_kv] and come with tail_start")
+        row_end = row_end.contiguous()
+    check(lib.nats_decode_fwd(_ptr(qc), _ptr(cache_k), _ptr(cache_v), _ptr(valid), _ptr(row_end),
+                              0 if tail_start is None else int(tail_start), _ptr(out), B, Hq, Hkv, D, n_rows,
                               i64_array(cache_k.stride()[:3]), i64_array(valid.stride()[:2]), scale, _dtype_code(q),
                               _ptr(ws), ws.numel(), _stream(q)))
     return out.view(B, Hq, 1, D)

@@ -35,6 +35,8 @@ def ragged_cache(seed, B, Hkv, D, W, C, n_max_chunks, dtype, frac=(0.1, 1.0), fi
     if poison:
         k[~vt] = float("nan")
         v[~vt] = float("nan")
+    ragged_cache.row_end = torch.from_numpy(W + lens)  # per head: end of its global + local rows
+    ragged_cache.tail_start = base  # first row of the open chunk
     return k, v, vt, n_rows
 
 
@@ -49,6 +51,12 @@ def run_case(B, Hq, Hkv, D, W, C, n_max_chunks, dtype, seed=0, frac=(0.1, 1.0), 
     assert torch.isfinite(got).all(), "a row with valid == False was read (NaN poison leaked)"
     err = (got - want).abs().max().item()
     assert err <= TOL[dtype], f"max abs err {err}"
+    # the same call with the dead-region hint the cache object passes
+    got2 = ops.decode_attention(q.cuda(), k.cuda(), v.cuda(), valid.cuda(), n_rows, row_end=ragged_cache.row_end.cuda(),
+                                tail_start=ragged_cache.tail_start).cpu().float()
+    assert torch.isfinite(got2).all()
+    err2 = (got2 - want).abs().max().item()
+    assert err2 <= TOL[dtype], f"max abs err with hint {err2}"
 
 
 @pytest.mark.parametrize("n_rep", [1, 2, 4, 8])
