@@ -51,12 +51,13 @@ __device__ __forceinline__ float exp2_guard(float x) { return __builtin_amdgcn_e
 constexpr float kDecodeRescaleSlack = 8.0f;
 constexpr int kDecTile = 32;
 
-constexpr int kMaxBalancedHeads = 2048;  // (b, kv head) streams whose tile prefix sums fit in LDS
+constexpr int kMaxBalancedHeads = 1024;  // (b, kv head) streams whose tile prefix sums fit in LDS
 
 template <int D, int NREP>
 struct DecodeSmem {
-  uint16_t v[4][2][kDecTile * D];  // [wave][buffer]
-  float wacc[4][NREP][D];
+  // [wave][buffer]; after a head's tile loop the wavefront's own buffers hold its accumulators
+  // (NREP * D floats <= 2 * kDecTile * D bf16 for NREP <= 16)
+  uint16_t v[4][2][kDecTile * D];
   float wm[4][NREP];
   float wl[4][NREP];
   int tile_prefix[kMaxBalancedHeads + 1];  // exclusive prefix of 32-row tiles per (b, kv head)
@@ -74,14 +75,21 @@ __device__ __forceinline__ void block_exclusive_scan(int* dst, int n, int* tmp) 
   for (int i = lo; i < hi; ++i) sum += dst[i];
   tmp[tid] = sum;
   __syncthreads();
-  if (tid == 0) {
-    int run = 0;
-    for (int i = 0; i < 256; ++i) {
-      int x = tmp[i];
-      tmp[i] = run;
-      run += x;
+  if (tid < kWave) {  // wavefront 0 scans the 256 partial sums, 4 per lane
+    int x0 = tmp[tid * 4], x1 = tmp[tid * 4 + 1], x2 = tmp[tid * 4 + 2], x3 = tmp[tid * 4 + 3];
+    int mine = x0 + x1 + x2 + x3;
+    int incl = mine;
+#pragma unroll
+    for (int o = 1; o < kWave; o <<= 1) {
+      int y = __shfl_up(incl, o);
+      if (tid >= o) incl += y;
     }
-    dst[n] = run;
+    int run = incl - mine;
+    tmp[tid * 4] = run;
+    tmp[tid * 4 + 1] = run + x0;
+    tmp[tid * 4 + 2] = run + x0 + x1;
+    tmp[tid * 4 + 3] = run + x0 + x1 + x2;
+    if (tid == kWave - 1) dst[n] = incl;
   }
   __syncthreads();
   int run = tmp[tid];
@@ -316,11 +324,12 @@ __global__ __launch_bounds__(256) void decode_split_mfma_kernel(DecodeArgs a) {
     // ---- merge the wavefronts of the workgroup, emit this head's partial ------------------------------
     l_run += __shfl_xor(l_run, 16);
     l_run += __shfl_xor(l_run, 32);
+    float* wacc_mine = reinterpret_cast<float*>(&sm.v[wave][0][0]);  // [NREP][D], this wavefront's tiles are consumed
     if (l16 < NREP) {
 #pragma unroll
       for (int db = 0; db < DB; ++db)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) sm.wacc[wave][l16][db * 16 + lg * 4 + i] = oacc[db][i];
+        for (int i = 0; i < 4; ++i) wacc_mine[l16 * D + db * 16 + lg * 4 + i] = oacc[db][i];
     }
     if (lane < NREP) {
       sm.wm[wave][lane] = m_run;
@@ -335,7 +344,7 @@ __global__ __launch_bounds__(256) void decode_split_mfma_kernel(DecodeArgs a) {
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
           float f = exp2_guard(sm.wm[w][h] - M);
-          sum += sm.wacc[w][h][d] * f;
+          sum += reinterpret_cast<const float*>(&sm.v[w][0][0])[h * D + d] * f;
           lsum += sm.wl[w][h] * f;
         }
       }
