@@ -28,6 +28,13 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
+# HBM bytes per launch of the dominant kernels at the default workloads, from rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE scaled by a 1 GiB device copy (read factor 2.0, write factor 1.0); see profiles/.
+MEASURED_TRAFFIC = {
+    "prefill": {"fetch_bytes": 232628 * 1024 * 2.0, "write_bytes": 294866 * 1024 * 1.0},
+    "decode": {"fetch_bytes": 887027 * 1024 * 2.0, "write_bytes": 1560 * 1024 * 1.0},
+    "evict": {"fetch_bytes": 272937 * 1024 * 2.0, "write_bytes": 554050 * 1024 * 1.0},
+}
 PEAK_HBM_GBS = 8000.0
 PEAK_BF16_TFLOPS = 2500.0
 METRIC = "NAtS prefill ms @32k (MFMA util); sparse-KV decode tok/s (HBM GB/s %peak)"
@@ -302,17 +309,19 @@ def main():
     }
     if pre:
         line["roofline"] = {"bound": "mfma", "achieved": pre["tflops_visited"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                            "frac": pre["tflops_visited"] / PEAK_BF16_TFLOPS, "traffic": None,
+                            "frac": pre["tflops_visited"] / PEAK_BF16_TFLOPS,
+                            "traffic": MEASURED_TRAFFIC["prefill"] if args.prefill_len == 32768 else None,
                             "kernel": "prefill_mfma_kernel<128>"}
     if "decode" in res:
         d = res["decode"]
         line["roofline_decode"] = {"bound": "hbm", "achieved": d["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                                   "frac": d["frac_of_hbm_peak"], "traffic": None,
-                                   "kernel": "decode_split_mfma_kernel<128,4> + decode_merge_kernel"}
+                                   "frac": d["frac_of_hbm_peak"], "traffic": MEASURED_TRAFFIC["decode"],
+                                   "kernel": "decode_split_mfma_kernel<128,4> + decode_merge_balanced_kernel"}
     if "evict" in res:
         e = res["evict"]
         line["roofline_evict"] = {"bound": "hbm", "achieved": e["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                                  "frac": e["frac_of_hbm_peak"], "traffic": None, "kernel": "evict_apply_first_kernel"}
+                                  "frac": e["frac_of_hbm_peak"], "traffic": MEASURED_TRAFFIC["evict"],
+                                  "kernel": "evict_plan_* + evict_apply_first_kernel (whole post_update)"}
     line["cpu_baseline"] = cpu
     line.update(res)
     print(json.dumps(line))
