@@ -30,10 +30,10 @@ if ROOT not in sys.path:
 
 # HBM bytes per launch of the dominant kernels at the default workloads, from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE scaled by a 1 GiB device copy (read factor 2.0, write factor 1.0); see profiles/.
-MEASURED_TRAFFIC = {
-    "prefill": {"fetch_bytes": 232628 * 1024 * 2.0, "write_bytes": 294866 * 1024 * 1.0},
-    "decode": {"fetch_bytes": 887027 * 1024 * 2.0, "write_bytes": 1560 * 1024 * 1.0},
-    "evict": {"fetch_bytes": 272937 * 1024 * 2.0, "write_bytes": 554050 * 1024 * 1.0},
+MEASURED_TRAFFIC = {  # bytes read + written per launch
+    "prefill": 232628 * 1024 * 2.0 + 294866 * 1024 * 1.0,
+    "decode": 887027 * 1024 * 2.0 + 1560 * 1024 * 1.0,
+    "evict": 272937 * 1024 * 2.0 + 554050 * 1024 * 1.0,
 }
 PEAK_HBM_GBS = 8000.0
 PEAK_BF16_TFLOPS = 2500.0
