@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define NATS_ABI_VERSION 1
+#define NATS_ABI_VERSION 2
 
 typedef enum {
   NATS_OK = 0,
@@ -43,7 +43,7 @@ int nats_abi_version(void);
 const char* nats_last_error(void);
 
 /* ------------------------------------------------------------------------------------------------
- * (a-1) role assignment.  Replaces BaseNAtSAttentionLayer._sample_for_token_info_values_inference
+ * Role assignment.  Replaces BaseNAtSAttentionLayer._sample_for_token_info_values_inference
  * (models/transformer/attention/nats_attention.py:96-109) and the open-chunk rule of
  * models/transformer/attention/nats_chunk_attention.py:92-94.
  *   logits  [B, S, H_kv, 3] contiguous, dtype bf16 or f32
@@ -56,7 +56,7 @@ int nats_roles_from_logits(const void* logits, int dtype, int64_t B, int64_t S, 
                            int force_first_global, int force_last_global, uint8_t* roles, void* one_hot,
                            void* stream);
 
-/* (a-2) next-global index and the per-slot visibility limit derived from it.
+/* next-global index and the per-slot visibility limit derived from it.
  * Replaces the first half of generate_hard_seq_masks (components/masks/utils.py:85-87).
  *   roles    [B, H_kv, S] uint8
  *   end_idx  [B, H_kv, S] int64 out, may be NULL: first global slot >= n, the last slot counting as global
@@ -67,24 +67,24 @@ int nats_role_scan(const uint8_t* roles, int64_t B, int64_t H_kv, int64_t S, int
                    int32_t* vis_lim, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
- * (a-3) debug / parity output: the token-level bool mask of a prefill from an empty cache, as
+ * debug / parity output: the token-level bool mask of a prefill from an empty cache, as
  * NAtSChunkLayerCache.generate_mask builds it (components/cache/nats_chunk_layer_cache.py:589-620),
- * evaluated with the same predicate the prefill kernels use.
- *   vis_lim [B, H_kv, S] int32 from nats_role_scan, S = ceil(L / C)
- *   mask    [B, H_kv, L, L] uint8 out (1 = attend)
+ * evaluated with the same per-key limits the prefill kernels use.
+ *   roles     [B, H_kv, S] uint8, S = ceil(L / C)
+ *   mask      [B, H_kv, L, L] uint8 out (1 = attend)
+ *   workspace nats_prefill_workspace_bytes(B, *, H_kv, L, *, C) bytes
  */
-int nats_prefill_mask(const int32_t* vis_lim, int64_t B, int64_t H_kv, int64_t L, int64_t C, uint8_t* mask,
-                      void* stream);
+int nats_prefill_mask(const uint8_t* roles, int64_t B, int64_t H_kv, int64_t L, int64_t C, int64_t W, uint8_t* mask,
+                      void* workspace, size_t workspace_bytes, void* stream);
 
-/* (a-3) debug / parity output: the block-sparse tile-skip map the prefill kernel walks.
- *   tile_lim_ws  B * H_kv * T * 8 bytes of scratch, T = ceil(L / 64)
- *   tiles        [B, H_kv, T, T] uint8 out: 1 = the 64x64 tile (query tile, key tile) is loaded
+/* debug / parity output: the block-sparse tile-skip map the prefill kernel walks.
+ *   tiles  [B, H_kv, T, T] uint8 out, T = ceil(L / 64): 1 = the 64x64 tile (query tile, key tile) is loaded
  */
-int nats_prefill_tile_map(const int32_t* vis_lim, int64_t B, int64_t H_kv, int64_t L, int64_t C, void* tile_lim_ws,
-                          uint8_t* tiles, void* stream);
+int nats_prefill_tile_map(const uint8_t* roles, int64_t B, int64_t H_kv, int64_t L, int64_t C, int64_t W,
+                          uint8_t* tiles, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
- * (a-4, a-5) role-masked chunked flash-attention prefill from an empty cache.
+ * role-masked chunked flash-attention prefill from an empty cache.
  * Replaces nats_prefill(...) with global_kv_size=None (models/transformer/triton/nats_flashattn_fwd.py:617-692)
  * and the generate_mask + SDPA branch of multi_head_attention
  * (models/transformer/attention/nats_chunk_attention.py:130-149).
@@ -92,7 +92,7 @@ int nats_prefill_tile_map(const int32_t* vis_lim, int64_t B, int64_t H_kv, int64
  *   three strides are given in elements (stride_b, stride_h, stride_l)
  *   roles [B, H_kv, S] uint8, S = ceil(L / C)
  *   workspace: nats_prefill_workspace_bytes(...) bytes of device memory (contents need not be kept)
- * D in {64, 128}; C a power of two in [1, 64] or a multiple of 64; W % C == 0; H_q % H_kv == 0.
+ * D in {64, 128}; C a power of two; W % C == 0; H_q % H_kv == 0.
  * dtype bf16 runs QK^T and PV on bf16 MFMA with fp32 softmax state; dtype f32 runs an fp32 FMA kernel.
  */
 size_t nats_prefill_workspace_bytes(int64_t B, int64_t H_q, int64_t H_kv, int64_t L, int64_t D, int64_t C);
@@ -103,7 +103,49 @@ int nats_prefill_fwd(const void* q, const void* k, const void* v, const uint8_t*
                      int dtype, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
- * (a-8) one-token decode attention over the evicted, ragged cache.
+ * A multi-token segment over a cache that earlier segments have filled and evicted.
+ * Replaces NAtSChunkLayerCache._generate_mask for x_len > 1 over a non-empty cache
+ * (components/cache/nats_chunk_layer_cache.py:462-511, with _fit_sliding_queue_masks :658-713) followed by
+ * SDPA over cache_k / cache_v[:, :, :n_ctx_data + x_len]
+ * (models/transformer/attention/nats_chunk_attention.py:130-149).  Call it after the cache update that
+ * appended the segment's keys / values and before the eviction of that segment.
+ *
+ * nats_past_state holds the cache scalars as they stand before the segment is evicted:
+ */
+typedef struct {
+  int64_t n_ctx_data; /* live rows before the segment was appended (the segment sits at rows
+                         [n_ctx_data, n_ctx_data + x_len)) */
+  int64_t old_fill;   /* tokens of the open chunk cached before the segment: chunk_fill_size - x_len */
+  int64_t gmin;       /* _n_global_min */
+  int64_t tail;       /* sliding_queue_tail */
+  int64_t seen;       /* _seen_tokens (not yet counting the segment) */
+  int64_t fill_last;  /* chunk_fill_size_last */
+} nats_past_state;
+
+/*   q [B, H_q, x_len, D], o like q; cache_k / cache_v [B, H_kv, >= n_ctx_data + x_len, D]
+ *   valid [B, H_kv, >= n_ctx_data] uint8 (valid_tokens), strides (stride_b, stride_h)
+ *   size_global / size_local [B, H_kv] int64 contiguous
+ *   roles [B, H_kv, S] uint8, S = ceil((old_fill + x_len) / C): one slot per chunk of the open-chunk region
+ *   workspace: nats_prefill_past_workspace_bytes(B, H_kv, n_ctx_data + x_len, S) bytes
+ * Query i is token old_fill + i of the region that starts at row n_ctx_data - old_fill.
+ */
+size_t nats_prefill_past_workspace_bytes(int64_t B, int64_t H_kv, int64_t n_rows, int64_t S);
+
+int nats_prefill_past_fwd(const void* q, const void* cache_k, const void* cache_v, const uint8_t* valid,
+                          const int64_t* size_global, const int64_t* size_local, const uint8_t* roles, void* o,
+                          int64_t B, int64_t H_q, int64_t H_kv, int64_t x_len, int64_t D, int64_t C, int64_t W,
+                          const nats_past_state* state, const int64_t* q_strides, const int64_t* k_strides,
+                          const int64_t* v_strides, const int64_t* valid_strides, const int64_t* o_strides,
+                          float sm_scale, int dtype, void* workspace, size_t workspace_bytes, void* stream);
+
+/* debug / parity output: the mask of that segment, [B, H_kv, x_len, n_ctx_data + x_len] uint8 */
+int nats_prefill_past_mask(const uint8_t* valid, const int64_t* size_global, const int64_t* size_local,
+                           const uint8_t* roles, int64_t B, int64_t H_kv, int64_t x_len, int64_t C, int64_t W,
+                           const nats_past_state* state, const int64_t* valid_strides, uint8_t* mask, void* workspace,
+                           size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * one-token decode attention over the evicted, ragged cache.
  * Replaces _generate_mask_one_step + SDPA (components/cache/nats_chunk_layer_cache.py:622-632,
  * models/transformer/attention/nats_chunk_attention.py:131-142) and the flattened varlen call of
  * models/transformer/hf/llama.py:274-295.
@@ -125,7 +167,7 @@ int nats_decode_fwd(const void* q, const void* cache_k, const void* cache_v, con
                     void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
- * (a-7) KV eviction + compaction: NAtSChunkLayerCache._post_update from its ring insert to its
+ * KV eviction + compaction: NAtSChunkLayerCache._post_update from its ring insert to its
  * valid_tokens rewrite (components/cache/nats_chunk_layer_cache.py:270-371, 391-437, 634-656, 715-868)
  * with merge_local_to_global_caches (components/cache/cache_update.py:25-76).
  *

@@ -18,7 +18,7 @@ c_i64p = ctypes.POINTER(ctypes.c_int64)
 NATS_DTYPE_BF16 = 0
 NATS_DTYPE_F32 = 1
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 
 class EvictParams(ctypes.Structure):
@@ -33,6 +33,11 @@ class EvictResult(ctypes.Structure):
                 ("n_ctx_data", "gmin", "all_sw", "all_local", "max_keep", "max_end", "moved_rows", "reserved")]
 
 
+class PastState(ctypes.Structure):
+    """nats_past_state"""
+    _fields_ = [(n, c_i64) for n in ("n_ctx_data", "old_fill", "gmin", "tail", "seen", "fill_last")]
+
+
 # every symbol include/nats_hip.h declares: name -> (restype, argtypes)
 SIGNATURES = {
     "nats_abi_version": (ctypes.c_int, []),
@@ -40,12 +45,17 @@ SIGNATURES = {
     "nats_roles_from_logits": (ctypes.c_int, [c_p, ctypes.c_int, c_i64, c_i64, c_i64, ctypes.c_float, ctypes.c_int,
                                               ctypes.c_int, c_p, c_p, c_p]),
     "nats_role_scan": (ctypes.c_int, [c_p, c_i64, c_i64, c_i64, c_i64, c_i64, c_p, c_p, c_p]),
-    "nats_prefill_mask": (ctypes.c_int, [c_p, c_i64, c_i64, c_i64, c_i64, c_p, c_p]),
-    "nats_prefill_tile_map": (ctypes.c_int, [c_p, c_i64, c_i64, c_i64, c_i64, c_p, c_p, c_p]),
+    "nats_prefill_mask": (ctypes.c_int, [c_p, c_i64, c_i64, c_i64, c_i64, c_i64, c_p, c_p, ctypes.c_size_t, c_p]),
+    "nats_prefill_tile_map": (ctypes.c_int, [c_p, c_i64, c_i64, c_i64, c_i64, c_i64, c_p, c_p, ctypes.c_size_t, c_p]),
     "nats_prefill_workspace_bytes": (ctypes.c_size_t, [c_i64] * 6),
     "nats_prefill_fwd": (ctypes.c_int, [c_p, c_p, c_p, c_p, c_p, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64,
                                         c_i64p, c_i64p, c_i64p, c_i64p, ctypes.c_float, ctypes.c_int, c_p,
                                         ctypes.c_size_t, c_p]),
+    "nats_prefill_past_workspace_bytes": (ctypes.c_size_t, [c_i64] * 4),
+    "nats_prefill_past_fwd": (ctypes.c_int, [c_p] * 8 + [c_i64] * 7 + [ctypes.POINTER(PastState)] + [c_i64p] * 5 +
+                              [ctypes.c_float, ctypes.c_int, c_p, ctypes.c_size_t, c_p]),
+    "nats_prefill_past_mask": (ctypes.c_int, [c_p] * 4 + [c_i64] * 5 + [ctypes.POINTER(PastState), c_i64p, c_p, c_p,
+                                                                         ctypes.c_size_t, c_p]),
     "nats_decode_workspace_bytes": (ctypes.c_size_t, [c_i64] * 5),
     "nats_decode_fwd": (ctypes.c_int, [c_p, c_p, c_p, c_p, c_p, c_i64, c_p, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64p,
                                        c_i64p, ctypes.c_float, ctypes.c_int, c_p, ctypes.c_size_t, c_p]),

@@ -8,8 +8,8 @@ outside this build).  Differences a caller can see:
 * keys / values are never repeated to H_q heads: the kernels read the kv heads directly (``repeat_kv_values``
   returns its arguments);
 * no [B, H, L, N] mask is built: ``multi_head_attention`` calls the prefill kernel for a multi-token segment
-  over an empty cache and the decode kernel for one token; ``cache.generate_mask`` stays available for
-  inspection.
+  (over an empty cache, or over the rows earlier segments left) and the decode kernel for one token;
+  ``cache.generate_mask`` stays available for inspection.
 """
 from __future__ import annotations
 
@@ -179,7 +179,7 @@ class BaseNAtSChunkAttentionLayer(BaseNAtSAttentionLayer):
             output = ops.prefill_attention(xq, keys, values, roles, self.chunk_size, self.local_seq_max_length,
                                            self.sm_scale)
         else:
-            raise NotImplementedError("a multi-token segment over a non-empty cache is not built yet")
+            output = layer.segment_attention(xq, self.sm_scale)
         if self.executor is not None:
             self._cache_is_till_updating = self.executor.submit(cache.post_update, layer_idx=self.layer_id, x_len=x_len)
             self._cache_is_till_updating.result()

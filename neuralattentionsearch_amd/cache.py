@@ -209,7 +209,28 @@ class NAtSChunkLayerCache:
             if self._roles is None:
                 raise ValueError("generate_mask needs the roles handed to update")
             return ops.prefill_mask(self._roles, x_len, self.chunk_size, self.sliding_window_size)
-        raise NotImplementedError("masks of a multi-token segment over an existing cache are not built yet")
+        return ops.prefill_past_mask(self._buf_valid, self.size_global_kv, self.size_local_kv, self.segment_roles(),
+                                     x_len, self.chunk_size, self.sliding_window_size, self.past_state(x_len))
+
+    def past_state(self, x_len: int):
+        """The scalars a segment of x_len tokens, appended by the last update and not yet evicted, is masked
+        with (nats_chunk_layer_cache.py:462-511)."""
+        return ops.past_state(self.n_ctx_data, self.chunk_fill_size - x_len, self._n_global_min, self.sliding_queue_tail,
+                              self._seen_tokens, self.chunk_fill_size_last)
+
+    def segment_roles(self):
+        """Roles handed to the last update; one global slot while the open chunk is not complete (:589-596)."""
+        if self._roles is not None:
+            return self._roles
+        return torch.zeros(self.bsz, self.n_msks, 1, dtype=torch.uint8, device=self.device)
+
+    def segment_attention(self, q: torch.Tensor, sm_scale: float | None = None):
+        """Attention of the multi-token segment the last update appended, over the whole cache: what the
+        reference computes as SDPA(q, cache_k, cache_v, generate_mask(x_len)) for a non-empty cache."""
+        x_len = q.shape[2]
+        return ops.prefill_past_attention(q, self._buf_k, self._buf_v, self._buf_valid, self.size_global_kv,
+                                          self.size_local_kv, self.segment_roles(), self.chunk_size,
+                                          self.sliding_window_size, self.past_state(x_len), sm_scale)
 
     # -- evict + compact (nats_chunk_layer_cache.py:258-389) -------------------------------------
     def post_update(self, x_len: int):

@@ -52,6 +52,43 @@ __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
   return uint16_t(u >> 16);
 }
 
+// ---- key visibility limits shared by the prefill kernels and the mask / tile-map outputs ----------------
+// State an earlier segment left in the cache, as the segment kernels need it.
+struct PastView {
+  const uint8_t* valid;  // valid_tokens, [B, H_kv, >= base]
+  int64_t valid_s_b, valid_s_h;
+  const int64_t* size_global;  // [B * H_kv]
+  const int64_t* size_local;   // [B * H_kv]
+  int64_t base;                // first cache row of the open-chunk region = n_ctx_data - old_fill
+  int64_t gmin, tail, seen, fill_last;
+};
+
+struct KeyLimArgs {
+  const int32_t* vis_lim;       // [streams, S] slot-level limits of the segment's roles
+  const int32_t* first_global;  // [streams] first global slot of the segment
+  const uint8_t* valid;
+  int64_t valid_s_b, valid_s_h;
+  const int64_t* size_global;
+  const int64_t* size_local;
+  int32_t* tok_lim;  // [streams, N] out
+  int2* tile_lim;    // [streams, Tk] out {max, min}
+  int Hkv, S, N, Tk, c_shift, C, W;
+  int base, gmin, tail, seen, fill_last;
+};
+
+struct PrefillWorkspace {
+  int32_t* vis_lim;
+  int32_t* first_global;
+  int32_t* tok_lim;
+  int2* tile_lim;
+  size_t bytes;
+};
+
+PrefillWorkspace carve_prefill_workspace(void* ws, int64_t n_streams, int64_t S, int64_t N);
+int prepare_key_limits(const uint8_t* roles, int64_t B, int64_t H_kv, int64_t S, int64_t N, int64_t C, int64_t W,
+                       const PastView* past, const PrefillWorkspace& w, hipStream_t st);
+int check_past_state(const char* who, const nats_past_state* ps, int64_t x_len, int64_t C, int64_t W);
+
 // Orders LDS traffic between the lanes of one wavefront (no workgroup barrier needed for wave-private LDS).
 __device__ __forceinline__ void wave_lds_sync() {
   __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");

@@ -4,35 +4,36 @@
 //   prefill_mfma_kernel   bf16, QK^T and PV on v_mfma_f32_32x32x16_bf16, fp32 online softmax
 //   prefill_simple_kernel fp32 (or bf16) FMA kernel, one query row per lane; the fp32 parity path
 //
-// Mask semantics (components/masks/utils.py:89-94, components/cache/nats_chunk_layer_cache.py:603-616):
-// query token m sees key token n iff n <= m and slot(m) <= vis_lim[slot(n)].
+// Mask semantics (components/masks/utils.py:89-94, components/cache/nats_chunk_layer_cache.py:462-511, 603-616):
+// the queries are tokens [r_begin, r_end) of the open-chunk region, which starts at key row `base`; every key
+// row carries the last region token that sees it (tok_lim, built from the roles of the segment and, for
+// rows below base, from the state earlier segments left in the cache).  Query token r sees key row n iff
+//   r <= tok_lim[n]  and  n - base <= r          (rows below base are older than every query).
+// A prefill from an empty cache is the case base = 0, r_begin = 0.
 #include "nats_common.h"
 
 namespace nats {
-
-int launch_role_scan(const uint8_t* roles, int64_t n_streams, int64_t S, int64_t W, int64_t C, int64_t* end_idx,
-                     int32_t* vis_lim, hipStream_t st);
-int launch_tile_lim(const int32_t* vis_lim, int64_t n_streams, int64_t S, int64_t T, int64_t C, int2* tile_lim,
-                    hipStream_t st);
 
 struct PrefillArgs {
   const void* q;
   const void* k;
   const void* v;
   void* o;
-  const int32_t* vis_lim;  // [B*Hkv, S]
-  const int2* tile_lim;    // [B*Hkv, T] {max, min}
+  const int32_t* tok_lim;  // [B*Hkv, N]
+  const int2* tile_lim;    // [B*Hkv, Tk] {max, min}
   int64_t qs_b, qs_h, qs_l;
   int64_t ks_b, ks_h, ks_l;
   int64_t vs_b, vs_h, vs_l;
   int64_t os_b, os_h, os_l;
   int B, Hq, Hkv, n_rep;
-  int L, S, T;
-  int c_shift;
+  int N, Tk;             // key rows and 64-row key tiles
+  int base;              // first key row of the region
+  int r_begin, r_end;    // region tokens that are queries; query i of q / o is token r_begin + i
+  int qt_first, qt_last; // 64-token region tiles that hold queries
   int hpw;       // q heads of one kv head handled by one workgroup (mfma kernel)
   int qpw;       // 64-row query tiles handled by one workgroup (mfma kernel)
   int n_hg;      // head groups per kv head = n_rep / hpw
-  int n_qg;      // query tile groups = ceil(T / qpw)
+  int n_qg;      // query tile groups = ceil(n query tiles / qpw)
   int xcd_mode;  // 1: workgroups of one kv stream share an XCD (needs B*Hkv % 8 == 0)
   float scale;   // softmax scale
 };
@@ -63,44 +64,43 @@ __global__ __launch_bounds__(64) void prefill_simple_kernel(PrefillArgs a) {
   __shared__ int limk[SUB];
 
   const int lane = threadIdx.x;
-  const int qt = a.T - 1 - (int)blockIdx.x;  // heavy query tiles first
+  const int qt = a.qt_last - (int)blockIdx.x;  // heavy query tiles first
   const int bh = blockIdx.y;
   const int b = bh / a.Hq, hq = bh % a.Hq, hkv = hq / a.n_rep;
   const int stream = b * a.Hkv + hkv;
-  const int32_t* lim = a.vis_lim + (int64_t)stream * a.S;
+  const int32_t* lim = a.tok_lim + (int64_t)stream * a.N;
   const T* qp = static_cast<const T*>(a.q) + b * a.qs_b + hq * a.qs_h;
   const T* kp = static_cast<const T*>(a.k) + b * a.ks_b + hkv * a.ks_h;
   const T* vp = static_cast<const T*>(a.v) + b * a.vs_b + hkv * a.vs_h;
   T* op = static_cast<T*>(a.o) + b * a.os_b + hq * a.os_h;
 
-  const int m = qt * kTile + lane;
-  const bool row_ok = m < a.L;
-  const int m_slot = m >> a.c_shift;
-  const int m0_slot = (qt * kTile) >> a.c_shift;
+  const int m = qt * kTile + lane;  // region token of this lane
+  const bool row_ok = m >= a.r_begin && m < a.r_end;
+  const int r0 = max(qt * kTile, a.r_begin);
 
   float qv[D], acc[D];
 #pragma unroll
   for (int d = 0; d < D; ++d) {
-    qv[d] = row_ok ? load_as_f32<T>(qp + (int64_t)m * a.qs_l + d) : 0.f;
+    qv[d] = row_ok ? load_as_f32<T>(qp + (int64_t)(m - a.r_begin) * a.qs_l + d) : 0.f;
     acc[d] = 0.f;
   }
   float m_run = -INFINITY, l_run = 0.f;
 
-  const int last_key = min(qt * kTile + kTile - 1, a.L - 1);
+  const int last_key = a.base + min(qt * kTile + kTile - 1, a.r_end - 1);
   for (int k0 = 0; k0 <= last_key; k0 += SUB) {
-    // does any slot of this sub-tile reach the first query slot of the tile?
+    // does any row of this sub-tile reach the first query of the tile?
     int key = k0 + lane;
-    bool reach = lane < SUB && key < a.L && lim[key >> a.c_shift] >= m0_slot;
+    bool reach = lane < SUB && key < a.N && lim[key] >= r0;
     if (__ballot(reach) == 0) continue;
     __syncthreads();  // previous sub-tile fully consumed
     for (int idx = lane; idx < SUB * D; idx += kWave) {
       int r = idx / D, d = idx % D;
       int n = k0 + r;
-      bool ok = n < a.L;
+      bool ok = n < a.N;
       Ks[r][d] = ok ? load_as_f32<T>(kp + (int64_t)n * a.ks_l + d) : 0.f;
       Vs[r][d] = ok ? load_as_f32<T>(vp + (int64_t)n * a.vs_l + d) : 0.f;
     }
-    if (lane < SUB) limk[lane] = key < a.L ? lim[key >> a.c_shift] : -1;
+    if (lane < SUB) limk[lane] = key < a.N ? lim[key] : -1;
     __syncthreads();
 
     float tmax = -INFINITY;
@@ -109,7 +109,7 @@ __global__ __launch_bounds__(64) void prefill_simple_kernel(PrefillArgs a) {
 #pragma unroll
       for (int d = 0; d < D; ++d) dot = fmaf(qv[d], Ks[j][d], dot);
       int n = k0 + j;
-      bool vis = row_ok && n <= m && m_slot <= limk[j];
+      bool vis = row_ok && n - a.base <= m && m <= limk[j];
       float s = vis ? dot * a.scale : -INFINITY;
       Ss[j][lane] = s;
       tmax = fmaxf(tmax, s);
@@ -132,7 +132,7 @@ __global__ __launch_bounds__(64) void prefill_simple_kernel(PrefillArgs a) {
   if (row_ok) {
     float inv = 1.f / l_run;
 #pragma unroll
-    for (int d = 0; d < D; ++d) store_from_f32<T>(op + (int64_t)m * a.os_l + d, acc[d] * inv);
+    for (int d = 0; d < D; ++d) store_from_f32<T>(op + (int64_t)(m - a.r_begin) * a.os_l + d, acc[d] * inv);
   }
 }
 
@@ -165,7 +165,7 @@ struct PrefillSmem {
   uint16_t k[2][kTile * D];
   uint16_t v[2][kTile * D];
   int limk[2][kTile];
-  int4 vlist[kWin];  // visited key tiles of the current window: {tile, max vis_lim, min vis_lim, -}
+  int4 vlist[kWin];  // visited key tiles of the current window: {tile, max limit, min limit, -}
   int vcount;
 };
 
@@ -206,20 +206,24 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
   const int qg = a.n_qg - 1 - rank;  // heavy query groups first
   const int b = ks / a.Hkv, hkv = ks % a.Hkv;
   const int hq = hkv * a.n_rep + hg * a.hpw + (wave % a.hpw);
-  const int qt_lo = qg * a.qpw;
-  const int qt_hi = min(qt_lo + a.qpw - 1, a.T - 1);
+  const int qt_lo = a.qt_first + qg * a.qpw;
+  const int qt_hi = min(qt_lo + a.qpw - 1, a.qt_last);
   const int my_qt = qt_lo + wave / a.hpw;
   const bool wave_live = my_qt <= qt_hi;
-  const int q0 = my_qt * kTile;
+  const int q0 = my_qt * kTile;  // region token of this wavefront's first row
 
-  const int2* tl = a.tile_lim + (int64_t)ks * a.T;
-  const int32_t* lim = a.vis_lim + (int64_t)ks * a.S;
+  const int2* tl = a.tile_lim + (int64_t)ks * a.Tk;
+  const int32_t* lim = a.tok_lim + (int64_t)ks * a.N;
   const uint16_t* kp = static_cast<const uint16_t*>(a.k) + b * a.ks_b + hkv * a.ks_h;
   const uint16_t* vp = static_cast<const uint16_t*>(a.v) + b * a.vs_b + hkv * a.vs_h;
 
-  const int m0_group = (qt_lo * kTile) >> a.c_shift;
-  const int my_m0 = q0 >> a.c_shift;
-  const int my_mlast = (min(q0 + kTile - 1, a.L - 1)) >> a.c_shift;
+  // first / last query token of the group and of this wavefront, and the last key tile either may see
+  const int r0_group = max(qt_lo * kTile, a.r_begin);
+  const int rlast_group = min(qt_hi * kTile + kTile - 1, a.r_end - 1);
+  const int my_r0 = max(q0, a.r_begin);
+  const int my_rlast = min(q0 + kTile - 1, a.r_end - 1);
+  const int kt_end_group = (a.base + rlast_group) / kTile;
+  const int my_kt_end = (a.base + my_rlast) / kTile;
 
   // ---- Q fragments: B operand, lane (query l32, k-group hl) --------------------------------------
   bf16x8 qreg[2][DSTEPS];
@@ -227,7 +231,7 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
     const uint16_t* qp = static_cast<const uint16_t*>(a.q) + b * a.qs_b + hq * a.qs_h;
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) {
-      int row = min(q0 + qb * 32 + l32, a.L - 1);
+      int row = min(max(q0 + qb * 32 + l32, a.r_begin), a.r_end - 1) - a.r_begin;
       if (!wave_live) row = 0;
       const uint4* rp = reinterpret_cast<const uint4*>(qp + (int64_t)row * a.qs_l + hl * 8);
 #pragma unroll
@@ -246,7 +250,7 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
   float l_run[2] = {0.f, 0.f};
   const float c = a.scale * 1.4426950408889634f;
 
-  // global -> LDS, one 64-key tile of K and of V; rows beyond L repeat row L-1 (their scores are masked,
+  // global -> LDS, one 64-key tile of K and of V; rows beyond N repeat row N-1 (their scores are masked,
   // so their probabilities are exactly 0 and a finite V row contributes nothing)
   auto issue_tile = [&](int kt, int buf, bool need_lim) {
 #pragma unroll
@@ -254,7 +258,7 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
       const int inst = wave * DMA_PER_WAVE + j;  // uniform
       const int q = inst * kWave + lane;         // chunk slot in the LDS tile
       const int row = q / OCT, pos = q % OCT;
-      const int n = min(kt * kTile + row, a.L - 1);
+      const int n = min(kt * kTile + row, a.N - 1);
       const int kchunk = pos ^ (row % OCT);
       const int vchunk = pos ^ ((row & 3) << 1);
       __builtin_amdgcn_global_load_lds(kp + (int64_t)n * a.ks_l + kchunk * 8,
@@ -264,7 +268,7 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
     }
     if (need_lim && tid < kTile) {
       int n = kt * kTile + tid;
-      sm.limk[buf][tid] = n < a.L ? lim[n >> a.c_shift] : -1;
+      sm.limk[buf][tid] = n < a.N ? lim[n] : -1;
     }
   };
 
@@ -301,11 +305,11 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
           const int lv[4] = {lm.x, lm.y, lm.z, lm.w};
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            int key = kt * kTile + kk + e;
+            int key = kt * kTile + kk + e - a.base;  // region token of the key row (negative: older row)
 #pragma unroll
             for (int qb = 0; qb < 2; ++qb) {
               int qtok = q0 + qb * 32 + l32;
-              bool vis = key <= qtok && (qtok >> a.c_shift) <= lv[e];
+              bool vis = key <= qtok && qtok <= lv[e];
               if (!vis) sacc[kb][qb][g4 * 4 + e] = -INFINITY;
             }
           }
@@ -374,22 +378,21 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
     }
   };
 
-  const int mlast_group = (min(qt_hi * kTile + kTile - 1, a.L - 1)) >> a.c_shift;
   int cur = 0;
-  for (int w0 = 0; w0 <= qt_hi; w0 += kWin) {
+  for (int w0 = 0; w0 <= kt_end_group; w0 += kWin) {
     // ---- visit list of this window: wavefront 0 compacts the tiles some query tile of the group sees ----
     if (wave == 0) {
       int2 vals[kWin / kWave];
 #pragma unroll
       for (int j = 0; j < kWin / kWave; ++j) {
         int t = w0 + j * kWave + lane;
-        vals[j] = t <= qt_hi ? tl[t] : make_int2(-1, -1);
+        vals[j] = t <= kt_end_group ? tl[t] : make_int2(-1, -1);
       }
       int count = 0;
 #pragma unroll
       for (int j = 0; j < kWin / kWave; ++j) {
         int t = w0 + j * kWave + lane;
-        bool v = t <= qt_hi && vals[j].x >= m0_group;
+        bool v = t <= kt_end_group && vals[j].x >= r0_group;
         uint64_t bits = __ballot(v);
         if (v) sm.vlist[count + __builtin_popcountll(bits & ((uint64_t(1) << lane) - 1))] = make_int4(t, vals[j].x, vals[j].y, 0);
         count += __builtin_popcountll(bits);
@@ -409,11 +412,12 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
       if (idx + 1 < n_vis) {
         const int4 en = sm.vlist[idx + 1];
         // the element mask is only evaluated on diagonal tiles and on tiles with mixed visibility
-        issue_tile(en.x, cur ^ 1, en.x >= qt_lo || en.z < mlast_group);
+        issue_tile(en.x, cur ^ 1, en.x * kTile + kTile - 1 - a.base > r0_group || en.z < rlast_group);
       }
-      const bool visit = wave_live && kt <= my_qt && ent.y >= my_m0;
+      const bool visit = wave_live && kt <= my_kt_end && ent.y >= my_r0;
       if (visit) {
-        const bool full = kt < my_qt && ent.z >= my_mlast;
+        // no masked score: every key row is at or before the first query and visible to the last one
+        const bool full = kt * kTile + kTile - 1 - a.base <= my_r0 && ent.z >= my_rlast;
         compute_tile(kt, cur, full);
       }
       __builtin_amdgcn_s_waitcnt(0);  // the next tile has landed in LDS
@@ -430,8 +434,8 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
       float l = l_run[qb] + __shfl_xor(l_run[qb], 32);
       float inv = 1.f / l;
       int qtok = q0 + qb * 32 + l32;
-      if (qtok < a.L) {
-        uint16_t* rp = op + (int64_t)qtok * a.os_l;
+      if (qtok >= a.r_begin && qtok < a.r_end) {
+        uint16_t* rp = op + (int64_t)(qtok - a.r_begin) * a.os_l;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
 #pragma unroll
@@ -468,76 +472,66 @@ static int launch_prefill_mfma(const PrefillArgs& a, int64_t n_wg, hipStream_t s
 
 using namespace nats;
 
-extern "C" size_t nats_prefill_workspace_bytes(int64_t B, int64_t H_q, int64_t H_kv, int64_t L, int64_t D, int64_t C) {
-  (void)H_q;
-  (void)D;
-  if (B <= 0 || H_kv <= 0 || L <= 0 || C <= 0) return 0;
-  int64_t S = (L + C - 1) / C;
-  int64_t T = (L + kTile - 1) / kTile;
-  size_t lim_bytes = ((size_t)(B * H_kv * S) * sizeof(int32_t) + 255) & ~size_t(255);
-  size_t tl_bytes = (size_t)(B * H_kv * T) * sizeof(int2);
-  return lim_bytes + tl_bytes;
-}
+namespace {
 
-extern "C" int nats_prefill_fwd(const void* q, const void* k, const void* v, const uint8_t* roles, void* o, int64_t B,
-                                int64_t H_q, int64_t H_kv, int64_t L, int64_t D, int64_t C, int64_t W,
-                                const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
-                                const int64_t* o_strides, float sm_scale, int dtype, void* workspace,
-                                size_t workspace_bytes, void* stream) {
-  NATS_REQUIRE(q && k && v && roles && o && workspace, NATS_ERR_NULL_POINTER, "nats_prefill_fwd: NULL pointer argument");
-  NATS_REQUIRE(q_strides && k_strides && v_strides && o_strides, NATS_ERR_NULL_POINTER,
-               "nats_prefill_fwd: NULL stride array");
-  NATS_REQUIRE(B > 0 && H_q > 0 && H_kv > 0 && L > 0, NATS_ERR_BAD_SHAPE, "nats_prefill_fwd: B=%lld H_q=%lld H_kv=%lld L=%lld",
-               (long long)B, (long long)H_q, (long long)H_kv, (long long)L);
-  NATS_REQUIRE(H_q % H_kv == 0, NATS_ERR_BAD_SHAPE, "nats_prefill_fwd: H_q=%lld is not a multiple of H_kv=%lld",
-               (long long)H_q, (long long)H_kv);
-  NATS_REQUIRE(D == 64 || D == 128, NATS_ERR_UNSUPPORTED, "nats_prefill_fwd: head_dim %lld (supported: 64, 128)",
-               (long long)D);
-  NATS_REQUIRE(is_pow2(C), NATS_ERR_UNSUPPORTED, "nats_prefill_fwd: chunk size %lld is not a power of two", (long long)C);
-  NATS_REQUIRE(W >= 0 && W % C == 0, NATS_ERR_BAD_SHAPE, "nats_prefill_fwd: window %lld is not a multiple of chunk size %lld",
-               (long long)W, (long long)C);
-  NATS_REQUIRE(dtype == NATS_DTYPE_BF16 || dtype == NATS_DTYPE_F32, NATS_ERR_BAD_DTYPE, "nats_prefill_fwd: dtype %d", dtype);
-  NATS_REQUIRE(L < (int64_t(1) << 30), NATS_ERR_BAD_SHAPE, "nats_prefill_fwd: L=%lld too long", (long long)L);
-  size_t need = nats_prefill_workspace_bytes(B, H_q, H_kv, L, D, C);
-  NATS_REQUIRE(workspace_bytes >= need, NATS_ERR_WORKSPACE, "nats_prefill_fwd: workspace %zu bytes < %zu", workspace_bytes,
-               need);
+struct SegmentShape {
+  int64_t B, H_q, H_kv, D, C, W;
+  int64_t x_len;    // queries
+  int64_t N;        // key rows
+  int64_t base;     // first key row of the open-chunk region
+  int64_t r_begin;  // region token of query 0
+};
+
+int check_common(const char* who, const SegmentShape& g, const int64_t* q_strides, const int64_t* k_strides,
+                 const int64_t* v_strides, const int64_t* o_strides, const void* q, const void* k, const void* v,
+                 const void* o, int dtype) {
+  NATS_REQUIRE(g.B > 0 && g.H_q > 0 && g.H_kv > 0 && g.x_len > 0, NATS_ERR_BAD_SHAPE, "%s: B=%lld H_q=%lld H_kv=%lld L=%lld",
+               who, (long long)g.B, (long long)g.H_q, (long long)g.H_kv, (long long)g.x_len);
+  NATS_REQUIRE(g.H_q % g.H_kv == 0, NATS_ERR_BAD_SHAPE, "%s: H_q=%lld is not a multiple of H_kv=%lld", who,
+               (long long)g.H_q, (long long)g.H_kv);
+  NATS_REQUIRE(g.D == 64 || g.D == 128, NATS_ERR_UNSUPPORTED, "%s: head_dim %lld (supported: 64, 128)", who, (long long)g.D);
+  NATS_REQUIRE(is_pow2(g.C), NATS_ERR_UNSUPPORTED, "%s: chunk size %lld is not a power of two", who, (long long)g.C);
+  NATS_REQUIRE(g.W >= 0 && g.W % g.C == 0, NATS_ERR_BAD_SHAPE, "%s: window %lld is not a multiple of chunk size %lld", who,
+               (long long)g.W, (long long)g.C);
+  NATS_REQUIRE(dtype == NATS_DTYPE_BF16 || dtype == NATS_DTYPE_F32, NATS_ERR_BAD_DTYPE, "%s: dtype %d", who, dtype);
+  NATS_REQUIRE(g.N < (int64_t(1) << 30), NATS_ERR_BAD_SHAPE, "%s: %lld key rows are too many", who, (long long)g.N);
   if (dtype == NATS_DTYPE_BF16) {
     // 16-byte vector loads of rows
     NATS_REQUIRE(q_strides[2] % 8 == 0 && k_strides[2] % 8 == 0 && v_strides[2] % 8 == 0 && o_strides[2] % 4 == 0 &&
                      q_strides[1] % 8 == 0 && k_strides[1] % 8 == 0 && v_strides[1] % 8 == 0 && o_strides[1] % 4 == 0 &&
                      q_strides[0] % 8 == 0 && k_strides[0] % 8 == 0 && v_strides[0] % 8 == 0 && o_strides[0] % 4 == 0,
-                 NATS_ERR_BAD_SHAPE, "nats_prefill_fwd: bf16 strides must keep rows 16-byte aligned");
+                 NATS_ERR_BAD_SHAPE, "%s: bf16 strides must keep rows 16-byte aligned", who);
     NATS_REQUIRE((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v)) % 16 == 0 &&
                      reinterpret_cast<uintptr_t>(o) % 8 == 0,
-                 NATS_ERR_BAD_SHAPE, "nats_prefill_fwd: bf16 tensors must be 16-byte aligned");
+                 NATS_ERR_BAD_SHAPE, "%s: bf16 tensors must be 16-byte aligned", who);
   }
+  return NATS_OK;
+}
 
-  hipStream_t st = static_cast<hipStream_t>(stream);
-  const int64_t S = (L + C - 1) / C;
-  const int64_t T = (L + kTile - 1) / kTile;
-  int32_t* vis_lim = static_cast<int32_t*>(workspace);
-  size_t lim_bytes = ((size_t)(B * H_kv * S) * sizeof(int32_t) + 255) & ~size_t(255);
-  int2* tile_lim = reinterpret_cast<int2*>(static_cast<char*>(workspace) + lim_bytes);
-  if (int rc = launch_role_scan(roles, B * H_kv, S, W, C, nullptr, vis_lim, st)) return rc;
-  if (int rc = launch_tile_lim(vis_lim, B * H_kv, S, T, C, tile_lim, st)) return rc;
-
+// key limits are in the workspace; launches the attention kernel of the segment
+int launch_segment(const char* who, const SegmentShape& g, const void* q, const void* k, const void* v, void* o,
+                   const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                   const int64_t* o_strides, float sm_scale, int dtype, const PrefillWorkspace& w, hipStream_t st) {
   PrefillArgs a;
   a.q = q; a.k = k; a.v = v; a.o = o;
-  a.vis_lim = vis_lim; a.tile_lim = tile_lim;
+  a.tok_lim = w.tok_lim; a.tile_lim = w.tile_lim;
   a.qs_b = q_strides[0]; a.qs_h = q_strides[1]; a.qs_l = q_strides[2];
   a.ks_b = k_strides[0]; a.ks_h = k_strides[1]; a.ks_l = k_strides[2];
   a.vs_b = v_strides[0]; a.vs_h = v_strides[1]; a.vs_l = v_strides[2];
   a.os_b = o_strides[0]; a.os_h = o_strides[1]; a.os_l = o_strides[2];
-  a.B = (int)B; a.Hq = (int)H_q; a.Hkv = (int)H_kv; a.n_rep = (int)(H_q / H_kv);
-  a.L = (int)L; a.S = (int)S; a.T = (int)T;
-  a.c_shift = ilog2(C);
+  a.B = (int)g.B; a.Hq = (int)g.H_q; a.Hkv = (int)g.H_kv; a.n_rep = (int)(g.H_q / g.H_kv);
+  a.N = (int)g.N; a.Tk = (int)((g.N + kTile - 1) / kTile);
+  a.base = (int)g.base;
+  a.r_begin = (int)g.r_begin; a.r_end = (int)(g.r_begin + g.x_len);
+  a.qt_first = a.r_begin / kTile; a.qt_last = (a.r_end - 1) / kTile;
+  const int64_t n_qt = a.qt_last - a.qt_first + 1;
   a.scale = sm_scale;
-  a.hpw = 1; a.qpw = 1; a.n_hg = 1; a.n_qg = (int)T; a.xcd_mode = 0;
+  a.hpw = 1; a.qpw = 1; a.n_hg = 1; a.n_qg = (int)n_qt; a.xcd_mode = 0;
 
   if (dtype == NATS_DTYPE_F32) {
-    NATS_REQUIRE(B * H_q <= 65535, NATS_ERR_BAD_SHAPE, "nats_prefill_fwd: B*H_q too large for the fp32 kernel");
-    dim3 grid((unsigned)T, (unsigned)(B * H_q));
-    if (D == 64) {
+    NATS_REQUIRE(g.B * g.H_q <= 65535, NATS_ERR_BAD_SHAPE, "%s: B*H_q too large for the fp32 kernel", who);
+    dim3 grid((unsigned)n_qt, (unsigned)(g.B * g.H_q));
+    if (g.D == 64) {
       hipLaunchKernelGGL((prefill_simple_kernel<float, 64>), grid, dim3(64), 0, st, a);
     } else {
       hipLaunchKernelGGL((prefill_simple_kernel<float, 128>), grid, dim3(64), 0, st, a);
@@ -550,13 +544,73 @@ extern "C" int nats_prefill_fwd(const void* q, const void* k, const void* v, con
   int n_rep = a.n_rep;
   int hpw = n_rep >= 4 ? 4 : n_rep;
   NATS_REQUIRE(n_rep % hpw == 0 && (4 % hpw) == 0, NATS_ERR_UNSUPPORTED,
-               "nats_prefill_fwd: GQA group size %d (supported: 1, 2, 4 and multiples of 4)", n_rep);
+               "%s: GQA group size %d (supported: 1, 2, 4 and multiples of 4)", who, n_rep);
   a.hpw = hpw;
   a.qpw = 4 / hpw;
   a.n_hg = n_rep / hpw;
-  a.n_qg = (int)((T + a.qpw - 1) / a.qpw);
-  a.xcd_mode = ((B * H_kv) % 8 == 0) ? 1 : 0;
-  int64_t n_wg = B * H_kv * a.n_hg * a.n_qg;
-  NATS_REQUIRE(n_wg < (int64_t(1) << 31), NATS_ERR_BAD_SHAPE, "nats_prefill_fwd: grid too large");
-  return D == 64 ? launch_prefill_mfma<64>(a, n_wg, st) : launch_prefill_mfma<128>(a, n_wg, st);
+  a.n_qg = (int)((n_qt + a.qpw - 1) / a.qpw);
+  a.xcd_mode = ((g.B * g.H_kv) % 8 == 0) ? 1 : 0;
+  int64_t n_wg = g.B * g.H_kv * a.n_hg * a.n_qg;
+  NATS_REQUIRE(n_wg < (int64_t(1) << 31), NATS_ERR_BAD_SHAPE, "%s: grid too large", who);
+  return g.D == 64 ? launch_prefill_mfma<64>(a, n_wg, st) : launch_prefill_mfma<128>(a, n_wg, st);
+}
+
+}  // namespace
+
+extern "C" size_t nats_prefill_workspace_bytes(int64_t B, int64_t H_q, int64_t H_kv, int64_t L, int64_t D, int64_t C) {
+  (void)H_q;
+  (void)D;
+  if (B <= 0 || H_kv <= 0 || L <= 0 || C <= 0) return 0;
+  return carve_prefill_workspace(nullptr, B * H_kv, (L + C - 1) / C, L).bytes;
+}
+
+extern "C" size_t nats_prefill_past_workspace_bytes(int64_t B, int64_t H_kv, int64_t n_rows, int64_t S) {
+  if (B <= 0 || H_kv <= 0 || n_rows <= 0 || S <= 0) return 0;
+  return carve_prefill_workspace(nullptr, B * H_kv, S, n_rows).bytes;
+}
+
+extern "C" int nats_prefill_fwd(const void* q, const void* k, const void* v, const uint8_t* roles, void* o, int64_t B,
+                                int64_t H_q, int64_t H_kv, int64_t L, int64_t D, int64_t C, int64_t W,
+                                const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                                const int64_t* o_strides, float sm_scale, int dtype, void* workspace,
+                                size_t workspace_bytes, void* stream) {
+  const char* who = "nats_prefill_fwd";
+  NATS_REQUIRE(q && k && v && roles && o && workspace, NATS_ERR_NULL_POINTER, "%s: NULL pointer argument", who);
+  NATS_REQUIRE(q_strides && k_strides && v_strides && o_strides, NATS_ERR_NULL_POINTER, "%s: NULL stride array", who);
+  SegmentShape g{B, H_q, H_kv, D, C, W, L, L, 0, 0};
+  if (int rc = check_common(who, g, q_strides, k_strides, v_strides, o_strides, q, k, v, o, dtype)) return rc;
+  const int64_t S = (L + C - 1) / C;
+  PrefillWorkspace w = carve_prefill_workspace(workspace, B * H_kv, S, L);
+  NATS_REQUIRE(workspace_bytes >= w.bytes, NATS_ERR_WORKSPACE, "%s: workspace %zu bytes < %zu", who, workspace_bytes, w.bytes);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (int rc = prepare_key_limits(roles, B, H_kv, S, L, C, W, nullptr, w, st)) return rc;
+  return launch_segment(who, g, q, k, v, o, q_strides, k_strides, v_strides, o_strides, sm_scale, dtype, w, st);
+}
+
+extern "C" int nats_prefill_past_fwd(const void* q, const void* cache_k, const void* cache_v, const uint8_t* valid,
+                                     const int64_t* size_global, const int64_t* size_local, const uint8_t* roles, void* o,
+                                     int64_t B, int64_t H_q, int64_t H_kv, int64_t x_len, int64_t D, int64_t C, int64_t W,
+                                     const nats_past_state* state, const int64_t* q_strides, const int64_t* k_strides,
+                                     const int64_t* v_strides, const int64_t* valid_strides, const int64_t* o_strides,
+                                     float sm_scale, int dtype, void* workspace, size_t workspace_bytes, void* stream) {
+  const char* who = "nats_prefill_past_fwd";
+  NATS_REQUIRE(q && cache_k && cache_v && valid && size_global && size_local && roles && o && workspace,
+               NATS_ERR_NULL_POINTER, "%s: NULL pointer argument", who);
+  NATS_REQUIRE(q_strides && k_strides && v_strides && valid_strides && o_strides, NATS_ERR_NULL_POINTER,
+               "%s: NULL stride array", who);
+  NATS_REQUIRE(is_pow2(C) && W >= 0 && W % C == 0, NATS_ERR_BAD_SHAPE, "%s: chunk size %lld, window %lld", who,
+               (long long)C, (long long)W);
+  if (int rc = check_past_state(who, state, x_len, C, W)) return rc;
+  const int64_t base = state->n_ctx_data - state->old_fill;
+  const int64_t N = state->n_ctx_data + x_len;
+  SegmentShape g{B, H_q, H_kv, D, C, W, x_len, N, base, state->old_fill};
+  if (int rc = check_common(who, g, q_strides, k_strides, v_strides, o_strides, q, cache_k, cache_v, o, dtype)) return rc;
+  const int64_t S = (state->old_fill + x_len + C - 1) / C;
+  PrefillWorkspace w = carve_prefill_workspace(workspace, B * H_kv, S, N);
+  NATS_REQUIRE(workspace_bytes >= w.bytes, NATS_ERR_WORKSPACE, "%s: workspace %zu bytes < %zu", who, workspace_bytes, w.bytes);
+  PastView pv{valid, valid_strides[0], valid_strides[1], size_global, size_local, base,
+              state->gmin, state->tail, state->seen, state->fill_last};
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (int rc = prepare_key_limits(roles, B, H_kv, S, N, C, W, &pv, w, st)) return rc;
+  return launch_segment(who, g, q, cache_k, cache_v, o, q_strides, k_strides, v_strides, o_strides, sm_scale, dtype, w, st);
 }

@@ -77,7 +77,8 @@ __global__ void roles_kernel(const void* __restrict__ logits, int64_t B, int64_t
 // (components/masks/utils.py:92 and components/cache/nats_chunk_layer_cache.py:603-611).
 // ---------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(64) void role_scan_kernel(const uint8_t* __restrict__ roles, int64_t S, int32_t wc,
-                                                      int64_t* __restrict__ end_idx, int32_t* __restrict__ vis_lim) {
+                                                      int64_t* __restrict__ end_idx, int32_t* __restrict__ vis_lim,
+                                                      int32_t* __restrict__ first_global) {
   const int64_t stream = blockIdx.x;
   const uint8_t* r = roles + stream * S;
   const int lane = lane_id();
@@ -106,64 +107,158 @@ __global__ __launch_bounds__(64) void role_scan_kernel(const uint8_t* __restrict
     }
     if (bits) carry = base + __builtin_ctzll(bits);
   }
+  if (first_global && lane == 0) first_global[stream] = int32_t(carry);  // end_idx[0]
 }
 
-// Per 64-key tile: the largest and the smallest vis_lim over the role slots the tile touches.
-// tile_lim[stream][t] = {max, min}.  A query tile whose first slot is m0 must load key tile t iff
-// max >= m0; every score of the pair is unmasked iff t lies strictly below the query tile and min >= the
-// query tile's last slot.
-__global__ void tile_lim_kernel(const int32_t* __restrict__ vis_lim, int64_t S, int64_t T, int c_shift,
-                                int2* __restrict__ tile_lim) {
-  int64_t idx = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
-  int64_t stream = blockIdx.y;
-  if (idx >= T) return;
-  int64_t n0 = (idx * kTile) >> c_shift;
-  int64_t n1 = ((idx * kTile + kTile - 1) >> c_shift);
-  if (n1 > S - 1) n1 = S - 1;
-  int32_t mx = -1, mn = kLimGlobal;
-  for (int64_t n = n0; n <= n1; ++n) {
-    int32_t v = vis_lim[stream * S + n];
-    mx = v > mx ? v : mx;
-    mn = v < mn ? v : mn;
+// Per key row the last query token (counted from the start of the open-chunk region) that sees it, and
+// per 64-row key tile the largest and the smallest of these limits: tile_lim[stream][t] = {max, min}.
+// A query tile whose first token is r0 must load key tile t iff max >= r0; every score of the pair is
+// unmasked iff all keys of t lie at or before the query tile's first token and min >= its last token.
+//
+// Rows of the region (row >= base) follow the roles of the segment: a slot visible up to query slot
+// vis_lim is visible up to token (vis_lim + 1) * C - 1.  Rows below base are what an earlier segment left
+// in the cache (components/cache/nats_chunk_layer_cache.py:462-511, 658-713):
+//   ring rows [0, W)            valid and not older than the window for that query
+//   rows [W, gmin)              valid_tokens as stored
+//   rows [gmin, size_global)    always (kept globals)
+//   rows [size_global, +local)  up to the first global slot of the segment
+//   beyond                      never (rows that longer heads use)
+template <bool kPast>
+__global__ __launch_bounds__(256) void key_lim_kernel(KeyLimArgs a) {
+  const int stream = blockIdx.y;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int tile = blockIdx.x * 4 + wave;
+  if (tile >= a.Tk) return;
+  const int row = tile * kTile + lane;
+  int32_t lim = -1;
+  if (row < a.N) {
+    if (!kPast || row >= a.base) {
+      int32_t v = a.vis_lim[(int64_t)stream * a.S + ((row - a.base) >> a.c_shift)];
+      int64_t t = (int64_t(v) + 1) * a.C - 1;
+      lim = (v == kLimGlobal || t >= kLimGlobal) ? kLimGlobal : int32_t(t);
+    } else {
+      const int b = stream / a.Hkv, h = stream % a.Hkv;
+      const bool val = a.valid[b * a.valid_s_b + h * a.valid_s_h + row] != 0;
+      const int C = a.C;
+      if (row < a.W) {
+        const int s = row >> a.c_shift;
+        if (!val) {
+          lim = -1;
+        } else if (a.seen >= a.W) {
+          lim = ((s + 1) * C + a.W - 1 - a.tail) % a.W;  // queue offset of the slot's newest row (:687-707)
+        } else if (s < a.seen / C) {
+          int t = (a.W / C - s) * C - 1 - a.fill_last;  // (r + fill_last) / C + s < W / C  (:666-676)
+          lim = t < 0 ? -1 : t;
+        } else {
+          lim = kLimGlobal;
+        }
+      } else {
+        const int ncc = (a.base - a.gmin) / C;
+        if (row < a.gmin || row >= a.gmin + ncc * C) {
+          lim = val ? kLimGlobal : -1;
+        } else {
+          const int cc = (row - a.gmin) / C;
+          const int64_t sg = a.size_global[stream], sl = a.size_local[stream];
+          const int64_t lo = (sg - a.gmin) / C, hi = (sg + sl - a.gmin) / C;
+          if (cc >= hi) {
+            lim = -1;
+          } else if (cc < lo) {
+            lim = kLimGlobal;
+          } else {
+            lim = (a.first_global[stream] + 1) * C - 1;  // query slot <= first global slot of the segment (:480-494)
+          }
+        }
+      }
+    }
+    a.tok_lim[(int64_t)stream * a.N + row] = lim;
   }
-  tile_lim[stream * T + idx] = make_int2(mx, mn);
+  int32_t mx = lim, mn = row < a.N ? lim : kLimGlobal;
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    mx = max(mx, __shfl_xor(mx, off));
+    mn = min(mn, __shfl_xor(mn, off));
+  }
+  if (lane == 0) a.tile_lim[(int64_t)stream * a.Tk + tile] = make_int2(mx, mn);
 }
 
-// token-level mask, one thread per (query, key) pair
-__global__ void mask_kernel(const int32_t* __restrict__ vis_lim, int64_t S, int64_t L, int c_shift,
-                            uint8_t* __restrict__ mask) {
-  int64_t n = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
-  int64_t m = blockIdx.y;
+// token-level mask from the per-row limits: query i of the segment is region token r = r_begin + i
+__global__ void mask_rows_kernel(const int32_t* __restrict__ tok_lim, int64_t N, int64_t x_len, int64_t base,
+                                 int64_t r_begin, uint8_t* __restrict__ mask) {
+  int64_t row = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  int64_t i = blockIdx.y;
   int64_t stream = blockIdx.z;
-  if (n >= L) return;
-  bool vis = n <= m && (m >> c_shift) <= int64_t(vis_lim[stream * S + (n >> c_shift)]);
-  mask[(stream * L + m) * L + n] = vis ? 1 : 0;
+  if (row >= N) return;
+  int64_t r = r_begin + i;
+  bool vis = r <= int64_t(tok_lim[stream * N + row]) && row - base <= r;
+  mask[(stream * x_len + i) * N + row] = vis ? 1 : 0;
 }
 
-__global__ void tile_map_kernel(const int2* __restrict__ tile_lim, int64_t T, int c_shift, uint8_t* __restrict__ tiles) {
+__global__ void tile_map_kernel(const int2* __restrict__ tile_lim, int64_t T, uint8_t* __restrict__ tiles) {
   int64_t kt = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
   int64_t qt = blockIdx.y;
   int64_t stream = blockIdx.z;
   if (kt >= T) return;
-  int64_t m0 = (qt * kTile) >> c_shift;
-  bool visit = kt <= qt && int64_t(tile_lim[stream * T + kt].x) >= m0;
+  bool visit = kt <= qt && int64_t(tile_lim[stream * T + kt].x) >= qt * kTile;
   tiles[(stream * T + qt) * T + kt] = visit ? 1 : 0;
 }
 
 int launch_role_scan(const uint8_t* roles, int64_t n_streams, int64_t S, int64_t W, int64_t C, int64_t* end_idx,
-                     int32_t* vis_lim, hipStream_t st) {
+                     int32_t* vis_lim, int32_t* first_global, hipStream_t st) {
   hipLaunchKernelGGL(role_scan_kernel, dim3((unsigned)n_streams), dim3(kWave), 0, st, roles, S, int32_t(W / C), end_idx,
-                     vis_lim);
+                     vis_lim, first_global);
   NATS_CHECK_LAUNCH("role_scan_kernel");
   return NATS_OK;
 }
 
-int launch_tile_lim(const int32_t* vis_lim, int64_t n_streams, int64_t S, int64_t T, int64_t C, int2* tile_lim,
-                    hipStream_t st) {
-  dim3 grid((unsigned)((T + 255) / 256), (unsigned)n_streams);
-  hipLaunchKernelGGL(tile_lim_kernel, grid, dim3(256), 0, st, vis_lim, S, T, ilog2(C), tile_lim);
-  NATS_CHECK_LAUNCH("tile_lim_kernel");
+int launch_key_lim(const KeyLimArgs& a, int64_t n_streams, bool past, hipStream_t st) {
+  NATS_REQUIRE(n_streams <= 65535, NATS_ERR_BAD_SHAPE, "too many (batch, kv head) streams: %lld", (long long)n_streams);
+  dim3 grid((unsigned)((a.Tk + 3) / 4), (unsigned)n_streams);
+  if (past) {
+    hipLaunchKernelGGL(key_lim_kernel<true>, grid, dim3(256), 0, st, a);
+  } else {
+    hipLaunchKernelGGL(key_lim_kernel<false>, grid, dim3(256), 0, st, a);
+  }
+  NATS_CHECK_LAUNCH("key_lim_kernel");
   return NATS_OK;
+}
+
+PrefillWorkspace carve_prefill_workspace(void* ws, int64_t n_streams, int64_t S, int64_t N) {
+  auto up = [](size_t x) { return (x + 255) & ~size_t(255); };
+  const int64_t Tk = (N + kTile - 1) / kTile;
+  PrefillWorkspace w;
+  char* p = static_cast<char*>(ws);
+  size_t off = 0;
+  w.vis_lim = reinterpret_cast<int32_t*>(p + off);
+  off += up((size_t)(n_streams * S) * sizeof(int32_t));
+  w.first_global = reinterpret_cast<int32_t*>(p + off);
+  off += up((size_t)n_streams * sizeof(int32_t));
+  w.tok_lim = reinterpret_cast<int32_t*>(p + off);
+  off += up((size_t)(n_streams * N) * sizeof(int32_t));
+  w.tile_lim = reinterpret_cast<int2*>(p + off);
+  off += up((size_t)(n_streams * Tk) * sizeof(int2));
+  w.bytes = off;
+  return w;
+}
+
+// roles -> vis_lim, first_global -> tok_lim, tile_lim.  `past` may be NULL (prefill from an empty cache).
+int prepare_key_limits(const uint8_t* roles, int64_t B, int64_t H_kv, int64_t S, int64_t N, int64_t C, int64_t W,
+                       const PastView* past, const PrefillWorkspace& w, hipStream_t st) {
+  const int64_t n_streams = B * H_kv;
+  if (int rc = launch_role_scan(roles, n_streams, S, W, C, nullptr, w.vis_lim, w.first_global, st)) return rc;
+  KeyLimArgs a{};
+  a.vis_lim = w.vis_lim;
+  a.first_global = w.first_global;
+  a.tok_lim = w.tok_lim;
+  a.tile_lim = w.tile_lim;
+  a.Hkv = (int)H_kv; a.S = (int)S; a.N = (int)N; a.Tk = (int)((N + kTile - 1) / kTile);
+  a.c_shift = ilog2(C); a.C = (int)C; a.W = (int)W;
+  if (past) {
+    a.valid = past->valid; a.valid_s_b = past->valid_s_b; a.valid_s_h = past->valid_s_h;
+    a.size_global = past->size_global; a.size_local = past->size_local;
+    a.base = (int)past->base; a.gmin = (int)past->gmin; a.tail = (int)past->tail; a.seen = (int)past->seen;
+    a.fill_last = (int)past->fill_last;
+  }
+  return launch_key_lim(a, n_streams, past != nullptr, st);
 }
 
 }  // namespace nats
@@ -208,36 +303,89 @@ extern "C" int nats_role_scan(const uint8_t* roles, int64_t B, int64_t H_kv, int
   NATS_REQUIRE(B > 0 && H_kv > 0 && S > 0 && S < (int64_t(1) << 30), NATS_ERR_BAD_SHAPE,
                "nats_role_scan: B=%lld H_kv=%lld S=%lld", (long long)B, (long long)H_kv, (long long)S);
   if (int rc = check_cw("nats_role_scan", C, W)) return rc;
-  return launch_role_scan(roles, B * H_kv, S, W, C, end_idx, vis_lim, static_cast<hipStream_t>(stream));
+  return launch_role_scan(roles, B * H_kv, S, W, C, end_idx, vis_lim, nullptr, static_cast<hipStream_t>(stream));
 }
 
-extern "C" int nats_prefill_mask(const int32_t* vis_lim, int64_t B, int64_t H_kv, int64_t L, int64_t C, uint8_t* mask,
-                                 void* stream) {
-  NATS_REQUIRE(vis_lim && mask, NATS_ERR_NULL_POINTER, "nats_prefill_mask: NULL pointer");
-  NATS_REQUIRE(B > 0 && H_kv > 0 && L > 0 && L <= 65535, NATS_ERR_BAD_SHAPE, "nats_prefill_mask: B=%lld H_kv=%lld L=%lld",
-               (long long)B, (long long)H_kv, (long long)L);
-  NATS_REQUIRE(is_pow2(C), NATS_ERR_UNSUPPORTED, "nats_prefill_mask: chunk size %lld", (long long)C);
-  NATS_REQUIRE(B * H_kv <= 65535, NATS_ERR_BAD_SHAPE, "nats_prefill_mask: too many streams");
-  int64_t S = (L + C - 1) / C;
-  dim3 grid((unsigned)((L + 255) / 256), (unsigned)L, (unsigned)(B * H_kv));
-  hipLaunchKernelGGL(mask_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream), vis_lim, S, L, ilog2(C), mask);
-  NATS_CHECK_LAUNCH("mask_kernel");
+static int launch_mask_rows(const PrefillWorkspace& w, int64_t n_streams, int64_t N, int64_t x_len, int64_t base,
+                            int64_t r_begin, uint8_t* mask, hipStream_t st) {
+  NATS_REQUIRE(x_len <= 65535 && n_streams <= 65535, NATS_ERR_BAD_SHAPE, "mask output: grid too large");
+  dim3 grid((unsigned)((N + 255) / 256), (unsigned)x_len, (unsigned)n_streams);
+  hipLaunchKernelGGL(mask_rows_kernel, grid, dim3(256), 0, st, w.tok_lim, N, x_len, base, r_begin, mask);
+  NATS_CHECK_LAUNCH("mask_rows_kernel");
   return NATS_OK;
 }
 
-extern "C" int nats_prefill_tile_map(const int32_t* vis_lim, int64_t B, int64_t H_kv, int64_t L, int64_t C,
-                                     void* tile_lim_ws, uint8_t* tiles, void* stream) {
-  NATS_REQUIRE(vis_lim && tiles && tile_lim_ws, NATS_ERR_NULL_POINTER, "nats_prefill_tile_map: NULL pointer");
+extern "C" int nats_prefill_mask(const uint8_t* roles, int64_t B, int64_t H_kv, int64_t L, int64_t C, int64_t W,
+                                 uint8_t* mask, void* workspace, size_t workspace_bytes, void* stream) {
+  NATS_REQUIRE(roles && mask && workspace, NATS_ERR_NULL_POINTER, "nats_prefill_mask: NULL pointer");
+  NATS_REQUIRE(B > 0 && H_kv > 0 && L > 0, NATS_ERR_BAD_SHAPE, "nats_prefill_mask: B=%lld H_kv=%lld L=%lld",
+               (long long)B, (long long)H_kv, (long long)L);
+  if (int rc = check_cw("nats_prefill_mask", C, W)) return rc;
+  const int64_t S = (L + C - 1) / C;
+  PrefillWorkspace w = carve_prefill_workspace(workspace, B * H_kv, S, L);
+  NATS_REQUIRE(workspace_bytes >= w.bytes, NATS_ERR_WORKSPACE, "nats_prefill_mask: workspace %zu bytes < %zu",
+               workspace_bytes, w.bytes);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (int rc = prepare_key_limits(roles, B, H_kv, S, L, C, W, nullptr, w, st)) return rc;
+  return launch_mask_rows(w, B * H_kv, L, L, 0, 0, mask, st);
+}
+
+extern "C" int nats_prefill_tile_map(const uint8_t* roles, int64_t B, int64_t H_kv, int64_t L, int64_t C, int64_t W,
+                                     uint8_t* tiles, void* workspace, size_t workspace_bytes, void* stream) {
+  NATS_REQUIRE(roles && tiles && workspace, NATS_ERR_NULL_POINTER, "nats_prefill_tile_map: NULL pointer");
   NATS_REQUIRE(B > 0 && H_kv > 0 && L > 0, NATS_ERR_BAD_SHAPE, "nats_prefill_tile_map: B=%lld H_kv=%lld L=%lld",
                (long long)B, (long long)H_kv, (long long)L);
-  NATS_REQUIRE(is_pow2(C), NATS_ERR_UNSUPPORTED, "nats_prefill_tile_map: chunk size %lld", (long long)C);
-  int64_t S = (L + C - 1) / C;
-  int64_t T = (L + kTile - 1) / kTile;
+  if (int rc = check_cw("nats_prefill_tile_map", C, W)) return rc;
+  const int64_t S = (L + C - 1) / C;
+  const int64_t T = (L + kTile - 1) / kTile;
   NATS_REQUIRE(T <= 65535 && B * H_kv <= 65535, NATS_ERR_BAD_SHAPE, "nats_prefill_tile_map: grid too large");
+  PrefillWorkspace w = carve_prefill_workspace(workspace, B * H_kv, S, L);
+  NATS_REQUIRE(workspace_bytes >= w.bytes, NATS_ERR_WORKSPACE, "nats_prefill_tile_map: workspace %zu bytes < %zu",
+               workspace_bytes, w.bytes);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (int rc = launch_tile_lim(vis_lim, B * H_kv, S, T, C, static_cast<int2*>(tile_lim_ws), st)) return rc;
+  if (int rc = prepare_key_limits(roles, B, H_kv, S, L, C, W, nullptr, w, st)) return rc;
   dim3 grid((unsigned)((T + 255) / 256), (unsigned)T, (unsigned)(B * H_kv));
-  hipLaunchKernelGGL(tile_map_kernel, grid, dim3(256), 0, st, static_cast<const int2*>(tile_lim_ws), T, ilog2(C), tiles);
+  hipLaunchKernelGGL(tile_map_kernel, grid, dim3(256), 0, st, w.tile_lim, T, tiles);
   NATS_CHECK_LAUNCH("tile_map_kernel");
   return NATS_OK;
+}
+
+int nats::check_past_state(const char* who, const nats_past_state* ps, int64_t x_len, int64_t C, int64_t W) {
+  NATS_REQUIRE(ps, NATS_ERR_NULL_POINTER, "%s: NULL past state", who);
+  NATS_REQUIRE(x_len > 0, NATS_ERR_BAD_SHAPE, "%s: x_len=%lld", who, (long long)x_len);
+  NATS_REQUIRE(ps->old_fill >= 0 && ps->old_fill < C, NATS_ERR_BAD_SHAPE, "%s: old_fill=%lld outside [0, %lld)", who,
+               (long long)ps->old_fill, (long long)C);
+  NATS_REQUIRE(ps->n_ctx_data >= W + ps->old_fill && ps->n_ctx_data + x_len < (int64_t(1) << 30), NATS_ERR_BAD_SHAPE,
+               "%s: n_ctx_data=%lld with window %lld and %lld open-chunk tokens", who, (long long)ps->n_ctx_data,
+               (long long)W, (long long)ps->old_fill);
+  NATS_REQUIRE(ps->gmin >= W && ps->gmin <= ps->n_ctx_data - ps->old_fill, NATS_ERR_BAD_SHAPE,
+               "%s: gmin=%lld outside [W, first open-chunk row]", who, (long long)ps->gmin);
+  NATS_REQUIRE(ps->tail >= 0 && (W == 0 ? ps->tail == 0 : ps->tail < W), NATS_ERR_BAD_SHAPE, "%s: tail=%lld", who,
+               (long long)ps->tail);
+  NATS_REQUIRE(ps->seen >= 0 && ps->fill_last >= 0 && ps->fill_last < C, NATS_ERR_BAD_SHAPE, "%s: seen=%lld fill_last=%lld",
+               who, (long long)ps->seen, (long long)ps->fill_last);
+  return NATS_OK;
+}
+
+extern "C" int nats_prefill_past_mask(const uint8_t* valid, const int64_t* size_global, const int64_t* size_local,
+                                      const uint8_t* roles, int64_t B, int64_t H_kv, int64_t x_len, int64_t C, int64_t W,
+                                      const nats_past_state* ps, const int64_t* valid_strides, uint8_t* mask,
+                                      void* workspace, size_t workspace_bytes, void* stream) {
+  NATS_REQUIRE(valid && size_global && size_local && roles && mask && workspace && valid_strides, NATS_ERR_NULL_POINTER,
+               "nats_prefill_past_mask: NULL pointer");
+  NATS_REQUIRE(B > 0 && H_kv > 0, NATS_ERR_BAD_SHAPE, "nats_prefill_past_mask: B=%lld H_kv=%lld", (long long)B,
+               (long long)H_kv);
+  if (int rc = check_cw("nats_prefill_past_mask", C, W)) return rc;
+  if (int rc = check_past_state("nats_prefill_past_mask", ps, x_len, C, W)) return rc;
+  const int64_t fill = ps->old_fill + x_len;
+  const int64_t S = (fill + C - 1) / C;
+  const int64_t N = ps->n_ctx_data + x_len;
+  PrefillWorkspace w = carve_prefill_workspace(workspace, B * H_kv, S, N);
+  NATS_REQUIRE(workspace_bytes >= w.bytes, NATS_ERR_WORKSPACE, "nats_prefill_past_mask: workspace %zu bytes < %zu",
+               workspace_bytes, w.bytes);
+  PastView pv{valid, valid_strides[0], valid_strides[1], size_global, size_local, ps->n_ctx_data - ps->old_fill,
+              ps->gmin, ps->tail, ps->seen, ps->fill_last};
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (int rc = prepare_key_limits(roles, B, H_kv, S, N, C, W, &pv, w, st)) return rc;
+  return launch_mask_rows(w, B * H_kv, N, x_len, pv.base, ps->old_fill, mask, st);
 }

@@ -12,7 +12,7 @@ import math
 import torch
 
 from . import _lib
-from ._lib import NATS_DTYPE_BF16, NATS_DTYPE_F32, EvictParams, EvictResult, check, i64_array
+from ._lib import NATS_DTYPE_BF16, NATS_DTYPE_F32, EvictParams, EvictResult, PastState, check, i64_array
 
 ROLE_GLOBAL, ROLE_LOCAL, ROLE_SW = 0, 1, 2
 TILE = 64
@@ -96,23 +96,26 @@ def role_scan(roles: torch.Tensor, W: int, C: int):
 
 def prefill_mask(roles: torch.Tensor, L: int, C: int, W: int) -> torch.Tensor:
     """Bool [B, H_kv, L, L]: the mask NAtSChunkLayerCache.generate_mask returns for a prefill from empty."""
+    _require_cuda(roles)
     lib = _lib.load()
-    _, vis_lim = role_scan(roles, W, C)
+    roles = roles.contiguous()
     B, H, _ = roles.shape
     mask = torch.empty(B, H, L, L, dtype=torch.uint8, device=roles.device)
-    check(lib.nats_prefill_mask(_ptr(vis_lim), B, H, L, C, _ptr(mask), _stream(roles)))
+    ws = workspace(roles.device, "prefill", lib.nats_prefill_workspace_bytes(B, H, H, L, 0, C))
+    check(lib.nats_prefill_mask(_ptr(roles), B, H, L, C, W, _ptr(mask), _ptr(ws), ws.numel(), _stream(roles)))
     return mask.bool()
 
 
 def prefill_tile_map(roles: torch.Tensor, L: int, C: int, W: int) -> torch.Tensor:
     """Bool [B, H_kv, T, T], T = ceil(L / 64): the 64x64 tiles the prefill kernel loads."""
+    _require_cuda(roles)
     lib = _lib.load()
-    _, vis_lim = role_scan(roles, W, C)
+    roles = roles.contiguous()
     B, H, _ = roles.shape
     T = (L + TILE - 1) // TILE
-    scratch = torch.empty(B * H * T * 8, dtype=torch.uint8, device=roles.device)
     tiles = torch.empty(B, H, T, T, dtype=torch.uint8, device=roles.device)
-    check(lib.nats_prefill_tile_map(_ptr(vis_lim), B, H, L, C, _ptr(scratch), _ptr(tiles), _stream(roles)))
+    ws = workspace(roles.device, "prefill", lib.nats_prefill_workspace_bytes(B, H, H, L, 0, C))
+    check(lib.nats_prefill_tile_map(_ptr(roles), B, H, L, C, W, _ptr(tiles), _ptr(ws), ws.numel(), _stream(roles)))
     return tiles.bool()
 
 
@@ -153,6 +156,77 @@ def prefill_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, roles: 
     return out
 
 
+def past_state(n_ctx_data: int, old_fill: int, gmin: int, tail: int, seen: int, fill_last: int) -> PastState:
+    return PastState(int(n_ctx_data), int(old_fill), int(gmin), int(tail), int(seen), int(fill_last))
+
+
+def _check_past(valid, size_global, size_local, roles, B, Hkv, x_len, C, state: PastState):
+    S = math.ceil((state.old_fill + x_len) / C)
+    if tuple(roles.shape) != (B, Hkv, S) or roles.dtype != torch.uint8:
+        raise ValueError(f"roles must be uint8 [B, H_kv, {S}], got {roles.dtype} {tuple(roles.shape)}")
+    if valid.dtype not in (torch.uint8, torch.bool) or valid.dim() != 3 or valid.shape[:2] != (B, Hkv) \
+            or valid.shape[2] < state.n_ctx_data or valid.stride(2) != 1:
+        raise ValueError("valid must be bool / uint8 [B, H_kv, >= n_ctx_data] with contiguous rows")
+    for t in (size_global, size_local):
+        if t.dtype != torch.int64 or tuple(t.shape) != (B, Hkv) or not t.is_contiguous():
+            raise ValueError("size_global / size_local must be contiguous int64 [B, H_kv]")
+    return S
+
+
+def prefill_past_mask(valid: torch.Tensor, size_global: torch.Tensor, size_local: torch.Tensor, roles: torch.Tensor,
+                      x_len: int, C: int, W: int, state: PastState) -> torch.Tensor:
+    """Bool [B, H_kv, x_len, n_ctx_data + x_len]: the mask NAtSChunkLayerCache.generate_mask returns for a
+    multi-token segment over a non-empty cache (components/cache/nats_chunk_layer_cache.py:462-511)."""
+    _require_cuda(valid, size_global, size_local, roles)
+    lib = _lib.load()
+    B, Hkv = valid.shape[:2]
+    roles = roles.contiguous()
+    S = _check_past(valid, size_global, size_local, roles, B, Hkv, x_len, C, state)
+    N = state.n_ctx_data + x_len
+    mask = torch.empty(B, Hkv, x_len, N, dtype=torch.uint8, device=valid.device)
+    ws = workspace(valid.device, "prefill", lib.nats_prefill_past_workspace_bytes(B, Hkv, N, S))
+    valid_u8 = valid.view(torch.uint8) if valid.dtype == torch.bool else valid
+    check(lib.nats_prefill_past_mask(_ptr(valid_u8), _ptr(size_global), _ptr(size_local), _ptr(roles), B, Hkv, x_len, C, W,
+                                     ctypes.byref(state), i64_array(valid.stride()[:2]), _ptr(mask), _ptr(ws), ws.numel(),
+                                     _stream(valid)))
+    return mask.bool()
+
+
+def prefill_past_attention(q: torch.Tensor, cache_k: torch.Tensor, cache_v: torch.Tensor, valid: torch.Tensor,
+                           size_global: torch.Tensor, size_local: torch.Tensor, roles: torch.Tensor, chunk_size: int,
+                           window: int, state: PastState, sm_scale: float | None = None) -> torch.Tensor:
+    """Attention of a multi-token segment over a cache that earlier segments filled and evicted.
+
+    q [B, H_q, x_len, D]; cache_k / cache_v [B, H_kv, >= n_ctx_data + x_len, D] with the segment already
+    appended at rows [n_ctx_data, n_ctx_data + x_len); valid / size_global / size_local are the cache's
+    valid_tokens, size_global_kv, size_local_kv; roles uint8 [B, H_kv, ceil((old_fill + x_len) / chunk_size)].
+    Equals SDPA(q, cache_k[:, :, :N], cache_v[:, :, :N], generate_mask(x_len)) of the reference."""
+    _require_cuda(q, cache_k, cache_v, valid, size_global, size_local, roles)
+    lib = _lib.load()
+    B, Hq, x_len, D = q.shape
+    Hkv = cache_k.shape[1]
+    N = state.n_ctx_data + x_len
+    if cache_k.shape != cache_v.shape or cache_k.shape[0] != B or cache_k.shape[3] != D or cache_k.shape[2] < N:
+        raise ValueError(f"cache_k / cache_v must be [B, H_kv, >= {N}, D], got {tuple(cache_k.shape)}, {tuple(cache_v.shape)}")
+    if not (q.dtype == cache_k.dtype == cache_v.dtype):
+        raise ValueError("q and the cache must share one dtype")
+    if cache_k.stride(-1) != 1 or cache_v.stride(-1) != 1:
+        raise ValueError("cache_k / cache_v need a contiguous last dimension")
+    roles = roles.contiguous()
+    S = _check_past(valid, size_global, size_local, roles, B, Hkv, x_len, chunk_size, state)
+    q = q if q.stride(-1) == 1 else q.contiguous()
+    out = torch.empty(B, Hq, x_len, D, dtype=q.dtype, device=q.device)
+    scale = (1.0 / math.sqrt(D)) if sm_scale is None else float(sm_scale)
+    ws = workspace(q.device, "prefill", lib.nats_prefill_past_workspace_bytes(B, Hkv, N, S))
+    valid_u8 = valid.view(torch.uint8) if valid.dtype == torch.bool else valid
+    check(lib.nats_prefill_past_fwd(_ptr(q), _ptr(cache_k), _ptr(cache_v), _ptr(valid_u8), _ptr(size_global),
+                                    _ptr(size_local), _ptr(roles), _ptr(out), B, Hq, Hkv, x_len, D, chunk_size, window,
+                                    ctypes.byref(state), i64_array(q.stride()[:3]), i64_array(cache_k.stride()[:3]),
+                                    i64_array(cache_v.stride()[:3]), i64_array(valid.stride()[:2]),
+                                    i64_array(out.stride()[:3]), scale, _dtype_code(q), _ptr(ws), ws.numel(), _stream(q)))
+    return out
+
+
 def nats_prefill(q, k, v, end_seqs_idx, sliding_tokens, sm_scale, nats_chunk_size: int = 1, global_kv_size=None,
                  local_kv_size=None, valid_sw_tokens=None, n_ctx_data=None, sw_token_tails=None, n_rep: int = 1,
                  n_tokens_in_first_chunk: int = 0, local_seq_max_length: int = 4, return_masks: bool = False,
@@ -164,7 +238,11 @@ def nats_prefill(q, k, v, end_seqs_idx, sliding_tokens, sm_scale, nats_chunk_siz
     sliding_tokens [B, H_kv, S] is option 2 of token_states_info.  A slot is global iff
     end_seqs_idx[n] == n (nats_flashattn_fwd.py:110)."""
     if global_kv_size is not None:
-        raise NotImplementedError("prefill over an existing evicted cache (HAS_PAST_INFO) is not built yet")
+        # the reference's only caller of this form (hf/llama.py:237-252) unpacks four results from a function
+        # that returns two; the working path for such a segment is generate_mask + SDPA, which
+        # prefill_past_attention stands in for
+        raise NotImplementedError("the HAS_PAST_INFO form is not mirrored: use prefill_past_attention, the "
+                                  "replacement of generate_mask + SDPA for a segment over an existing cache")
     if q.shape[1] // k.shape[1] != n_rep:
         raise ValueError(f"n_rep={n_rep} does not match {q.shape[1]} q heads / {k.shape[1]} kv heads")
     S = end_seqs_idx.shape[-1]

@@ -56,7 +56,7 @@ def test_window_not_multiple_of_chunk_is_rejected():
 def test_prefill_rejects_bad_head_dim_and_small_workspace():
     lib = _lib.load()
     fake = ctypes.c_void_p(256)
-    st = _lib.i64_array([1, 1, 1])
+    st = _lib.i64_array([8, 8, 8])
     rc = lib.nats_prefill_fwd(fake, fake, fake, fake, fake, 1, 4, 2, 128, 96, 64, 128, st, st, st, st, 1.0, 0, fake, 1 << 20,
                               None)
     assert rc == -4
@@ -65,6 +65,23 @@ def test_prefill_rejects_bad_head_dim_and_small_workspace():
     rc = lib.nats_prefill_fwd(fake, fake, fake, fake, fake, 1, 5, 2, 128, 128, 64, 128, st, st, st, st, 1.0, 0, fake, 1 << 20,
                               None)
     assert rc == -2
+
+
+def test_past_state_is_validated():
+    lib = _lib.load()
+    fake = ctypes.c_void_p(256)
+    st = _lib.i64_array([8, 8, 8])
+    args = lambda ps, ws=1 << 24: (fake, fake, fake, fake, fake, fake, fake, fake, 1, 4, 2, 100, 128, 16, 32,
+                                   ctypes.byref(ps), st, st, st, st, st, 1.0, 0, fake, ws, None)
+    ok = _lib.PastState(320, 5, 64, 16, 400, 5)
+    assert lib.nats_prefill_past_fwd(*args(ok, 8)) == -5  # everything valid but the workspace
+    assert lib.nats_prefill_past_fwd(*args(_lib.PastState(320, 16, 64, 16, 400, 5))) == -2  # old_fill >= C
+    assert lib.nats_prefill_past_fwd(*args(_lib.PastState(320, 5, 16, 16, 400, 5))) == -2  # gmin < W
+    assert lib.nats_prefill_past_fwd(*args(_lib.PastState(320, 5, 64, 32, 400, 5))) == -2  # tail >= W
+    assert lib.nats_prefill_past_fwd(*args(_lib.PastState(20, 5, 64, 16, 400, 5))) == -2  # n_ctx_data < W + old_fill
+    assert b"n_ctx_data" in lib.nats_last_error()
+    need = lib.nats_prefill_past_workspace_bytes(1, 2, 420, 7)
+    assert need >= 2 * (7 * 4 + 4 + 420 * 4 + 7 * 8)
 
 
 def test_evict_params_are_validated():

@@ -22,9 +22,19 @@ def rope_tables(B, start, n, D, device):
 
 @pytest.mark.parametrize("L,C,W,steps", [(100, 16, 32, 40), (64, 16, 32, 20), (5, 8, 16, 30)])
 def test_module_prefill_and_decode(L, C, W, steps):
+    run_module([L] + [1] * steps, C, W)
+
+
+@pytest.mark.parametrize("lens,C,W", [([70, 45, 1, 1, 33, 16, 1, 90], 16, 32), ([3, 9, 40, 1, 1, 1, 25], 8, 16)])
+def test_module_segments_over_a_filled_cache(lens, C, W):
+    """Multi-token segments after the first one run the segment kernel over the evicted cache."""
+    run_module(lens, C, W)
+
+
+def run_module(lens, C, W):
     from neuralattentionsearch_amd.attention import LlamaNAtSChunkAttentionLayer, apply_rotary_pos_emb
     from neuralattentionsearch_amd.cache import NAtSCache
-    say("attention module", L, C, W, steps)
+    say("attention module", lens, C, W)
     torch.manual_seed(0)
     B, dim, Hq, Hkv = 2, 512, 8, 2
     D = dim // Hq
@@ -48,8 +58,7 @@ def test_module_prefill_and_decode(L, C, W, steps):
 
     fill, seen = 0, 0
     with torch.no_grad():
-        for step in range(steps + 1):
-            n = L if step == 0 else 1
+        for step, n in enumerate(lens):
             x = torch.randn(B, n, dim, device="cuda")
             q, k, v, pos = qkv(x, seen)
             logits_seen.clear()
@@ -69,6 +78,8 @@ def test_module_prefill_and_decode(L, C, W, steps):
             if seen == 0:
                 mask = orc.prefill_mask(roles, n, C, W)
                 att = orc.masked_attention(q.cpu(), ko, vo, mask)
+            elif n > 1:
+                att = orc.masked_attention(q.cpu(), ko, vo, st.generate_mask(n))
             else:
                 att = orc.decode_attention(q.cpu(), ko, vo, torch.from_numpy(st.valid), st.n_ctx_data + 1)
             st.post_update(n)

@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 import torch
 
-from oracle.nats_oracle import ChunkCacheOracle, one_hot_roles
+from oracle.nats_oracle import ChunkCacheOracle, masked_attention, one_hot_roles
 from tests.golden_io import Golden
 from tests.gpu_util import say
 
@@ -32,8 +32,9 @@ def compare(hip, st, where):
         assert np.array_equal(hip.token_positions.cpu().numpy().astype(np.int64), st.pos_k), (where, "index map")
 
 
-def drive(name, B, H, D, C, W, segs, dtype, seed, check_masks=True):
-    """segs: list of (x_len, roles uint8 [B, H, S])."""
+def drive(name, B, H, D, C, W, segs, dtype, seed, check_masks=True, attend_n_rep=0):
+    """segs: list of (x_len, roles uint8 [B, H, S]).  With attend_n_rep > 0 every multi-token segment over a
+    non-empty cache also runs the segment attention kernel against masked attention on the oracle's cache."""
     from neuralattentionsearch_amd.cache import NAtSChunkLayerCache
     hip = NAtSChunkLayerCache(B, H, W, chunk_size=C, device="cuda", track_positions=True)
     st = ChunkCacheOracle(B=B, H=H, W=W, C=C)
@@ -48,8 +49,18 @@ def drive(name, B, H, D, C, W, segs, dtype, seed, check_masks=True):
         kh, vh = hip.update(k.cuda(), v.cuda(), tsi.cuda())
         assert torch.equal(kh.cpu().view(torch.int16 if dtype == torch.bfloat16 else torch.int32),
                            ko.contiguous().view(torch.int16 if dtype == torch.bfloat16 else torch.int32)), (name, oi, "update K")
-        if check_masks and (x_len == 1 or t_seen == 0):
-            assert np.array_equal(hip.generate_mask(x_len).cpu().numpy(), st.generate_mask(x_len)), (name, oi, "mask")
+        if check_masks:
+            want_mask = st.generate_mask(x_len)
+            got_mask = hip.generate_mask(x_len).cpu().numpy()
+            assert got_mask.shape == want_mask.shape, (name, oi, "mask shape", got_mask.shape, want_mask.shape)
+            assert np.array_equal(got_mask, want_mask), (name, oi, "mask", np.argwhere(got_mask != want_mask)[:8])
+        if attend_n_rep and x_len > 1 and t_seen > 0:
+            q = torch.randn(B, H * attend_n_rep, x_len, D, generator=g).to(dtype)
+            want = masked_attention(q.float(), ko.float(), vo.float(), st.generate_mask(x_len))
+            got = hip.segment_attention(q.cuda()).float().cpu()
+            err = (got - want).abs().max().item()
+            tol = 2e-2 if dtype == torch.bfloat16 else 1e-5
+            assert err <= tol, (name, oi, "segment attention", err)
         st.post_update(x_len)
         hip.post_update(x_len)
         compare(hip, st, (name, oi, x_len))
@@ -63,6 +74,17 @@ def test_replay_reference_scenarios(name, dtype):
     si, sc = GOLD.scenario(name)
     segs = [(op["x_len"], GOLD.op(si, oi)["roles"]) for oi, op in enumerate(sc["ops"])]
     drive(name, sc["B"], sc["H"], 8, sc["C"], sc["W"], segs, dtype, seed=si)
+
+
+@pytest.mark.parametrize("name", [n for n in GOLD.scenario_names()
+                                  if sum(op["x_len"] > 1 for op in GOLD.scenario(n)[1]["ops"]) > 1])
+@pytest.mark.parametrize("dtype,D,n_rep", [(torch.float32, 64, 2), (torch.bfloat16, 128, 4)])
+def test_segment_attention_on_reference_scenarios(name, dtype, D, n_rep):
+    """Multi-token segments over a non-empty cache: mask (bit exact against the oracle, which the golden
+    vectors pin) and attention output of the segment kernel."""
+    si, sc = GOLD.scenario(name)
+    segs = [(op["x_len"], GOLD.op(si, oi)["roles"]) for oi, op in enumerate(sc["ops"])]
+    drive(name, sc["B"], sc["H"], D, sc["C"], sc["W"], segs, dtype, seed=si, attend_n_rep=n_rep)
 
 
 def role_stream(rng, B, H, C, lens, p):
@@ -100,7 +122,17 @@ def test_multi_segment_and_streaming_random(C, W):
     rng = np.random.default_rng(C)
     lens = [10 * C, 4 * C, C, C, 3 * C + 7, 2 * C - 7, 1, 1, 5 * C] + [C] * 6
     drive(f"multiseg_C{C}", 2, 3, 128, C, W, role_stream(rng, 2, 3, C, lens, (0.15, 0.25, 0.6)), torch.bfloat16, seed=C,
-          check_masks=True)
+          check_masks=True, attend_n_rep=4)
+
+
+@pytest.mark.parametrize("C,W,D,dtype,n_rep", [(64, 256, 128, torch.bfloat16, 4), (8, 32, 64, torch.bfloat16, 2),
+                                               (16, 64, 64, torch.float32, 1), (128, 256, 128, torch.bfloat16, 4)])
+def test_segments_before_the_window_is_full_and_ragged_segments(C, W, D, dtype, n_rep):
+    """Short first segments (cache seen < W, open chunks carried between segments), then long ones."""
+    rng = np.random.default_rng(7 * C + W)
+    lens = [C // 2 + 1, C // 2, C + 3, 2 * C - 5, 5, W + 2 * C + 1, 3, C - 1, 6 * C + 9, 1, 1, 2 * C]
+    drive(f"ragged_C{C}", 2, 2, D, C, W, role_stream(rng, 2, 2, C, lens, (0.2, 0.3, 0.5)), dtype, seed=C + 1,
+          attend_n_rep=n_rep)
 
 
 def test_surviving_index_map_semantics():
