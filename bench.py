@@ -1,6 +1,6 @@
 """Benchmark of the NAtS sparse-attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-cpu] [--only prefill|decode|evict]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-cpu] [--only prefill|decode|evict|evict_stream|llama]
 
 One step = one pass of a kernel family over one batch of synthetic input that is already resident in HBM:
 
@@ -206,6 +206,78 @@ def bench_evict(args, ops):
     }
 
 
+def bench_evict_stream(args, ops):
+    """The streamed form of the eviction workload: the same 16 x 8 x 65536 x 128 cache filled chunk by chunk,
+    1024 x (update(64 tokens) + post_update(64)); every post_update runs the in-place plan + apply kernels."""
+    from neuralattentionsearch_amd.cache import NAtSChunkLayerCache
+    B, Hkv, L, D, C, W = 16, 8, 65536, 128, 64, 512
+    dev = "cuda"
+    n_chunks = L // C
+    g = torch.Generator(device=dev).manual_seed(0)
+    k = torch.randn(B, Hkv, C, D, generator=g, device=dev).bfloat16()
+    v = torch.randn(B, Hkv, C, D, generator=g, device=dev).bfloat16()
+    roles_np = draw_roles(0, B, Hkv, n_chunks, (0.10, 0.15, 0.75))
+    tsi_all = torch.zeros(B, Hkv, n_chunks, 3, dtype=torch.bfloat16, device=dev)
+    tsi_all.scatter_(-1, torch.from_numpy(roles_np.astype(np.int64)).to(dev).unsqueeze(-1), 1.0)
+    tsis = [tsi_all[:, :, i:i + 1].contiguous() for i in range(n_chunks)]
+    cache = NAtSChunkLayerCache(B, Hkv, W, chunk_size=C, device=dev)
+
+    def run():
+        cache.reset_cache()
+        for i in range(n_chunks):
+            cache.update(k, v, tsis[i])
+            cache.post_update(C)
+
+    run()  # warm-up: sizes the capacity buffers
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    run()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return {"total_s": wall, "us_per_chunk_step": wall / n_chunks * 1e6, "chunks": n_chunks,
+            "cache_rows_after": int(cache.cache_k.shape[2]),
+            "note": "host-driven loop: update (append 64 tokens) + post_update (plan, result readback, in-place apply)",
+            "shape": dict(B=B, Hkv=Hkv, L=L, D=D, C=C, W=W)}
+
+
+def bench_llama(args):
+    """End to end at the Llama-3-8B shape with random weights: one prefill, then greedy decode steps with
+    eviction live in all 32 layers."""
+    from neuralattentionsearch_amd.llama import NAtSLlamaConfig, NAtSLlamaForCausalLM
+    cfg = NAtSLlamaConfig.llama3_8b()
+    model = NAtSLlamaForCausalLM.random_init(cfg, seed=0)
+    g = torch.Generator().manual_seed(0)
+    ids = torch.randint(0, cfg.vocab_size, (1, args.llama_prefill), generator=g).cuda()
+    warm = model.new_cache()
+    logits = model(ids[:, :2048], 0, warm)  # loads every kernel and the GEMM heuristics once
+    for i in range(3):
+        logits = model(logits.argmax(-1, keepdim=True), 2048 + i, warm)
+    del warm
+    cache = model.new_cache()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    logits = model(ids, 0, cache)
+    torch.cuda.synchronize()
+    t_prefill = time.perf_counter() - t0
+    pos = args.llama_prefill
+    t0 = time.perf_counter()
+    for i in range(args.llama_decode):
+        logits = model(logits.argmax(-1, keepdim=True), pos, cache)
+        pos += 1
+    torch.cuda.synchronize()
+    t_decode = time.perf_counter() - t0
+    kept = [float(l.valid_tokens[:, :, :l.n_ctx_data].sum().item()) / (cfg.num_key_value_heads * pos) for l in cache.cache_model]
+    return {"prefill_s": t_prefill, "prefill_tokens_per_s": args.llama_prefill / t_prefill,
+            "decode_s": t_decode, "decode_tokens_per_s": args.llama_decode / t_decode,
+            "decode_ms_per_token": t_decode / args.llama_decode * 1e3,
+            "kept_fraction_mean": float(np.mean(kept)), "kept_fraction_min": float(np.min(kept)),
+            "kept_fraction_max": float(np.max(kept)),
+            "shape": dict(layers=cfg.num_hidden_layers, d_model=cfg.hidden_size, heads="32/8", head_dim=cfg.head_dim,
+                          ffn=cfg.intermediate_size, vocab=cfg.vocab_size, prefill=args.llama_prefill,
+                          decode_steps=args.llama_decode, chunk=cfg.chunk_size, window=cfg.local_seq_max_length),
+            "note": "random weights give near-uniform roles; projections / MLP / norms are library GEMMs and torch ops"}
+
+
 # --------------------------------------------------------------------------------------------------
 def cpu_baseline(args):
     """The oracle (a port of the reference's PyTorch path) on this host's cores, bounded samples."""
@@ -267,7 +339,9 @@ def main():
     ap.add_argument("--prefill-len", type=int, default=32768)
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--no-compare", action="store_true", help="skip the dense comparators of the prefill leg")
-    ap.add_argument("--only", choices=["prefill", "decode", "evict", "copy"], default=None)
+    ap.add_argument("--only", choices=["prefill", "decode", "evict", "copy", "evict_stream", "llama"], default=None)
+    ap.add_argument("--llama-prefill", type=int, default=16384)
+    ap.add_argument("--llama-decode", type=int, default=512)
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures the one-GPU hot path; it does not run on more than one GPU (--gpus 1 only)",
@@ -292,8 +366,12 @@ def main():
         res["decode"] = bench_decode(args, ops)
     if args.only in (None, "evict"):
         res["evict"] = bench_evict(args, ops)
+    if args.only == "evict_stream":  # not part of the default run
+        res["evict_stream"] = bench_evict_stream(args, ops)
+    if args.only == "llama":  # not part of the default run
+        res["llama_e2e"] = bench_llama(args)
     torch.cuda.synchronize()
-    cpu = None if args.skip_cpu else cpu_baseline(args)
+    cpu = None if args.skip_cpu or args.only in ("evict_stream", "llama") else cpu_baseline(args)
 
     pre = res.get("prefill")
     line = {

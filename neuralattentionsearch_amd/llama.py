@@ -1,0 +1,210 @@
+"""A Llama-architecture inference model whose attention layers follow the call order of the reference's
+Hugging Face twin, forward_llama_nats_chunk_one_way (src/nats/models/transformer/hf/llama_nats_chunk.py:171-292):
+
+    q / k / v projections -> pooled role logits -> argmax roles -> RoPE -> cache.update -> attention kernel
+    -> cache.post_update -> o_proj
+
+The attention itself, the roles and the cache run on the HIP kernels of this package; embeddings, RMSNorm,
+the SwiGLU MLP and the projections are plain torch modules (library GEMMs), as they are in the reference.
+Differences from BaseNAtSChunkAttentionLayer that this twin has and that are kept: no bias on the global
+logit (:206-214 takes the plain maximum) and `position_ids[0, 0] == 0` decides between the prefill kernel
+and the cached paths (:194, :238-270).
+
+Weights are random-initialised (there is no checkpoint loader here); `NAtSLlamaConfig.llama3_8b()` gives the
+Llama-3-8B shape.
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+
+import torch
+from torch import nn
+
+from . import ops
+from .attention import apply_rotary_pos_emb
+from .cache import ChunkMergeType, NAtSCache
+
+
+@dataclass
+class NAtSLlamaConfig:
+    vocab_size: int = 128256
+    hidden_size: int = 4096
+    intermediate_size: int = 14336
+    num_hidden_layers: int = 32
+    num_attention_heads: int = 32
+    num_key_value_heads: int = 8
+    rms_norm_eps: float = 1e-5
+    rope_theta: float = 500000.0
+    chunk_size: int = 64
+    local_seq_max_length: int = 256  # sliding window, in tokens
+    chunk_merge_method: str = "mean"
+
+    @property
+    def head_dim(self) -> int:
+        return self.hidden_size // self.num_attention_heads
+
+    @staticmethod
+    def llama3_8b(**kw) -> "NAtSLlamaConfig":
+        return NAtSLlamaConfig(**kw)
+
+
+class RMSNorm(nn.Module):
+    def __init__(self, dim: int, eps: float):
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(dim))
+        self.eps = eps
+
+    def forward(self, x):
+        h = x.float()
+        h = h * torch.rsqrt(h.pow(2).mean(-1, keepdim=True) + self.eps)
+        return self.weight * h.to(x.dtype)
+
+
+class LlamaMLP(nn.Module):
+    def __init__(self, cfg: NAtSLlamaConfig):
+        super().__init__()
+        self.gate_proj = nn.Linear(cfg.hidden_size, cfg.intermediate_size, bias=False)
+        self.up_proj = nn.Linear(cfg.hidden_size, cfg.intermediate_size, bias=False)
+        self.down_proj = nn.Linear(cfg.intermediate_size, cfg.hidden_size, bias=False)
+
+    def forward(self, x):
+        return self.down_proj(nn.functional.silu(self.gate_proj(x)) * self.up_proj(x))
+
+
+def rotary_tables(position_ids: torch.Tensor, head_dim: int, theta: float, dtype: torch.dtype):
+    """cos / sin [B, L, head_dim], computed in fp32 and cast, the Hugging Face Llama convention."""
+    inv = 1.0 / (theta ** (torch.arange(0, head_dim, 2, device=position_ids.device, dtype=torch.float32) / head_dim))
+    freqs = position_ids[:, :, None].float() * inv[None, None, :]
+    emb = torch.cat([freqs, freqs], dim=-1)
+    return emb.cos().to(dtype), emb.sin().to(dtype)
+
+
+class NAtSLlamaAttention(nn.Module):
+    """llama_nats_chunk.py:171-292 with the attention, the roles and the cache on the HIP kernels."""
+
+    def __init__(self, cfg: NAtSLlamaConfig, layer_idx: int):
+        super().__init__()
+        self.layer_idx = layer_idx
+        self.hidden_size = cfg.hidden_size
+        self.num_heads = cfg.num_attention_heads
+        self.num_key_value_heads = cfg.num_key_value_heads
+        self.num_key_value_groups = self.num_heads // self.num_key_value_heads
+        self.head_dim = cfg.head_dim
+        self.chunk_size = cfg.chunk_size
+        self.local_seq_max_length = cfg.local_seq_max_length
+        if cfg.chunk_merge_method not in ("mean", "max"):
+            raise NotImplementedError(cfg.chunk_merge_method)
+        self.chunk_merge_method = ChunkMergeType.MEAN if cfg.chunk_merge_method == "mean" else ChunkMergeType.MAX
+        self.q_proj = nn.Linear(cfg.hidden_size, self.num_heads * self.head_dim, bias=False)
+        self.k_proj = nn.Linear(cfg.hidden_size, self.num_key_value_heads * self.head_dim, bias=False)
+        self.v_proj = nn.Linear(cfg.hidden_size, self.num_key_value_heads * self.head_dim, bias=False)
+        self.o_proj = nn.Linear(self.num_heads * self.head_dim, cfg.hidden_size, bias=False)
+        self.proj_layer = nn.Linear(cfg.hidden_size, self.num_key_value_heads * 3, bias=False)  # :315-318
+
+    def forward(self, hidden_states: torch.Tensor, position_embeddings, start_pos: int, past_key_value: NAtSCache):
+        bsz, q_len, _ = hidden_states.shape
+        C, idx = self.chunk_size, self.layer_idx
+        q = self.q_proj(hidden_states).view(bsz, q_len, self.num_heads, self.head_dim).transpose(1, 2)
+        k = self.k_proj(hidden_states).view(bsz, q_len, self.num_key_value_heads, self.head_dim).transpose(1, 2)
+        v = self.v_proj(hidden_states).view(bsz, q_len, self.num_key_value_heads, self.head_dim).transpose(1, 2)
+
+        pre_fill = past_key_value.get_nats_chunk_fill_size(idx)
+        is_pre_filling = start_pos == 0
+        if pre_fill + q_len < C:
+            past_key_value.update_nats_cached_x_in_chunk(hidden_states, idx, self.chunk_merge_method)
+            roles = torch.zeros(bsz, self.num_key_value_heads, 1, dtype=torch.uint8, device=hidden_states.device)
+            tsi = torch.zeros(bsz, self.num_key_value_heads, 1, 3, dtype=hidden_states.dtype, device=hidden_states.device)
+            tsi[..., 0] = 1
+        else:
+            pooled, pad = past_key_value.update_nats_cached_x_across_chunk(hidden_states, pre_fill, idx,
+                                                                           self.chunk_merge_method)
+            logit = self.proj_layer(pooled).unflatten(-1, (self.num_key_value_heads, 3))
+            roles, tsi = ops.roles_from_logits(logit, 0.0, force_first_global=start_pos < C, force_last_global=pad != 0)
+
+        cos, sin = position_embeddings
+        q, k = apply_rotary_pos_emb(q, k, cos, sin)
+        keys, values = past_key_value.update(k, v, idx, cache_kwargs={"token_states_info": tsi})
+        layer = past_key_value.cache_model[idx]
+        scale = 1.0 / math.sqrt(self.head_dim)
+        if is_pre_filling:
+            out = ops.prefill_attention(q, keys, values, roles, C, self.local_seq_max_length, scale)
+        elif q_len > 1:
+            out = layer.segment_attention(q, scale)
+        else:
+            out = ops.decode_attention(q, keys, values, layer.valid_tokens, keys.shape[2], scale,
+                                       row_end=layer.size_global_kv + layer.size_local_kv,
+                                       tail_start=layer.n_ctx_data - (layer.chunk_fill_size - 1))
+        past_key_value.post_update(layer_idx=idx, x_len=q_len)
+        return self.o_proj(out.transpose(1, 2).reshape(bsz, q_len, -1))
+
+
+class NAtSLlamaDecoderLayer(nn.Module):
+    def __init__(self, cfg: NAtSLlamaConfig, layer_idx: int):
+        super().__init__()
+        self.self_attn = NAtSLlamaAttention(cfg, layer_idx)
+        self.mlp = LlamaMLP(cfg)
+        self.input_layernorm = RMSNorm(cfg.hidden_size, cfg.rms_norm_eps)
+        self.post_attention_layernorm = RMSNorm(cfg.hidden_size, cfg.rms_norm_eps)
+
+    def forward(self, x, position_embeddings, start_pos: int, cache: NAtSCache):
+        x = x + self.self_attn(self.input_layernorm(x), position_embeddings, start_pos, cache)
+        return x + self.mlp(self.post_attention_layernorm(x))
+
+
+class NAtSLlamaForCausalLM(nn.Module):
+    def __init__(self, cfg: NAtSLlamaConfig):
+        super().__init__()
+        self.config = cfg
+        self.embed_tokens = nn.Embedding(cfg.vocab_size, cfg.hidden_size)
+        self.layers = nn.ModuleList([NAtSLlamaDecoderLayer(cfg, i) for i in range(cfg.num_hidden_layers)])
+        self.norm = RMSNorm(cfg.hidden_size, cfg.rms_norm_eps)
+        self.lm_head = nn.Linear(cfg.hidden_size, cfg.vocab_size, bias=False)
+
+    @staticmethod
+    def random_init(cfg: NAtSLlamaConfig, device="cuda", dtype=torch.bfloat16, seed: int = 0, std: float = 0.02):
+        """Builds the model on `device` without a host copy of the weights."""
+        with torch.device("meta"):
+            model = NAtSLlamaForCausalLM(cfg)
+        model = model.to_empty(device=device).to(dtype)
+        g = torch.Generator(device=device).manual_seed(seed)
+        with torch.no_grad():
+            for name, p in model.named_parameters():
+                if name.endswith("layernorm.weight") or name == "norm.weight":
+                    p.fill_(1.0)
+                else:
+                    p.normal_(0.0, std, generator=g)
+        return model.eval()
+
+    def new_cache(self, track_positions: bool = False) -> NAtSCache:
+        return NAtSCache(sliding_window_size=self.config.local_seq_max_length, chunk_size=self.config.chunk_size,
+                         track_positions=track_positions)
+
+    @torch.no_grad()
+    def forward(self, input_ids: torch.Tensor, start_pos: int, cache: NAtSCache, all_logits: bool = False):
+        """input_ids [B, L] -> logits of the last position [B, vocab] (or of every position)."""
+        bsz, q_len = input_ids.shape
+        x = self.embed_tokens(input_ids)
+        pos = torch.arange(start_pos, start_pos + q_len, device=input_ids.device)[None].expand(bsz, -1)
+        position_embeddings = rotary_tables(pos, self.config.head_dim, self.config.rope_theta, x.dtype)
+        for layer in self.layers:
+            x = layer(x, position_embeddings, start_pos, cache)
+        x = self.norm(x if all_logits else x[:, -1:])
+        logits = self.lm_head(x)
+        return logits if all_logits else logits[:, 0]
+
+    @torch.no_grad()
+    def generate(self, input_ids: torch.Tensor, max_new_tokens: int, cache: NAtSCache | None = None):
+        """Greedy decoding with eviction live.  Returns (new tokens [B, max_new_tokens], cache)."""
+        cache = self.new_cache() if cache is None else cache
+        start = cache.get_seq_length(0) if len(cache.cache_model) else 0
+        logits = self.forward(input_ids, start, cache)
+        pos = start + input_ids.shape[1]
+        out = []
+        for i in range(max_new_tokens):
+            tok = logits.argmax(-1, keepdim=True)
+            out.append(tok)
+            if i + 1 < max_new_tokens:
+                logits = self.forward(tok, pos, cache)
+                pos += 1
+        return torch.cat(out, dim=1) if out else input_ids[:, :0], cache

@@ -1,0 +1,133 @@
+"""GPU: the Llama-architecture harness, layer by layer against the oracle.
+
+Every attention layer of the model is observed through hooks: its input hidden states, its role logits
+and the attention output it hands to o_proj.  The oracle side recomputes, per layer, roles -> cache update ->
+mask -> attention -> eviction from the same q / k / v and logits and must agree on the attention output, on
+the cache bookkeeping after every call and on the roles."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import nats_oracle as orc
+from tests.gpu_util import say
+
+pytestmark = pytest.mark.gpu
+
+
+class LayerProbe:
+    def __init__(self, attn):
+        self.attn = attn
+        self.hidden = self.logits = self.att = None
+        attn.register_forward_pre_hook(self._pre)
+        attn.proj_layer.register_forward_hook(self._logit)
+        attn.o_proj.register_forward_pre_hook(self._att)
+
+    def _pre(self, m, args):
+        self.hidden, self.pos_emb, self.start_pos = args[0].detach(), args[1], args[2]
+        self.logits = None
+
+    def _logit(self, m, i, o):
+        self.logits = o.detach().float().cpu()
+
+    def _att(self, m, args):
+        self.att = args[0].detach()
+
+
+def run(cfg, dtype, lens, tol, B=2, seed=0, std=0.05):
+    from neuralattentionsearch_amd.attention import apply_rotary_pos_emb
+    from neuralattentionsearch_amd.llama import NAtSLlamaForCausalLM
+    model = NAtSLlamaForCausalLM.random_init(cfg, dtype=dtype, seed=seed, std=std)
+    with torch.no_grad():
+        for layer in model.layers:
+            layer.self_attn.proj_layer.weight.mul_(6.0)  # spread the role logits
+    probes = [LayerProbe(layer.self_attn) for layer in model.layers]
+    cache = model.new_cache()
+    C, W = cfg.chunk_size, cfg.local_seq_max_length
+    Hq, Hkv, D = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
+    states = [orc.ChunkCacheOracle(B=B, H=Hkv, W=W, C=C) for _ in model.layers]
+    fills = [0] * len(model.layers)
+    g = torch.Generator().manual_seed(seed)
+    seen = 0
+    role_counts = np.zeros(3, dtype=np.int64)
+    for step, n in enumerate(lens):
+        say("llama harness", dtype, "step", step, "tokens", n)
+        ids = torch.randint(0, cfg.vocab_size, (B, n), generator=g).cuda()
+        logits = model(ids, seen, cache)
+        assert logits.shape == (B, cfg.vocab_size) and torch.isfinite(logits).all()
+        for li, (pr, st) in enumerate(zip(probes, states)):
+            a = pr.attn
+            with torch.no_grad():
+                q = a.q_proj(pr.hidden).view(B, n, Hq, D).transpose(1, 2)
+                k = a.k_proj(pr.hidden).view(B, n, Hkv, D).transpose(1, 2)
+                v = a.v_proj(pr.hidden).view(B, n, Hkv, D).transpose(1, 2)
+                q, k = apply_rotary_pos_emb(q, k, *pr.pos_emb)
+            total = fills[li] + n
+            if total < C:
+                roles = np.zeros((B, Hkv, 1), dtype=np.uint8)
+                assert pr.logits is None
+                fills[li] = total
+            else:
+                lg = pr.logits.unflatten(-1, (Hkv, 3)).to(dtype)
+                roles = orc.roles_from_logits(lg, 0.0, force_first_global=seen < C, force_last_global=total % C != 0)
+                assert roles.shape[-1] == math.ceil(total / C)
+                fills[li] = total % C
+                role_counts += np.bincount(roles.ravel(), minlength=3)
+            ko, vo = st.update(k.cpu(), v.cpu(), roles)
+            if seen == 0:
+                att = orc.masked_attention(q.cpu().float(), ko.float(), vo.float(), orc.prefill_mask(roles, n, C, W))
+            elif n > 1:
+                att = orc.masked_attention(q.cpu().float(), ko.float(), vo.float(), st.generate_mask(n))
+            else:
+                att = orc.decode_attention(q.cpu(), ko, vo, torch.from_numpy(st.valid), st.n_ctx_data + 1).float()
+            st.post_update(n)
+            got = pr.att.float().cpu().view(B, n, Hq, D).transpose(1, 2)
+            err = (got - att).abs().max().item()
+            assert err <= tol, (step, li, err)
+            lc = cache.cache_model[li]
+            assert lc.n_ctx_data == st.n_ctx_data, (step, li)
+            assert np.array_equal(lc.valid_tokens.cpu().numpy(), st.valid), (step, li)
+            assert np.array_equal(lc.size_global_kv.cpu().numpy(), st.size_global), (step, li)
+            assert np.array_equal(lc.size_local_kv.cpu().numpy(), st.size_local), (step, li)
+        seen += n
+    assert (role_counts > 0).all(), role_counts  # the run exercised all three roles
+    return model, cache
+
+
+def test_small_fp32_model_layer_by_layer():
+    from neuralattentionsearch_amd.llama import NAtSLlamaConfig
+    cfg = NAtSLlamaConfig(vocab_size=1000, hidden_size=512, intermediate_size=1024, num_hidden_layers=3,
+                          num_attention_heads=8, num_key_value_heads=2, chunk_size=16, local_seq_max_length=32)
+    run(cfg, torch.float32, [100, 37] + [1] * 40 + [50, 1, 1], tol=2e-5)
+
+
+def test_llama_head_shape_bf16_layer_by_layer():
+    """32 q heads / 8 kv heads / head_dim 128, chunk 64, window 256, two layers."""
+    from neuralattentionsearch_amd.llama import NAtSLlamaConfig
+    cfg = NAtSLlamaConfig(vocab_size=512, hidden_size=4096, intermediate_size=1024, num_hidden_layers=2,
+                          chunk_size=64, local_seq_max_length=256)
+    run(cfg, torch.bfloat16, [1500, 200] + [1] * 70, tol=2e-2, B=1, std=4096 ** -0.5)  # q, k, v of unit scale
+
+
+def test_generate_is_deterministic_and_matches_stepwise_forward():
+    from neuralattentionsearch_amd.llama import NAtSLlamaConfig, NAtSLlamaForCausalLM
+    say("llama generate")
+    cfg = NAtSLlamaConfig(vocab_size=777, hidden_size=512, intermediate_size=512, num_hidden_layers=2,
+                          num_attention_heads=8, num_key_value_heads=4, chunk_size=8, local_seq_max_length=16)
+    model = NAtSLlamaForCausalLM.random_init(cfg, dtype=torch.float32, seed=3, std=0.08)
+    ids = torch.randint(0, 777, (2, 45), generator=torch.Generator().manual_seed(1)).cuda()
+    a, cache_a = model.generate(ids, 30)
+    b, _ = model.generate(ids, 30)
+    assert torch.equal(a, b) and a.shape == (2, 30)
+    cache = model.new_cache()
+    logits = model(ids, 0, cache)
+    toks = []
+    for i in range(30):
+        tok = logits.argmax(-1, keepdim=True)
+        toks.append(tok)
+        logits = model(tok, 45 + i, cache)
+    assert torch.equal(torch.cat(toks, 1), a)
+    # eviction was live: the cache holds fewer rows than tokens seen for at least one layer
+    assert cache_a.get_seq_length(0) == 45 + 29
+    assert min(l.n_ctx_data for l in cache_a.cache_model) < 45 + 29 + 16
