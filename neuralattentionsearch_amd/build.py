@@ -27,7 +27,7 @@ def build(verbose: bool = True) -> str:
             print(" ".join(cmd), flush=True)
         subprocess.run(cmd, check=True)
         objs.append(obj)
-    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", *objs, "-o", LIB_PATH]
+    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", "-Wl,-z,defs", *objs, "-o", LIB_PATH]
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.run(cmd, check=True)

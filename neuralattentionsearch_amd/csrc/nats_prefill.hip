@@ -158,6 +158,26 @@ __global__ __launch_bounds__(64) void prefill_simple_kernel(PrefillArgs a) {
 // ---------------------------------------------------------------------------------------------------
 constexpr float kRescaleSlack = 8.0f;
 
+// Register-file constraints and the in-place scaling of an accumulation register.  The host pass of the
+// single-source compile never runs this code and has no such registers, so the statements are empty there.
+#if defined(__HIP_DEVICE_COMPILE__)
+#define NATS_PIN_ACC(x) asm volatile("" : "+a"(x))
+#define NATS_PIN_ARCH(x) asm volatile("" : "+v"(x))
+#define NATS_SCALE_ACC(e, alpha)                                                                          \
+  do {                                                                                                    \
+    float t__;                                                                                            \
+    asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\tv_accvgpr_write_b32 %0, %1"       \
+                 : "+a"(e), "=&v"(t__)                                                                    \
+                 : "v"(alpha));                                                                           \
+  } while (0)
+#define NATS_ACC_SETTLE() asm volatile("s_nop 7")
+#else
+#define NATS_PIN_ACC(x) (void)(x)
+#define NATS_PIN_ARCH(x) (void)(x)
+#define NATS_SCALE_ACC(e, alpha) (e) *= (alpha)
+#define NATS_ACC_SETTLE() (void)0
+#endif
+
 constexpr int kWin = 1024;  // key tiles whose visit list is built at once
 
 template <int D>
@@ -180,7 +200,7 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
   PrefillSmem<D>& sm = *reinterpret_cast<PrefillSmem<D>*>(smem_raw);
 
   const int tid = threadIdx.x;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform, and the compiler may know it
   const int lane = tid & 63;
   const int l32 = lane & 31;
   const int hl = lane >> 5;
@@ -250,21 +270,59 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
   float l_run[2] = {0.f, 0.f};
   const float c = a.scale * 1.4426950408889634f;
 
-  // global -> LDS, one 64-key tile of K and of V; rows beyond N repeat row N-1 (their scores are masked,
-  // so their probabilities are exactly 0 and a finite V row contributes nothing)
-  auto issue_tile = [&](int kt, int buf, bool need_lim) {
+  // Register file placement.  The matrix instructions read their operands from either half of the unified
+  // register file; the vector ALU only from the architectural half.  Q fragments (read by MFMA only) and the
+  // output accumulators (touched by the vector ALU only on a rescale) belong in the accumulation half,
+  // scores and probabilities in the architectural half.  The empty statements below constrain the
+  // allocator accordingly at the points where the values are merged.
+  auto pin_q = [&]() {
 #pragma unroll
-    for (int j = 0; j < DMA_PER_WAVE; ++j) {
-      const int inst = wave * DMA_PER_WAVE + j;  // uniform
-      const int q = inst * kWave + lane;         // chunk slot in the LDS tile
-      const int row = q / OCT, pos = q % OCT;
-      const int n = min(kt * kTile + row, a.N - 1);
-      const int kchunk = pos ^ (row % OCT);
-      const int vchunk = pos ^ ((row & 3) << 1);
-      __builtin_amdgcn_global_load_lds(kp + (int64_t)n * a.ks_l + kchunk * 8,
-                                       (uint32_t __attribute__((address_space(3)))*)(&sm.k[buf][inst * kWave * 8]), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds(vp + (int64_t)n * a.vs_l + vchunk * 8,
-                                       (uint32_t __attribute__((address_space(3)))*)(&sm.v[buf][inst * kWave * 8]), 16, 0, 0);
+    for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+      for (int s = 0; s < DSTEPS; ++s) NATS_PIN_ACC(qreg[qb][s]);
+  };
+  auto pin_o = [&]() {
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb) NATS_PIN_ACC(oacc[dt][qb]);
+  };
+
+  // global -> LDS, one 64-key tile of K and of V; rows beyond N repeat row N-1 (their scores are masked,
+  // so their probabilities are exactly 0 and a finite V row contributes nothing).  The lane's share of a
+  // tile sits at fixed offsets from the tile's first row, computed once.
+  int koff[DMA_PER_WAVE], voff[DMA_PER_WAVE];
+#pragma unroll
+  for (int j = 0; j < DMA_PER_WAVE; ++j) {
+    const int q = (wave * DMA_PER_WAVE + j) * kWave + lane;  // chunk slot in the LDS tile
+    const int row = q / OCT, pos = q % OCT;
+    koff[j] = int(row * a.ks_l + (pos ^ (row % OCT)) * 8);
+    voff[j] = int(row * a.vs_l + (pos ^ ((row & 3) << 1)) * 8);
+  }
+  auto issue_tile = [&](int kt, int buf, bool need_lim) {
+    if (kt * kTile + kTile <= a.N) {
+      const uint16_t* kb = kp + (int64_t)kt * kTile * a.ks_l;  // uniform
+      const uint16_t* vb = vp + (int64_t)kt * kTile * a.vs_l;
+#pragma unroll
+      for (int j = 0; j < DMA_PER_WAVE; ++j) {
+        const int inst = wave * DMA_PER_WAVE + j;
+        __builtin_amdgcn_global_load_lds(kb + (int)koff[j], (uint32_t __attribute__((address_space(3)))*)(&sm.k[buf][inst * kWave * 8]), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(vb + (int)voff[j], (uint32_t __attribute__((address_space(3)))*)(&sm.v[buf][inst * kWave * 8]), 16, 0, 0);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < DMA_PER_WAVE; ++j) {
+        const int inst = wave * DMA_PER_WAVE + j;  // uniform
+        const int q = inst * kWave + lane;
+        const int row = q / OCT, pos = q % OCT;
+        const int n = min(kt * kTile + row, a.N - 1);
+        const int kchunk = pos ^ (row % OCT);
+        const int vchunk = pos ^ ((row & 3) << 1);
+        __builtin_amdgcn_global_load_lds(kp + (int64_t)n * a.ks_l + kchunk * 8,
+                                         (uint32_t __attribute__((address_space(3)))*)(&sm.k[buf][inst * kWave * 8]), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(vp + (int64_t)n * a.vs_l + vchunk * 8,
+                                         (uint32_t __attribute__((address_space(3)))*)(&sm.v[buf][inst * kWave * 8]), 16, 0, 0);
+      }
     }
     if (need_lim && tid < kTile) {
       int n = kt * kTile + tid;
@@ -272,11 +330,9 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
     }
   };
 
-  auto compute_tile = [&](int kt, int cur, bool full) {
+  // ---- S^T = K Q^T, the mask, and the scaled row maxima ----------------------------------------------
+  auto score_tile = [&](int kt, int cur, bool full, f32x16 (&sacc)[2][2], float (&mx)[2]) {
     const uint16_t* Kt = sm.k[cur];
-    const uint16_t* Vt = sm.v[cur];
-    // ---- S^T = K Q^T ---------------------------------------------------------------------------
-    f32x16 sacc[2][2];
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
       const int row = kb * 32 + l32;
@@ -294,8 +350,13 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
         }
       }
     }
-    // ---- mask (diagonal tile, or a tile whose slots are not uniformly visible) -----------------
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb) NATS_PIN_ARCH(sacc[kb][qb]);
+    // mask (diagonal tile, or a tile whose rows are not uniformly visible)
     if (!full) {
+      asm volatile("" ::: "memory");  // keeps this a branch: most tiles skip it
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
@@ -316,26 +377,47 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
         }
       }
     }
-    // ---- online softmax, one query per lane and q block ----------------------------------------
-    bf16x8 pb[2][4];
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) {
-      float mx = -INFINITY;
+      float m = -INFINITY;
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) mx = fmaxf(mx, sacc[kb][qb][i]);
-      mx = fmaxf(mx, __shfl_xor(mx, 32)) * c;
-      if (__ballot(mx > m_run[qb] + kRescaleSlack)) {
-        float m_new = fmaxf(m_run[qb], mx);
+        for (int i = 0; i < 16; ++i) m = fmaxf(m, sacc[kb][qb][i]);
+      mx[qb] = fmaxf(m, __shfl_xor(m, 32)) * c;
+    }
+  };
+
+  // ---- raise the running maxima (rare): O and l shrink by 2^(old - new) ------------------------------
+  auto rescale = [&](const float (&mx)[2]) {
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) {
+      if (__ballot(mx[qb] > m_run[qb] + kRescaleSlack)) {
+        float m_new = fmaxf(m_run[qb], mx[qb]);
         float alpha = m_run[qb] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_run[qb] - m_new);
         l_run[qb] *= alpha;
         m_run[qb] = m_new;
+        // scaled in place in the accumulation registers, one element at a time through a temporary
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
+        for (int dt = 0; dt < DT; ++dt) {
 #pragma unroll
-          for (int i = 0; i < 16; ++i) oacc[dt][qb][i] *= alpha;
+          for (int i = 0; i < 16; ++i) {
+            float e = oacc[dt][qb][i];
+            NATS_SCALE_ACC(e, alpha);
+            oacc[dt][qb][i] = e;
+          }
+        }
+        NATS_ACC_SETTLE();  // the matrix instructions that follow read these registers
       }
+    }
+  };
+
+  // ---- probabilities and O^T += V^T P^T ---------------------------------------------------------------
+  auto finish_tile = [&](int cur, const f32x16 (&sacc)[2][2]) {
+    const uint16_t* Vt = sm.v[cur];
+    bf16x8 pb[2][4];
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) {
       const float m_use = m_run[qb] == -INFINITY ? 0.f : m_run[qb];
       float rs = 0.f;
 #pragma unroll
@@ -349,7 +431,6 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
       }
       l_run[qb] += rs;
     }
-    // ---- O^T += V^T P^T ------------------------------------------------------------------------
     // ds_read_b64_tr_b16: within 16 lanes, lane r reads 4 dims of key (K0 + r / 4) starting at dim
     // D0 + 4 * (r % 4) and receives keys K0 .. K0 + 3 of dim D0 + r.
     const int r16 = lane & 15;
@@ -400,25 +481,36 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
       if (lane == 0) sm.vcount = count;
     }
     __syncthreads();
-    const int n_vis = sm.vcount;
+    const int n_vis = __builtin_amdgcn_readfirstlane(sm.vcount);
     if (n_vis > 0) {
-      issue_tile(sm.vlist[0].x, cur, true);
+      issue_tile(__builtin_amdgcn_readfirstlane(sm.vlist[0].x), cur, true);
       __builtin_amdgcn_s_waitcnt(0);
       __syncthreads();
     }
     for (int idx = 0; idx < n_vis; ++idx) {
+      // the list entries are the same for every lane: keep them in scalar registers
       const int4 ent = sm.vlist[idx];
-      const int kt = ent.x;
+      const int kt = __builtin_amdgcn_readfirstlane(ent.x);
+      const int ent_max = __builtin_amdgcn_readfirstlane(ent.y);
+      const int ent_min = __builtin_amdgcn_readfirstlane(ent.z);
+      pin_o();
+      pin_q();
       if (idx + 1 < n_vis) {
         const int4 en = sm.vlist[idx + 1];
+        const int nkt = __builtin_amdgcn_readfirstlane(en.x);
+        const int nmin = __builtin_amdgcn_readfirstlane(en.z);
         // the element mask is only evaluated on diagonal tiles and on tiles with mixed visibility
-        issue_tile(en.x, cur ^ 1, en.x * kTile + kTile - 1 - a.base > r0_group || en.z < rlast_group);
+        issue_tile(nkt, cur ^ 1, nkt * kTile + kTile - 1 - a.base > r0_group || nmin < rlast_group);
       }
-      const bool visit = wave_live && kt <= my_kt_end && ent.y >= my_r0;
-      if (visit) {
+      if (wave_live && kt <= my_kt_end && ent_max >= my_r0) {
         // no masked score: every key row is at or before the first query and visible to the last one
-        const bool full = kt * kTile + kTile - 1 - a.base <= my_r0 && ent.z >= my_rlast;
-        compute_tile(kt, cur, full);
+        const bool full = kt * kTile + kTile - 1 - a.base <= my_r0 && ent_min >= my_rlast;
+        f32x16 sacc[2][2];
+        float mx[2];
+        score_tile(kt, cur, full, sacc, mx);
+        if (__ballot(mx[0] > m_run[0] + kRescaleSlack || mx[1] > m_run[1] + kRescaleSlack)) rescale(mx);
+        pin_o();
+        finish_tile(cur, sacc);
       }
       __builtin_amdgcn_s_waitcnt(0);  // the next tile has landed in LDS
       __syncthreads();                // ... for every wavefront, and this tile is no longer read
