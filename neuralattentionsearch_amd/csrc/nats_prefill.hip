@@ -184,12 +184,14 @@ template <int D>
 struct PrefillSmem {
   uint16_t k[2][kTile * D];
   uint16_t v[2][kTile * D];
-  int limk[2][kTile];
+  int limk[4][kTile];
   int4 vlist[kWin];  // visited key tiles of the current window: {tile, max limit, min limit, -}
   int vcount;
 };
 
-template <int D>
+// kUniform: the four wavefronts are the four q heads of one query tile (GQA groups of 4 and more), so every
+// tile of the visit list is visited by every wavefront and the tile loop has no per-wavefront branches.
+template <int D, bool kUniform>
 __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
   constexpr int OCT = D / 8;              // 16-byte chunks per row
   constexpr int DMA_PER_WAVE = OCT / 4;   // 1 KiB global->LDS transfers per wavefront and tensor
@@ -299,15 +301,14 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
     koff[j] = int(row * a.ks_l + (pos ^ (row % OCT)) * 8);
     voff[j] = int(row * a.vs_l + (pos ^ ((row & 3) << 1)) * 8);
   }
-  auto issue_tile = [&](int kt, int buf, bool need_lim) {
+  auto issue_rows = [&](const uint16_t* base, int64_t stride, const int (&off)[DMA_PER_WAVE], uint16_t* dst, int kt,
+                        bool is_v) {
     if (kt * kTile + kTile <= a.N) {
-      const uint16_t* kb = kp + (int64_t)kt * kTile * a.ks_l;  // uniform
-      const uint16_t* vb = vp + (int64_t)kt * kTile * a.vs_l;
+      const uint16_t* tb = base + (int64_t)kt * kTile * stride;  // uniform
 #pragma unroll
       for (int j = 0; j < DMA_PER_WAVE; ++j) {
         const int inst = wave * DMA_PER_WAVE + j;
-        __builtin_amdgcn_global_load_lds(kb + (int)koff[j], (uint32_t __attribute__((address_space(3)))*)(&sm.k[buf][inst * kWave * 8]), 16, 0, 0);
-        __builtin_amdgcn_global_load_lds(vb + (int)voff[j], (uint32_t __attribute__((address_space(3)))*)(&sm.v[buf][inst * kWave * 8]), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(tb + (int)off[j], (uint32_t __attribute__((address_space(3)))*)(dst + inst * kWave * 8), 16, 0, 0);
       }
     } else {
 #pragma unroll
@@ -316,23 +317,25 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
         const int q = inst * kWave + lane;
         const int row = q / OCT, pos = q % OCT;
         const int n = min(kt * kTile + row, a.N - 1);
-        const int kchunk = pos ^ (row % OCT);
-        const int vchunk = pos ^ ((row & 3) << 1);
-        __builtin_amdgcn_global_load_lds(kp + (int64_t)n * a.ks_l + kchunk * 8,
-                                         (uint32_t __attribute__((address_space(3)))*)(&sm.k[buf][inst * kWave * 8]), 16, 0, 0);
-        __builtin_amdgcn_global_load_lds(vp + (int64_t)n * a.vs_l + vchunk * 8,
-                                         (uint32_t __attribute__((address_space(3)))*)(&sm.v[buf][inst * kWave * 8]), 16, 0, 0);
+        const int chunk = is_v ? pos ^ ((row & 3) << 1) : pos ^ (row % OCT);
+        __builtin_amdgcn_global_load_lds(base + (int64_t)n * stride + chunk * 8,
+                                         (uint32_t __attribute__((address_space(3)))*)(dst + inst * kWave * 8), 16, 0, 0);
       }
     }
+  };
+  // K tile and the visibility limits of its rows; the limits go to slot (list index & 3)
+  auto issue_k = [&](int kt, int buf, int slot, bool need_lim) {
+    issue_rows(kp, a.ks_l, koff, sm.k[buf], kt, false);
     if (need_lim && tid < kTile) {
       int n = kt * kTile + tid;
-      sm.limk[buf][tid] = n < a.N ? lim[n] : -1;
+      sm.limk[slot][tid] = n < a.N ? lim[n] : -1;
     }
   };
+  auto issue_v = [&](int kt, int buf) { issue_rows(vp, a.vs_l, voff, sm.v[buf], kt, true); };
 
-  // ---- S^T = K Q^T, the mask, and the scaled row maxima ----------------------------------------------
-  auto score_tile = [&](int kt, int cur, bool full, f32x16 (&sacc)[2][2], float (&mx)[2]) {
-    const uint16_t* Kt = sm.k[cur];
+  // ---- S^T = K Q^T into the accumulation registers ----------------------------------------------------
+  auto qk_tile = [&](int buf, f32x16 (&sacc)[2][2]) {
+    const uint16_t* Kt = sm.k[buf];
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
       const int row = kb * 32 + l32;
@@ -350,40 +353,37 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
         }
       }
     }
+  };
+  // ---- mask of a diagonal tile, or of a tile whose rows are not uniformly visible ---------------------
+  auto mask_scores = [&](int kt, int slot, f32x16 (&sv)[2][2]) {
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
+    for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
-      for (int qb = 0; qb < 2; ++qb) NATS_PIN_ARCH(sacc[kb][qb]);
-    // mask (diagonal tile, or a tile whose rows are not uniformly visible)
-    if (!full) {
-      asm volatile("" ::: "memory");  // keeps this a branch: most tiles skip it
+      for (int g4 = 0; g4 < 4; ++g4) {
+        int kk = kb * 32 + g4 * 8 + hl * 4;  // key offset in tile of accumulator 4*g4
+        int4 lm = *reinterpret_cast<const int4*>(&sm.limk[slot][kk]);
+        const int lv[4] = {lm.x, lm.y, lm.z, lm.w};
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb) {
+        for (int e = 0; e < 4; ++e) {
+          int key = kt * kTile + kk + e - a.base;  // region token of the key row (negative: older row)
 #pragma unroll
-        for (int g4 = 0; g4 < 4; ++g4) {
-          int kk = kb * 32 + g4 * 8 + hl * 4;  // key offset in tile of accumulator 4*g4
-          int4 lm = *reinterpret_cast<const int4*>(&sm.limk[cur][kk]);
-          const int lv[4] = {lm.x, lm.y, lm.z, lm.w};
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            int key = kt * kTile + kk + e - a.base;  // region token of the key row (negative: older row)
-#pragma unroll
-            for (int qb = 0; qb < 2; ++qb) {
-              int qtok = q0 + qb * 32 + l32;
-              bool vis = key <= qtok && qtok <= lv[e];
-              if (!vis) sacc[kb][qb][g4 * 4 + e] = -INFINITY;
-            }
+          for (int qb = 0; qb < 2; ++qb) {
+            int qtok = q0 + qb * 32 + l32;
+            bool vis = key <= qtok && qtok <= lv[e];
+            if (!vis) sv[kb][qb][g4 * 4 + e] = -INFINITY;
           }
         }
       }
     }
+  };
+  auto row_max = [&](const f32x16 (&sv)[2][2], float (&mx)[2]) {
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) {
       float m = -INFINITY;
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) m = fmaxf(m, sacc[kb][qb][i]);
+        for (int i = 0; i < 16; ++i) m = fmaxf(m, sv[kb][qb][i]);
       mx[qb] = fmaxf(m, __shfl_xor(m, 32)) * c;
     }
   };
@@ -412,35 +412,39 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
     }
   };
 
-  // ---- probabilities and O^T += V^T P^T ---------------------------------------------------------------
-  auto finish_tile = [&](int cur, const f32x16 (&sacc)[2][2]) {
-    const uint16_t* Vt = sm.v[cur];
-    bf16x8 pb[2][4];
+  // ---- probabilities (bf16, B-operand layout) and the row sums, in the order O^T += V^T P^T eats them ----
+  auto probs = [&](const f32x16 (&sv)[2][2], bf16x8 (&pb)[2][4]) {
+    float m_use[2], rs[2] = {0.f, 0.f};
 #pragma unroll
-    for (int qb = 0; qb < 2; ++qb) {
-      const float m_use = m_run[qb] == -INFINITY ? 0.f : m_run[qb];
-      float rs = 0.f;
+    for (int qb = 0; qb < 2; ++qb) m_use[qb] = m_run[qb] == -INFINITY ? 0.f : m_run[qb];
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb) {
+    for (int t = 0; t < 4; ++t) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          float p = __builtin_amdgcn_exp2f(fmaf(sacc[kb][qb][i], c, -m_use));
-          rs += p;
-          pb[qb][kb * 2 + (i >> 3)][i & 7] = (__bf16)p;
+      for (int qb = 0; qb < 2; ++qb) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          float p = __builtin_amdgcn_exp2f(fmaf(sv[t >> 1][qb][(t & 1) * 8 + i], c, -m_use[qb]));
+          rs[qb] += p;
+          pb[qb][t][i] = (__bf16)p;
         }
       }
-      l_run[qb] += rs;
     }
-    // ds_read_b64_tr_b16: within 16 lanes, lane r reads 4 dims of key (K0 + r / 4) starting at dim
-    // D0 + 4 * (r % 4) and receives keys K0 .. K0 + 3 of dim D0 + r.
+    l_run[0] += rs[0];
+    l_run[1] += rs[1];
+  };
+  // ---- O^T += V^T P^T, 16 keys (one B operand per q block) at a time -----------------------------------
+  // ds_read_b64_tr_b16: within 16 lanes, lane r reads 4 dims of key (K0 + r / 4) starting at dim
+  // D0 + 4 * (r % 4) and receives keys K0 .. K0 + 3 of dim D0 + r.
+  auto pv_tile = [&](int buf, const bf16x8 (&pb)[2][4]) {
+    const uint16_t* Vt = sm.v[buf];
     const int r16 = lane & 15;
     const int dsel = (lane >> 4) & 1;
+    const int half = r16 & 1;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      const int chunk0 = dt * 4 + dsel * 2 + ((r16 & 3) >> 1);
-      const int half = r16 & 1;
+    for (int t = 0; t < 4; ++t) {
 #pragma unroll
-      for (int t = 0; t < 4; ++t) {
+      for (int dt = 0; dt < DT; ++dt) {
+        const int chunk0 = dt * 4 + dsel * 2 + ((r16 & 3) >> 1);
         bf16x4 lo, hi;
         {
           const int row = t * 16 + hl * 4 + (r16 >> 2);
@@ -458,8 +462,122 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
       }
     }
   };
+  // ---- the fused step: scores of the next tile, probabilities of this one, O += P V of this one ----------
+  // A matrix instruction occupies the matrix pipe for 8 passes, during which the wavefront can issue vector
+  // ALU work.  The step is therefore written as slots of one MFMA followed by a slice of the exponentials,
+  // fenced so that the compiler keeps the slots in this order:
+  //   phase A  score MFMAs of the next tile        + probabilities of keys  0..31 of this tile
+  //   phase B  O += P V for keys 0..31             + probabilities of keys 32..63
+  //   phase C  O += P V for keys 32..63
+  // LDS operands are fetched one slot ahead of the MFMA that consumes them.
+  auto fused_step = [&](int kbuf_next, int vbuf, const f32x16 (&sv)[2][2], f32x16 (&sacc)[2][2]) {
+    const uint16_t* Kt = sm.k[kbuf_next];
+    const uint16_t* Vt = sm.v[vbuf];
+    constexpr int N_QK = 4 * DSTEPS;      // score MFMAs
+    constexpr int N_PV = 8 * DT;          // PV MFMAs
+    constexpr int VA = 32 / N_QK;         // probabilities per slot in phase A
+    constexpr int VB = 32 / (N_PV / 2);   // ... in phase B
+    float m_use[2], rs[2] = {0.f, 0.f};
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) m_use[qb] = m_run[qb] == -INFINITY ? 0.f : m_run[qb];
+    bf16x8 pb[2][4];
+    auto pval = [&](int n) {  // n-th probability in the order the PV MFMAs consume them
+      const int t = n >> 4, qb = (n >> 3) & 1, i = n & 7;
+      float p = __builtin_amdgcn_exp2f(fmaf(sv[t >> 1][qb][(t & 1) * 8 + i], c, -m_use[qb]));
+      rs[qb] += p;
+      pb[qb][t][i] = (__bf16)p;
+    };
+    auto k_frag = [&](int kb, int s) {
+      const int row = kb * 32 + l32;
+      const int chunk = (s * 2 + hl) ^ (row % OCT);
+      return *reinterpret_cast<const bf16x8*>(Kt + row * D + chunk * 8);
+    };
+    const int r16 = lane & 15;
+    const int dsel = (lane >> 4) & 1;
+    const int half = r16 & 1;
+    auto v_frag = [&](int t, int dt) {
+      const int chunk0 = dt * 4 + dsel * 2 + ((r16 & 3) >> 1);
+      const int row_lo = t * 16 + hl * 4 + (r16 >> 2);
+      const int row_hi = row_lo + 8;
+      const uint16_t* pl = Vt + row_lo * D + ((chunk0 ^ ((row_lo & 3) << 1)) * 8) + half * 4;
+      const uint16_t* ph = Vt + row_hi * D + ((chunk0 ^ ((row_hi & 3) << 1)) * 8) + half * 4;
+      bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((bf16x4 __attribute__((address_space(3)))*)pl);
+      bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((bf16x4 __attribute__((address_space(3)))*)ph);
+      bf16x8 va = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      return va;
+    };
 
-  int cur = 0;
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- phase A ----
+    bf16x8 ka = k_frag(0, 0);
+    int n = 0;
+#pragma unroll
+    for (int s = 0; s < DSTEPS; ++s) {
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) {
+        const bf16x8 cur = ka;
+        if (kb == 0) {
+          ka = k_frag(1, s);
+        } else if (s + 1 < DSTEPS) {
+          ka = k_frag(0, s + 1);
+        }
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb) {
+          if (s == 0) {
+            const f32x16 z = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            sacc[kb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cur, qreg[qb][s], z, 0, 0, 0);
+          } else {
+            sacc[kb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cur, qreg[qb][s], sacc[kb][qb], 0, 0, 0);
+          }
+#pragma unroll
+          for (int e = 0; e < VA; ++e) pval(n++);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+    }
+    // ---- phases B and C ----
+    bf16x8 va = v_frag(0, 0);
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        const bf16x8 cur = va;
+        if (dt + 1 < DT) {
+          va = v_frag(t, dt + 1);
+        } else if (t + 1 < 4) {
+          va = v_frag(t + 1, 0);
+        }
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb) {
+          oacc[dt][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cur, pb[qb][t], oacc[dt][qb], 0, 0, 0);
+          if (t < 2) {
+#pragma unroll
+            for (int e = 0; e < VB; ++e) pval(n++);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+    }
+    l_run[0] += rs[0];
+    l_run[1] += rs[1];
+  };
+
+  // Scores of the tile that the next step turns into probabilities; they stay in the accumulation registers
+  // from the step that computes them to the step that reads them.
+  f32x16 sacc[2][2];
+#pragma unroll
+  for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) sacc[kb][qb][i] = 0.f;
+  auto pin_s = [&]() {
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb) NATS_PIN_ACC(sacc[kb][qb]);
+  };
+
   for (int w0 = 0; w0 <= kt_end_group; w0 += kWin) {
     // ---- visit list of this window: wavefront 0 compacts the tiles some query tile of the group sees ----
     if (wave == 0) {
@@ -482,39 +600,84 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
     }
     __syncthreads();
     const int n_vis = __builtin_amdgcn_readfirstlane(sm.vcount);
-    if (n_vis > 0) {
-      issue_tile(__builtin_amdgcn_readfirstlane(sm.vlist[0].x), cur, true);
-      __builtin_amdgcn_s_waitcnt(0);
-      __syncthreads();
+    if (n_vis == 0) continue;
+
+    // The list entries are the same for every lane: they are kept in scalar registers.
+    // Step j of the pipeline: loads of K tile j+2 and V tile j+1 are put in flight; the scores of tile j
+    // (computed by step j-1) leave the accumulation registers; the matrix pipe computes the scores of tile
+    // j+1 while the vector ALU turns those of tile j into probabilities; then O += P V for tile j.
+    // Buffers: K tile j in k[j & 1], V tile j in v[j & 1], row limits of tile j in limk[j & 3].
+    auto entry = [&](int j, int& kt, int& emax, int& emin) {
+      const int4 e = sm.vlist[j];
+      kt = __builtin_amdgcn_readfirstlane(e.x);
+      emax = __builtin_amdgcn_readfirstlane(e.y);
+      emin = __builtin_amdgcn_readfirstlane(e.z);
+    };
+    // the element mask is only evaluated on diagonal tiles and on tiles with mixed visibility
+    auto group_needs_lim = [&](int kt, int emin) { return kt * kTile + kTile - 1 - a.base > r0_group || emin < rlast_group; };
+    auto visits = [&](int kt, int emax) { return kUniform || (wave_live && kt <= my_kt_end && emax >= my_r0); };
+
+    int kt_c, emax_c, emin_c;  // tile of the current step
+    int kt_n = 0, emax_n = 0, emin_n = 0;  // tile of the next step
+    entry(0, kt_c, emax_c, emin_c);
+    issue_k(kt_c, 0, 0, group_needs_lim(kt_c, emin_c));
+    issue_v(kt_c, 0);
+    if (n_vis > 1) {
+      entry(1, kt_n, emax_n, emin_n);
+      issue_k(kt_n, 1, 1, group_needs_lim(kt_n, emin_n));
     }
-    for (int idx = 0; idx < n_vis; ++idx) {
-      // the list entries are the same for every lane: keep them in scalar registers
-      const int4 ent = sm.vlist[idx];
-      const int kt = __builtin_amdgcn_readfirstlane(ent.x);
-      const int ent_max = __builtin_amdgcn_readfirstlane(ent.y);
-      const int ent_min = __builtin_amdgcn_readfirstlane(ent.z);
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    pin_q();
+    if (visits(kt_c, emax_c)) qk_tile(0, sacc);
+    pin_s();
+    __syncthreads();  // k[0] may be overwritten from here on
+
+    for (int j = 0; j < n_vis; ++j) {
       pin_o();
       pin_q();
-      if (idx + 1 < n_vis) {
-        const int4 en = sm.vlist[idx + 1];
-        const int nkt = __builtin_amdgcn_readfirstlane(en.x);
-        const int nmin = __builtin_amdgcn_readfirstlane(en.z);
-        // the element mask is only evaluated on diagonal tiles and on tiles with mixed visibility
-        issue_tile(nkt, cur ^ 1, nkt * kTile + kTile - 1 - a.base > r0_group || nmin < rlast_group);
+      pin_s();
+      if (j + 2 < n_vis) {
+        int kt2, emax2, emin2;
+        entry(j + 2, kt2, emax2, emin2);
+        issue_k(kt2, j & 1, (j + 2) & 3, group_needs_lim(kt2, emin2));
       }
-      if (wave_live && kt <= my_kt_end && ent_max >= my_r0) {
+      if (j + 1 < n_vis) issue_v(kt_n, (j + 1) & 1);
+      const bool vis_c = visits(kt_c, emax_c);
+      // (uniform case: the last step computes scores of a stale tile that nobody reads, which keeps the
+      // step free of branches around the matrix instructions)
+      const bool vis_n = kUniform || (j + 1 < n_vis && visits(kt_n, emax_n));
+      if (vis_c) {
+        f32x16 sv[2][2];
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int qb = 0; qb < 2; ++qb) {
+            sv[kb][qb] = sacc[kb][qb];
+            NATS_PIN_ARCH(sv[kb][qb]);
+          }
         // no masked score: every key row is at or before the first query and visible to the last one
-        const bool full = kt * kTile + kTile - 1 - a.base <= my_r0 && ent_min >= my_rlast;
-        f32x16 sacc[2][2];
+        const bool full = kt_c * kTile + kTile - 1 - a.base <= my_r0 && emin_c >= my_rlast;
+        if (!full) mask_scores(kt_c, j & 3, sv);
         float mx[2];
-        score_tile(kt, cur, full, sacc, mx);
+        row_max(sv, mx);
         if (__ballot(mx[0] > m_run[0] + kRescaleSlack || mx[1] > m_run[1] + kRescaleSlack)) rescale(mx);
         pin_o();
-        finish_tile(cur, sacc);
+        if (vis_n) {
+          fused_step((j + 1) & 1, j & 1, sv, sacc);
+        } else {
+          bf16x8 pb[2][4];
+          probs(sv, pb);
+          pv_tile(j & 1, pb);
+        }
+      } else if (vis_n) {
+        qk_tile((j + 1) & 1, sacc);
       }
-      __builtin_amdgcn_s_waitcnt(0);  // the next tile has landed in LDS
-      __syncthreads();                // ... for every wavefront, and this tile is no longer read
-      cur ^= 1;
+      pin_s();
+      kt_c = kt_n; emax_c = emax_n; emin_c = emin_n;
+      if (j + 2 < n_vis) entry(j + 2, kt_n, emax_n, emin_n);
+      __builtin_amdgcn_s_waitcnt(0);  // the tiles in flight have landed in LDS
+      __syncthreads();                // ... for every wavefront, and the tiles of this step are no longer read
     }
   }
 
@@ -545,17 +708,17 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
   }
 }
 
-template <int D>
+template <int D, bool kUniform>
 static int launch_prefill_mfma(const PrefillArgs& a, int64_t n_wg, hipStream_t st) {
-  static bool configured = false;  // per process and head size; the attribute is a property of the kernel
+  static bool configured = false;  // per process and instantiation; the attribute is a property of the kernel
   const size_t smem = sizeof(PrefillSmem<D>);
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_mfma_kernel<D>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_mfma_kernel<D, kUniform>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return fail(NATS_ERR_LAUNCH, "hipFuncSetAttribute(%zu bytes of LDS): %s", smem, hipGetErrorString(e));
     configured = true;
   }
-  hipLaunchKernelGGL((prefill_mfma_kernel<D>), dim3((unsigned)n_wg), dim3(256), smem, st, a);
+  hipLaunchKernelGGL((prefill_mfma_kernel<D, kUniform>), dim3((unsigned)n_wg), dim3(256), smem, st, a);
   NATS_CHECK_LAUNCH("prefill_mfma_kernel");
   return NATS_OK;
 }
@@ -644,7 +807,8 @@ int launch_segment(const char* who, const SegmentShape& g, const void* q, const 
   a.xcd_mode = ((g.B * g.H_kv) % 8 == 0) ? 1 : 0;
   int64_t n_wg = g.B * g.H_kv * a.n_hg * a.n_qg;
   NATS_REQUIRE(n_wg < (int64_t(1) << 31), NATS_ERR_BAD_SHAPE, "%s: grid too large", who);
-  return g.D == 64 ? launch_prefill_mfma<64>(a, n_wg, st) : launch_prefill_mfma<128>(a, n_wg, st);
+  if (hpw == 4) return g.D == 64 ? launch_prefill_mfma<64, true>(a, n_wg, st) : launch_prefill_mfma<128, true>(a, n_wg, st);
+  return g.D == 64 ? launch_prefill_mfma<64, false>(a, n_wg, st) : launch_prefill_mfma<128, false>(a, n_wg, st);
 }
 
 }  // namespace
