@@ -139,8 +139,10 @@ __global__ __launch_bounds__(64) void prefill_simple_kernel(PrefillArgs a) {
 // ---------------------------------------------------------------------------------------------------
 // bf16 MFMA kernel.
 //
-// Workgroup = 4 wavefronts = (hpw q heads of one kv head) x (qpw query tiles of 64 rows); every wavefront
-// owns 64 query rows of one q head and all wavefronts share each 64-key K / V tile through LDS.
+// Workgroup = 8 wavefronts = (hpw q heads of one kv head) x (qpw query tiles of 64 rows) x (2 halves of 32
+// rows); every wavefront owns 32 query rows of one q head and all wavefronts share each 64-key K / V tile
+// through LDS.  With 256 registers per lane two wavefronts share a SIMD, so that the vector ALU work of
+// one (exponentials) runs under the matrix instructions of the other.
 //
 // K / V tiles travel global -> LDS without passing through registers (global_load_lds, 16 bytes per lane),
 // double buffered, row major with 256-byte rows whose 16-byte chunks are XOR-swizzled (the lane supplies
@@ -157,27 +159,7 @@ __global__ __launch_bounds__(64) void prefill_simple_kernel(PrefillArgs a) {
 // operands hold without loss, and O is not touched.
 // ---------------------------------------------------------------------------------------------------
 constexpr float kRescaleSlack = 8.0f;
-
-// Register-file constraints and the in-place scaling of an accumulation register.  The host pass of the
-// single-source compile never runs this code and has no such registers, so the statements are empty there.
-#if defined(__HIP_DEVICE_COMPILE__)
-#define NATS_PIN_ACC(x) asm volatile("" : "+a"(x))
-#define NATS_PIN_ARCH(x) asm volatile("" : "+v"(x))
-#define NATS_SCALE_ACC(e, alpha)                                                                          \
-  do {                                                                                                    \
-    float t__;                                                                                            \
-    asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\tv_accvgpr_write_b32 %0, %1"       \
-                 : "+a"(e), "=&v"(t__)                                                                    \
-                 : "v"(alpha));                                                                           \
-  } while (0)
-#define NATS_ACC_SETTLE() asm volatile("s_nop 7")
-#else
-#define NATS_PIN_ACC(x) (void)(x)
-#define NATS_PIN_ARCH(x) (void)(x)
-#define NATS_SCALE_ACC(e, alpha) (e) *= (alpha)
-#define NATS_ACC_SETTLE() (void)0
-#endif
-
+constexpr int kPrefillWaves = 8;
 constexpr int kWin = 1024;  // key tiles whose visit list is built at once
 
 template <int D>
@@ -189,20 +171,24 @@ struct PrefillSmem {
   int vcount;
 };
 
-// kUniform: the four wavefronts are the four q heads of one query tile (GQA groups of 4 and more), so every
-// tile of the visit list is visited by every wavefront and the tile loop has no per-wavefront branches.
+// kUniform: the wavefronts are the q heads of ONE query tile (GQA groups of 4 and more), so every tile of
+// the visit list is visited by every wavefront and the tile loop has no per-wavefront branches.
 template <int D, bool kUniform>
-__global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
-  constexpr int OCT = D / 8;              // 16-byte chunks per row
-  constexpr int DMA_PER_WAVE = OCT / 4;   // 1 KiB global->LDS transfers per wavefront and tensor
+__global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(PrefillArgs a) {
+  constexpr int OCT = D / 8;                          // 16-byte chunks per row
+  constexpr int DMA_PER_WAVE = OCT / kPrefillWaves;   // 1 KiB global->LDS transfers per wavefront and tensor
   constexpr int DSTEPS = D / 16;
   constexpr int DT = D / 32;
+  constexpr int kHalf = kTile / 2;
+  static_assert(DMA_PER_WAVE >= 1, "tile rows are split over the wavefronts in 1 KiB transfers");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   PrefillSmem<D>& sm = *reinterpret_cast<PrefillSmem<D>*>(smem_raw);
 
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform, and the compiler may know it
+  const int sub = wave & 3;    // which (head, query tile) of the workgroup; wavefronts sub and sub + 4 share a SIMD
+  const int half = wave >> 2;  // which 32 rows of the query tile
   const int lane = tid & 63;
   const int l32 = lane & 31;
   const int hl = lane >> 5;
@@ -227,70 +213,50 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
   }
   const int qg = a.n_qg - 1 - rank;  // heavy query groups first
   const int b = ks / a.Hkv, hkv = ks % a.Hkv;
-  const int hq = hkv * a.n_rep + hg * a.hpw + (wave % a.hpw);
+  const int hq = hkv * a.n_rep + hg * a.hpw + (sub % a.hpw);
   const int qt_lo = a.qt_first + qg * a.qpw;
   const int qt_hi = min(qt_lo + a.qpw - 1, a.qt_last);
-  const int my_qt = qt_lo + wave / a.hpw;
+  const int my_qt = qt_lo + sub / a.hpw;
   const bool wave_live = my_qt <= qt_hi;
-  const int q0 = my_qt * kTile;  // region token of this wavefront's first row
+  const int q0 = my_qt * kTile + half * kHalf;  // region token of this wavefront's first row
 
   const int2* tl = a.tile_lim + (int64_t)ks * a.Tk;
   const int32_t* lim = a.tok_lim + (int64_t)ks * a.N;
   const uint16_t* kp = static_cast<const uint16_t*>(a.k) + b * a.ks_b + hkv * a.ks_h;
   const uint16_t* vp = static_cast<const uint16_t*>(a.v) + b * a.vs_b + hkv * a.vs_h;
 
-  // first / last query token of the group and of this wavefront, and the last key tile either may see
+  // first / last query token of the group, of this wavefront's query tile and of its 32 rows, and the last
+  // key tile the group / the query tile may see
   const int r0_group = max(qt_lo * kTile, a.r_begin);
   const int rlast_group = min(qt_hi * kTile + kTile - 1, a.r_end - 1);
+  const int tile_r0 = max(my_qt * kTile, a.r_begin);
+  const int tile_rlast = min(my_qt * kTile + kTile - 1, a.r_end - 1);
   const int my_r0 = max(q0, a.r_begin);
-  const int my_rlast = min(q0 + kTile - 1, a.r_end - 1);
+  const int my_rlast = min(q0 + kHalf - 1, a.r_end - 1);
   const int kt_end_group = (a.base + rlast_group) / kTile;
-  const int my_kt_end = (a.base + my_rlast) / kTile;
+  const int my_kt_end = (a.base + tile_rlast) / kTile;
 
   // ---- Q fragments: B operand, lane (query l32, k-group hl) --------------------------------------
-  bf16x8 qreg[2][DSTEPS];
+  bf16x8 qreg[DSTEPS];
   {
     const uint16_t* qp = static_cast<const uint16_t*>(a.q) + b * a.qs_b + hq * a.qs_h;
+    int row = min(max(q0 + l32, a.r_begin), a.r_end - 1) - a.r_begin;
+    if (!wave_live) row = 0;
+    const uint4* rp = reinterpret_cast<const uint4*>(qp + (int64_t)row * a.qs_l + hl * 8);
 #pragma unroll
-    for (int qb = 0; qb < 2; ++qb) {
-      int row = min(max(q0 + qb * 32 + l32, a.r_begin), a.r_end - 1) - a.r_begin;
-      if (!wave_live) row = 0;
-      const uint4* rp = reinterpret_cast<const uint4*>(qp + (int64_t)row * a.qs_l + hl * 8);
-#pragma unroll
-      for (int s = 0; s < DSTEPS; ++s) qreg[qb][s] = __builtin_bit_cast(bf16x8, rp[s * 2]);
-    }
+    for (int s = 0; s < DSTEPS; ++s) qreg[s] = __builtin_bit_cast(bf16x8, rp[s * 2]);
   }
 
-  f32x16 oacc[DT][2];
+  f32x16 oacc[DT];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-    for (int qb = 0; qb < 2; ++qb)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) oacc[dt][qb][i] = 0.f;
-  float m_run[2] = {-INFINITY, -INFINITY};
-  float l_run[2] = {0.f, 0.f};
+    for (int i = 0; i < 16; ++i) oacc[dt][i] = 0.f;
+  float m_run = -INFINITY;
+  float l_run = 0.f;
   const float c = a.scale * 1.4426950408889634f;
 
-  // Register file placement.  The matrix instructions read their operands from either half of the unified
-  // register file; the vector ALU only from the architectural half.  Q fragments (read by MFMA only) and the
-  // output accumulators (touched by the vector ALU only on a rescale) belong in the accumulation half,
-  // scores and probabilities in the architectural half.  The empty statements below constrain the
-  // allocator accordingly at the points where the values are merged.
-  auto pin_q = [&]() {
-#pragma unroll
-    for (int qb = 0; qb < 2; ++qb)
-#pragma unroll
-      for (int s = 0; s < DSTEPS; ++s) NATS_PIN_ACC(qreg[qb][s]);
-  };
-  auto pin_o = [&]() {
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-      for (int qb = 0; qb < 2; ++qb) NATS_PIN_ACC(oacc[dt][qb]);
-  };
-
-  // global -> LDS, one 64-key tile of K and of V; rows beyond N repeat row N-1 (their scores are masked,
+  // global -> LDS, one 64-key tile of K or of V; rows beyond N repeat row N-1 (their scores are masked,
   // so their probabilities are exactly 0 and a finite V row contributes nothing).  The lane's share of a
   // tile sits at fixed offsets from the tile's first row, computed once.
   int koff[DMA_PER_WAVE], voff[DMA_PER_WAVE];
@@ -333,29 +299,48 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
   };
   auto issue_v = [&](int kt, int buf) { issue_rows(vp, a.vs_l, voff, sm.v[buf], kt, true); };
 
-  // ---- S^T = K Q^T into the accumulation registers ----------------------------------------------------
-  auto qk_tile = [&](int buf, f32x16 (&sacc)[2][2]) {
+  auto k_frag = [&](const uint16_t* Kt, int kb, int s) {
+    const int row = kb * 32 + l32;
+    const int chunk = (s * 2 + hl) ^ (row % OCT);
+    return *reinterpret_cast<const bf16x8*>(Kt + row * D + chunk * 8);
+  };
+  // ds_read_b64_tr_b16: within 16 lanes, lane r reads 4 dims of key (K0 + r / 4) starting at dim
+  // D0 + 4 * (r % 4) and receives keys K0 .. K0 + 3 of dim D0 + r.
+  const int r16 = lane & 15;
+  const int dsel = (lane >> 4) & 1;
+  auto v_frag = [&](const uint16_t* Vt, int t, int dt) {
+    const int chunk0 = dt * 4 + dsel * 2 + ((r16 & 3) >> 1);
+    const int half4 = (r16 & 1) * 4;
+    const int row_lo = t * 16 + hl * 4 + (r16 >> 2);
+    const int row_hi = row_lo + 8;
+    const uint16_t* pl = Vt + row_lo * D + ((chunk0 ^ ((row_lo & 3) << 1)) * 8) + half4;
+    const uint16_t* ph = Vt + row_hi * D + ((chunk0 ^ ((row_hi & 3) << 1)) * 8) + half4;
+    bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((bf16x4 __attribute__((address_space(3)))*)pl);
+    bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((bf16x4 __attribute__((address_space(3)))*)ph);
+    bf16x8 va = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    return va;
+  };
+
+  // ---- S^T = K Q^T -----------------------------------------------------------------------------------
+  auto qk_tile = [&](int buf, f32x16 (&sacc)[2]) {
     const uint16_t* Kt = sm.k[buf];
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
-      const int row = kb * 32 + l32;
+    for (int s = 0; s < DSTEPS; ++s) {
 #pragma unroll
-      for (int s = 0; s < DSTEPS; ++s) {
-        const int chunk = (s * 2 + hl) ^ (row % OCT);
-        bf16x8 ka = *reinterpret_cast<const bf16x8*>(Kt + row * D + chunk * 8);
+      for (int kb = 0; kb < 2; ++kb) {
+        bf16x8 ka = k_frag(Kt, kb, s);
         if (s == 0) {
           const f32x16 z = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-          sacc[kb][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qreg[0][s], z, 0, 0, 0);
-          sacc[kb][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qreg[1][s], z, 0, 0, 0);
+          sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qreg[s], z, 0, 0, 0);
         } else {
-          sacc[kb][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qreg[0][s], sacc[kb][0], 0, 0, 0);
-          sacc[kb][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qreg[1][s], sacc[kb][1], 0, 0, 0);
+          sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qreg[s], sacc[kb], 0, 0, 0);
         }
       }
     }
   };
   // ---- mask of a diagonal tile, or of a tile whose rows are not uniformly visible ---------------------
-  auto mask_scores = [&](int kt, int slot, f32x16 (&sv)[2][2]) {
+  auto mask_scores = [&](int kt, int slot, f32x16 (&sv)[2]) {
+    const int qtok = q0 + l32;
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
@@ -366,217 +351,126 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           int key = kt * kTile + kk + e - a.base;  // region token of the key row (negative: older row)
-#pragma unroll
-          for (int qb = 0; qb < 2; ++qb) {
-            int qtok = q0 + qb * 32 + l32;
-            bool vis = key <= qtok && qtok <= lv[e];
-            if (!vis) sv[kb][qb][g4 * 4 + e] = -INFINITY;
-          }
+          bool vis = key <= qtok && qtok <= lv[e];
+          if (!vis) sv[kb][g4 * 4 + e] = -INFINITY;
         }
       }
     }
   };
-  auto row_max = [&](const f32x16 (&sv)[2][2], float (&mx)[2]) {
+  auto row_max = [&](const f32x16 (&sv)[2]) {
+    float m = -INFINITY;
 #pragma unroll
-    for (int qb = 0; qb < 2; ++qb) {
-      float m = -INFINITY;
+    for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) m = fmaxf(m, sv[kb][qb][i]);
-      mx[qb] = fmaxf(m, __shfl_xor(m, 32)) * c;
-    }
+      for (int i = 0; i < 16; ++i) m = fmaxf(m, sv[kb][i]);
+    return fmaxf(m, __shfl_xor(m, 32)) * c;
   };
-
-  // ---- raise the running maxima (rare): O and l shrink by 2^(old - new) ------------------------------
-  auto rescale = [&](const float (&mx)[2]) {
+  // ---- raise the running maximum (rare): O and l shrink by 2^(old - new) ----------------------------
+  auto rescale = [&](float mx) {
+    float m_new = fmaxf(m_run, mx);
+    float alpha = m_run == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_run - m_new);
+    l_run *= alpha;
+    m_run = m_new;
 #pragma unroll
-    for (int qb = 0; qb < 2; ++qb) {
-      if (__ballot(mx[qb] > m_run[qb] + kRescaleSlack)) {
-        float m_new = fmaxf(m_run[qb], mx[qb]);
-        float alpha = m_run[qb] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_run[qb] - m_new);
-        l_run[qb] *= alpha;
-        m_run[qb] = m_new;
-        // scaled in place in the accumulation registers, one element at a time through a temporary
+    for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-#pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            float e = oacc[dt][qb][i];
-            NATS_SCALE_ACC(e, alpha);
-            oacc[dt][qb][i] = e;
-          }
-        }
-        NATS_ACC_SETTLE();  // the matrix instructions that follow read these registers
-      }
-    }
+      for (int i = 0; i < 16; ++i) oacc[dt][i] *= alpha;
   };
-
-  // ---- probabilities (bf16, B-operand layout) and the row sums, in the order O^T += V^T P^T eats them ----
-  auto probs = [&](const f32x16 (&sv)[2][2], bf16x8 (&pb)[2][4]) {
-    float m_use[2], rs[2] = {0.f, 0.f};
-#pragma unroll
-    for (int qb = 0; qb < 2; ++qb) m_use[qb] = m_run[qb] == -INFINITY ? 0.f : m_run[qb];
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-#pragma unroll
-      for (int qb = 0; qb < 2; ++qb) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          float p = __builtin_amdgcn_exp2f(fmaf(sv[t >> 1][qb][(t & 1) * 8 + i], c, -m_use[qb]));
-          rs[qb] += p;
-          pb[qb][t][i] = (__bf16)p;
-        }
-      }
-    }
-    l_run[0] += rs[0];
-    l_run[1] += rs[1];
+  // n-th probability of the tile in the order the PV MFMAs consume them (16 keys per B operand)
+  auto prob = [&](const f32x16 (&sv)[2], int n, float m_use, float& rs, bf16x8 (&pb)[4]) {
+    const int t = n >> 3, i = n & 7;
+    float p = __builtin_amdgcn_exp2f(fmaf(sv[t >> 1][(t & 1) * 8 + i], c, -m_use));
+    rs += p;
+    pb[t][i] = (__bf16)p;
   };
-  // ---- O^T += V^T P^T, 16 keys (one B operand per q block) at a time -----------------------------------
-  // ds_read_b64_tr_b16: within 16 lanes, lane r reads 4 dims of key (K0 + r / 4) starting at dim
-  // D0 + 4 * (r % 4) and receives keys K0 .. K0 + 3 of dim D0 + r.
-  auto pv_tile = [&](int buf, const bf16x8 (&pb)[2][4]) {
-    const uint16_t* Vt = sm.v[buf];
-    const int r16 = lane & 15;
-    const int dsel = (lane >> 4) & 1;
-    const int half = r16 & 1;
+  // ---- plain step: probabilities, then O^T += V^T P^T ------------------------------------------------
+  auto finish_tile = [&](int vbuf, const f32x16 (&sv)[2]) {
+    const uint16_t* Vt = sm.v[vbuf];
+    const float m_use = m_run == -INFINITY ? 0.f : m_run;
+    float rs = 0.f;
+    bf16x8 pb[4];
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
+    for (int n = 0; n < 32; ++n) prob(sv, n, m_use, rs, pb);
+    l_run += rs;
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        const int chunk0 = dt * 4 + dsel * 2 + ((r16 & 3) >> 1);
-        bf16x4 lo, hi;
-        {
-          const int row = t * 16 + hl * 4 + (r16 >> 2);
-          const uint16_t* pa = Vt + row * D + ((chunk0 ^ ((row & 3) << 1)) * 8) + half * 4;
-          lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((bf16x4 __attribute__((address_space(3)))*)pa);
-        }
-        {
-          const int row = t * 16 + 8 + hl * 4 + (r16 >> 2);
-          const uint16_t* pa = Vt + row * D + ((chunk0 ^ ((row & 3) << 1)) * 8) + half * 4;
-          hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((bf16x4 __attribute__((address_space(3)))*)pa);
-        }
-        bf16x8 va = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        oacc[dt][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb[0][t], oacc[dt][0], 0, 0, 0);
-        oacc[dt][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb[1][t], oacc[dt][1], 0, 0, 0);
-      }
-    }
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v_frag(Vt, t, dt), pb[t], oacc[dt], 0, 0, 0);
   };
-  // ---- the fused step: scores of the next tile, probabilities of this one, O += P V of this one ----------
-  // A matrix instruction occupies the matrix pipe for 8 passes, during which the wavefront can issue vector
-  // ALU work.  The step is therefore written as slots of one MFMA followed by a slice of the exponentials,
-  // fenced so that the compiler keeps the slots in this order:
-  //   phase A  score MFMAs of the next tile        + probabilities of keys  0..31 of this tile
-  //   phase B  O += P V for keys 0..31             + probabilities of keys 32..63
+  // ---- fused step: scores of the next tile, probabilities of this one, O += P V of this one ----------
+  // A matrix instruction occupies the matrix pipe for 8 passes, during which vector ALU work can issue.  The
+  // step is written as slots of one MFMA followed by a slice of the exponentials, fenced so that the compiler
+  // keeps the slots in this order:
+  //   phase A  score MFMAs of the next tile   + probabilities of keys  0..31 of this tile
+  //   phase B  O += P V for keys 0..31        + probabilities of keys 32..63
   //   phase C  O += P V for keys 32..63
   // LDS operands are fetched one slot ahead of the MFMA that consumes them.
-  auto fused_step = [&](int kbuf_next, int vbuf, const f32x16 (&sv)[2][2], f32x16 (&sacc)[2][2]) {
+  auto fused_step = [&](int kbuf_next, int vbuf, const f32x16 (&sv)[2], f32x16 (&sacc)[2]) {
     const uint16_t* Kt = sm.k[kbuf_next];
     const uint16_t* Vt = sm.v[vbuf];
-    constexpr int N_QK = 4 * DSTEPS;      // score MFMAs
-    constexpr int N_PV = 8 * DT;          // PV MFMAs
-    constexpr int VA = 32 / N_QK;         // probabilities per slot in phase A
-    constexpr int VB = 32 / (N_PV / 2);   // ... in phase B
-    float m_use[2], rs[2] = {0.f, 0.f};
-#pragma unroll
-    for (int qb = 0; qb < 2; ++qb) m_use[qb] = m_run[qb] == -INFINITY ? 0.f : m_run[qb];
-    bf16x8 pb[2][4];
-    auto pval = [&](int n) {  // n-th probability in the order the PV MFMAs consume them
-      const int t = n >> 4, qb = (n >> 3) & 1, i = n & 7;
-      float p = __builtin_amdgcn_exp2f(fmaf(sv[t >> 1][qb][(t & 1) * 8 + i], c, -m_use[qb]));
-      rs[qb] += p;
-      pb[qb][t][i] = (__bf16)p;
-    };
-    auto k_frag = [&](int kb, int s) {
-      const int row = kb * 32 + l32;
-      const int chunk = (s * 2 + hl) ^ (row % OCT);
-      return *reinterpret_cast<const bf16x8*>(Kt + row * D + chunk * 8);
-    };
-    const int r16 = lane & 15;
-    const int dsel = (lane >> 4) & 1;
-    const int half = r16 & 1;
-    auto v_frag = [&](int t, int dt) {
-      const int chunk0 = dt * 4 + dsel * 2 + ((r16 & 3) >> 1);
-      const int row_lo = t * 16 + hl * 4 + (r16 >> 2);
-      const int row_hi = row_lo + 8;
-      const uint16_t* pl = Vt + row_lo * D + ((chunk0 ^ ((row_lo & 3) << 1)) * 8) + half * 4;
-      const uint16_t* ph = Vt + row_hi * D + ((chunk0 ^ ((row_hi & 3) << 1)) * 8) + half * 4;
-      bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((bf16x4 __attribute__((address_space(3)))*)pl);
-      bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((bf16x4 __attribute__((address_space(3)))*)ph);
-      bf16x8 va = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-      return va;
-    };
-
-    __builtin_amdgcn_sched_barrier(0);
-    // ---- phase A ----
-    bf16x8 ka = k_frag(0, 0);
+    constexpr int N_QK = 2 * DSTEPS;         // score MFMAs
+    constexpr int N_PV = 4 * DT;             // PV MFMAs
+    constexpr int VA = 16 / N_QK > 0 ? 16 / N_QK : 1;  // probabilities per slot in phase A
+    constexpr int VB = 16 / (N_PV / 2);      // ... in phase B
+    const float m_use = m_run == -INFINITY ? 0.f : m_run;
+    float rs = 0.f;
+    bf16x8 pb[4];
     int n = 0;
+    __builtin_amdgcn_sched_barrier(0);
+    bf16x8 ka = k_frag(Kt, 0, 0);
 #pragma unroll
     for (int s = 0; s < DSTEPS; ++s) {
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb) {
         const bf16x8 cur = ka;
         if (kb == 0) {
-          ka = k_frag(1, s);
+          ka = k_frag(Kt, 1, s);
         } else if (s + 1 < DSTEPS) {
-          ka = k_frag(0, s + 1);
+          ka = k_frag(Kt, 0, s + 1);
         }
-#pragma unroll
-        for (int qb = 0; qb < 2; ++qb) {
-          if (s == 0) {
-            const f32x16 z = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-            sacc[kb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cur, qreg[qb][s], z, 0, 0, 0);
-          } else {
-            sacc[kb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cur, qreg[qb][s], sacc[kb][qb], 0, 0, 0);
-          }
-#pragma unroll
-          for (int e = 0; e < VA; ++e) pval(n++);
-          __builtin_amdgcn_sched_barrier(0);
+        if (s == 0) {
+          const f32x16 z = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+          sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cur, qreg[s], z, 0, 0, 0);
+        } else {
+          sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cur, qreg[s], sacc[kb], 0, 0, 0);
         }
+        if (n < 16) {
+#pragma unroll
+          for (int e = 0; e < VA; ++e) prob(sv, n++, m_use, rs, pb);
+        }
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
-    // ---- phases B and C ----
-    bf16x8 va = v_frag(0, 0);
+#pragma unroll
+    for (; n < 16;) prob(sv, n++, m_use, rs, pb);
+    bf16x8 va = v_frag(Vt, 0, 0);
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) {
         const bf16x8 cur = va;
         if (dt + 1 < DT) {
-          va = v_frag(t, dt + 1);
+          va = v_frag(Vt, t, dt + 1);
         } else if (t + 1 < 4) {
-          va = v_frag(t + 1, 0);
+          va = v_frag(Vt, t + 1, 0);
         }
+        oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cur, pb[t], oacc[dt], 0, 0, 0);
+        if (t < 2) {
 #pragma unroll
-        for (int qb = 0; qb < 2; ++qb) {
-          oacc[dt][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cur, pb[qb][t], oacc[dt][qb], 0, 0, 0);
-          if (t < 2) {
-#pragma unroll
-            for (int e = 0; e < VB; ++e) pval(n++);
-          }
-          __builtin_amdgcn_sched_barrier(0);
+          for (int e = 0; e < VB; ++e) prob(sv, n++, m_use, rs, pb);
         }
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
-    l_run[0] += rs[0];
-    l_run[1] += rs[1];
+    l_run += rs;
   };
 
-  // Scores of the tile that the next step turns into probabilities; they stay in the accumulation registers
-  // from the step that computes them to the step that reads them.
-  f32x16 sacc[2][2];
+  // Scores of the tile that the next step turns into probabilities.
+  f32x16 sacc[2];
 #pragma unroll
   for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-    for (int qb = 0; qb < 2; ++qb)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) sacc[kb][qb][i] = 0.f;
-  auto pin_s = [&]() {
-#pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-      for (int qb = 0; qb < 2; ++qb) NATS_PIN_ACC(sacc[kb][qb]);
-  };
+    for (int i = 0; i < 16; ++i) sacc[kb][i] = 0.f;
 
   for (int w0 = 0; w0 <= kt_end_group; w0 += kWin) {
     // ---- visit list of this window: wavefront 0 compacts the tiles some query tile of the group sees ----
@@ -600,109 +494,102 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs a) {
     }
     __syncthreads();
     const int n_vis = __builtin_amdgcn_readfirstlane(sm.vcount);
-    if (n_vis == 0) continue;
+    if (n_vis > 0) {
+      // The list entries are the same for every lane: they are kept in scalar registers.
+      // Step j of the pipeline: loads of K tile j+2 and V tile j+1 are put in flight; the matrix pipe computes
+      // the scores of tile j+1 while the vector ALU turns those of tile j into probabilities; then O += P V
+      // for tile j.  Buffers: K tile j in k[j & 1], V tile j in v[j & 1], row limits of tile j in limk[j & 3].
+      auto entry = [&](int j, int& kt, int& emax, int& emin) {
+        const int4 e = sm.vlist[j];
+        kt = __builtin_amdgcn_readfirstlane(e.x);
+        emax = __builtin_amdgcn_readfirstlane(e.y);
+        emin = __builtin_amdgcn_readfirstlane(e.z);
+      };
+      // the element mask is only evaluated on diagonal tiles and on tiles with mixed visibility
+      auto group_needs_lim = [&](int kt, int emin) { return kt * kTile + kTile - 1 - a.base > r0_group || emin < rlast_group; };
+      auto visits = [&](int kt, int emax) { return kUniform || (wave_live && kt <= my_kt_end && emax >= tile_r0); };
 
-    // The list entries are the same for every lane: they are kept in scalar registers.
-    // Step j of the pipeline: loads of K tile j+2 and V tile j+1 are put in flight; the scores of tile j
-    // (computed by step j-1) leave the accumulation registers; the matrix pipe computes the scores of tile
-    // j+1 while the vector ALU turns those of tile j into probabilities; then O += P V for tile j.
-    // Buffers: K tile j in k[j & 1], V tile j in v[j & 1], row limits of tile j in limk[j & 3].
-    auto entry = [&](int j, int& kt, int& emax, int& emin) {
-      const int4 e = sm.vlist[j];
-      kt = __builtin_amdgcn_readfirstlane(e.x);
-      emax = __builtin_amdgcn_readfirstlane(e.y);
-      emin = __builtin_amdgcn_readfirstlane(e.z);
-    };
-    // the element mask is only evaluated on diagonal tiles and on tiles with mixed visibility
-    auto group_needs_lim = [&](int kt, int emin) { return kt * kTile + kTile - 1 - a.base > r0_group || emin < rlast_group; };
-    auto visits = [&](int kt, int emax) { return kUniform || (wave_live && kt <= my_kt_end && emax >= my_r0); };
-
-    int kt_c, emax_c, emin_c;  // tile of the current step
-    int kt_n = 0, emax_n = 0, emin_n = 0;  // tile of the next step
-    entry(0, kt_c, emax_c, emin_c);
-    issue_k(kt_c, 0, 0, group_needs_lim(kt_c, emin_c));
-    issue_v(kt_c, 0);
-    if (n_vis > 1) {
-      entry(1, kt_n, emax_n, emin_n);
-      issue_k(kt_n, 1, 1, group_needs_lim(kt_n, emin_n));
-    }
-    __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();
-    pin_q();
-    if (visits(kt_c, emax_c)) qk_tile(0, sacc);
-    pin_s();
-    __syncthreads();  // k[0] may be overwritten from here on
-
-    for (int j = 0; j < n_vis; ++j) {
-      pin_o();
-      pin_q();
-      pin_s();
-      if (j + 2 < n_vis) {
-        int kt2, emax2, emin2;
-        entry(j + 2, kt2, emax2, emin2);
-        issue_k(kt2, j & 1, (j + 2) & 3, group_needs_lim(kt2, emin2));
+      int kt_c, emax_c, emin_c;              // tile of the current step
+      int kt_n = 0, emax_n = 0, emin_n = 0;  // tile of the next step
+      entry(0, kt_c, emax_c, emin_c);
+      issue_k(kt_c, 0, 0, group_needs_lim(kt_c, emin_c));
+      issue_v(kt_c, 0);
+      if (n_vis > 1) {
+        entry(1, kt_n, emax_n, emin_n);
+        issue_k(kt_n, 1, 1, group_needs_lim(kt_n, emin_n));
       }
-      if (j + 1 < n_vis) issue_v(kt_n, (j + 1) & 1);
-      const bool vis_c = visits(kt_c, emax_c);
-      // (uniform case: the last step computes scores of a stale tile that nobody reads, which keeps the
-      // step free of branches around the matrix instructions)
-      const bool vis_n = kUniform || (j + 1 < n_vis && visits(kt_n, emax_n));
-      if (vis_c) {
-        f32x16 sv[2][2];
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-          for (int qb = 0; qb < 2; ++qb) {
-            sv[kb][qb] = sacc[kb][qb];
-            NATS_PIN_ARCH(sv[kb][qb]);
-          }
-        // no masked score: every key row is at or before the first query and visible to the last one
-        const bool full = kt_c * kTile + kTile - 1 - a.base <= my_r0 && emin_c >= my_rlast;
-        if (!full) mask_scores(kt_c, j & 3, sv);
-        float mx[2];
-        row_max(sv, mx);
-        if (__ballot(mx[0] > m_run[0] + kRescaleSlack || mx[1] > m_run[1] + kRescaleSlack)) rescale(mx);
-        pin_o();
-        if (vis_n) {
-          fused_step((j + 1) & 1, j & 1, sv, sacc);
-        } else {
-          bf16x8 pb[2][4];
-          probs(sv, pb);
-          pv_tile(j & 1, pb);
+      __builtin_amdgcn_s_waitcnt(0);
+      __syncthreads();
+      if (visits(kt_c, emax_c)) qk_tile(0, sacc);
+      __syncthreads();  // k[0] may be overwritten from here on
+
+      for (int j = 0; j < n_vis; ++j) {
+        if (j + 2 < n_vis) {
+          int kt2, emax2, emin2;
+          entry(j + 2, kt2, emax2, emin2);
+          issue_k(kt2, j & 1, (j + 2) & 3, group_needs_lim(kt2, emin2));
         }
-      } else if (vis_n) {
-        qk_tile((j + 1) & 1, sacc);
+        if (j + 1 < n_vis) issue_v(kt_n, (j + 1) & 1);
+        const bool vis_c = visits(kt_c, emax_c);
+        // (uniform case: the last step computes scores of a stale tile that nobody reads, which keeps the
+        // step free of branches around the matrix instructions)
+        const bool vis_n = kUniform || (j + 1 < n_vis && visits(kt_n, emax_n));
+        if (vis_c) {
+          f32x16 sv[2] = {sacc[0], sacc[1]};
+          // no masked score: every key row is at or before the first query and visible to the last one
+          const bool full = kt_c * kTile + kTile - 1 - a.base <= my_r0 && emin_c >= my_rlast;
+          if (!full) mask_scores(kt_c, j & 3, sv);
+          const float mx = row_max(sv);
+          if (__ballot(mx > m_run + kRescaleSlack)) rescale(mx);
+          if (vis_n) {
+            fused_step((j + 1) & 1, j & 1, sv, sacc);
+          } else {
+            finish_tile(j & 1, sv);
+          }
+        } else if (vis_n) {
+          qk_tile((j + 1) & 1, sacc);
+        }
+        kt_c = kt_n; emax_c = emax_n; emin_c = emin_n;
+        if (j + 2 < n_vis) entry(j + 2, kt_n, emax_n, emin_n);
+        __builtin_amdgcn_s_waitcnt(0);  // the tiles in flight have landed in LDS
+        __syncthreads();                // ... for every wavefront, and the tiles of this step are no longer read
       }
-      pin_s();
-      kt_c = kt_n; emax_c = emax_n; emin_c = emin_n;
-      if (j + 2 < n_vis) entry(j + 2, kt_n, emax_n, emin_n);
-      __builtin_amdgcn_s_waitcnt(0);  // the tiles in flight have landed in LDS
-      __syncthreads();                // ... for every wavefront, and the tiles of this step are no longer read
     }
   }
 
-  // ---- epilogue -----------------------------------------------------------------------------------
+  // ---- epilogue: O rows go through LDS so that every row leaves as whole 16-byte pieces ----------------
+  // (all wavefronts are past the last barrier of the tile loop: the tile buffers are free)
+  constexpr int kRowPitch = D * 2 + 16;  // bytes; the pad spreads the rows over the banks
+  static_assert(kPrefillWaves * kHalf * kRowPitch <= sizeof(PrefillSmem<D>), "staging area fits the tile buffers");
+  unsigned char* stage = smem_raw + wave * (kHalf * kRowPitch);
+  {
+    const float l = l_run + __shfl_xor(l_run, 32);
+    const float inv = 1.f / l;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+      for (int g4 = 0; g4 < 4; ++g4) {
+        int d = dt * 32 + g4 * 8 + hl * 4;
+        uint32_t lo = uint32_t(f32_to_bf16_bits(oacc[dt][g4 * 4 + 0] * inv)) |
+                      (uint32_t(f32_to_bf16_bits(oacc[dt][g4 * 4 + 1] * inv)) << 16);
+        uint32_t hi = uint32_t(f32_to_bf16_bits(oacc[dt][g4 * 4 + 2] * inv)) |
+                      (uint32_t(f32_to_bf16_bits(oacc[dt][g4 * 4 + 3] * inv)) << 16);
+        *reinterpret_cast<uint2*>(stage + l32 * kRowPitch + d * 2) = make_uint2(lo, hi);
+      }
+    }
+  }
+  wave_lds_sync();
   if (wave_live) {
     uint16_t* op = static_cast<uint16_t*>(a.o) + b * a.os_b + hq * a.os_h;
+    constexpr int kPieces = kHalf * OCT / kWave;  // 16-byte pieces per lane
 #pragma unroll
-    for (int qb = 0; qb < 2; ++qb) {
-      float l = l_run[qb] + __shfl_xor(l_run[qb], 32);
-      float inv = 1.f / l;
-      int qtok = q0 + qb * 32 + l32;
+    for (int i = 0; i < kPieces; ++i) {
+      const int id = i * kWave + lane;
+      const int row = id / OCT, piece = id % OCT;
+      const int qtok = q0 + row;
       if (qtok >= a.r_begin && qtok < a.r_end) {
-        uint16_t* rp = op + (int64_t)(qtok - a.r_begin) * a.os_l;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-#pragma unroll
-          for (int g4 = 0; g4 < 4; ++g4) {
-            int d = dt * 32 + g4 * 8 + hl * 4;
-            uint32_t lo = uint32_t(f32_to_bf16_bits(oacc[dt][qb][g4 * 4 + 0] * inv)) |
-                          (uint32_t(f32_to_bf16_bits(oacc[dt][qb][g4 * 4 + 1] * inv)) << 16);
-            uint32_t hi = uint32_t(f32_to_bf16_bits(oacc[dt][qb][g4 * 4 + 2] * inv)) |
-                          (uint32_t(f32_to_bf16_bits(oacc[dt][qb][g4 * 4 + 3] * inv)) << 16);
-            *reinterpret_cast<uint2*>(rp + d) = make_uint2(lo, hi);
-          }
-        }
+        uint4 val = *reinterpret_cast<const uint4*>(stage + row * kRowPitch + piece * 16);
+        *reinterpret_cast<uint4*>(op + (int64_t)(qtok - a.r_begin) * a.os_l + piece * 8) = val;
       }
     }
   }
@@ -718,7 +605,7 @@ static int launch_prefill_mfma(const PrefillArgs& a, int64_t n_wg, hipStream_t s
     if (e != hipSuccess) return fail(NATS_ERR_LAUNCH, "hipFuncSetAttribute(%zu bytes of LDS): %s", smem, hipGetErrorString(e));
     configured = true;
   }
-  hipLaunchKernelGGL((prefill_mfma_kernel<D, kUniform>), dim3((unsigned)n_wg), dim3(256), smem, st, a);
+  hipLaunchKernelGGL((prefill_mfma_kernel<D, kUniform>), dim3((unsigned)n_wg), dim3(kPrefillWaves * kWave), smem, st, a);
   NATS_CHECK_LAUNCH("prefill_mfma_kernel");
   return NATS_OK;
 }
@@ -750,14 +637,17 @@ int check_common(const char* who, const SegmentShape& g, const int64_t* q_stride
                (long long)g.W, (long long)g.C);
   NATS_REQUIRE(dtype == NATS_DTYPE_BF16 || dtype == NATS_DTYPE_F32, NATS_ERR_BAD_DTYPE, "%s: dtype %d", who, dtype);
   NATS_REQUIRE(g.N < (int64_t(1) << 30), NATS_ERR_BAD_SHAPE, "%s: %lld key rows are too many", who, (long long)g.N);
+  NATS_REQUIRE(k_strides[2] * kTile < (int64_t(1) << 30) && v_strides[2] * kTile < (int64_t(1) << 30) && k_strides[2] > 0 &&
+                   v_strides[2] > 0,
+               NATS_ERR_BAD_SHAPE, "%s: row strides %lld / %lld of k / v", who, (long long)k_strides[2], (long long)v_strides[2]);
   if (dtype == NATS_DTYPE_BF16) {
-    // 16-byte vector loads of rows
-    NATS_REQUIRE(q_strides[2] % 8 == 0 && k_strides[2] % 8 == 0 && v_strides[2] % 8 == 0 && o_strides[2] % 4 == 0 &&
-                     q_strides[1] % 8 == 0 && k_strides[1] % 8 == 0 && v_strides[1] % 8 == 0 && o_strides[1] % 4 == 0 &&
-                     q_strides[0] % 8 == 0 && k_strides[0] % 8 == 0 && v_strides[0] % 8 == 0 && o_strides[0] % 4 == 0,
+    // 16-byte vector loads and stores of rows
+    NATS_REQUIRE(q_strides[2] % 8 == 0 && k_strides[2] % 8 == 0 && v_strides[2] % 8 == 0 && o_strides[2] % 8 == 0 &&
+                     q_strides[1] % 8 == 0 && k_strides[1] % 8 == 0 && v_strides[1] % 8 == 0 && o_strides[1] % 8 == 0 &&
+                     q_strides[0] % 8 == 0 && k_strides[0] % 8 == 0 && v_strides[0] % 8 == 0 && o_strides[0] % 8 == 0,
                  NATS_ERR_BAD_SHAPE, "%s: bf16 strides must keep rows 16-byte aligned", who);
-    NATS_REQUIRE((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v)) % 16 == 0 &&
-                     reinterpret_cast<uintptr_t>(o) % 8 == 0,
+    NATS_REQUIRE((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
+                  reinterpret_cast<uintptr_t>(o)) % 16 == 0,
                  NATS_ERR_BAD_SHAPE, "%s: bf16 tensors must be 16-byte aligned", who);
   }
   return NATS_OK;
