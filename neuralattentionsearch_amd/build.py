@@ -13,7 +13,7 @@ HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
     # hipcc -O3 may otherwise form packed fp32 ops; keep them off
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    "-Wno-unknown-warning-option", "-Wno-unused-command-line-argument",
+    "-Wno-unknown-warning-option", "-Wno-unused-command-line-argument", "-Wno-inline-asm",
 ]
 
 
