@@ -160,33 +160,12 @@ __global__ __launch_bounds__(64) void prefill_simple_kernel(PrefillArgs a) {
 // ---------------------------------------------------------------------------------------------------
 constexpr float kRescaleSlack = 8.0f;
 constexpr int kPrefillWaves = 8;
-
-// Global -> LDS transfers (16 or 4 bytes per lane, LDS address = uniform base + lane * size).  They are
-// issued from assembly so that the kernel itself decides when to wait for them (s_waitcnt vmcnt(n), they
-// complete in order): the compiler, not knowing which buffer an LDS read touches, would otherwise wait for
-// every transfer in flight before every LDS read and serialise loads and compute.
-// The host pass of the single-source compile never runs this code.
-#if defined(__HIP_DEVICE_COMPILE__)
-__device__ __forceinline__ void lds_dma16(const void* gptr, uint32_t lds_addr) {
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(lds_addr) : "memory", "m0");
-}
-__device__ __forceinline__ void lds_dma4(const void* gptr, uint32_t lds_addr) {
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(gptr), "s"(lds_addr) : "memory", "m0");
-}
-#else
-__device__ __forceinline__ void lds_dma16(const void*, uint32_t) {}
-__device__ __forceinline__ void lds_dma4(const void*, uint32_t) {}
-#endif
-__device__ __forceinline__ uint32_t lds_address(const void* p) {
-  return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) unsigned char*)p;
-}
 constexpr int kWin = 1024;  // key tiles whose visit list is built at once
-constexpr int kStages = 4;   // K / V tile buffers (a power of two); loads run two to three steps ahead of their use
 
 template <int D>
 struct PrefillSmem {
-  uint16_t k[kStages][kTile * D];
-  uint16_t v[kStages][kTile * D];
+  uint16_t k[2][kTile * D];
+  uint16_t v[2][kTile * D];
   int limk[4][kTile];
   int4 vlist[kWin];  // visited key tiles of the current window: {tile, max limit, min limit, -}
   int vcount;
@@ -295,7 +274,7 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
 #pragma unroll
       for (int j = 0; j < DMA_PER_WAVE; ++j) {
         const int inst = wave * DMA_PER_WAVE + j;
-        lds_dma16(tb + (int)off[j], __builtin_amdgcn_readfirstlane(lds_address(dst + inst * kWave * 8)));
+        __builtin_amdgcn_global_load_lds(tb + (int)off[j], (uint32_t __attribute__((address_space(3)))*)(dst + inst * kWave * 8), 16, 0, 0);
       }
     } else {
 #pragma unroll
@@ -305,37 +284,20 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
         const int row = q / OCT, pos = q % OCT;
         const int n = min(kt * kTile + row, a.N - 1);
         const int chunk = is_v ? pos ^ ((row & 3) << 1) : pos ^ (row % OCT);
-        lds_dma16(base + (int64_t)n * stride + chunk * 8, __builtin_amdgcn_readfirstlane(lds_address(dst + inst * kWave * 8)));
+        __builtin_amdgcn_global_load_lds(base + (int64_t)n * stride + chunk * 8,
+                                         (uint32_t __attribute__((address_space(3)))*)(dst + inst * kWave * 8), 16, 0, 0);
       }
     }
   };
   // K tile and the visibility limits of its rows; the limits go to slot (list index & 3)
-  // Returns the number of transfers this wavefront put in flight.  Rows beyond N take the limit of row
-  // N-1: they lie after every query, so causality masks them.
   auto issue_k = [&](int kt, int buf, int slot, bool need_lim) {
     issue_rows(kp, a.ks_l, koff, sm.k[buf], kt, false);
-    if (need_lim && wave == 0) {
-      const int n = min(kt * kTile + lane, a.N - 1);
-      lds_dma4(lim + n, __builtin_amdgcn_readfirstlane(lds_address(&sm.limk[slot][0])));
-      return DMA_PER_WAVE + 1;
-    }
-    return DMA_PER_WAVE;
-  };
-  auto issue_v = [&](int kt, int buf) {
-    issue_rows(vp, a.vs_l, voff, sm.v[buf], kt, true);
-    return DMA_PER_WAVE;
-  };
-  // waits until at most `n` of this wavefront's transfers are still in flight (they complete in order)
-  auto wait_in_flight = [&](int n) {
-    switch (n) {
-      case 0: __builtin_amdgcn_s_waitcnt(0x0f70 | 0); break;
-      case 1: __builtin_amdgcn_s_waitcnt(0x0f70 | 1); break;
-      case 2: __builtin_amdgcn_s_waitcnt(0x0f70 | 2); break;
-      case 3: __builtin_amdgcn_s_waitcnt(0x0f70 | 3); break;
-      case 4: __builtin_amdgcn_s_waitcnt(0x0f70 | 4); break;
-      default: __builtin_amdgcn_s_waitcnt(0x0f70 | 5); break;
+    if (need_lim && tid < kTile) {
+      int n = kt * kTile + tid;
+      sm.limk[slot][tid] = n < a.N ? lim[n] : -1;
     }
   };
+  auto issue_v = [&](int kt, int buf) { issue_rows(vp, a.vs_l, voff, sm.v[buf], kt, true); };
 
   auto k_frag = [&](const uint16_t* Kt, int kb, int s) {
     const int row = kb * 32 + l32;
@@ -549,35 +511,25 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
 
       int kt_c, emax_c, emin_c;              // tile of the current step
       int kt_n = 0, emax_n = 0, emin_n = 0;  // tile of the next step
-      int kt_2 = 0, emax_2 = 0, emin_2 = 0;  // tile after that
       entry(0, kt_c, emax_c, emin_c);
       issue_k(kt_c, 0, 0, group_needs_lim(kt_c, emin_c));
       issue_v(kt_c, 0);
       if (n_vis > 1) {
         entry(1, kt_n, emax_n, emin_n);
         issue_k(kt_n, 1, 1, group_needs_lim(kt_n, emin_n));
-        issue_v(kt_n, 1);
       }
-      int flying = 0;  // transfers of this wavefront that the next step does not need yet
-      if (n_vis > 2) {
-        entry(2, kt_2, emax_2, emin_2);
-        flying = issue_k(kt_2, 2, 2, group_needs_lim(kt_2, emin_2));
-      }
-      wait_in_flight(flying);
+      __builtin_amdgcn_s_waitcnt(0);
       __syncthreads();
       if (visits(kt_c, emax_c)) qk_tile(0, sacc);
       __syncthreads();  // k[0] may be overwritten from here on
 
       for (int j = 0; j < n_vis; ++j) {
-        // tile j+3's keys and tile j+2's values go in flight; at the end of the step tile j+2's keys and tile
-        // j+1's values (in flight since the previous step) must have landed
-        flying = 0;
-        if (j + 3 < n_vis) {
-          int kt3, emax3, emin3;
-          entry(j + 3, kt3, emax3, emin3);
-          flying += issue_k(kt3, (j + 3) % kStages, (j + 3) & 3, group_needs_lim(kt3, emin3));
+        if (j + 2 < n_vis) {
+          int kt2, emax2, emin2;
+          entry(j + 2, kt2, emax2, emin2);
+          issue_k(kt2, j & 1, (j + 2) & 3, group_needs_lim(kt2, emin2));
         }
-        if (j + 2 < n_vis) flying += issue_v(kt_2, (j + 2) % kStages);
+        if (j + 1 < n_vis) issue_v(kt_n, (j + 1) & 1);
         const bool vis_c = visits(kt_c, emax_c);
         // (uniform case: the last step computes scores of a stale tile that nobody reads, which keeps the
         // step free of branches around the matrix instructions)
@@ -590,18 +542,17 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
           const float mx = row_max(sv);
           if (__ballot(mx > m_run + kRescaleSlack)) rescale(mx);
           if (vis_n) {
-            fused_step((j + 1) % kStages, j % kStages, sv, sacc);
+            fused_step((j + 1) & 1, j & 1, sv, sacc);
           } else {
-            finish_tile(j % kStages, sv);
+            finish_tile(j & 1, sv);
           }
         } else if (vis_n) {
-          qk_tile((j + 1) % kStages, sacc);
+          qk_tile((j + 1) & 1, sacc);
         }
         kt_c = kt_n; emax_c = emax_n; emin_c = emin_n;
-        kt_n = kt_2; emax_n = emax_2; emin_n = emin_2;
-        if (j + 3 < n_vis) entry(j + 3, kt_2, emax_2, emin_2);
-        wait_in_flight(flying);  // everything older than this step's transfers has landed in LDS
-        __syncthreads();         // ... for every wavefront, and the tiles of this step are no longer read
+        if (j + 2 < n_vis) entry(j + 2, kt_n, emax_n, emin_n);
+        __builtin_amdgcn_s_waitcnt(0);  // the tiles in flight have landed in LDS
+        __syncthreads();                // ... for every wavefront, and the tiles of this step are no longer read
       }
     }
   }
