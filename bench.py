@@ -31,7 +31,7 @@ if ROOT not in sys.path:
 # HBM bytes per launch of the dominant kernels at the default workloads, from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE scaled by a 1 GiB device copy (read factor 2.0, write factor 1.0); see profiles/.
 MEASURED_TRAFFIC = {  # bytes read + written per launch
-    "prefill": 232628 * 1024 * 2.0 + 294866 * 1024 * 1.0,
+    "prefill": 228539 * 1024 * 2.0 + 262144 * 1024 * 1.0,
     "decode": 887027 * 1024 * 2.0 + 1560 * 1024 * 1.0,
     "evict": 272937 * 1024 * 2.0 + 554050 * 1024 * 1.0,
 }
@@ -389,7 +389,7 @@ def main():
         line["roofline"] = {"bound": "mfma", "achieved": pre["tflops_visited"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                             "frac": pre["tflops_visited"] / PEAK_BF16_TFLOPS,
                             "traffic": MEASURED_TRAFFIC["prefill"] if args.prefill_len == 32768 else None,
-                            "kernel": "prefill_mfma_kernel<128>"}
+                            "kernel": "prefill_mfma_kernel<128, true>"}
     if "decode" in res:
         d = res["decode"]
         line["roofline_decode"] = {"bound": "hbm", "achieved": d["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
