@@ -56,6 +56,32 @@ int nats_roles_from_logits(const void* logits, int dtype, int64_t B, int64_t S, 
                            int force_first_global, int force_last_global, uint8_t* roles, void* one_hot,
                            void* stream);
 
+/* ------------------------------------------------------------------------------------------------
+ * Fused role step: chunk pooling of the hidden states, role projection, bias, argmax with forced globals and
+ * the next-global scan in one call.  Replaces NAtSCache.update_nats_cached_x_across_chunk / _in_chunk
+ * (components/cache/dyn_cache.py:117-171) with the pooling of chunk_utils.py:13-62, followed by proj_layer and
+ * _sample_for_token_info_values_inference (models/transformer/attention/nats_chunk_attention.py:64-95,
+ * nats_attention.py:96-109) and the index scan of components/masks/utils.py:85-87.
+ *   x         [B, L, dim] hidden states of the new tokens, strides (stride_b, stride_l), last dimension contiguous
+ *   carry_in  [B, dim] running statistic of the open chunk (sum of x / C, or max); required when pre_fill > 0
+ *   weight    [H_kv * 3, dim] contiguous, the role projection (bias free)
+ *   pre_fill  tokens already in the open chunk (chunk_fill_size before this call), 0 <= pre_fill < C
+ *   merge_max 0 = mean pooling, 1 = max pooling
+ * With total = pre_fill + L:  total < C  -> no chunk completes, only carry_out = statistic so far is written;
+ * otherwise S = ceil(total / C) role slots are produced, the open last one (total % C != 0) forced global and
+ * its statistic written to carry_out.
+ *   roles     [B, H_kv, S] uint8 out
+ *   one_hot   [B, H_kv, S, 3] out, dtype of x, may be NULL
+ *   logits    [B, S, H_kv, 3] out (before the bias), dtype of x, may be NULL
+ *   end_idx / vis_lim  [B, H_kv, S] as nats_role_scan, may be NULL
+ * The pooled statistic and the logits are rounded to the dtype of x where the torch ops round them; logits
+ * are accumulated in fp32 in an order of their own, so they agree with a library GEMM to rounding only.
+ */
+int nats_role_step(const void* x, const void* carry_in, const void* weight, int dtype, int64_t B, int64_t L, int64_t dim,
+                   int64_t H_kv, int64_t C, int64_t W, int64_t pre_fill, int merge_max, float global_bias,
+                   int force_first_global, const int64_t* x_strides, uint8_t* roles, void* one_hot, void* logits,
+                   void* carry_out, int64_t* end_idx, int32_t* vis_lim, void* stream);
+
 /* next-global index and the per-slot visibility limit derived from it.
  * Replaces the first half of generate_hard_seq_masks (components/masks/utils.py:85-87).
  *   roles    [B, H_kv, S] uint8

@@ -44,6 +44,8 @@ SIGNATURES = {
     "nats_last_error": (ctypes.c_char_p, []),
     "nats_roles_from_logits": (ctypes.c_int, [c_p, ctypes.c_int, c_i64, c_i64, c_i64, ctypes.c_float, ctypes.c_int,
                                               ctypes.c_int, c_p, c_p, c_p]),
+    "nats_role_step": (ctypes.c_int, [c_p, c_p, c_p, ctypes.c_int, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64,
+                                      ctypes.c_int, ctypes.c_float, ctypes.c_int, c_i64p, c_p, c_p, c_p, c_p, c_p, c_p, c_p]),
     "nats_role_scan": (ctypes.c_int, [c_p, c_i64, c_i64, c_i64, c_i64, c_i64, c_p, c_p, c_p]),
     "nats_prefill_mask": (ctypes.c_int, [c_p, c_i64, c_i64, c_i64, c_i64, c_i64, c_p, c_p, ctypes.c_size_t, c_p]),
     "nats_prefill_tile_map": (ctypes.c_int, [c_p, c_i64, c_i64, c_i64, c_i64, c_i64, c_p, c_p, ctypes.c_size_t, c_p]),

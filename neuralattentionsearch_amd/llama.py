@@ -39,6 +39,7 @@ class NAtSLlamaConfig:
     chunk_size: int = 64
     local_seq_max_length: int = 256  # sliding window, in tokens
     chunk_merge_method: str = "mean"
+    fused_role_step: bool = False  # pooling + role projection + argmax in one kernel instead of torch ops
 
     @property
     def head_dim(self) -> int:
@@ -101,6 +102,7 @@ class NAtSLlamaAttention(nn.Module):
         self.v_proj = nn.Linear(cfg.hidden_size, self.num_key_value_heads * self.head_dim, bias=False)
         self.o_proj = nn.Linear(self.num_heads * self.head_dim, cfg.hidden_size, bias=False)
         self.proj_layer = nn.Linear(cfg.hidden_size, self.num_key_value_heads * 3, bias=False)  # :315-318
+        self.fused_role_step = cfg.fused_role_step
 
     def forward(self, hidden_states: torch.Tensor, position_embeddings, start_pos: int, past_key_value: NAtSCache):
         bsz, q_len, _ = hidden_states.shape
@@ -111,7 +113,18 @@ class NAtSLlamaAttention(nn.Module):
 
         pre_fill = past_key_value.get_nats_chunk_fill_size(idx)
         is_pre_filling = start_pos == 0
-        if pre_fill + q_len < C:
+        if self.fused_role_step:
+            step = ops.role_step(hidden_states, self.proj_layer.weight, C, self.local_seq_max_length, pre_fill=pre_fill,
+                                 carry_in=past_key_value.get_nats_cached_x_in_chunk(idx) if pre_fill else None,
+                                 merge_max=self.chunk_merge_method == ChunkMergeType.MAX, global_bias=0.0,
+                                 force_first_global=start_pos < C)
+            past_key_value._update_cache_x(step["carry"], idx)
+            roles, tsi = step["roles"], step["token_states_info"]
+            if roles is None:
+                roles = torch.zeros(bsz, self.num_key_value_heads, 1, dtype=torch.uint8, device=hidden_states.device)
+                tsi = torch.zeros(bsz, self.num_key_value_heads, 1, 3, dtype=hidden_states.dtype, device=hidden_states.device)
+                tsi[..., 0] = 1
+        elif pre_fill + q_len < C:
             past_key_value.update_nats_cached_x_in_chunk(hidden_states, idx, self.chunk_merge_method)
             roles = torch.zeros(bsz, self.num_key_value_heads, 1, dtype=torch.uint8, device=hidden_states.device)
             tsi = torch.zeros(bsz, self.num_key_value_heads, 1, 3, dtype=hidden_states.dtype, device=hidden_states.device)

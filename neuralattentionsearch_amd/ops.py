@@ -74,6 +74,50 @@ def roles_from_logits(logits: torch.Tensor, global_bias: float = 0.1, force_firs
     return roles, one_hot
 
 
+def role_step(x: torch.Tensor, weight: torch.Tensor, chunk_size: int, window: int, pre_fill: int = 0,
+              carry_in: torch.Tensor | None = None, merge_max: bool = False, global_bias: float = 0.1,
+              force_first_global: bool = False, with_one_hot: bool = True, with_logits: bool = False,
+              with_scan: bool = False) -> dict:
+    """Chunk pooling of hidden states + role projection + argmax (+ next-global scan) in one call.
+
+    x [B, L, dim] hidden states of the new tokens, weight [H_kv * 3, dim] (proj_layer.weight), carry_in
+    [B, 1, dim] or [B, dim] the running statistic of the open chunk (required when pre_fill > 0).
+    Returns a dict with `roles` uint8 [B, H_kv, S] (None while no chunk completes), `token_states_info`,
+    `logits` [B, S, H_kv, 3], `carry` [B, 1, dim] (statistic of the open chunk, None if every chunk is
+    complete), `end_idx`, `vis_lim`, and `pad`.
+    components/cache/dyn_cache.py:117-171, models/transformer/attention/nats_chunk_attention.py:64-95."""
+    _require_cuda(x, weight, carry_in)
+    lib = _lib.load()
+    if x.dim() != 3 or weight.dim() != 2 or weight.shape[1] != x.shape[2] or weight.shape[0] % 3 != 0:
+        raise ValueError(f"x must be [B, L, dim] and weight [H_kv * 3, dim], got {tuple(x.shape)}, {tuple(weight.shape)}")
+    if weight.dtype != x.dtype or (carry_in is not None and carry_in.dtype != x.dtype):
+        raise ValueError("x, weight and carry_in must share one dtype")
+    B, L, dim = x.shape
+    H = weight.shape[0] // 3
+    C = chunk_size
+    if x.stride(-1) != 1:
+        x = x.contiguous()
+    weight = weight.contiguous()
+    if carry_in is not None:
+        carry_in = carry_in.reshape(B, dim).contiguous()
+    total = pre_fill + L
+    S = 0 if total < C else math.ceil(total / C)
+    pad = 0 if S == 0 else S * C - total
+    dev, dt = x.device, x.dtype
+    roles = torch.empty(B, H, S, dtype=torch.uint8, device=dev) if S else None
+    one_hot = torch.empty(B, H, S, 3, dtype=dt, device=dev) if S and with_one_hot else None
+    logits = torch.empty(B, S, H, 3, dtype=dt, device=dev) if S and with_logits else None
+    carry = torch.empty(B, 1, dim, dtype=dt, device=dev) if (S == 0 or pad) else None
+    end_idx = torch.empty(B, H, S, dtype=torch.int64, device=dev) if S and with_scan else None
+    vis_lim = torch.empty(B, H, S, dtype=torch.int32, device=dev) if S and with_scan else None
+    check(lib.nats_role_step(_ptr(x), _ptr(carry_in), _ptr(weight), _dtype_code(x), B, L, dim, H, C, window, pre_fill,
+                             int(merge_max), float(global_bias), int(force_first_global), i64_array(x.stride()[:2]),
+                             _ptr(roles), _ptr(one_hot), _ptr(logits), _ptr(carry), _ptr(end_idx), _ptr(vis_lim),
+                             _stream(x)))
+    return {"roles": roles, "token_states_info": one_hot, "logits": logits, "carry": carry, "end_idx": end_idx,
+            "vis_lim": vis_lim, "pad": pad}
+
+
 def roles_from_one_hot(token_states_info: torch.Tensor) -> torch.Tensor:
     """[B, H_kv, S, 3] one-hot float -> uint8 roles (index of the 1)."""
     t = token_states_info

@@ -23,6 +23,9 @@ How each function is pinned (see tests/test_oracle_*.py):
                                  every byte of cache_k, cache_v, valid_tokens, sizes and scalars
 * decode_attention ............. equals masked_attention restricted to the valid rows (gather, then dense
                                  softmax); checked against torch SDPA
+* pooled_role_logits ........... closed forms (constant chunks, one-hot projection rows), zero padding of the
+                                 open chunk, and the invariant that any split of a stream into calls gives
+                                 the statistics of one call (dyn_cache.py:98-171, chunk_utils.py:13-62)
 
 Functions with parity unpinned: none of the above; the per-token cache (chunk_size == 1,
 components/cache/nats_layer_cache.py) is not restated here.
@@ -70,6 +73,54 @@ def roles_from_logits(logits: torch.Tensor, global_bias: float = 0.1, force_firs
     if force_last_global:
         roles[:, :, -1] = ROLE_GLOBAL
     return roles
+
+
+def pooled_role_logits(x: torch.Tensor, weight: torch.Tensor, chunk_size: int, pre_fill: int = 0,
+                       carry_in: torch.Tensor | None = None, merge_max: bool = False):
+    """Hidden states of the new tokens -> (pooled [B, S, dim], logits [B, S, H_kv, 3], carry, pad), with the
+    torch ops the reference runs, in the dtype of x.
+
+    components/cache/dyn_cache.py:98-115 (running statistic: sum of x / C, or max), :130-171 (chunks touched by
+    the new tokens: the open chunk completed with its carried statistic, whole chunks pooled with
+    chunk_utils.py:13-62, zero padding of an open last chunk) and proj_layer (nats_chunk_attention.py:87).
+    While no chunk completes (pre_fill + L < C) pooled and logits are None and only the carry is returned."""
+    B, L, dim = x.shape
+    C = chunk_size
+
+    def merge(cache, new):  # dyn_cache.py:98-113
+        if merge_max:
+            return new.max(1, keepdim=True)[0] if cache is None else torch.max(torch.cat([cache, new], 1), 1, keepdim=True)[0]
+        add = (new / C).sum(1, keepdim=True)
+        return add if cache is None else cache + add
+
+    def pool(t, pad):  # chunk_utils.py:13-62
+        if pad:
+            t = torch.nn.functional.pad(t, (0, 0, 0, pad))
+        t = t.unflatten(1, (-1, C))
+        return t.max(2)[0] if merge_max else t.mean(2)
+
+    if carry_in is not None:
+        carry_in = carry_in.reshape(B, 1, dim)
+    if pre_fill + L < C:  # dyn_cache.py:117-124
+        return None, None, merge(carry_in if pre_fill else None, x), 0
+    if pre_fill:
+        head_len = C - pre_fill
+        head = merge(carry_in, x[:, :head_len])
+        rest = L - head_len
+        if rest == 0:
+            pad, pooled = 0, head
+        else:
+            pad = (-rest) % C
+            pooled = torch.cat([head, pool(x[:, head_len:], pad)], 1)
+    else:
+        pad = (-L) % C
+        pooled = pool(x, pad)
+    carry = None
+    if pad:
+        tail = x[:, pad - C:]
+        carry = tail.max(1, keepdim=True)[0] if merge_max else (tail / C).sum(1, keepdim=True)
+    logits = torch.nn.functional.linear(pooled, weight).unflatten(-1, (-1, 3))
+    return pooled, logits, carry, pad
 
 
 def one_hot_roles(roles: np.ndarray, dtype=torch.float32) -> torch.Tensor:

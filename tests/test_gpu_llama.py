@@ -131,3 +131,21 @@ def test_generate_is_deterministic_and_matches_stepwise_forward():
     # eviction was live: the cache holds fewer rows than tokens seen for at least one layer
     assert cache_a.get_seq_length(0) == 45 + 29
     assert min(l.n_ctx_data for l in cache_a.cache_model) < 45 + 29 + 16
+
+
+def test_fused_role_step_gives_the_same_generation():
+    """The harness with the fused role-step kernel against the same model with torch pooling + projection (fp32:
+    the two differ in summation order only, which the seeded logits' gaps absorb)."""
+    from neuralattentionsearch_amd.llama import NAtSLlamaConfig, NAtSLlamaForCausalLM
+    say("llama fused role step")
+    kw = dict(vocab_size=777, hidden_size=512, intermediate_size=512, num_hidden_layers=2, num_attention_heads=8,
+              num_key_value_heads=4, chunk_size=8, local_seq_max_length=16)
+    ids = torch.randint(0, 777, (2, 45), generator=torch.Generator().manual_seed(1)).cuda()
+    outs, kept = [], []
+    for fused in (False, True):
+        model = NAtSLlamaForCausalLM.random_init(NAtSLlamaConfig(fused_role_step=fused, **kw), dtype=torch.float32, seed=3, std=0.08)
+        toks, cache = model.generate(ids, 30)
+        outs.append(toks)
+        kept.append([l.valid_tokens.sum().item() for l in cache.cache_model])
+    assert torch.equal(outs[0], outs[1])
+    assert kept[0] == kept[1]

@@ -3,6 +3,7 @@ import itertools
 import math
 
 import numpy as np
+import pytest
 import torch
 
 from oracle import nats_oracle as orc
@@ -130,3 +131,51 @@ def test_masked_attention_explicit_form_matches_sdpa():
     a = orc.masked_attention(q, k, v, mask)
     b = orc.masked_attention(q, k, v, mask, explicit=True)
     assert (a - b).abs().max().item() < 1e-5
+
+
+# ---- pooled_role_logits ---------------------------------------------------------------------------
+def test_pooling_closed_forms():
+    """Constant chunks pool to their constant; an open last chunk is averaged over C with zero padding (max
+    pooling sees the zeros too); one-hot projection rows pick single pooled columns."""
+    C, dim, H = 4, 6, 2
+    x = torch.zeros(1, 10, dim)
+    x[0, 0:4] = 2.0
+    x[0, 4:8] = -3.0
+    x[0, 8:10] = 5.0
+    w = torch.zeros(H * 3, dim)
+    for o in range(H * 3):
+        w[o, o] = 1.0
+    pooled, logits, carry, pad = orc.pooled_role_logits(x, w, C)
+    assert pad == 2 and pooled.shape == (1, 3, dim) and logits.shape == (1, 3, H, 3)
+    assert torch.equal(pooled[0, :, 0], torch.tensor([2.0, -3.0, 2.5]))  # 2 * 5 / 4: zeros count in the mean
+    assert torch.equal(logits[0, :, 1, 2], pooled[0, :, 5])
+    assert torch.equal(carry[0, 0], torch.full((dim,), 2.5))
+    pooled_m, _, carry_m, _ = orc.pooled_role_logits(-x, w, C, merge_max=True)
+    assert torch.equal(pooled_m[0, :, 0], torch.tensor([-2.0, 3.0, 0.0]))  # the zero padding wins over -5
+    assert torch.equal(carry_m[0, 0], torch.full((dim,), -5.0))  # ... but is not carried on
+
+
+@pytest.mark.parametrize("merge_max", [False, True])
+def test_pooling_is_independent_of_how_the_stream_is_cut(merge_max):
+    C, dim, H, B = 8, 16, 3, 2
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(B, 61, dim, generator=g)
+    w = torch.randn(H * 3, dim, generator=g)
+    whole, logits_whole, _, _ = orc.pooled_role_logits(x, w, C, merge_max=merge_max)
+    n_full = 61 // C
+    for cuts in ([61], [3, 2, 9, 1, 1, 30, 15], [8, 8, 8, 37], [5, 56]):
+        pre, carry, pos, got = 0, None, 0, []
+        for n in cuts:
+            pooled, logits, carry_new, pad = orc.pooled_role_logits(x[:, pos:pos + n], w, C, pre_fill=pre, carry_in=carry,
+                                                                    merge_max=merge_max)
+            total = pre + n
+            if pooled is not None:
+                done = total // C
+                got.append(pooled[:, :done])
+                carry = carry_new
+            else:
+                carry = carry_new
+            pre, pos = total % C, pos + n
+        got = torch.cat(got, 1)
+        assert got.shape[1] == n_full
+        assert torch.allclose(got, whole[:, :n_full], atol=1e-6)
