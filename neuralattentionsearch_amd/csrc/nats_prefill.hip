@@ -541,10 +541,12 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
           if (!full) mask_scores(kt_c, j & 3, sv);
           const float mx = row_max(sv);
           if (__ballot(mx > m_run + kRescaleSlack)) rescale(mx);
-          if (vis_n) {
+          if (kUniform) {
             fused_step((j + 1) & 1, j & 1, sv, sacc);
           } else {
+            // wavefronts with different query tiles: the same pipeline, its two halves one after the other
             finish_tile(j & 1, sv);
+            if (vis_n) qk_tile((j + 1) & 1, sacc);
           }
         } else if (vis_n) {
           qk_tile((j + 1) & 1, sacc);
