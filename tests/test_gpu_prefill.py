@@ -46,7 +46,8 @@ def test_bf16_gqa_group_sizes(n_rep):
 
 
 @pytest.mark.parametrize("L,C,W,D", [(1000, 64, 256, 128), (777, 32, 64, 128), (512, 16, 64, 64), (2048, 64, 128, 64),
-                                     (1536, 128, 256, 128), (200, 8, 16, 128), (63, 64, 64, 128), (65, 64, 64, 128)])
+                                     (1536, 128, 256, 128), (200, 8, 16, 128), (63, 64, 64, 128), (65, 64, 64, 128),
+                                     (900, 1, 64, 128), (333, 2, 8, 64)])  # per-token roles (chunk size 1) included
 def test_bf16_shapes(L, C, W, D):
     run_case(2, 8, 2, L, D, C, W, torch.bfloat16, seed=L + C)
 
