@@ -164,9 +164,9 @@ constexpr int kWin = 1024;  // key tiles whose visit list is built at once
 
 template <int D>
 struct PrefillSmem {
-  uint16_t k[2][kTile * D];
-  uint16_t v[2][kTile * D];
-  int limk[4][kTile];
+  uint16_t k[4][kTile * D];  // tile j of the visit list in k[j & 3]
+  uint16_t v[4][kTile * D];
+  int limk[8][kTile];        // row limits of tile j in limk[j & 7]
   int4 vlist[kWin];  // visited key tiles of the current window: {tile, max limit, min limit, -}
   int vcount;
 };
@@ -509,50 +509,68 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
       auto group_needs_lim = [&](int kt, int emin) { return kt * kTile + kTile - 1 - a.base > r0_group || emin < rlast_group; };
       auto visits = [&](int kt, int emax) { return kUniform || (wave_live && kt <= my_kt_end && emax >= tile_r0); };
 
-      int kt_c, emax_c, emin_c;              // tile of the current step
-      int kt_n = 0, emax_n = 0, emin_n = 0;  // tile of the next step
-      entry(0, kt_c, emax_c, emin_c);
-      issue_k(kt_c, 0, 0, group_needs_lim(kt_c, emin_c));
-      issue_v(kt_c, 0);
-      if (n_vis > 1) {
-        entry(1, kt_n, emax_n, emin_n);
-        issue_k(kt_n, 1, 1, group_needs_lim(kt_n, emin_n));
-      }
-      __builtin_amdgcn_s_waitcnt(0);
-      __syncthreads();
-      if (visits(kt_c, emax_c)) qk_tile(0, sacc);
-      __syncthreads();  // k[0] may be overwritten from here on
-
-      for (int j = 0; j < n_vis; ++j) {
-        if (j + 2 < n_vis) {
-          int kt2, emax2, emin2;
-          entry(j + 2, kt2, emax2, emin2);
-          issue_k(kt2, j & 1, (j + 2) & 3, group_needs_lim(kt2, emin2));
+      // One step handles two tiles of the list (2s, 2s + 1) between two workgroup barriers.  At its start the
+      // K tiles 2s + 1, 2s + 2 and the V tiles 2s, 2s + 1 are in LDS and the scores of tile 2s in registers; the
+      // step puts K tiles 2s + 3, 2s + 4 and V tiles 2s + 2, 2s + 3 in flight.
+      struct Entry {
+        int kt, emax, emin;
+      };
+      auto read_entry = [&](int j) {
+        Entry r = {0, 0, 0};
+        if (j < n_vis) {
+          int kt, emax, emin;
+          entry(j, kt, emax, emin);
+          r.kt = kt; r.emax = emax; r.emin = emin;
         }
-        if (j + 1 < n_vis) issue_v(kt_n, (j + 1) & 1);
-        const bool vis_c = visits(kt_c, emax_c);
-        // (uniform case: the last step computes scores of a stale tile that nobody reads, which keeps the
-        // step free of branches around the matrix instructions)
-        const bool vis_n = kUniform || (j + 1 < n_vis && visits(kt_n, emax_n));
+        return r;
+      };
+      auto load_k = [&](int j, const Entry& e) { if (j < n_vis) issue_k(e.kt, j & 3, j & 7, group_needs_lim(e.kt, e.emin)); };
+      auto load_v = [&](int j, const Entry& e) { if (j < n_vis) issue_v(e.kt, j & 3); };
+      // tile t: its scores (in sacc) become probabilities while the scores of tile t + 1 are computed, then O += P V
+      auto process_tile = [&](int t, const Entry& ec, const Entry& en) {
+        const bool vis_c = visits(ec.kt, ec.emax);
+        // (uniform case: the last tile computes scores of a stale tile that nobody reads, which keeps the step
+        // free of branches around the matrix instructions)
+        const bool vis_n = kUniform || (t + 1 < n_vis && visits(en.kt, en.emax));
         if (vis_c) {
           f32x16 sv[2] = {sacc[0], sacc[1]};
           // no masked score: every key row is at or before the first query and visible to the last one
-          const bool full = kt_c * kTile + kTile - 1 - a.base <= my_r0 && emin_c >= my_rlast;
-          if (!full) mask_scores(kt_c, j & 3, sv);
+          const bool full = ec.kt * kTile + kTile - 1 - a.base <= my_r0 && ec.emin >= my_rlast;
+          if (!full) mask_scores(ec.kt, t & 7, sv);
           const float mx = row_max(sv);
           if (__ballot(mx > m_run + kRescaleSlack)) rescale(mx);
           if (kUniform) {
-            fused_step((j + 1) & 1, j & 1, sv, sacc);
+            fused_step((t + 1) & 3, t & 3, sv, sacc);
           } else {
             // wavefronts with different query tiles: the same pipeline, its two halves one after the other
-            finish_tile(j & 1, sv);
-            if (vis_n) qk_tile((j + 1) & 1, sacc);
+            finish_tile(t & 3, sv);
+            if (vis_n) qk_tile((t + 1) & 3, sacc);
           }
         } else if (vis_n) {
-          qk_tile((j + 1) & 1, sacc);
+          qk_tile((t + 1) & 3, sacc);
         }
-        kt_c = kt_n; emax_c = emax_n; emin_c = emin_n;
-        if (j + 2 < n_vis) entry(j + 2, kt_n, emax_n, emin_n);
+      };
+
+      Entry e0 = read_entry(0), e1 = read_entry(1), e2 = read_entry(2);
+      load_k(0, e0);
+      load_v(0, e0);
+      load_k(1, e1);
+      load_v(1, e1);
+      load_k(2, e2);
+      __builtin_amdgcn_s_waitcnt(0);
+      __syncthreads();
+      if (visits(e0.kt, e0.emax)) qk_tile(0, sacc);
+      __syncthreads();  // k[0] is overwritten by the first step
+
+      for (int t = 0; t < n_vis; t += 2) {
+        const Entry e3 = read_entry(t + 3), e4 = read_entry(t + 4);
+        load_k(t + 3, e3);
+        load_k(t + 4, e4);
+        load_v(t + 2, e2);
+        load_v(t + 3, e3);
+        process_tile(t, e0, e1);
+        if (t + 1 < n_vis) process_tile(t + 1, e1, e2);
+        e0 = e2; e1 = e3; e2 = e4;
         __builtin_amdgcn_s_waitcnt(0);  // the tiles in flight have landed in LDS
         __syncthreads();                // ... for every wavefront, and the tiles of this step are no longer read
       }
