@@ -120,8 +120,7 @@ def role_step(x: torch.Tensor, weight: torch.Tensor, chunk_size: int, window: in
 
 def roles_from_one_hot(token_states_info: torch.Tensor) -> torch.Tensor:
     """[B, H_kv, S, 3] one-hot float -> uint8 roles (index of the 1)."""
-    t = token_states_info
-    return (t[..., 1] > 0).to(torch.uint8) + 2 * (t[..., 2] > 0).to(torch.uint8)
+    return token_states_info.argmax(-1).to(torch.uint8)
 
 
 def role_scan(roles: torch.Tensor, W: int, C: int):
