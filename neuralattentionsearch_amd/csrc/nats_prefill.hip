@@ -417,50 +417,44 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
     bf16x8 pb[4];
     int n = 0;
     __builtin_amdgcn_sched_barrier(0);
-    bf16x8 ka = k_frag(Kt, 0, 0);
+    // LDS operands are fetched two slots ahead of the MFMA that consumes them (rings of three fragments)
+    auto k_at = [&](int i) { return k_frag(Kt, i & 1, i >> 1); };   // i-th score MFMA: (kb, s) = (i & 1, i >> 1)
+    auto v_at = [&](int i) { return v_frag(Vt, i / DT, i % DT); };  // i-th PV MFMA: (t, dt) = (i / DT, i % DT)
+    bf16x8 kf[3], vf[3];
+    kf[0] = k_at(0);
+    kf[1] = k_at(1);
 #pragma unroll
-    for (int s = 0; s < DSTEPS; ++s) {
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb) {
-        const bf16x8 cur = ka;
-        if (kb == 0) {
-          ka = k_frag(Kt, 1, s);
-        } else if (s + 1 < DSTEPS) {
-          ka = k_frag(Kt, 0, s + 1);
-        }
-        if (s == 0) {
-          const f32x16 z = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-          sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cur, qreg[s], z, 0, 0, 0);
-        } else {
-          sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cur, qreg[s], sacc[kb], 0, 0, 0);
-        }
-        if (n < 16) {
-#pragma unroll
-          for (int e = 0; e < VA; ++e) prob(sv, n++, m_use, rs, pb);
-        }
-        __builtin_amdgcn_sched_barrier(0);
+    for (int i = 0; i < N_QK; ++i) {
+      const int s = i >> 1, kb = i & 1;
+      if (i + 2 < N_QK) {
+        kf[(i + 2) % 3] = k_at(i + 2);
+      } else {
+        vf[(i + 2 - N_QK) % 3] = v_at(i + 2 - N_QK);
       }
+      if (s == 0) {
+        const f32x16 z = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i % 3], qreg[s], z, 0, 0, 0);
+      } else {
+        sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i % 3], qreg[s], sacc[kb], 0, 0, 0);
+      }
+      if (n < 16) {
+#pragma unroll
+        for (int e = 0; e < VA; ++e) prob(sv, n++, m_use, rs, pb);
+      }
+      __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
     for (; n < 16;) prob(sv, n++, m_use, rs, pb);
-    bf16x8 va = v_frag(Vt, 0, 0);
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
+    for (int i = 0; i < N_PV; ++i) {
+      const int t = i / DT, dt = i % DT;
+      if (i + 2 < N_PV) vf[(i + 2) % 3] = v_at(i + 2);
+      oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[i % 3], pb[t], oacc[dt], 0, 0, 0);
+      if (t < 2) {
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        const bf16x8 cur = va;
-        if (dt + 1 < DT) {
-          va = v_frag(Vt, t, dt + 1);
-        } else if (t + 1 < 4) {
-          va = v_frag(Vt, t + 1, 0);
-        }
-        oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cur, pb[t], oacc[dt], 0, 0, 0);
-        if (t < 2) {
-#pragma unroll
-          for (int e = 0; e < VB; ++e) prob(sv, n++, m_use, rs, pb);
-        }
-        __builtin_amdgcn_sched_barrier(0);
+        for (int e = 0; e < VB; ++e) prob(sv, n++, m_use, rs, pb);
       }
+      __builtin_amdgcn_sched_barrier(0);
     }
     l_run += rs;
   };
