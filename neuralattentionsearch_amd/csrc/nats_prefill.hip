@@ -160,6 +160,16 @@ __global__ __launch_bounds__(64) void prefill_simple_kernel(PrefillArgs a) {
 // ---------------------------------------------------------------------------------------------------
 constexpr float kRescaleSlack = 8.0f;
 constexpr int kPrefillWaves = 8;
+
+// both halves of the wavefront get max / sum over lane and lane ^ 32 (one cross-half swap, no LDS round trip)
+__device__ __forceinline__ float half_swap_max(float v) {
+  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float half_swap_sum(float v) {
+  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
 constexpr int kWin = 1024;  // key tiles whose visit list is built at once
 
 template <int D>
@@ -363,7 +373,7 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
       for (int i = 0; i < 16; ++i) m = fmaxf(m, sv[kb][i]);
-    return fmaxf(m, __shfl_xor(m, 32)) * c;
+    return half_swap_max(m) * c;
   };
   // ---- raise the running maximum (rare): O and l shrink by 2^(old - new) ----------------------------
   auto rescale = [&](float mx) {
@@ -577,7 +587,7 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
   static_assert(kPrefillWaves * kHalf * kRowPitch <= sizeof(PrefillSmem<D>), "staging area fits the tile buffers");
   unsigned char* stage = smem_raw + wave * (kHalf * kRowPitch);
   {
-    const float l = l_run + __shfl_xor(l_run, 32);
+    const float l = half_swap_sum(l_run);
     const float inv = 1.f / l;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
