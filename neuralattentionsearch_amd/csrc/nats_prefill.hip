@@ -299,7 +299,7 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
       }
     }
   };
-  // K tile and the visibility limits of its rows; the limits go to slot (list index & 3)
+  // K tile and the visibility limits of its rows; the limits go to slot (list index & 7)
   auto issue_k = [&](int kt, int buf, int slot, bool need_lim) {
     issue_rows(kp, a.ks_l, koff, sm.k[buf], kt, false);
     if (need_lim && tid < kTile) {
@@ -414,7 +414,6 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
   //   phase A  score MFMAs of the next tile   + probabilities of keys  0..31 of this tile
   //   phase B  O += P V for keys 0..31        + probabilities of keys 32..63
   //   phase C  O += P V for keys 32..63
-  // LDS operands are fetched one slot ahead of the MFMA that consumes them.
   auto fused_step = [&](int kbuf_next, int vbuf, const f32x16 (&sv)[2], f32x16 (&sacc)[2]) {
     const uint16_t* Kt = sm.k[kbuf_next];
     const uint16_t* Vt = sm.v[vbuf];
@@ -500,9 +499,9 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
     const int n_vis = __builtin_amdgcn_readfirstlane(sm.vcount);
     if (n_vis > 0) {
       // The list entries are the same for every lane: they are kept in scalar registers.
-      // Step j of the pipeline: loads of K tile j+2 and V tile j+1 are put in flight; the matrix pipe computes
-      // the scores of tile j+1 while the vector ALU turns those of tile j into probabilities; then O += P V
-      // for tile j.  Buffers: K tile j in k[j & 1], V tile j in v[j & 1], row limits of tile j in limk[j & 3].
+      // Tile j of the list: the matrix pipe computes the scores of tile j+1 while the vector ALU turns those of
+      // tile j into probabilities; then O += P V for tile j.  Buffers: K tile j in k[j & 3], V tile j in
+      // v[j & 3], row limits of tile j in limk[j & 7].
       auto entry = [&](int j, int& kt, int& emax, int& emin) {
         const int4 e = sm.vlist[j];
         kt = __builtin_amdgcn_readfirstlane(e.x);
