@@ -286,7 +286,7 @@ def bench_llama(args):
             "shape": dict(layers=cfg.num_hidden_layers, d_model=cfg.hidden_size, heads="32/8", head_dim=cfg.head_dim,
                           ffn=cfg.intermediate_size, vocab=cfg.vocab_size, prefill=args.llama_prefill,
                           decode_steps=args.llama_decode, chunk=cfg.chunk_size, window=cfg.local_seq_max_length),
-            "note": "random weights give near-uniform roles; projections / MLP / norms are library GEMMs and torch ops"}
+            "note": "random weights give near-uniform roles; projections are library GEMMs; one-token steps use the fused norm / rotary + append / gate kernels"}
 
 
 # --------------------------------------------------------------------------------------------------

@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define NATS_ABI_VERSION 2
+#define NATS_ABI_VERSION 3
 
 typedef enum {
   NATS_OK = 0,
@@ -257,6 +257,43 @@ int nats_evict_apply_first(const void* src_k, const void* src_v, void* cache_k, 
                            const nats_evict_params* params, const int64_t* src_strides, const int64_t* kv_strides,
                            const int64_t* valid_strides, int elem_bytes, const void* workspace,
                            const nats_evict_result* result, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Decode-step glue of the HF-shaped caller (models/transformer/hf/llama_nats_chunk.py:171-292 inside a Llama
+ * decoder layer): the elementwise work around the attention, fused so that a layer costs a dozen launches.
+ * Each entry point keeps the rounding points of the torch ops it replaces.
+ */
+
+/* x += delta (optional); out = RMSNorm(x) * weight, normalised in fp32, cast to the dtype, then multiplied
+ * (models/transformer/components.py:14-26, the HF LlamaRMSNorm form).  Optionally also the running chunk
+ * statistic of the role step for an open chunk (NAtSCache.merge_new_x_values_in_chunk,
+ * components/cache/dyn_cache.py:98-124, called from hf/llama_nats_chunk.py:198) from the normalised row:
+ *   carry_mode 0 none; 1 carry = out / chunk_size; 2 carry += out / chunk_size; 3 carry = out; 4 carry = max(carry, out)
+ *   x [rows, dim] in / out, delta [rows, dim] or NULL, weight [dim], out [rows, dim], carry [rows, dim] or NULL;
+ *   all contiguous, dim <= 8192
+ */
+int nats_add_rms_norm(void* x, const void* delta, const void* weight, void* out, void* carry, int64_t rows,
+                      int64_t dim, float eps, int carry_mode, int64_t chunk_size, int dtype, void* stream);
+
+/* out[r, c] = silu(gate_up[r, c]) * gate_up[r, inter + c]: act_fn(gate_proj(x)) * up_proj(x) of the Llama MLP
+ * with the two projections stored as one matrix.  gate_up [rows, 2 * inter], out [rows, inter], contiguous.
+ */
+int nats_silu_mul(const void* gate_up, void* out, int64_t rows, int64_t inter, int dtype, void* stream);
+
+/* Rotary embedding of q and k (transformers' apply_rotary_pos_emb, hf/llama_nats_chunk.py:227) and the row
+ * write of NAtSChunkLayerCache.update (components/cache/nats_chunk_layer_cache.py:243-256) in one launch:
+ *   q_out[b, h, l]            = rope(q[b, h, l])            [B, H_q, x_len, D] contiguous
+ *   cache_k[b, h, row0 + l]   = rope(k[b, h, l]),  cache_v[b, h, row0 + l] = v[b, h, l]
+ *   valid[b, h, row0 + l] = 1, pos[b, h, row0 + l] = pos0 + l (pos may be NULL)
+ *   q [B, H_q, x_len, D], k / v [B, H_kv, x_len, D]: strides (b, h, l), last dimension contiguous
+ *   cos / sin [B, x_len, D]: strides (b, l);  cache_k / cache_v [B, H_kv, n_alloc, D]: strides (b, h, row)
+ *   valid / pos [B, H_kv, n_alloc]: strides (b, h)
+ */
+int nats_rope_append(const void* q, const void* k, const void* v, const void* cos, const void* sin, void* q_out,
+                     void* cache_k, void* cache_v, uint8_t* valid, int32_t* pos, int64_t B, int64_t H_q, int64_t H_kv,
+                     int64_t x_len, int64_t D, int64_t row0, int64_t n_alloc, int64_t pos0, const int64_t* q_strides,
+                     const int64_t* k_strides, const int64_t* v_strides, const int64_t* cos_strides,
+                     const int64_t* cache_strides, const int64_t* valid_strides, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

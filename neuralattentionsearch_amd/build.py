@@ -7,7 +7,7 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 INCLUDE = os.path.join(os.path.dirname(PKG_DIR), "include")
 LIB_PATH = os.path.join(PKG_DIR, "libnats_hip.so")
-SOURCES = ["nats_roles.hip", "nats_rolestep.hip", "nats_prefill.hip", "nats_decode.hip", "nats_evict.hip"]
+SOURCES = ["nats_roles.hip", "nats_rolestep.hip", "nats_prefill.hip", "nats_decode.hip", "nats_evict.hip", "nats_glue.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",

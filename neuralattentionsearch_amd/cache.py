@@ -169,18 +169,26 @@ class NAtSChunkLayerCache:
             self._buf_pos[:, :, W:W + x_len] = torch.arange(x_len, dtype=torch.int32, device=k.device)
 
     # -- append (nats_chunk_layer_cache.py:171-256) ----------------------------------------------
-    def update(self, key_states: torch.Tensor, value_states: torch.Tensor, token_states_info: torch.Tensor | None):
+    def _note_roles(self, token_states_info, roles):
+        self._tokens_info = token_states_info
+        if roles is not None:
+            self._roles = roles.contiguous()
+        else:
+            self._roles = None if token_states_info is None else ops.roles_from_one_hot(token_states_info).contiguous()
+
+    def update(self, key_states: torch.Tensor, value_states: torch.Tensor, token_states_info: torch.Tensor | None,
+               roles: torch.Tensor | None = None):
+        """`roles` (uint8 [B, H, S]) may be handed over beside the one-hot tensor by a caller that has them already."""
         if not key_states.is_cuda:
             raise ValueError("NAtSChunkLayerCache.update takes GPU tensors")
         x_len = key_states.shape[2]
         self.chunk_fill_size += x_len
-        if token_states_info is None:
+        if token_states_info is None and roles is None:
             assert self.chunk_fill_size < self.chunk_size, \
                 "a new token_states_info must be generated once the open chunk is full"
         if x_len == 0:
             return self.cache_k[:, :, :self.n_ctx_data], self.cache_v[:, :, :self.n_ctx_data]
-        self._tokens_info = token_states_info
-        self._roles = None if token_states_info is None else ops.roles_from_one_hot(token_states_info).contiguous()
+        self._note_roles(token_states_info, roles)
         if self._buf_k is None and self._pending is None:
             self._pending = (key_states, value_states)
             if self.chunk_fill_size < self.chunk_size:
@@ -197,6 +205,28 @@ class NAtSChunkLayerCache:
             self._buf_pos[:, :, start:end] = torch.arange(self._seen_tokens, self._seen_tokens + x_len,
                                                           dtype=torch.int32, device=self.device)
         return self._buf_k[:, :, :end], self._buf_v[:, :, :end]
+
+    def append_rotated(self, q: torch.Tensor, key_states: torch.Tensor, value_states: torch.Tensor, cos: torch.Tensor,
+                       sin: torch.Tensor, token_states_info: torch.Tensor | None = None,
+                       roles: torch.Tensor | None = None):
+        """`update` for a cache that already holds rows, with the rotary embedding of q and k applied on the way
+        (one kernel: hf/llama_nats_chunk.py:227 + nats_chunk_layer_cache.py:243-256).  q / k / v are the projections
+        before the rotary embedding; returns (rotated q, keys, values)."""
+        if self._buf_k is None and self._pending is None:
+            raise ValueError("append_rotated needs a cache that holds rows; the first segment goes through update")
+        x_len = key_states.shape[2]
+        self.chunk_fill_size += x_len
+        if token_states_info is None and roles is None:
+            assert self.chunk_fill_size < self.chunk_size, \
+                "roles must be generated once the open chunk is full"
+        self._note_roles(token_states_info, roles)
+        self._materialize_pending()
+        start = self.n_ctx_data
+        end = start + x_len
+        self._grow(math.ceil(end / self.chunk_size) * self.chunk_size)
+        q_rot = ops.rope_append(q, key_states, value_states, cos, sin, self._buf_k, self._buf_v, self._buf_valid,
+                                self._buf_pos, start, self._seen_tokens)
+        return q_rot, self._buf_k[:, :, :end], self._buf_v[:, :, :end]
 
     # -- masks (nats_chunk_layer_cache.py:156-163, 444-460, 622-632) ------------------------------
     def generate_mask(self, x_len: int):

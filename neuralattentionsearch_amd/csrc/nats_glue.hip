@@ -1,0 +1,299 @@
+// Small fused kernels around the attention of a decode step, so that a decoder layer of the HF-shaped caller
+// costs a dozen launches instead of fifty: residual add + RMSNorm (+ the running chunk statistic of the role
+// step), rotary embedding + cache append, SiLU gate.
+//
+// Each follows the rounding points of the torch ops the reference runs, so that in bf16 the results equal those
+// ops element for element wherever the arithmetic is elementwise:
+//   * RMSNorm: models/transformer/components.py:14-26 (the HF LlamaRMSNorm form: normalise in fp32, cast to the
+//     input dtype, then multiply by the weight in that dtype); the mean of squares is an fp32 reduction whose
+//     order differs from the library's.
+//   * running chunk statistic: NAtSCache.merge_new_x_values_in_chunk (components/cache/dyn_cache.py:98-115),
+//     called for an open chunk by update_nats_cached_x_in_chunk (:117-124) from hf/llama_nats_chunk.py:198.
+//   * rotary embedding: transformers' apply_rotary_pos_emb as imported by hf/llama_nats_chunk.py:7 and called at
+//     :227 (q * cos + rotate_half(q) * sin, every product and the sum rounded to the dtype), followed by the
+//     row write of NAtSChunkLayerCache.update (components/cache/nats_chunk_layer_cache.py:243-256).
+//   * SiLU gate: act_fn(gate_proj(x)) * up_proj(x) of the HF Llama MLP the reference keeps unchanged.
+#include "nats_common.h"
+
+namespace nats {
+
+template <bool kBf16>
+__device__ __forceinline__ float g_load(const void* p, int64_t i) {
+  if (kBf16) return bf16_bits_to_f32(static_cast<const uint16_t*>(p)[i]);
+  return static_cast<const float*>(p)[i];
+}
+template <bool kBf16>
+__device__ __forceinline__ float g_round(float v) {
+  return kBf16 ? bf16_bits_to_f32(f32_to_bf16_bits(v)) : v;
+}
+template <bool kBf16>
+__device__ __forceinline__ void g_store(void* p, int64_t i, float v) {
+  if (kBf16) {
+    static_cast<uint16_t*>(p)[i] = f32_to_bf16_bits(v);
+  } else {
+    static_cast<float*>(p)[i] = v;
+  }
+}
+
+struct AddNormArgs {
+  void* x;            // [rows, dim] in / out (x += delta)
+  const void* delta;  // [rows, dim] or null
+  const void* weight; // [dim]
+  void* out;          // [rows, dim]
+  void* carry;        // [rows, dim] or null
+  int dim;
+  int carry_mode;     // 0 none, 1 mean (first token of the chunk), 2 mean (later token), 3 max (first), 4 max (later)
+  float eps, chunk;
+};
+
+// One workgroup of 256 threads per row; the row is kept in registers between the two passes.  VEC consecutive
+// columns per thread and step: 8 (16-byte loads of bf16, two 16-byte loads of fp32) when dim % 8 == 0, else 1.
+constexpr int kNormThreads = 256;
+constexpr int kNormMaxDim = 8192;
+
+template <bool kBf16, int VEC>
+__device__ __forceinline__ void load_vec(const void* p, int64_t i, float (&v)[VEC]) {
+  if (VEC == 8 && kBf16) {
+    const uint4 u = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(p) + i);
+    const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      v[2 * e] = __uint_as_float(w[e] << 16);
+      v[2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
+    }
+  } else if (VEC == 8) {
+    const float4 a = *reinterpret_cast<const float4*>(static_cast<const float*>(p) + i);
+    const float4 b = *reinterpret_cast<const float4*>(static_cast<const float*>(p) + i + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+  } else {
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) v[e] = g_load<kBf16>(p, i + e);
+  }
+}
+template <bool kBf16, int VEC>
+__device__ __forceinline__ void store_vec(void* p, int64_t i, const float (&v)[VEC]) {
+  if (VEC == 8 && kBf16) {
+    uint32_t w[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) w[e] = uint32_t(f32_to_bf16_bits(v[2 * e])) | (uint32_t(f32_to_bf16_bits(v[2 * e + 1])) << 16);
+    *reinterpret_cast<uint4*>(static_cast<uint16_t*>(p) + i) = make_uint4(w[0], w[1], w[2], w[3]);
+  } else if (VEC == 8) {
+    *reinterpret_cast<float4*>(static_cast<float*>(p) + i) = make_float4(v[0], v[1], v[2], v[3]);
+    *reinterpret_cast<float4*>(static_cast<float*>(p) + i + 4) = make_float4(v[4], v[5], v[6], v[7]);
+  } else {
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) g_store<kBf16>(p, i + e, v[e]);
+  }
+}
+
+template <bool kBf16, int VEC>
+__global__ __launch_bounds__(kNormThreads) void add_rms_norm_kernel(AddNormArgs a) {
+  constexpr int STEPS = kNormMaxDim / (kNormThreads * VEC);
+  __shared__ float part[kNormThreads / kWave];
+  const int64_t base = (int64_t)blockIdx.x * a.dim;
+  const int tid = threadIdx.x;
+  float v[STEPS][VEC];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < STEPS; ++j) {
+    const int c = (j * kNormThreads + tid) * VEC;
+    if (c < a.dim) {
+      load_vec<kBf16, VEC>(a.x, base + c, v[j]);
+      if (a.delta) {
+        float d[VEC];
+        load_vec<kBf16, VEC>(a.delta, base + c, d);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) v[j][e] = g_round<kBf16>(v[j][e] + d[e]);
+        store_vec<kBf16, VEC>(a.x, base + c, v[j]);
+      }
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) ss += v[j][e] * v[j][e];
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+  if ((tid & 63) == 0) part[tid >> 6] = ss;
+  __syncthreads();
+  float tot = 0.f;
+#pragma unroll
+  for (int w = 0; w < kNormThreads / kWave; ++w) tot += part[w];
+  const float r = rsqrtf(tot / (float)a.dim + a.eps);
+#pragma unroll
+  for (int j = 0; j < STEPS; ++j) {
+    const int c = (j * kNormThreads + tid) * VEC;
+    if (c < a.dim) {
+      float w[VEC], h[VEC];
+      load_vec<kBf16, VEC>(a.weight, c, w);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) h[e] = g_round<kBf16>(g_round<kBf16>(v[j][e] * r) * w[e]);
+      store_vec<kBf16, VEC>(a.out, base + c, h);
+      if (a.carry_mode) {
+        float cv[VEC];
+        if (a.carry_mode == 2 || a.carry_mode == 4) load_vec<kBf16, VEC>(a.carry, base + c, cv);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          if (a.carry_mode <= 2) {
+            const float add = g_round<kBf16>(h[e] / a.chunk);
+            cv[e] = a.carry_mode == 1 ? add : g_round<kBf16>(cv[e] + add);
+          } else {
+            cv[e] = a.carry_mode == 3 ? h[e] : fmaxf(cv[e], h[e]);
+          }
+        }
+        store_vec<kBf16, VEC>(a.carry, base + c, cv);
+      }
+    }
+  }
+}
+
+template <bool kBf16>
+__global__ __launch_bounds__(256) void silu_mul_kernel(const void* __restrict__ gate_up, void* __restrict__ out, int64_t rows,
+                                                        int inter) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= rows * inter) return;
+  const int64_t r = i / inter;
+  const int c = (int)(i - r * inter);
+  const float g = g_load<kBf16>(gate_up, r * 2 * inter + c);
+  const float u = g_load<kBf16>(gate_up, r * 2 * inter + inter + c);
+  const float s = g_round<kBf16>(g / (1.f + expf(-g)));
+  g_store<kBf16>(out, i, s * u);
+}
+
+struct RopeAppendArgs {
+  const void *q, *k, *v, *cos, *sin;
+  void *q_out, *cache_k, *cache_v;
+  uint8_t* valid;
+  int32_t* pos;
+  int64_t qs[3], ks[3], vs[3];  // strides (b, h, l) of q, k, v; last dim contiguous
+  int64_t cs[2];                // strides (b, l) of cos / sin
+  int64_t cache_s[3];           // strides (b, h, row) of cache_k / cache_v
+  int64_t valid_s[2];           // strides (b, h) of valid / pos
+  int Hq, Hkv, x_len, D;
+  int64_t row0;
+  int pos0;
+};
+
+// grid (x_len, Hq + 2 * Hkv, B); one thread per element of the head vector (D <= 256)
+template <bool kBf16>
+__global__ void rope_append_kernel(RopeAppendArgs a) {
+#pragma clang fp contract(off)  // the two products and their sum round separately, as the torch ops do (fp32 too)
+  const int l = blockIdx.x, hh = blockIdx.y, b = blockIdx.z;
+  const int d = threadIdx.x;
+  if (d >= a.D) return;
+  const int half = a.D / 2;
+  const int64_t cidx = b * a.cs[0] + l * a.cs[1];
+  if (hh < a.Hq + a.Hkv) {
+    const bool is_q = hh < a.Hq;
+    const int h = is_q ? hh : hh - a.Hq;
+    const void* src = is_q ? a.q : a.k;
+    const int64_t* st = is_q ? a.qs : a.ks;
+    const int64_t s0 = b * st[0] + h * st[1] + l * st[2];
+    const float x = g_load<kBf16>(src, s0 + d);
+    const float xr = d < half ? -g_load<kBf16>(src, s0 + d + half) : g_load<kBf16>(src, s0 + d - half);
+    const float p1 = g_round<kBf16>(x * g_load<kBf16>(a.cos, cidx + d));
+    const float p2 = g_round<kBf16>(xr * g_load<kBf16>(a.sin, cidx + d));
+    const float y = p1 + p2;
+    if (is_q) {
+      g_store<kBf16>(a.q_out, (((int64_t)b * a.Hq + h) * a.x_len + l) * a.D + d, y);
+    } else {
+      g_store<kBf16>(a.cache_k, b * a.cache_s[0] + h * a.cache_s[1] + (a.row0 + l) * a.cache_s[2] + d, y);
+      if (d == 0) {
+        a.valid[b * a.valid_s[0] + h * a.valid_s[1] + a.row0 + l] = 1;
+        if (a.pos) a.pos[b * a.valid_s[0] + h * a.valid_s[1] + a.row0 + l] = a.pos0 + l;
+      }
+    }
+  } else {
+    const int h = hh - a.Hq - a.Hkv;
+    const float x = g_load<kBf16>(a.v, b * a.vs[0] + h * a.vs[1] + l * a.vs[2] + d);
+    g_store<kBf16>(a.cache_v, b * a.cache_s[0] + h * a.cache_s[1] + (a.row0 + l) * a.cache_s[2] + d, x);
+  }
+}
+
+}  // namespace nats
+
+using namespace nats;
+
+extern "C" int nats_add_rms_norm(void* x, const void* delta, const void* weight, void* out, void* carry, int64_t rows,
+                                 int64_t dim, float eps, int carry_mode, int64_t chunk_size, int dtype, void* stream) {
+  NATS_REQUIRE(x && weight && out, NATS_ERR_NULL_POINTER, "nats_add_rms_norm: NULL pointer");
+  NATS_REQUIRE(rows > 0 && dim > 0 && dim <= kNormMaxDim && rows <= 0x7fffffff, NATS_ERR_BAD_SHAPE,
+               "nats_add_rms_norm: rows=%lld dim=%lld (dim <= %d)", (long long)rows, (long long)dim, kNormMaxDim);
+  NATS_REQUIRE(dtype == NATS_DTYPE_BF16 || dtype == NATS_DTYPE_F32, NATS_ERR_BAD_DTYPE, "nats_add_rms_norm: dtype %d", dtype);
+  NATS_REQUIRE(carry_mode >= 0 && carry_mode <= 4 && (carry_mode == 0 || (carry && chunk_size > 0)), NATS_ERR_BAD_SHAPE,
+               "nats_add_rms_norm: carry_mode %d needs a carry buffer and a chunk size", carry_mode);
+  AddNormArgs a{x, delta, weight, out, carry, (int)dim, carry_mode, eps, (float)chunk_size};
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  auto aligned16 = [](const void* p) { return p == nullptr || reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+  const bool vec = dim % 8 == 0 && aligned16(x) && aligned16(delta) && aligned16(weight) && aligned16(out) && aligned16(carry);
+  const dim3 grid((unsigned)rows), block(kNormThreads);
+  if (dtype == NATS_DTYPE_BF16) {
+    if (vec) {
+      hipLaunchKernelGGL((add_rms_norm_kernel<true, 8>), grid, block, 0, st, a);
+    } else {
+      hipLaunchKernelGGL((add_rms_norm_kernel<true, 1>), grid, block, 0, st, a);
+    }
+  } else {
+    if (vec) {
+      hipLaunchKernelGGL((add_rms_norm_kernel<false, 8>), grid, block, 0, st, a);
+    } else {
+      hipLaunchKernelGGL((add_rms_norm_kernel<false, 1>), grid, block, 0, st, a);
+    }
+  }
+  NATS_CHECK_LAUNCH("add_rms_norm_kernel");
+  return NATS_OK;
+}
+
+extern "C" int nats_silu_mul(const void* gate_up, void* out, int64_t rows, int64_t inter, int dtype, void* stream) {
+  NATS_REQUIRE(gate_up && out, NATS_ERR_NULL_POINTER, "nats_silu_mul: NULL pointer");
+  NATS_REQUIRE(rows > 0 && inter > 0 && inter <= 0x3fffffff && rows * inter <= (int64_t)0x7fffffff * 256, NATS_ERR_BAD_SHAPE,
+               "nats_silu_mul: rows=%lld inter=%lld", (long long)rows, (long long)inter);
+  NATS_REQUIRE(dtype == NATS_DTYPE_BF16 || dtype == NATS_DTYPE_F32, NATS_ERR_BAD_DTYPE, "nats_silu_mul: dtype %d", dtype);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const unsigned blocks = (unsigned)((rows * inter + 255) / 256);
+  if (dtype == NATS_DTYPE_BF16) {
+    hipLaunchKernelGGL(silu_mul_kernel<true>, dim3(blocks), dim3(256), 0, st, gate_up, out, rows, (int)inter);
+  } else {
+    hipLaunchKernelGGL(silu_mul_kernel<false>, dim3(blocks), dim3(256), 0, st, gate_up, out, rows, (int)inter);
+  }
+  NATS_CHECK_LAUNCH("silu_mul_kernel");
+  return NATS_OK;
+}
+
+extern "C" int nats_rope_append(const void* q, const void* k, const void* v, const void* cos, const void* sin, void* q_out,
+                                void* cache_k, void* cache_v, uint8_t* valid, int32_t* pos, int64_t B, int64_t H_q,
+                                int64_t H_kv, int64_t x_len, int64_t D, int64_t row0, int64_t n_alloc, int64_t pos0,
+                                const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                                const int64_t* cos_strides, const int64_t* cache_strides, const int64_t* valid_strides,
+                                int dtype, void* stream) {
+  NATS_REQUIRE(q && k && v && cos && sin && q_out && cache_k && cache_v && valid, NATS_ERR_NULL_POINTER,
+               "nats_rope_append: NULL pointer");
+  NATS_REQUIRE(q_strides && k_strides && v_strides && cos_strides && cache_strides && valid_strides, NATS_ERR_NULL_POINTER,
+               "nats_rope_append: NULL stride array");
+  NATS_REQUIRE(B > 0 && H_q > 0 && H_kv > 0 && x_len > 0 && B <= 65535 && H_q + 2 * H_kv <= 65535, NATS_ERR_BAD_SHAPE,
+               "nats_rope_append: B=%lld H_q=%lld H_kv=%lld x_len=%lld", (long long)B, (long long)H_q, (long long)H_kv,
+               (long long)x_len);
+  NATS_REQUIRE(D > 0 && D % 2 == 0 && D <= 256, NATS_ERR_UNSUPPORTED, "nats_rope_append: head_dim %lld", (long long)D);
+  NATS_REQUIRE(row0 >= 0 && row0 + x_len <= n_alloc, NATS_ERR_BAD_SHAPE, "nats_rope_append: rows [%lld, %lld) of %lld",
+               (long long)row0, (long long)(row0 + x_len), (long long)n_alloc);
+  NATS_REQUIRE(dtype == NATS_DTYPE_BF16 || dtype == NATS_DTYPE_F32, NATS_ERR_BAD_DTYPE, "nats_rope_append: dtype %d", dtype);
+  RopeAppendArgs a{};
+  a.q = q; a.k = k; a.v = v; a.cos = cos; a.sin = sin;
+  a.q_out = q_out; a.cache_k = cache_k; a.cache_v = cache_v; a.valid = valid; a.pos = pos;
+  for (int i = 0; i < 3; ++i) {
+    a.qs[i] = q_strides[i]; a.ks[i] = k_strides[i]; a.vs[i] = v_strides[i]; a.cache_s[i] = cache_strides[i];
+  }
+  for (int i = 0; i < 2; ++i) {
+    a.cs[i] = cos_strides[i]; a.valid_s[i] = valid_strides[i];
+  }
+  a.Hq = (int)H_q; a.Hkv = (int)H_kv; a.x_len = (int)x_len; a.D = (int)D;
+  a.row0 = row0; a.pos0 = (int)pos0;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  dim3 grid((unsigned)x_len, (unsigned)(H_q + 2 * H_kv), (unsigned)B);
+  const unsigned threads = (unsigned)((D + 63) / 64 * 64);
+  if (dtype == NATS_DTYPE_BF16) {
+    hipLaunchKernelGGL(rope_append_kernel<true>, grid, dim3(threads), 0, st, a);
+  } else {
+    hipLaunchKernelGGL(rope_append_kernel<false>, grid, dim3(threads), 0, st, a);
+  }
+  NATS_CHECK_LAUNCH("rope_append_kernel");
+  return NATS_OK;
+}

@@ -10,6 +10,11 @@ Differences from BaseNAtSChunkAttentionLayer that this twin has and that are kep
 logit (:206-214 takes the plain maximum) and `position_ids[0, 0] == 0` decides between the prefill kernel
 and the cached paths (:194, :238-270).
 
+One-token steps take a shorter route through the same arithmetic (`fused_decode`): q / k / v and gate / up are
+one GEMM each over merged weights (the separate `*_proj.weight` parameters are views of them), the residual add,
+RMSNorm and the running chunk statistic are one kernel, the rotary embedding and the cache append another, the
+SiLU gate a third, so that a decoder layer is about a dozen launches.
+
 Weights are random-initialised (there is no checkpoint loader here); `NAtSLlamaConfig.llama3_8b()` gives the
 Llama-3-8B shape.
 """
@@ -40,6 +45,7 @@ class NAtSLlamaConfig:
     local_seq_max_length: int = 256  # sliding window, in tokens
     chunk_merge_method: str = "mean"
     fused_role_step: bool = False  # pooling + role projection + argmax in one kernel instead of torch ops
+    fused_decode: bool = True      # one-token steps: fused norm / rotary + append / gate kernels, merged projections
 
     @property
     def head_dim(self) -> int:
@@ -68,9 +74,27 @@ class LlamaMLP(nn.Module):
         self.gate_proj = nn.Linear(cfg.hidden_size, cfg.intermediate_size, bias=False)
         self.up_proj = nn.Linear(cfg.hidden_size, cfg.intermediate_size, bias=False)
         self.down_proj = nn.Linear(cfg.intermediate_size, cfg.hidden_size, bias=False)
+        self.gate_up_weight = None
+
+    def fuse(self):
+        """gate_proj / up_proj weights become views of one [2 * I, hidden] matrix."""
+        w = torch.cat([self.gate_proj.weight.data, self.up_proj.weight.data], dim=0)
+        n = self.gate_proj.weight.shape[0]
+        self.gate_proj.weight = nn.Parameter(w[:n], requires_grad=False)
+        self.up_proj.weight = nn.Parameter(w[n:], requires_grad=False)
+        self.gate_up_weight = w
+
+    def fused_ok(self):
+        w = self.gate_up_weight
+        return w is not None and w.data_ptr() == self.gate_proj.weight.data_ptr() and w.dtype == self.gate_proj.weight.dtype
 
     def forward(self, x):
         return self.down_proj(nn.functional.silu(self.gate_proj(x)) * self.up_proj(x))
+
+    def forward_fused(self, x):
+        if not self.fused_ok():
+            self.fuse()
+        return self.down_proj(ops.silu_mul(nn.functional.linear(x, self.gate_up_weight)))
 
 
 def rotary_tables(position_ids: torch.Tensor, head_dim: int, theta: float, dtype: torch.dtype):
@@ -103,10 +127,65 @@ class NAtSLlamaAttention(nn.Module):
         self.o_proj = nn.Linear(self.num_heads * self.head_dim, cfg.hidden_size, bias=False)
         self.proj_layer = nn.Linear(cfg.hidden_size, self.num_key_value_heads * 3, bias=False)  # :315-318
         self.fused_role_step = cfg.fused_role_step
+        self.qkv_weight = None
 
-    def forward(self, hidden_states: torch.Tensor, position_embeddings, start_pos: int, past_key_value: NAtSCache):
+    def fuse(self):
+        """q_proj / k_proj / v_proj weights become views of one [(H_q + 2 H_kv) * D, hidden] matrix."""
+        w = torch.cat([self.q_proj.weight.data, self.k_proj.weight.data, self.v_proj.weight.data], dim=0)
+        nq, nk = self.q_proj.weight.shape[0], self.k_proj.weight.shape[0]
+        self.q_proj.weight = nn.Parameter(w[:nq], requires_grad=False)
+        self.k_proj.weight = nn.Parameter(w[nq:nq + nk], requires_grad=False)
+        self.v_proj.weight = nn.Parameter(w[nq + nk:], requires_grad=False)
+        self.qkv_weight = w
+
+    def fused_ok(self):
+        w = self.qkv_weight
+        return w is not None and w.data_ptr() == self.q_proj.weight.data_ptr() and w.dtype == self.q_proj.weight.dtype
+
+    def _decode_one(self, hidden_states, position_embeddings, start_pos: int, past_key_value: NAtSCache,
+                    statistic_done: bool):
+        """One token over a cache that holds rows: the same steps as `forward`, with one GEMM for q / k / v and the
+        rotary embedding fused with the cache append.  `statistic_done`: the caller's norm kernel has already
+        merged this token into the running chunk statistic."""
+        bsz = hidden_states.shape[0]
+        C, idx = self.chunk_size, self.layer_idx
+        Hq, Hkv, D = self.num_heads, self.num_key_value_heads, self.head_dim
+        if not self.fused_ok():
+            self.fuse()
+        qkv = nn.functional.linear(hidden_states, self.qkv_weight).view(bsz, 1, Hq + 2 * Hkv, D).transpose(1, 2)
+        q, k, v = qkv[:, :Hq], qkv[:, Hq:Hq + Hkv], qkv[:, Hq + Hkv:]
+        pre_fill = past_key_value.get_nats_chunk_fill_size(idx)
+        roles = tsi = None
+        if pre_fill + 1 < C:
+            if not statistic_done:
+                past_key_value.update_nats_cached_x_in_chunk(hidden_states, idx, self.chunk_merge_method)
+        elif self.fused_role_step:
+            step = ops.role_step(hidden_states, self.proj_layer.weight, C, self.local_seq_max_length, pre_fill=pre_fill,
+                                 carry_in=past_key_value.get_nats_cached_x_in_chunk(idx) if pre_fill else None,
+                                 merge_max=self.chunk_merge_method == ChunkMergeType.MAX, global_bias=0.0,
+                                 force_first_global=start_pos < C)
+            past_key_value._update_cache_x(step["carry"], idx)
+            roles, tsi = step["roles"], step["token_states_info"]
+        else:
+            pooled, pad = past_key_value.update_nats_cached_x_across_chunk(hidden_states, pre_fill, idx,
+                                                                           self.chunk_merge_method)
+            logit = self.proj_layer(pooled).unflatten(-1, (Hkv, 3))
+            roles, tsi = ops.roles_from_logits(logit, 0.0, force_first_global=start_pos < C, force_last_global=pad != 0)
+        layer = past_key_value.cache_model[idx]
+        cos, sin = position_embeddings
+        q, keys, values = layer.append_rotated(q, k, v, cos, sin, tsi, roles)
+        out = ops.decode_attention(q, keys, values, layer.valid_tokens, keys.shape[2], 1.0 / math.sqrt(D),
+                                   row_end=layer.size_global_kv + layer.size_local_kv,
+                                   tail_start=layer.n_ctx_data - (layer.chunk_fill_size - 1))
+        past_key_value.post_update(layer_idx=idx, x_len=1)
+        return self.o_proj(out.transpose(1, 2).reshape(bsz, 1, -1))
+
+    def forward(self, hidden_states: torch.Tensor, position_embeddings, start_pos: int, past_key_value: NAtSCache,
+                fused_decode: bool = False, statistic_done: bool = False):
         bsz, q_len, _ = hidden_states.shape
         C, idx = self.chunk_size, self.layer_idx
+        if fused_decode:
+            return self._decode_one(hidden_states, position_embeddings, start_pos, past_key_value, statistic_done)
         q = self.q_proj(hidden_states).view(bsz, q_len, self.num_heads, self.head_dim).transpose(1, 2)
         k = self.k_proj(hidden_states).view(bsz, q_len, self.num_key_value_heads, self.head_dim).transpose(1, 2)
         v = self.v_proj(hidden_states).view(bsz, q_len, self.num_key_value_heads, self.head_dim).transpose(1, 2)
@@ -164,6 +243,29 @@ class NAtSLlamaDecoderLayer(nn.Module):
         x = x + self.self_attn(self.input_layernorm(x), position_embeddings, start_pos, cache)
         return x + self.mlp(self.post_attention_layernorm(x))
 
+    def decode_step(self, x, delta, position_embeddings, start_pos: int, cache: NAtSCache):
+        """One token.  `x` [B, 1, dim] is the residual stream, updated in place; `delta` is the branch output of the
+        previous layer that has not been added yet (None for the first layer).  Returns this layer's MLP output,
+        to be added by whoever normalises next."""
+        attn = self.self_attn
+        idx, C = attn.layer_idx, attn.chunk_size
+        pre_fill = cache.get_nats_chunk_fill_size(idx)
+        carry, mode = None, ops.CARRY_NONE
+        if pre_fill + 1 < C:  # the chunk stays open: its running statistic takes this token in (dyn_cache.py:117-124)
+            carry = cache.get_nats_cached_x_in_chunk(idx)
+            is_max = attn.chunk_merge_method == ChunkMergeType.MAX
+            if carry is None:
+                carry = torch.empty_like(x)
+                mode = ops.CARRY_MAX_FIRST if is_max else ops.CARRY_MEAN_FIRST
+            else:
+                mode = ops.CARRY_MAX_MERGE if is_max else ops.CARRY_MEAN_ADD
+        h = ops.add_rms_norm(x, delta, self.input_layernorm.weight, self.input_layernorm.eps, carry, mode, C)
+        if mode != ops.CARRY_NONE:
+            cache._update_cache_x(carry, idx)
+        att = attn(h, position_embeddings, start_pos, cache, fused_decode=True, statistic_done=mode != ops.CARRY_NONE)
+        h = ops.add_rms_norm(x, att, self.post_attention_layernorm.weight, self.post_attention_layernorm.eps)
+        return self.mlp.forward_fused(h)
+
 
 class NAtSLlamaForCausalLM(nn.Module):
     def __init__(self, cfg: NAtSLlamaConfig):
@@ -187,6 +289,10 @@ class NAtSLlamaForCausalLM(nn.Module):
                     p.fill_(1.0)
                 else:
                     p.normal_(0.0, std, generator=g)
+        if cfg.fused_decode:
+            for layer in model.layers:
+                layer.self_attn.fuse()
+                layer.mlp.fuse()
         return model.eval()
 
     def new_cache(self, track_positions: bool = False) -> NAtSCache:
@@ -200,6 +306,12 @@ class NAtSLlamaForCausalLM(nn.Module):
         x = self.embed_tokens(input_ids)
         pos = torch.arange(start_pos, start_pos + q_len, device=input_ids.device)[None].expand(bsz, -1)
         position_embeddings = rotary_tables(pos, self.config.head_dim, self.config.rope_theta, x.dtype)
+        if self.config.fused_decode and q_len == 1 and start_pos > 0 and len(cache.cache_model) == len(self.layers):
+            x = x.contiguous()
+            delta = None
+            for layer in self.layers:
+                delta = layer.decode_step(x, delta, position_embeddings, start_pos, cache)
+            return self.lm_head(ops.add_rms_norm(x, delta, self.norm.weight, self.norm.eps))[:, 0]
         for layer in self.layers:
             x = layer(x, position_embeddings, start_pos, cache)
         x = self.norm(x if all_logits else x[:, -1:])

@@ -395,3 +395,74 @@ def evict_apply_first(src_k, src_v, cache_k, cache_v, valid, pos, roles, size_gl
                                      i64_array(src_k.stride()[:3]), i64_array(cache_k.stride()[:3]),
                                      i64_array(v8.stride()[:2]), cache_k.element_size(), _ptr(ws), _ptr(result),
                                      _stream(cache_k)))
+
+
+# ------------------------------------------------------------------------------------------------
+# decode-step glue of the HF-shaped caller
+# ------------------------------------------------------------------------------------------------
+CARRY_NONE, CARRY_MEAN_FIRST, CARRY_MEAN_ADD, CARRY_MAX_FIRST, CARRY_MAX_MERGE = 0, 1, 2, 3, 4
+
+
+def add_rms_norm(x: torch.Tensor, delta: torch.Tensor | None, weight: torch.Tensor, eps: float,
+                 carry: torch.Tensor | None = None, carry_mode: int = CARRY_NONE, chunk_size: int = 1) -> torch.Tensor:
+    """x += delta (in place, if delta is given); returns RMSNorm(x) * weight (models/transformer/components.py:14-26).
+    With carry_mode != 0 the running chunk statistic `carry` [rows, dim] of the role step is updated from the
+    normalised rows (components/cache/dyn_cache.py:98-124)."""
+    _require_cuda(x, delta, weight, carry)
+    if not x.is_contiguous() or (delta is not None and (not delta.is_contiguous() or delta.shape != x.shape)):
+        raise ValueError("add_rms_norm takes contiguous x and delta of one shape")
+    dim = x.shape[-1]
+    rows = x.numel() // dim
+    if weight.shape != (dim,) or weight.dtype != x.dtype or not weight.is_contiguous():
+        raise ValueError("add_rms_norm: weight must be [dim] of x's dtype")
+    if carry_mode != CARRY_NONE and (carry is None or carry.numel() != x.numel() or not carry.is_contiguous()
+                                     or carry.dtype != x.dtype):
+        raise ValueError("add_rms_norm: the chunk statistic must be a contiguous tensor of x's size and dtype")
+    out = torch.empty_like(x)
+    check(_lib.load().nats_add_rms_norm(_ptr(x), _ptr(delta), _ptr(weight), _ptr(out), _ptr(carry), rows, dim, float(eps),
+                                        int(carry_mode), int(chunk_size), _dtype_code(x), _stream(x)))
+    return out
+
+
+def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
+    """[..., 2 * I] -> silu(gate_up[..., :I]) * gate_up[..., I:]."""
+    _require_cuda(gate_up)
+    if not gate_up.is_contiguous() or gate_up.shape[-1] % 2:
+        raise ValueError("silu_mul takes a contiguous [..., 2 * I] tensor")
+    inter = gate_up.shape[-1] // 2
+    out = torch.empty(*gate_up.shape[:-1], inter, dtype=gate_up.dtype, device=gate_up.device)
+    check(_lib.load().nats_silu_mul(_ptr(gate_up), _ptr(out), gate_up.numel() // (2 * inter), inter, _dtype_code(gate_up),
+                                    _stream(gate_up)))
+    return out
+
+
+def rope_append(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
+                cache_k: torch.Tensor, cache_v: torch.Tensor, valid: torch.Tensor, pos: torch.Tensor | None, row0: int,
+                pos0: int = 0) -> torch.Tensor:
+    """Rotary embedding of q and k, and k / v written to rows [row0, row0 + x_len) of the cache with their valid
+    bytes (and stream positions).  q [B, H_q, x_len, D], k / v [B, H_kv, x_len, D] (any strides, last dimension
+    contiguous), cos / sin [B, x_len, D].  Returns the rotated q, contiguous."""
+    _require_cuda(q, k, v, cos, sin, cache_k, cache_v, valid, pos)
+    B, Hq, x_len, D = q.shape
+    Hkv = k.shape[1]
+    if k.shape != (B, Hkv, x_len, D) or v.shape != k.shape or cos.shape != (B, x_len, D) or sin.shape != cos.shape:
+        raise ValueError("rope_append: q / k / v / cos / sin shapes do not fit")
+    ts = (q, k, v, cos, sin, cache_k, cache_v)
+    if any(t.dtype != q.dtype for t in ts) or any(t.stride(-1) != 1 for t in ts):
+        raise ValueError("rope_append: one dtype and a contiguous last dimension everywhere")
+    if cache_v.stride() != cache_k.stride() or cache_k.shape[:2] != (B, Hkv) or cache_k.shape[3] != D:
+        raise ValueError("rope_append: cache_k / cache_v must be [B, H_kv, rows, D] with equal strides")
+    if sin.stride() != cos.stride():
+        sin = sin.contiguous()
+        cos = cos.contiguous()
+    if valid.dtype != torch.uint8 or valid.stride(-1) != 1 or (pos is not None and (pos.stride() != valid.stride()
+                                                                                   or pos.dtype != torch.int32)):
+        raise ValueError("rope_append: valid must be uint8 rows (pos: int32 of the same layout)")
+    q_out = torch.empty(B, Hq, x_len, D, dtype=q.dtype, device=q.device)
+    n_alloc = min(cache_k.shape[2], valid.shape[2])
+    check(_lib.load().nats_rope_append(
+        _ptr(q), _ptr(k), _ptr(v), _ptr(cos), _ptr(sin), _ptr(q_out), _ptr(cache_k), _ptr(cache_v), _ptr(valid), _ptr(pos),
+        B, Hq, Hkv, x_len, D, int(row0), n_alloc, int(pos0), i64_array(q.stride()[:3]), i64_array(k.stride()[:3]),
+        i64_array(v.stride()[:3]), i64_array(cos.stride()[:2]), i64_array(cache_k.stride()[:3]),
+        i64_array(valid.stride()[:2]), _dtype_code(q), _stream(q)))
+    return q_out
