@@ -123,6 +123,15 @@ int nats_prefill_tile_map(const uint8_t* roles, int64_t B, int64_t H_kv, int64_t
  */
 size_t nats_prefill_workspace_bytes(int64_t B, int64_t H_q, int64_t H_kv, int64_t L, int64_t D, int64_t C);
 
+/* Extra workspace bytes (behind the ones above; already included in nats_prefill_workspace_bytes) that let bf16
+ * calls with GQA groups of 4 q heads or a multiple run the persistent kernel: one workgroup per CU walks a
+ * precomputed list of (query tile, key tile) visits instead of one workgroup per query tile building its own.
+ * A call whose workspace is smaller runs the per-tile kernel; results are the same to rounding.  0 for shapes
+ * that never use it.  n_queries: new tokens of the call, n_rows: key rows (L for a prefill from an empty cache,
+ * n_ctx_data + x_len over a filled one).
+ */
+size_t nats_prefill_sched_workspace_bytes(int64_t B, int64_t H_q, int64_t H_kv, int64_t n_queries, int64_t n_rows);
+
 int nats_prefill_fwd(const void* q, const void* k, const void* v, const uint8_t* roles, void* o, int64_t B,
                      int64_t H_q, int64_t H_kv, int64_t L, int64_t D, int64_t C, int64_t W, const int64_t* q_strides,
                      const int64_t* k_strides, const int64_t* v_strides, const int64_t* o_strides, float sm_scale,
@@ -152,7 +161,8 @@ typedef struct {
  *   valid [B, H_kv, >= n_ctx_data] uint8 (valid_tokens), strides (stride_b, stride_h)
  *   size_global / size_local [B, H_kv] int64 contiguous
  *   roles [B, H_kv, S] uint8, S = ceil((old_fill + x_len) / C): one slot per chunk of the open-chunk region
- *   workspace: nats_prefill_past_workspace_bytes(B, H_kv, n_ctx_data + x_len, S) bytes
+ *   workspace: nats_prefill_past_workspace_bytes(B, H_kv, n_ctx_data + x_len, S) bytes, optionally followed by
+ *              nats_prefill_sched_workspace_bytes(B, H_q, H_kv, x_len, n_ctx_data + x_len) more
  * Query i is token old_fill + i of the region that starts at row n_ctx_data - old_fill.
  */
 size_t nats_prefill_past_workspace_bytes(int64_t B, int64_t H_kv, int64_t n_rows, int64_t S);

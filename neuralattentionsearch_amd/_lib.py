@@ -50,6 +50,7 @@ SIGNATURES = {
     "nats_prefill_mask": (ctypes.c_int, [c_p, c_i64, c_i64, c_i64, c_i64, c_i64, c_p, c_p, ctypes.c_size_t, c_p]),
     "nats_prefill_tile_map": (ctypes.c_int, [c_p, c_i64, c_i64, c_i64, c_i64, c_i64, c_p, c_p, ctypes.c_size_t, c_p]),
     "nats_prefill_workspace_bytes": (ctypes.c_size_t, [c_i64] * 6),
+    "nats_prefill_sched_workspace_bytes": (ctypes.c_size_t, [c_i64] * 5),
     "nats_prefill_fwd": (ctypes.c_int, [c_p, c_p, c_p, c_p, c_p, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64,
                                         c_i64p, c_i64p, c_i64p, c_i64p, ctypes.c_float, ctypes.c_int, c_p,
                                         ctypes.c_size_t, c_p]),

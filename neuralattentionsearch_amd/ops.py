@@ -260,7 +260,8 @@ def prefill_past_attention(q: torch.Tensor, cache_k: torch.Tensor, cache_v: torc
     q = q if q.stride(-1) == 1 else q.contiguous()
     out = torch.empty(B, Hq, x_len, D, dtype=q.dtype, device=q.device)
     scale = (1.0 / math.sqrt(D)) if sm_scale is None else float(sm_scale)
-    ws = workspace(q.device, "prefill", lib.nats_prefill_past_workspace_bytes(B, Hkv, N, S))
+    ws = workspace(q.device, "prefill", lib.nats_prefill_past_workspace_bytes(B, Hkv, N, S) +
+                   lib.nats_prefill_sched_workspace_bytes(B, Hq, Hkv, x_len, N))
     valid_u8 = valid.view(torch.uint8) if valid.dtype == torch.bool else valid
     check(lib.nats_prefill_past_fwd(_ptr(q), _ptr(cache_k), _ptr(cache_v), _ptr(valid_u8), _ptr(size_global),
                                     _ptr(size_local), _ptr(roles), _ptr(out), B, Hq, Hkv, x_len, D, chunk_size, window,
