@@ -31,7 +31,7 @@ if ROOT not in sys.path:
 # HBM bytes per launch of the dominant kernels at the default workloads, from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE scaled by a 1 GiB device copy (read factor 2.0, write factor 1.0); see profiles/.
 MEASURED_TRAFFIC = {  # bytes read + written per launch
-    "prefill": 228890 * 1024 * 2.0 + 270264 * 1024 * 1.0,
+    "prefill": 225880 * 1024 * 2.0 + 262144 * 1024 * 1.0,
     "decode": 887027 * 1024 * 2.0 + 1560 * 1024 * 1.0,
     "evict": 272937 * 1024 * 2.0 + 554050 * 1024 * 1.0,
 }
