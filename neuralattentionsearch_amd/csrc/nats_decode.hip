@@ -522,13 +522,15 @@ static size_t align256(size_t x) { return (x + 255) & ~size_t(255); }
 
 template <int D, int NREP>
 static int launch_mfma(const DecodeArgs& a, int groups, hipStream_t st) {
-  static bool configured = false;  // the LDS attribute is a property of the kernel
+  static bool configured[64] = {};  // per instantiation; the LDS attribute is set once per device
   const size_t smem = sizeof(DecodeSmem<D, NREP>);
-  if (!configured) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return fail(NATS_ERR_LAUNCH, "decode: no current device");
+  if (!configured[dev]) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&decode_split_mfma_kernel<D, NREP>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return fail(NATS_ERR_LAUNCH, "hipFuncSetAttribute(%zu bytes of LDS): %s", smem, hipGetErrorString(e));
-    configured = true;
+    configured[dev] = true;
   }
   dim3 grid((unsigned)a.n_wg, 1u, (unsigned)groups);
   hipLaunchKernelGGL((decode_split_mfma_kernel<D, NREP>), grid, dim3(256), smem, st, a);

@@ -165,6 +165,7 @@ __global__ __launch_bounds__(64) void prefill_simple_kernel(PrefillArgs a) {
 // ---------------------------------------------------------------------------------------------------
 constexpr float kRescaleSlack = 8.0f;
 constexpr int kPrefillWaves = 8;
+constexpr int kMaxDevices = 64;
 
 // both halves of the wavefront get max / sum over lane and lane ^ 32 (one cross-half swap, no LDS round trip)
 __device__ __forceinline__ float half_swap_max(float v) {
@@ -1240,13 +1241,15 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_stream_kernel(P
 
 template <int D, bool kUniform>
 static int launch_prefill_mfma(const PrefillArgs& a, int64_t n_wg, hipStream_t st) {
-  static bool configured = false;  // per process and instantiation; the attribute is a property of the kernel
+  static bool configured[kMaxDevices] = {};  // per instantiation; the attribute is set once per device
   const size_t smem = sizeof(PrefillSmem<D>);
-  if (!configured) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail(NATS_ERR_LAUNCH, "prefill: no current device");
+  if (!configured[dev]) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_mfma_kernel<D, kUniform>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return fail(NATS_ERR_LAUNCH, "hipFuncSetAttribute(%zu bytes of LDS): %s", smem, hipGetErrorString(e));
-    configured = true;
+    configured[dev] = true;
   }
   hipLaunchKernelGGL((prefill_mfma_kernel<D, kUniform>), dim3((unsigned)n_wg), dim3(kPrefillWaves * kWave), smem, st, a);
   NATS_CHECK_LAUNCH("prefill_mfma_kernel");
@@ -1303,9 +1306,9 @@ static StreamSched carve_stream_sched(void* ws, int64_t B, int64_t H_q, int64_t 
 }
 
 static int device_cu_count() {
-  static int cached[64] = {0};
+  static int cached[kMaxDevices] = {0};
   int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 0;
   if (cached[dev] == 0) {
     int n = 0;
     if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
@@ -1337,13 +1340,15 @@ static int launch_prefill_stream(PrefillArgs a, const StreamSched& sw, hipStream
 
   a.entries = sw.entries;
   a.bounds = sw.bounds;
-  static bool configured = false;
+  static bool configured[kMaxDevices] = {};
   const size_t smem = sizeof(StreamSmem<D>);
-  if (!configured) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail(NATS_ERR_LAUNCH, "prefill: no current device");
+  if (!configured[dev]) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_stream_kernel<D>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return fail(NATS_ERR_LAUNCH, "hipFuncSetAttribute(%zu bytes of LDS): %s", smem, hipGetErrorString(e));
-    configured = true;
+    configured[dev] = true;
   }
   hipLaunchKernelGGL((prefill_stream_kernel<D>), dim3((unsigned)n_wg), dim3(kPrefillWaves * kWave), smem, st, a);
   NATS_CHECK_LAUNCH("prefill_stream_kernel");
