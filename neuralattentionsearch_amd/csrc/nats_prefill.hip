@@ -600,10 +600,11 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
 #pragma unroll
       for (int g4 = 0; g4 < 4; ++g4) {
         int d = dt * 32 + g4 * 8 + hl * 4;
-        uint32_t lo = uint32_t(f32_to_bf16_bits(oacc[dt][g4 * 4 + 0] * inv)) |
-                      (uint32_t(f32_to_bf16_bits(oacc[dt][g4 * 4 + 1] * inv)) << 16);
-        uint32_t hi = uint32_t(f32_to_bf16_bits(oacc[dt][g4 * 4 + 2] * inv)) |
-                      (uint32_t(f32_to_bf16_bits(oacc[dt][g4 * 4 + 3] * inv)) << 16);
+        // (the hardware conversion: round to nearest even, two values per instruction)
+        const bf16x4 ob = {(__bf16)(oacc[dt][g4 * 4 + 0] * inv), (__bf16)(oacc[dt][g4 * 4 + 1] * inv),
+                           (__bf16)(oacc[dt][g4 * 4 + 2] * inv), (__bf16)(oacc[dt][g4 * 4 + 3] * inv)};
+        const uint2 ou = __builtin_bit_cast(uint2, ob);
+        const uint32_t lo = ou.x, hi = ou.y;
         *reinterpret_cast<uint2*>(stage + l32 * kRowPitch + d * 2) = make_uint2(lo, hi);
       }
     }
@@ -1124,10 +1125,11 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_stream_kernel(P
 #pragma unroll
       for (int g4 = 0; g4 < 4; ++g4) {
         const int d = g4 * 8 + hl * 4;
-        uint32_t lo = uint32_t(f32_to_bf16_bits(oacc[dt][g4 * 4 + 0] * inv)) |
-                      (uint32_t(f32_to_bf16_bits(oacc[dt][g4 * 4 + 1] * inv)) << 16);
-        uint32_t hi = uint32_t(f32_to_bf16_bits(oacc[dt][g4 * 4 + 2] * inv)) |
-                      (uint32_t(f32_to_bf16_bits(oacc[dt][g4 * 4 + 3] * inv)) << 16);
+        // (the hardware conversion: round to nearest even, two values per instruction)
+        const bf16x4 ob = {(__bf16)(oacc[dt][g4 * 4 + 0] * inv), (__bf16)(oacc[dt][g4 * 4 + 1] * inv),
+                           (__bf16)(oacc[dt][g4 * 4 + 2] * inv), (__bf16)(oacc[dt][g4 * 4 + 3] * inv)};
+        const uint2 ou = __builtin_bit_cast(uint2, ob);
+        const uint32_t lo = ou.x, hi = ou.y;
         *reinterpret_cast<uint2*>(stage + l32 * kPitch + d * 2) = make_uint2(lo, hi);
       }
       wave_lds_sync();
