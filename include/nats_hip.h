@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define NATS_ABI_VERSION 3
+#define NATS_ABI_VERSION 4
 
 typedef enum {
   NATS_OK = 0,
@@ -289,6 +289,17 @@ int nats_add_rms_norm(void* x, const void* delta, const void* weight, void* out,
  * with the two projections stored as one matrix.  gate_up [rows, 2 * inter], out [rows, inter], contiguous.
  */
 int nats_silu_mul(const void* gate_up, void* out, int64_t rows, int64_t inter, int dtype, void* stream);
+
+/* y[r, n] = sum_k x[r, k] * w[n, k]: the nn.Linear projections (no bias) of a one-token step
+ * (hf/llama_nats_chunk.py:185-187 q / k / v, :290 o_proj, the gate / up / down projections of the HF Llama MLP
+ * the reference keeps, lm_head) for 1..4 rows of x.  fp32 accumulation, one rounding to the dtype.
+ *   w [n_out, k] (gate != 0: [2 * n_out, k], gate rows first, then up rows), x [x_rows, k], y [x_rows, n_out];
+ *   strides in elements, k contiguous; k and the strides of w and x multiples of 16 bytes, w and x 16-byte aligned
+ *   gate != 0: y[r, n] = silu(x[r] . w[n]) * (x[r] . w[n_out + n]) with the roundings of the separate ops
+ *   (nats_silu_mul after one projection over the stacked matrix)
+ */
+int nats_matvec(const void* w, const void* x, void* y, int64_t x_rows, int64_t n_out, int64_t k, int64_t w_stride,
+                int64_t x_stride, int64_t y_stride, int gate, int dtype, void* stream);
 
 /* Rotary embedding of q and k (transformers' apply_rotary_pos_emb, hf/llama_nats_chunk.py:227) and the row
  * write of NAtSChunkLayerCache.update (components/cache/nats_chunk_layer_cache.py:243-256) in one launch:

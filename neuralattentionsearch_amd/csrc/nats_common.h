@@ -40,6 +40,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));  // 16 bytes as the native vector the streaming load / store builtins take
 
 __device__ __forceinline__ int lane_id() { return threadIdx.x & (kWave - 1); }
 

@@ -49,6 +49,8 @@ __device__ __forceinline__ float exp2_guard(float x) { return __builtin_amdgcn_e
 // tile's first valid row instead (a cache hit), whose score is masked and whose probability is exactly 0.
 // ---------------------------------------------------------------------------------------------------
 constexpr float kDecodeRescaleSlack = 8.0f;
+// K and V rows are read once per step: their loads carry the streaming hint (no retention in the caches)
+constexpr int kAuxStream = 2;  // the "nt" bit of a global_load_lds
 constexpr int kDecTile = 32;
 
 constexpr int kMaxBalancedHeads = 1024;  // (b, kv head) streams whose tile prefix sums fit in LDS
@@ -214,7 +216,10 @@ __global__ __launch_bounds__(256) void decode_split_mfma_kernel(DecodeArgs a) {
         int row = ((vm >> kl) & 1) ? kl : fv;
         const uint16_t* rp = kp + (int64_t)(r0 + row) * a.ks_r + lg * 8;
 #pragma unroll
-        for (int s = 0; s < STEPS; ++s) kreg[g][s] = *reinterpret_cast<const uint4*>(rp + s * 32);
+        for (int s = 0; s < STEPS; ++s) {
+          const u32x4 w = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(rp + s * 32));
+          kreg[g][s] = make_uint4(w.x, w.y, w.z, w.w);
+        }
       }
     };
     auto issue_v = [&](int r0, uint32_t vm, int buf) {
@@ -227,7 +232,7 @@ __global__ __launch_bounds__(256) void decode_split_mfma_kernel(DecodeArgs a) {
         const int chunk = cpos ^ ((row & 3) << 1);
         __builtin_amdgcn_global_load_lds(vp + (int64_t)(r0 + src_row) * a.ks_r + chunk * 8,
                                          (uint32_t __attribute__((address_space(3)))*)(&sm.v[wave][buf][j * kWave * 8]), 16, 0,
-                                         0);
+                                         kAuxStream);
       }
     };
 

@@ -475,9 +475,10 @@ __global__ __launch_bounds__(256) void evict_apply_first_kernel(ApplyArgs a) {
       int row = u / upr, col = u % upr;
       int64_t drow = ci * C + row;
       int64_t tok = src_chunk < 0 ? -1 : src_chunk * C + row;
-      uint4 val = make_uint4(0, 0, 0, 0);
-      if (tok >= 0 && tok < L && drow < res.n_ctx_data) val = src[tok * s_stride + col];
-      dst[drow * d_stride + col] = val;
+      // every row is read once and written once: both sides carry the streaming hint
+      u32x4 val = {0u, 0u, 0u, 0u};
+      if (tok >= 0 && tok < L && drow < res.n_ctx_data) val = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src + tok * s_stride + col));
+      __builtin_nontemporal_store(val, reinterpret_cast<u32x4*>(dst + drow * d_stride + col));
     }
   } else {
     int32_t* dst = static_cast<int32_t*>(a.tensor[2]) + b * a.vs_b + h * a.vs_h;

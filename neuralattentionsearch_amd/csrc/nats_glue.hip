@@ -13,6 +13,9 @@
 //     :227 (q * cos + rotate_half(q) * sin, every product and the sum rounded to the dtype), followed by the
 //     row write of NAtSChunkLayerCache.update (components/cache/nats_chunk_layer_cache.py:243-256).
 //   * SiLU gate: act_fn(gate_proj(x)) * up_proj(x) of the HF Llama MLP the reference keeps unchanged.
+//   * matrix-vector products: the nn.Linear projections of a one-token step (hf/llama_nats_chunk.py:185-187 q / k / v,
+//     :290 o_proj, and the gate / up / down projections of the HF Llama MLP), fp32 accumulation over k, one
+//     rounding to the dtype at the end, as the library GEMM does; the order of the fp32 sum differs from the library's.
 #include "nats_common.h"
 
 namespace nats {
@@ -158,6 +161,125 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const void* __restrict__ 
   g_store<kBf16>(out, i, s * u);
 }
 
+// ---- y[r, n] = sum_k x[r, k] * w[n, k] for a few rows of x (the projections of a one-token step) --------------
+// The weights are read once from HBM and nothing else is: one wavefront owns WR output columns, its lanes walk
+// k in 16-byte pieces with UNROLL pieces of every weight row in flight, products and sums in fp32, one
+// butterfly reduction per (column, x row) at the end.  Weight loads bypass the caches' retention (each byte is
+// used once per step); x is re-read from cache by every wavefront.
+// kGate: w holds the gate rows [0, N) and the up rows [N, 2N); the wavefront computes both for its columns and
+// writes silu(gate) * up with the rounding points of the separate ops (projection, SiLU, product).
+struct MatvecArgs {
+  const void *w, *x;
+  void* y;
+  int64_t w_stride, x_stride, y_stride;  // elements
+  int n_out, k;
+};
+
+constexpr int kMatvecWaves = 4;
+constexpr int kMatvecUnroll = 4;
+
+// a 16-byte piece of a weight row; the load is marked as a stream (no reuse)
+__device__ __forceinline__ uint4 stream_load16(const unsigned char* p) {
+  const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+
+template <bool kBf16>
+__device__ __forceinline__ void unpack_piece(const uint4& u, float (&v)[8]) {
+  // (fp32: only v[0..3] are used)
+  if (kBf16) {
+    const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      v[2 * e] = __uint_as_float(w[e] << 16);
+      v[2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
+    }
+  } else {
+    v[0] = __uint_as_float(u.x); v[1] = __uint_as_float(u.y); v[2] = __uint_as_float(u.z); v[3] = __uint_as_float(u.w);
+  }
+}
+
+template <bool kBf16, int XR, int WR, bool kGate>
+__global__ __launch_bounds__(kMatvecWaves * kWave) void matvec_kernel(MatvecArgs a) {
+  constexpr int E = kBf16 ? 8 : 4;       // elements per 16-byte piece
+  constexpr int NW = kGate ? 2 * WR : WR;  // weight rows per wavefront
+  constexpr int ES = kBf16 ? 2 : 4;      // bytes per element
+  const int lane = lane_id();
+  const int n0 = (blockIdx.x * kMatvecWaves + (threadIdx.x >> 6)) * WR;
+  if (n0 >= a.n_out) return;
+  const unsigned char* wrow[NW];
+#pragma unroll
+  for (int j = 0; j < NW; ++j) {
+    // columns past the end repeat the last one (their results are not written)
+    const int col = min(n0 + (j % WR), a.n_out - 1);
+    const int64_t row = (kGate && j >= WR) ? (int64_t)a.n_out + col : col;
+    wrow[j] = static_cast<const unsigned char*>(a.w) + row * a.w_stride * ES;
+  }
+  const unsigned char* xp = static_cast<const unsigned char*>(a.x);
+  float acc[NW][XR];
+#pragma unroll
+  for (int j = 0; j < NW; ++j)
+#pragma unroll
+    for (int r = 0; r < XR; ++r) acc[j][r] = 0.f;
+
+  const int pieces = a.k / E;
+  auto step = [&](int p, const uint4 (&wv)[NW]) {
+    float xv[XR][8];
+#pragma unroll
+    for (int r = 0; r < XR; ++r) {
+      const uint4 u = *reinterpret_cast<const uint4*>(xp + (r * a.x_stride + (int64_t)p * E) * ES);
+      unpack_piece<kBf16>(u, xv[r]);
+    }
+#pragma unroll
+    for (int j = 0; j < NW; ++j) {
+      float wf[8];
+      unpack_piece<kBf16>(wv[j], wf);
+#pragma unroll
+      for (int r = 0; r < XR; ++r)
+#pragma unroll
+        for (int e = 0; e < E; ++e) acc[j][r] = fmaf(wf[e], xv[r][e], acc[j][r]);
+    }
+  };
+  int p = lane;
+  for (; p + (kMatvecUnroll - 1) * kWave < pieces; p += kMatvecUnroll * kWave) {
+    uint4 wv[kMatvecUnroll][NW];
+#pragma unroll
+    for (int u = 0; u < kMatvecUnroll; ++u)
+#pragma unroll
+      for (int j = 0; j < NW; ++j)
+        wv[u][j] = stream_load16(wrow[j] + (int64_t)(p + u * kWave) * 16);
+#pragma unroll
+    for (int u = 0; u < kMatvecUnroll; ++u) step(p + u * kWave, wv[u]);
+  }
+  for (; p < pieces; p += kWave) {
+    uint4 wv[NW];
+#pragma unroll
+    for (int j = 0; j < NW; ++j) wv[j] = stream_load16(wrow[j] + (int64_t)p * 16);
+    step(p, wv);
+  }
+#pragma unroll
+  for (int j = 0; j < NW; ++j)
+#pragma unroll
+    for (int r = 0; r < XR; ++r)
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) acc[j][r] += __shfl_xor(acc[j][r], o);
+  if (lane == 0) {
+#pragma unroll
+    for (int j = 0; j < WR; ++j) {
+      if (n0 + j >= a.n_out) break;
+#pragma unroll
+      for (int r = 0; r < XR; ++r) {
+        float v = acc[j][r];
+        if (kGate) {
+          const float g = g_round<kBf16>(v), u = g_round<kBf16>(acc[j + WR][r]);
+          v = g_round<kBf16>(g / (1.f + expf(-g))) * u;
+        }
+        g_store<kBf16>(a.y, r * a.y_stride + n0 + j, v);
+      }
+    }
+  }
+}
+
 struct RopeAppendArgs {
   const void *q, *k, *v, *cos, *sin;
   void *q_out, *cache_k, *cache_v;
@@ -255,6 +377,57 @@ extern "C" int nats_silu_mul(const void* gate_up, void* out, int64_t rows, int64
     hipLaunchKernelGGL(silu_mul_kernel<false>, dim3(blocks), dim3(256), 0, st, gate_up, out, rows, (int)inter);
   }
   NATS_CHECK_LAUNCH("silu_mul_kernel");
+  return NATS_OK;
+}
+
+template <bool kBf16, int XR, bool kGate>
+static void launch_matvec(const MatvecArgs& a, hipStream_t st) {
+  // wide outputs: two columns per wavefront (more bytes in flight per lane); narrow ones keep one column per
+  // wavefront so that every CU has wavefronts
+  const bool two = !kGate && a.n_out >= 8192;
+  const int per_wave = two ? 2 : 1;
+  const unsigned blocks = (unsigned)((a.n_out + per_wave * kMatvecWaves - 1) / (per_wave * kMatvecWaves));
+  if (two) {
+    hipLaunchKernelGGL((matvec_kernel<kBf16, XR, 2, kGate>), dim3(blocks), dim3(kMatvecWaves * kWave), 0, st, a);
+  } else {
+    hipLaunchKernelGGL((matvec_kernel<kBf16, XR, 1, kGate>), dim3(blocks), dim3(kMatvecWaves * kWave), 0, st, a);
+  }
+}
+
+template <bool kBf16, bool kGate>
+static void launch_matvec_rows(const MatvecArgs& a, int x_rows, hipStream_t st) {
+  switch (x_rows) {
+    case 1: launch_matvec<kBf16, 1, kGate>(a, st); break;
+    case 2: launch_matvec<kBf16, 2, kGate>(a, st); break;
+    case 3: launch_matvec<kBf16, 3, kGate>(a, st); break;
+    default: launch_matvec<kBf16, 4, kGate>(a, st); break;
+  }
+}
+
+extern "C" int nats_matvec(const void* w, const void* x, void* y, int64_t x_rows, int64_t n_out, int64_t k,
+                           int64_t w_stride, int64_t x_stride, int64_t y_stride, int gate, int dtype, void* stream) {
+  NATS_REQUIRE(w && x && y, NATS_ERR_NULL_POINTER, "nats_matvec: NULL pointer");
+  NATS_REQUIRE(dtype == NATS_DTYPE_BF16 || dtype == NATS_DTYPE_F32, NATS_ERR_BAD_DTYPE, "nats_matvec: dtype %d", dtype);
+  const int64_t e = dtype == NATS_DTYPE_BF16 ? 8 : 4;
+  NATS_REQUIRE(x_rows >= 1 && x_rows <= 4, NATS_ERR_UNSUPPORTED, "nats_matvec: %lld rows of x (1..4)", (long long)x_rows);
+  NATS_REQUIRE(n_out > 0 && n_out <= 0x3fffffff && k > 0 && k <= 0x3fffffff, NATS_ERR_BAD_SHAPE,
+               "nats_matvec: n_out=%lld k=%lld", (long long)n_out, (long long)k);
+  NATS_REQUIRE(k % e == 0 && w_stride % e == 0 && x_stride % e == 0 && w_stride >= k && x_stride >= k && y_stride >= n_out,
+               NATS_ERR_BAD_SHAPE, "nats_matvec: k=%lld and the strides of w (%lld) and x (%lld) must be multiples of %lld",
+               (long long)k, (long long)w_stride, (long long)x_stride, (long long)e);
+  NATS_REQUIRE((reinterpret_cast<uintptr_t>(w) & 15) == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0, NATS_ERR_BAD_SHAPE,
+               "nats_matvec: w and x must be 16-byte aligned");
+  MatvecArgs a{};
+  a.w = w; a.x = x; a.y = y;
+  a.w_stride = w_stride; a.x_stride = x_stride; a.y_stride = y_stride;
+  a.n_out = (int)n_out; a.k = (int)k;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == NATS_DTYPE_BF16) {
+    if (gate) launch_matvec_rows<true, true>(a, (int)x_rows, st); else launch_matvec_rows<true, false>(a, (int)x_rows, st);
+  } else {
+    if (gate) launch_matvec_rows<false, true>(a, (int)x_rows, st); else launch_matvec_rows<false, false>(a, (int)x_rows, st);
+  }
+  NATS_CHECK_LAUNCH("matvec_kernel");
   return NATS_OK;
 }
 

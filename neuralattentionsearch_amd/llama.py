@@ -68,6 +68,19 @@ class RMSNorm(nn.Module):
         return self.weight * h.to(x.dtype)
 
 
+def step_linear(x: torch.Tensor, proj) -> torch.Tensor:
+    """A bias-free projection of a one-token step: the matrix-vector kernel for the few rows it takes, the library
+    GEMM otherwise.  `proj` is a weight matrix or an nn.Linear; a module with hooks is called as a module, so that
+    whoever registered them still sees its inputs and outputs."""
+    if isinstance(proj, nn.Module):
+        if proj._forward_pre_hooks or proj._forward_hooks or proj.bias is not None:
+            return proj(x)
+        proj = proj.weight
+    if ops.matvec_ok(x, proj):
+        return ops.matvec(x, proj, _checked=True)
+    return nn.functional.linear(x, proj)
+
+
 class LlamaMLP(nn.Module):
     def __init__(self, cfg: NAtSLlamaConfig):
         super().__init__()
@@ -94,6 +107,8 @@ class LlamaMLP(nn.Module):
     def forward_fused(self, x):
         if not self.fused_ok():
             self.fuse()
+        if ops.matvec_ok(x, self.gate_up_weight):
+            return step_linear(ops.matvec(x, self.gate_up_weight, gate=True, _checked=True), self.down_proj)
         return self.down_proj(ops.silu_mul(nn.functional.linear(x, self.gate_up_weight)))
 
 
@@ -152,7 +167,7 @@ class NAtSLlamaAttention(nn.Module):
         Hq, Hkv, D = self.num_heads, self.num_key_value_heads, self.head_dim
         if not self.fused_ok():
             self.fuse()
-        qkv = nn.functional.linear(hidden_states, self.qkv_weight).view(bsz, 1, Hq + 2 * Hkv, D).transpose(1, 2)
+        qkv = step_linear(hidden_states, self.qkv_weight).view(bsz, 1, Hq + 2 * Hkv, D).transpose(1, 2)
         q, k, v = qkv[:, :Hq], qkv[:, Hq:Hq + Hkv], qkv[:, Hq + Hkv:]
         pre_fill = past_key_value.get_nats_chunk_fill_size(idx)
         roles = tsi = None
@@ -178,7 +193,7 @@ class NAtSLlamaAttention(nn.Module):
                                    row_end=layer.size_global_kv + layer.size_local_kv,
                                    tail_start=layer.n_ctx_data - (layer.chunk_fill_size - 1))
         past_key_value.post_update(layer_idx=idx, x_len=1)
-        return self.o_proj(out.transpose(1, 2).reshape(bsz, 1, -1))
+        return step_linear(out.transpose(1, 2).reshape(bsz, 1, -1), self.o_proj)
 
     def forward(self, hidden_states: torch.Tensor, position_embeddings, start_pos: int, past_key_value: NAtSCache,
                 fused_decode: bool = False, statistic_done: bool = False):
@@ -311,7 +326,7 @@ class NAtSLlamaForCausalLM(nn.Module):
             delta = None
             for layer in self.layers:
                 delta = layer.decode_step(x, delta, position_embeddings, start_pos, cache)
-            return self.lm_head(ops.add_rms_norm(x, delta, self.norm.weight, self.norm.eps))[:, 0]
+            return step_linear(ops.add_rms_norm(x, delta, self.norm.weight, self.norm.eps), self.lm_head)[:, 0]
         for layer in self.layers:
             x = layer(x, position_embeddings, start_pos, cache)
         x = self.norm(x if all_logits else x[:, -1:])

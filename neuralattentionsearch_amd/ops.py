@@ -20,7 +20,13 @@ TILE = 64
 _workspaces: dict = {}
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(t: torch.Tensor):
+    """The current stream of t's device as the handle the library takes."""
+    if _raw_stream is not None:
+        return ctypes.c_void_p(_raw_stream(t.device.index if t.device.index is not None else torch.cuda.current_device()))
     return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
 
 
@@ -435,6 +441,37 @@ def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
     check(_lib.load().nats_silu_mul(_ptr(gate_up), _ptr(out), gate_up.numel() // (2 * inter), inter, _dtype_code(gate_up),
                                     _stream(gate_up)))
     return out
+
+
+MATVEC_MAX_ROWS = 4
+
+
+def matvec_ok(x: torch.Tensor, weight: torch.Tensor) -> bool:
+    """Whether `matvec` takes this pair: at most four rows of x, 16-byte pieces along k."""
+    e = 16 // x.element_size()
+    k = x.shape[-1]
+    return (x.is_cuda and weight.is_cuda and x.dtype == weight.dtype and x.dtype in (torch.bfloat16, torch.float32)
+            and weight.dim() == 2 and weight.shape[1] == k and k % e == 0 and weight.stride(1) == 1
+            and weight.stride(0) % e == 0 and weight.data_ptr() % 16 == 0 and x.is_contiguous()
+            and x.data_ptr() % 16 == 0 and 1 <= x.numel() // k <= MATVEC_MAX_ROWS)
+
+
+def matvec(x: torch.Tensor, weight: torch.Tensor, gate: bool = False, _checked: bool = False) -> torch.Tensor:
+    """nn.functional.linear(x, weight) for up to four rows of x: [..., K] x [N, K] -> [..., N].
+    gate=True: weight is [2 * I, K] (gate rows, then up rows) and the result is silu(x W_g^T) * (x W_u^T), [..., I].
+    `_checked`: the caller has just evaluated matvec_ok(x, weight)."""
+    if not _checked and not matvec_ok(x, weight):
+        raise ValueError("matvec: x [<= 4 rows, K] contiguous and weight [N, K] of the same dtype, K a multiple of 16 bytes")
+    k = x.shape[-1]
+    n = weight.shape[0]
+    if gate:
+        if n % 2:
+            raise ValueError("matvec: a gate / up matrix has an even number of rows")
+        n //= 2
+    y = torch.empty(*x.shape[:-1], n, dtype=x.dtype, device=x.device)
+    check(_lib.load().nats_matvec(_ptr(weight), _ptr(x), _ptr(y), x.numel() // k, n, k, weight.stride(0), k, n,
+                                  1 if gate else 0, _dtype_code(x), _stream(x)))
+    return y
 
 
 def rope_append(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,

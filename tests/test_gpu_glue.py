@@ -1,6 +1,6 @@
 """GPU: the decode-step glue kernels (residual add + RMSNorm + running chunk statistic, rotary embedding + cache
-append, SiLU gate) against the torch ops the reference runs in their place, and the Llama harness with and
-without them.
+append, SiLU gate, matrix-vector products) against the torch ops the reference runs in their place, and the Llama
+harness with and without them.
 
 Elementwise arithmetic must agree bit for bit in bf16 (same rounding points); the RMSNorm's mean of squares is
 an fp32 reduction in another order, so its rows are compared to one unit in the last place of the dtype."""
@@ -108,6 +108,61 @@ def test_rope_append(dtype, B, Hq, Hkv, x_len, D):
     assert (tp[:, :, keep] == -1).all()
     with pytest.raises(ValueError):
         ops.rope_append(q, k, v, cos, sin, ck, cv, valid, tp, rows - x_len + 1, 0)  # rows past the allocation
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("rows,n_out,k", [(1, 4096, 4096), (1, 1, 64), (2, 7, 520), (3, 8200, 1032), (4, 24, 14336)])
+def test_matvec_against_an_fp64_product(dtype, rows, n_out, k):
+    """nn.functional.linear for a few rows: fp32 accumulation in another order than the library's, so the result is
+    held to the exact product (fp64) within the rounding of the dtype plus the fp32 accumulation error."""
+    from neuralattentionsearch_amd import ops
+    say("matvec", dtype, rows, n_out, k)
+    g = torch.Generator().manual_seed(rows * n_out + k)
+    x = torch.randn(rows, 1, k, generator=g).to(dtype).cuda()
+    big = (torch.randn(n_out + 3, k + 16, generator=g) / math.sqrt(k)).to(dtype).cuda()
+    for w in (big[:n_out, :k].contiguous(), big[2:2 + n_out, 16:16 + k]):  # packed rows, and rows of a wider matrix
+        got = ops.matvec(x, w)
+        assert got.shape == (rows, 1, n_out) and got.dtype == dtype
+        exact = x.double() @ w.double().T
+        mag = (x.double().abs() @ w.double().abs().T)
+        tol = (2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -23) * exact.abs() + 2.0 ** -20 * mag
+        assert ((got.double() - exact).abs() <= tol).all(), ((got.double() - exact).abs() / tol).max().item()
+        lib = torch.nn.functional.linear(x, w)
+        assert (got.float() - lib.float()).abs().max().item() <= (2.0 ** -6 if dtype == torch.bfloat16 else 1e-5)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("rows,inter,k", [(1, 1000, 512), (3, 14336, 1024), (4, 5, 64)])
+def test_matvec_with_the_silu_gate(dtype, rows, inter, k):
+    """gate=True equals the SiLU gate kernel applied to the plain product over the stacked matrix, bit for bit: the
+    same sums, the same rounding points."""
+    from neuralattentionsearch_amd import ops
+    say("matvec gate", dtype, rows, inter, k)
+    g = torch.Generator().manual_seed(inter + k)
+    x = torch.randn(rows, 1, k, generator=g).to(dtype).cuda()
+    w = (2 * torch.randn(2 * inter, k, generator=g) / math.sqrt(k)).to(dtype).cuda()
+    got = ops.matvec(x, w, gate=True)
+    want = ops.silu_mul(ops.matvec(x, w))
+    assert got.shape == (rows, 1, inter)
+    assert torch.equal(got, want)
+    ref = torch.nn.functional.silu(torch.nn.functional.linear(x, w[:inter])) * torch.nn.functional.linear(x, w[inter:])
+    scale = max(1.0, ref.float().abs().max().item())
+    assert (got.float() - ref.float()).abs().max().item() <= (2.0 ** -6 if dtype == torch.bfloat16 else 1e-5) * scale
+
+
+def test_matvec_rejects_what_it_does_not_take():
+    from neuralattentionsearch_amd import ops
+    x = torch.randn(5, 64).bfloat16().cuda()
+    w = torch.randn(8, 64).bfloat16().cuda()
+    with pytest.raises(ValueError):
+        ops.matvec(x, w)  # five rows
+    with pytest.raises(ValueError):
+        ops.matvec(x[:1, :60].contiguous(), w[:, :60].contiguous())  # k not in 16-byte pieces
+    with pytest.raises(ValueError):
+        ops.matvec(x[:1].float(), w)  # mixed dtypes
+    with pytest.raises(ValueError):
+        ops.matvec(x[:1], w[:7], gate=True)  # odd number of rows for gate / up
+    assert not ops.matvec_ok(x, w) and ops.matvec_ok(x[:4], w)
 
 
 @pytest.mark.parametrize("merge", ["mean", "max"])
