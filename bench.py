@@ -31,9 +31,9 @@ if ROOT not in sys.path:
 # HBM bytes per launch of the dominant kernels at the default workloads, from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE scaled by a 1 GiB device copy (read factor 2.0, write factor 1.0); see profiles/.
 MEASURED_TRAFFIC = {  # bytes read + written per launch
-    "prefill": 225880 * 1024 * 2.0 + 262144 * 1024 * 1.0,
-    "decode": 887027 * 1024 * 2.0 + 1560 * 1024 * 1.0,
-    "evict": 272937 * 1024 * 2.0 + 554050 * 1024 * 1.0,
+    "prefill": 225859 * 1024 * 2.0 + 262144 * 1024 * 1.0,
+    "decode": 889921 * 1024 * 2.0 + 1562 * 1024 * 1.0,
+    "evict": 272468 * 1024 * 2.0 + 554048 * 1024 * 1.0,
 }
 PEAK_HBM_GBS = 8000.0
 PEAK_BF16_TFLOPS = 2500.0
@@ -286,7 +286,7 @@ def bench_llama(args):
             "shape": dict(layers=cfg.num_hidden_layers, d_model=cfg.hidden_size, heads="32/8", head_dim=cfg.head_dim,
                           ffn=cfg.intermediate_size, vocab=cfg.vocab_size, prefill=args.llama_prefill,
                           decode_steps=args.llama_decode, chunk=cfg.chunk_size, window=cfg.local_seq_max_length),
-            "note": "random weights give near-uniform roles; projections are library GEMMs; one-token steps use the fused norm / rotary + append / gate kernels"}
+            "note": "random weights give near-uniform roles; prefill projections are library GEMMs; one-token steps use the matrix-vector, fused norm and rotary + append kernels"}
 
 
 # --------------------------------------------------------------------------------------------------
