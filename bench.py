@@ -74,21 +74,33 @@ def prefill_flops(roles: np.ndarray, L: int, C: int, W: int, D: int, n_rep: int)
 
 
 def time_gpu(fn, steps: int, warmup: int):
-    """Per-step time of `fn` on the current stream, from HIP events around every step."""
+    """Time of `fn` on the current stream: W untimed calls, then exactly K calls between one pair of HIP events
+    (and one pair of synchronisations), so that the launches follow each other as they do in use.  Returns
+    (host wall time per step, GPU time per step, best single step); the best step comes from a short extra loop
+    with an event pair around every call, which costs each call about ten microseconds of markers and is
+    therefore not what the mean is taken from."""
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
-    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-    stops = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
-    for i in range(steps):
+    start.record()
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3 / steps
+    mean = start.elapsed_time(stop) / steps
+    n = min(steps, 10)
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(n)]
+    stops = [torch.cuda.Event(enable_timing=True) for _ in range(n)]
+    for i in range(n):
         starts[i].record()
         fn()
         stops[i].record()
     torch.cuda.synchronize()
-    wall = (time.perf_counter() - t0) * 1e3 / steps
-    ev = [s.elapsed_time(e) for s, e in zip(starts, stops)]
-    return wall, float(np.mean(ev)), float(np.min(ev))
+    best = min(s.elapsed_time(e) for s, e in zip(starts, stops))
+    return wall, float(mean), float(min(best, mean))
 
 
 # --------------------------------------------------------------------------------------------------
