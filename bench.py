@@ -1,6 +1,6 @@
 """Benchmark of the NAtS sparse-attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-cpu] [--only prefill|decode|evict|evict_stream|llama]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-cpu] [--only prefill|decode|evict|evict_stream|segments|role_step|llama]
 
 One step = one pass of a kernel family over one batch of synthetic input that is already resident in HBM:
 
@@ -263,6 +263,73 @@ def bench_evict_stream(args, ops):
             "shape": dict(B=B, Hkv=Hkv, L=L, D=D, C=C, W=W)}
 
 
+def bench_segments(args, ops):
+    """The prefill workload cut into four segments of 8192 tokens over one cache: segment 1 is a first prefill, the
+    others attend over the evicted cache plus their own tokens (the multi-segment path); every segment is followed
+    by its eviction, as in the caller."""
+    from neuralattentionsearch_amd.cache import NAtSChunkLayerCache
+    B, Hq, Hkv, L, D, C, W = 1, 32, 8, args.prefill_len, 128, 64, 256
+    n_seg = 4
+    seg = L // n_seg
+    dev = "cuda"
+    g = torch.Generator(device=dev).manual_seed(0)
+    q = (torch.randn(B, Hq, L, D, generator=g, device=dev) / math.sqrt(D)).bfloat16()
+    k = (torch.randn(B, Hkv, L, D, generator=g, device=dev) / math.sqrt(D)).bfloat16()
+    v = (torch.randn(B, Hkv, L, D, generator=g, device=dev) / math.sqrt(D)).bfloat16()
+    roles_np = draw_roles(0, B, Hkv, L // C, (0.05, 0.15, 0.80))
+    roles = torch.from_numpy(roles_np).to(dev)
+    tsi = torch.zeros(B, Hkv, L // C, 3, dtype=torch.bfloat16, device=dev)
+    tsi.scatter_(-1, roles.long().unsqueeze(-1), 1.0)
+    sc = seg // C
+    parts = [(q[:, :, i * seg:(i + 1) * seg], k[:, :, i * seg:(i + 1) * seg], v[:, :, i * seg:(i + 1) * seg],
+              roles[:, :, i * sc:(i + 1) * sc].contiguous(), tsi[:, :, i * sc:(i + 1) * sc].contiguous()) for i in range(n_seg)]
+    cache = NAtSChunkLayerCache(B, Hkv, W, chunk_size=C, device=dev)
+    seen = {"pairs": 0, "rows": []}
+
+    def run(count: bool = False):
+        cache.reset_cache()
+        for i, (qs, ks, vs, rs, ts) in enumerate(parts):
+            kc, vc = cache.update(ks, vs, ts)
+            if i == 0:
+                ops.prefill_attention(qs, kc, vc, rs, C, W)
+            else:
+                if count:  # visible (query, key) pairs of this segment, from the mask the kernel implements
+                    seen["pairs"] += int(cache.generate_mask(seg).sum().item())
+                    seen["rows"].append(int(kc.shape[2]))
+                cache.segment_attention(qs)
+            cache.post_update(seg)
+
+    run(count=True)
+    first_pairs = int(ops.prefill_mask(parts[0][3], seg, C, W).sum().item())
+    flops = 4.0 * D * (Hq // Hkv) * (seen["pairs"] + first_pairs)
+    wall, ev_mean, ev_min = time_gpu(run, max(3, args.steps // 4), 2)
+    return {"ms": ev_mean, "ms_min": ev_min, "ms_wall": wall, "segments": n_seg, "segment_tokens": seg,
+            "key_rows_of_later_segments": seen["rows"], "algorithmic_tflop": flops / 1e12,
+            "tflops_visible_pairs": flops / (ev_mean * 1e-3) / 1e12,
+            "note": "per step: 4 x (cache update, attention, eviction); FLOPs counted on visible (query, key) pairs, "
+                    "not on visited tiles",
+            "shape": dict(B=B, Hq=Hq, Hkv=Hkv, L=L, D=D, C=C, W=W)}
+
+
+def bench_role_step(args, ops):
+    """The fused role step (chunk pooling of the hidden states, role projection, argmax, next-global scan) at the
+    Llama-3-8B width: a 32768-token prefill and the token that closes a chunk during decoding."""
+    B, L, dim, Hkv, C, W = 1, args.prefill_len, 4096, 8, 64, 256
+    dev = "cuda"
+    g = torch.Generator(device=dev).manual_seed(0)
+    x = torch.randn(B, L, dim, generator=g, device=dev).bfloat16()
+    w = (torch.randn(Hkv * 3, dim, generator=g, device=dev) * 0.02).bfloat16()
+    _, pre_ms, pre_min = time_gpu(lambda: ops.role_step(x, w, C, W, force_first_global=True, with_scan=True), args.steps, 3)
+    x1 = x[:, :1].contiguous()
+    carry = x[:, 1:2].contiguous()
+    _, one_ms, one_min = time_gpu(lambda: ops.role_step(x1, w, C, W, pre_fill=C - 1, carry_in=carry), args.steps, 3)
+    nbytes = x.numel() * 2
+    return {"prefill_ms": pre_ms, "prefill_ms_min": pre_min, "prefill_gbs": nbytes / (pre_ms * 1e-3) / 1e9,
+            "prefill_frac_of_hbm_peak": nbytes / (pre_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, "algorithmic_bytes": nbytes,
+            "chunk_closing_token_us": one_ms * 1e3, "chunk_closing_token_us_min": one_min * 1e3,
+            "shape": dict(B=B, L=L, dim=dim, Hkv=Hkv, C=C, W=W)}
+
+
 def bench_llama(args):
     """End to end at the Llama-3-8B shape with random weights: one prefill, then greedy decode steps with
     eviction live in all 32 layers."""
@@ -362,7 +429,7 @@ def main():
     ap.add_argument("--prefill-len", type=int, default=32768)
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--no-compare", action="store_true", help="skip the dense comparators of the prefill leg")
-    ap.add_argument("--only", choices=["prefill", "decode", "evict", "copy", "evict_stream", "llama"], default=None)
+    ap.add_argument("--only", choices=["prefill", "decode", "evict", "copy", "evict_stream", "segments", "role_step", "llama"], default=None)
     ap.add_argument("--llama-prefill", type=int, default=16384)
     ap.add_argument("--llama-decode", type=int, default=512)
     args = ap.parse_args()
@@ -391,10 +458,14 @@ def main():
         res["evict"] = bench_evict(args, ops)
     if args.only == "evict_stream":  # not part of the default run
         res["evict_stream"] = bench_evict_stream(args, ops)
+    if args.only == "segments":  # not part of the default run
+        res["segments"] = bench_segments(args, ops)
+    if args.only == "role_step":  # not part of the default run
+        res["role_step"] = bench_role_step(args, ops)
     if args.only == "llama":  # not part of the default run
         res["llama_e2e"] = bench_llama(args)
     torch.cuda.synchronize()
-    cpu = None if args.skip_cpu or args.only in ("evict_stream", "llama") else cpu_baseline(args)
+    cpu = None if args.skip_cpu or args.only in ("evict_stream", "segments", "role_step", "llama") else cpu_baseline(args)
 
     pre = res.get("prefill")
     line = {

@@ -71,9 +71,9 @@ __global__ __launch_bounds__(256) void role_step_kernel(RoleStepArgs a) {
     float acc[VEC];
 #pragma unroll
     for (int v = 0; v < VEC; ++v) acc[v] = a.merge_max ? -INFINITY : 0.f;
-    for (int t = t0; t < t1; ++t) {
+    // kAhead rows are requested before the first of them is used (the sums keep the order of the rows)
+    auto load_row = [&](int t, float (&e)[VEC]) {
       const char* row = xb + (b * a.xs_b + t * a.xs_l + d) * esz;
-      float e[VEC];
       if (VEC == 1) {
         e[0] = load_elem<kBf16>(row, 0);
       } else if (kBf16) {
@@ -87,6 +87,21 @@ __global__ __launch_bounds__(256) void role_step_kernel(RoleStepArgs a) {
 #pragma unroll
         for (int v = 0; v < VEC; ++v) e[v] = w[v];
       }
+    };
+    constexpr int kAhead = 8;
+    int t = t0;
+    for (; t + kAhead <= t1; t += kAhead) {
+      float e[kAhead][VEC];
+#pragma unroll
+      for (int u = 0; u < kAhead; ++u) load_row(t + u, e[u]);
+#pragma unroll
+      for (int u = 0; u < kAhead; ++u)
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) acc[v] = a.merge_max ? fmaxf(acc[v], e[u][v]) : acc[v] + e[u][v];
+    }
+    for (; t < t1; ++t) {
+      float e[VEC];
+      load_row(t, e);
 #pragma unroll
       for (int v = 0; v < VEC; ++v) acc[v] = a.merge_max ? fmaxf(acc[v], e[v]) : acc[v] + e[v];
     }
@@ -115,7 +130,28 @@ __global__ __launch_bounds__(256) void role_step_kernel(RoleStepArgs a) {
   const int n_out = a.Hkv * 3;
   for (int o = wave; o < n_out; o += 4) {
     float acc = 0.f;
-    for (int d = lane; d < a.dim; d += 64) acc = fmaf(pooled[d], load_elem<kBf16>(a.weight, (int64_t)o * a.dim + d), acc);
+    if (VEC > 1) {
+      // VEC consecutive weights per lane and step (one 16-byte load)
+      const char* wrow = static_cast<const char*>(a.weight) + (int64_t)o * a.dim * esz;
+      for (int d = lane * VEC; d < a.dim; d += 64 * VEC) {
+        float w[VEC];
+        if (kBf16) {
+          const uint4 raw = *reinterpret_cast<const uint4*>(wrow + d * 2);
+          const uint32_t u[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) w[v] = bf16_bits_to_f32(uint16_t(u[(v >> 1) & 3] >> ((v & 1) * 16)));
+        } else {
+          const float4 raw = *reinterpret_cast<const float4*>(wrow + d * 4);
+          const float f[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) w[v] = f[v & 3];
+        }
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) acc = fmaf(pooled[d + v], w[v], acc);
+      }
+    } else {
+      for (int d = lane; d < a.dim; d += 64) acc = fmaf(pooled[d], load_elem<kBf16>(a.weight, (int64_t)o * a.dim + d), acc);
+    }
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) acc += __shfl_xor(acc, off);
     if (lane == 0) logit_s[o] = round_elem<kBf16>(acc);
@@ -197,9 +233,10 @@ extern "C" int nats_role_step(const void* x, const void* carry_in, const void* w
     hipLaunchKernelGGL(kernel, grid, dim3(256), smem, st, a);
     return NATS_OK;
   };
-  // 16-byte loads of x when every row allows them
+  // 16-byte loads of x and of the projection weights when every row allows them
   const int vec = dtype == NATS_DTYPE_BF16 ? 8 : 4;
-  const bool wide = dim % vec == 0 && x_strides[0] % vec == 0 && x_strides[1] % vec == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0;
+  const bool wide = dim % vec == 0 && x_strides[0] % vec == 0 && x_strides[1] % vec == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
+                    reinterpret_cast<uintptr_t>(weight) % 16 == 0;
   int rc;
   if (dtype == NATS_DTYPE_BF16) {
     rc = wide ? launch(role_step_kernel<true, 8>) : launch(role_step_kernel<true, 1>);
