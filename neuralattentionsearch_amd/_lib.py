@@ -6,6 +6,7 @@ The library is loaded from the package directory; it is built by ``python -m neu
 from __future__ import annotations
 
 import ctypes
+import functools
 import os
 
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
@@ -117,5 +118,11 @@ def check(rc: int) -> None:
     raise NatsError(rc, msg)
 
 
+@functools.lru_cache(maxsize=4096)
+def _i64_array_of(values: tuple):
+    return (ctypes.c_int64 * len(values))(*values)
+
+
 def i64_array(values):
-    return (ctypes.c_int64 * len(values))(*[int(v) for v in values])
+    """A read-only int64[] argument (strides, sizes); equal tuples share one array."""
+    return _i64_array_of(tuple(int(v) for v in values))

@@ -71,12 +71,14 @@ class NAtSChunkLayerCache:
         self.track_positions = track_positions
         self.size_local_kv = torch.zeros(bsz, n_msks, device=device, dtype=torch.long)
         self.size_global_kv = torch.full([bsz, n_msks], sliding_window_size, device=device, dtype=torch.long)
+        self._row_end = None  # size_global_kv + size_local_kv, kept between evictions
         self.reset_cache()
 
     # -- state ----------------------------------------------------------------------------------
     def reset_cache(self):
         self.size_local_kv.zero_()
         self.size_global_kv.fill_(self.sliding_window_size)
+        self._row_end = None
         self.sliding_queue_tail = 0
         self.chunk_fill_size = 0
         self.chunk_fill_size_last = 0
@@ -262,6 +264,13 @@ class NAtSChunkLayerCache:
                                           self.size_local_kv, self.segment_roles(), self.chunk_size,
                                           self.sliding_window_size, self.past_state(x_len), sm_scale)
 
+    def row_end(self) -> torch.Tensor:
+        """int64 [B, H_kv]: the first cache row past a head's own global and local rows (size_global_kv +
+        size_local_kv), the hint `ops.decode_attention` takes.  Computed once per eviction."""
+        if self._row_end is None:
+            self._row_end = self.size_global_kv + self.size_local_kv
+        return self._row_end
+
     # -- evict + compact (nats_chunk_layer_cache.py:258-389) -------------------------------------
     def post_update(self, x_len: int):
         C, W = self.chunk_size, self.sliding_window_size
@@ -273,6 +282,7 @@ class NAtSChunkLayerCache:
         fill = self.chunk_fill_size
         partial, n_done = fill % C, fill // C
         first = self._seen_tokens == x_len
+        self._row_end = None  # the apply kernels below rewrite the sizes
         roles = self._roles
         if roles is None:
             raise ValueError("post_update needs the roles handed to the update that completed a chunk")

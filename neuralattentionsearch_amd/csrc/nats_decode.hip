@@ -366,36 +366,63 @@ __global__ __launch_bounds__(256) void decode_split_mfma_kernel(DecodeArgs a) {
   }
 }
 
-// merge the partials of one q head (balanced schedule): grid = B*Hq, block = D threads
+// merge the partials of one q head (balanced schedule): grid = B*Hq, block = D threads (one or two wavefronts).
+// The weights 2^(m_s - M) of the partials are computed side by side (thread s takes partial s) and kept in LDS;
+// the accumulators are then summed in partial order with four loads in flight.
 __global__ void decode_merge_balanced_kernel(const float* __restrict__ ws_acc, const float* __restrict__ ws_ml,
                                              const int2* __restrict__ head_table, uint16_t* __restrict__ o, int Hq, int Hkv,
                                              int D) {
+  extern __shared__ float merge_w[];  // [partials of the head] weights, then 2 x 4 floats for the block reductions
   const int head = blockIdx.x;  // b * Hq + hq
   const int d = threadIdx.x;
-  if (d >= D) return;
   const int n_rep = Hq / Hkv;
   const int b = head / Hq, hq = head % Hq;
   const int2 tab = head_table[b * Hkv + hq / n_rep];
   const int r = hq % n_rep;
-  float M = -INFINITY;
-  for (int s = 0; s < tab.y; ++s) M = fmaxf(M, ws_ml[((int64_t)(tab.x + s) * n_rep + r) * 2]);
-  float sum = 0.f, lsum = 0.f;
-  if (M != -INFINITY) {
-    for (int s = 0; s < tab.y; ++s) {
-      const int64_t prt = (int64_t)(tab.x + s) * n_rep + r;
-      float ms = ws_ml[prt * 2];
-      if (ms == -INFINITY) continue;
-      float f = exp2_guard(ms - M);
-      sum += ws_acc[prt * D + d] * f;
-      lsum += ws_ml[prt * 2 + 1] * f;
-    }
+  const int n = tab.y;
+  float* red = merge_w + n;
+  const int n_waves = (blockDim.x + kWave - 1) / kWave;
+
+  float mloc = -INFINITY;
+  for (int s = d; s < n; s += blockDim.x) mloc = fmaxf(mloc, ws_ml[((int64_t)(tab.x + s) * n_rep + r) * 2]);
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) mloc = fmaxf(mloc, __shfl_xor(mloc, off));
+  if ((d & 63) == 0) red[d >> 6] = mloc;
+  __syncthreads();
+  float M = red[0];
+  for (int w = 1; w < n_waves; ++w) M = fmaxf(M, red[w]);
+
+  float lloc = 0.f;
+  for (int s = d; s < n; s += blockDim.x) {
+    const int64_t prt = (int64_t)(tab.x + s) * n_rep + r;
+    const float ms = ws_ml[prt * 2];
+    const float f = (ms == -INFINITY) ? 0.f : exp2_guard(ms - M);
+    merge_w[s] = f;
+    lloc += ws_ml[prt * 2 + 1] * f;
   }
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) lloc += __shfl_xor(lloc, off);
+  if ((d & 63) == 0) red[4 + (d >> 6)] = lloc;
+  __syncthreads();
+  float lsum = red[4];
+  for (int w = 1; w < n_waves; ++w) lsum += red[4 + w];
+  if (d >= D) return;
+
+  float sum = 0.f;
+  const float* acc = ws_acc + ((int64_t)tab.x * n_rep + r) * D + d;
+  const int64_t step = (int64_t)n_rep * D;
+  int s = 0;
+  for (; s + 4 <= n; s += 4) {
+    const float a0 = acc[(s + 0) * step], a1 = acc[(s + 1) * step], a2 = acc[(s + 2) * step], a3 = acc[(s + 3) * step];
+    sum = fmaf(a0, merge_w[s], sum);
+    sum = fmaf(a1, merge_w[s + 1], sum);
+    sum = fmaf(a2, merge_w[s + 2], sum);
+    sum = fmaf(a3, merge_w[s + 3], sum);
+  }
+  for (; s < n; ++s) sum = fmaf(acc[s * step], merge_w[s], sum);
   o[(int64_t)head * D + d] = f32_to_bf16_bits(lsum > 0.f ? sum / lsum : 0.f);
 }
 
-// ---------------------------------------------------------------------------------------------------
-// fp32: one q head per workgroup, one key row per wavefront step; the parity path for fp32 caches.
-// ---------------------------------------------------------------------------------------------------
 template <int D>
 __global__ __launch_bounds__(256) void decode_split_f32_kernel(DecodeArgs a) {
   constexpr int PER = D / 64;
@@ -644,7 +671,9 @@ extern "C" int nats_decode_fwd(const void* q, const void* cache_k, const void* c
   }
   if (rc) return rc;
   NATS_CHECK_LAUNCH("decode_split_mfma_kernel");
-  hipLaunchKernelGGL(decode_merge_balanced_kernel, dim3((unsigned)(B * H_q)), dim3((unsigned)D), 0, st, a.ws_acc, a.ws_ml,
+  // (a head has at most one partial per workgroup plus one)
+  const size_t merge_smem = ((size_t)a.n_wg + 2 + 8) * sizeof(float);
+  hipLaunchKernelGGL(decode_merge_balanced_kernel, dim3((unsigned)(B * H_q)), dim3((unsigned)D), merge_smem, st, a.ws_acc, a.ws_ml,
                      a.head_table, static_cast<uint16_t*>(o), (int)H_q, (int)H_kv, (int)D);
   NATS_CHECK_LAUNCH("decode_merge_balanced_kernel");
   return NATS_OK;

@@ -95,13 +95,17 @@ __global__ __launch_bounds__(kNormThreads) void add_rms_norm_kernel(AddNormArgs 
   __shared__ float part[kNormThreads / kWave];
   const int64_t base = (int64_t)blockIdx.x * a.dim;
   const int tid = threadIdx.x;
-  float v[STEPS][VEC];
+  float v[STEPS][VEC], wv[STEPS][VEC], cv[STEPS][VEC];
+  const bool carry_read = a.carry_mode == 2 || a.carry_mode == 4;
   float ss = 0.f;
 #pragma unroll
   for (int j = 0; j < STEPS; ++j) {
     const int c = (j * kNormThreads + tid) * VEC;
     if (c < a.dim) {
       load_vec<kBf16, VEC>(a.x, base + c, v[j]);
+      // (what the second pass needs is requested now, so that it does not wait for memory again)
+      load_vec<kBf16, VEC>(a.weight, c, wv[j]);
+      if (carry_read) load_vec<kBf16, VEC>(a.carry, base + c, cv[j]);
       if (a.delta) {
         float d[VEC];
         load_vec<kBf16, VEC>(a.delta, base + c, d);
@@ -125,24 +129,22 @@ __global__ __launch_bounds__(kNormThreads) void add_rms_norm_kernel(AddNormArgs 
   for (int j = 0; j < STEPS; ++j) {
     const int c = (j * kNormThreads + tid) * VEC;
     if (c < a.dim) {
-      float w[VEC], h[VEC];
-      load_vec<kBf16, VEC>(a.weight, c, w);
+      float h[VEC];
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) h[e] = g_round<kBf16>(g_round<kBf16>(v[j][e] * r) * w[e]);
+      for (int e = 0; e < VEC; ++e) h[e] = g_round<kBf16>(g_round<kBf16>(v[j][e] * r) * wv[j][e]);
       store_vec<kBf16, VEC>(a.out, base + c, h);
       if (a.carry_mode) {
-        float cv[VEC];
-        if (a.carry_mode == 2 || a.carry_mode == 4) load_vec<kBf16, VEC>(a.carry, base + c, cv);
+        float cn[VEC];
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
           if (a.carry_mode <= 2) {
             const float add = g_round<kBf16>(h[e] / a.chunk);
-            cv[e] = a.carry_mode == 1 ? add : g_round<kBf16>(cv[e] + add);
+            cn[e] = a.carry_mode == 1 ? add : g_round<kBf16>(cv[j][e] + add);
           } else {
-            cv[e] = a.carry_mode == 3 ? h[e] : fmaxf(cv[e], h[e]);
+            cn[e] = a.carry_mode == 3 ? h[e] : fmaxf(cv[j][e], h[e]);
           }
         }
-        store_vec<kBf16, VEC>(a.carry, base + c, cv);
+        store_vec<kBf16, VEC>(a.carry, base + c, cn);
       }
     }
   }

@@ -68,17 +68,27 @@ class RMSNorm(nn.Module):
         return self.weight * h.to(x.dtype)
 
 
-def step_linear(x: torch.Tensor, proj) -> torch.Tensor:
+_plans: dict = {}
+
+
+def step_linear(x: torch.Tensor, proj, gate: bool = False) -> torch.Tensor:
     """A bias-free projection of a one-token step: the matrix-vector kernel for the few rows it takes, the library
     GEMM otherwise.  `proj` is a weight matrix or an nn.Linear; a module with hooks is called as a module, so that
-    whoever registered them still sees its inputs and outputs."""
+    whoever registered them still sees its inputs and outputs.  gate=True: `proj` is the stacked gate / up matrix
+    and the result is silu(gate) * up."""
     if isinstance(proj, nn.Module):
         if proj._forward_pre_hooks or proj._forward_hooks or proj.bias is not None:
             return proj(x)
         proj = proj.weight
-    if ops.matvec_ok(x, proj):
-        return ops.matvec(x, proj, _checked=True)
-    return nn.functional.linear(x, proj)
+    plan = _plans.get(id(proj))
+    if plan is None or plan.weight() is not proj or not plan.current(proj):
+        if len(_plans) > 4096:
+            _plans.clear()
+        plan = _plans[id(proj)] = ops.MatvecPlan(proj, gate)
+    if plan.takes(x):
+        return plan(x)
+    y = nn.functional.linear(x, proj)
+    return ops.silu_mul(y) if gate else y
 
 
 class LlamaMLP(nn.Module):
@@ -107,9 +117,7 @@ class LlamaMLP(nn.Module):
     def forward_fused(self, x):
         if not self.fused_ok():
             self.fuse()
-        if ops.matvec_ok(x, self.gate_up_weight):
-            return step_linear(ops.matvec(x, self.gate_up_weight, gate=True, _checked=True), self.down_proj)
-        return self.down_proj(ops.silu_mul(nn.functional.linear(x, self.gate_up_weight)))
+        return step_linear(step_linear(x, self.gate_up_weight, gate=True), self.down_proj)
 
 
 def rotary_tables(position_ids: torch.Tensor, head_dim: int, theta: float, dtype: torch.dtype):
@@ -190,7 +198,7 @@ class NAtSLlamaAttention(nn.Module):
         cos, sin = position_embeddings
         q, keys, values = layer.append_rotated(q, k, v, cos, sin, tsi, roles)
         out = ops.decode_attention(q, keys, values, layer.valid_tokens, keys.shape[2], 1.0 / math.sqrt(D),
-                                   row_end=layer.size_global_kv + layer.size_local_kv,
+                                   row_end=layer.row_end(),
                                    tail_start=layer.n_ctx_data - (layer.chunk_fill_size - 1))
         past_key_value.post_update(layer_idx=idx, x_len=1)
         return step_linear(out.transpose(1, 2).reshape(bsz, 1, -1), self.o_proj)

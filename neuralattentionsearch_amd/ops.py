@@ -8,6 +8,7 @@ from __future__ import annotations
 
 import ctypes
 import math
+import weakref
 
 import torch
 
@@ -26,12 +27,14 @@ _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 def _stream(t: torch.Tensor):
     """The current stream of t's device as the handle the library takes."""
     if _raw_stream is not None:
-        return ctypes.c_void_p(_raw_stream(t.device.index if t.device.index is not None else torch.cuda.current_device()))
-    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+        idx = t.device.index
+        return _raw_stream(idx if idx is not None else torch.cuda.current_device()) or None
+    return torch.cuda.current_stream(t.device).cuda_stream or None
 
 
 def _ptr(t: torch.Tensor | None):
-    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+    """Device address for a `void*` parameter (ctypes converts the integer; None is NULL)."""
+    return None if t is None else t.data_ptr()
 
 
 def _dtype_code(t: torch.Tensor) -> int:
@@ -446,32 +449,65 @@ def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
 MATVEC_MAX_ROWS = 4
 
 
+def _matvec_weight_ok(weight: torch.Tensor) -> bool:
+    e = 16 // weight.element_size()
+    return (weight.is_cuda and weight.dim() == 2 and weight.dtype in (torch.bfloat16, torch.float32)
+            and weight.shape[1] % e == 0 and weight.stride(1) == 1 and weight.stride(0) % e == 0
+            and weight.data_ptr() % 16 == 0)
+
+
 def matvec_ok(x: torch.Tensor, weight: torch.Tensor) -> bool:
     """Whether `matvec` takes this pair: at most four rows of x, 16-byte pieces along k."""
-    e = 16 // x.element_size()
     k = x.shape[-1]
-    return (x.is_cuda and weight.is_cuda and x.dtype == weight.dtype and x.dtype in (torch.bfloat16, torch.float32)
-            and weight.dim() == 2 and weight.shape[1] == k and k % e == 0 and weight.stride(1) == 1
-            and weight.stride(0) % e == 0 and weight.data_ptr() % 16 == 0 and x.is_contiguous()
-            and x.data_ptr() % 16 == 0 and 1 <= x.numel() // k <= MATVEC_MAX_ROWS)
+    return (_matvec_weight_ok(weight) and x.is_cuda and x.dtype == weight.dtype and weight.shape[1] == k
+            and x.is_contiguous() and x.data_ptr() % 16 == 0 and 1 <= x.numel() // k <= MATVEC_MAX_ROWS)
 
 
-def matvec(x: torch.Tensor, weight: torch.Tensor, gate: bool = False, _checked: bool = False) -> torch.Tensor:
+def matvec(x: torch.Tensor, weight: torch.Tensor, gate: bool = False) -> torch.Tensor:
     """nn.functional.linear(x, weight) for up to four rows of x: [..., K] x [N, K] -> [..., N].
-    gate=True: weight is [2 * I, K] (gate rows, then up rows) and the result is silu(x W_g^T) * (x W_u^T), [..., I].
-    `_checked`: the caller has just evaluated matvec_ok(x, weight)."""
-    if not _checked and not matvec_ok(x, weight):
+    gate=True: weight is [2 * I, K] (gate rows, then up rows) and the result is silu(x W_g^T) * (x W_u^T), [..., I]."""
+    _require_cuda(x, weight)
+    if not matvec_ok(x, weight):
         raise ValueError("matvec: x [<= 4 rows, K] contiguous and weight [N, K] of the same dtype, K a multiple of 16 bytes")
-    k = x.shape[-1]
-    n = weight.shape[0]
-    if gate:
-        if n % 2:
+    return MatvecPlan(weight, gate)(x)  # (x keeps `weight` alive for the call)
+
+
+class MatvecPlan:
+    """A weight matrix checked once for `matvec`, for callers that apply it step after step.  `ok` is False when
+    the kernel does not take the matrix; `takes(x)` is the per-call part of `matvec_ok`."""
+
+    __slots__ = ("weight", "ok", "gate", "n", "k", "w_ptr", "w_stride", "dtype", "code", "fn")
+
+    def __init__(self, weight: torch.Tensor, gate: bool = False):
+        self.weight = weakref.ref(weight)  # the plan must not keep the matrix alive
+        self.gate = 1 if gate else 0
+        self.ok = _matvec_weight_ok(weight) and not (gate and weight.shape[0] % 2)
+        if gate and weight.shape[0] % 2:
             raise ValueError("matvec: a gate / up matrix has an even number of rows")
-        n //= 2
-    y = torch.empty(*x.shape[:-1], n, dtype=x.dtype, device=x.device)
-    check(_lib.load().nats_matvec(_ptr(weight), _ptr(x), _ptr(y), x.numel() // k, n, k, weight.stride(0), k, n,
-                                  1 if gate else 0, _dtype_code(x), _stream(x)))
-    return y
+        self.n = weight.shape[0] // 2 if gate else weight.shape[0]
+        self.k = weight.shape[1]
+        self.w_ptr = weight.data_ptr()
+        self.w_stride = weight.stride(0)
+        self.dtype = weight.dtype
+        self.code = _dtype_code(weight) if self.ok else -1
+        self.fn = _lib.load().nats_matvec
+
+    def current(self, weight: torch.Tensor) -> bool:
+        """Whether the plan still describes `weight` (same storage, dtype and shape)."""
+        return weight.data_ptr() == self.w_ptr and weight.dtype == self.dtype and weight.shape[1] == self.k
+
+    def takes(self, x: torch.Tensor) -> bool:
+        k = self.k
+        return (self.ok and x.dtype == self.dtype and x.shape[-1] == k and x.is_cuda and x.is_contiguous()
+                and 1 <= x.numel() // k <= MATVEC_MAX_ROWS and x.data_ptr() % 16 == 0)
+
+    def __call__(self, x: torch.Tensor) -> torch.Tensor:
+        """x must satisfy `takes(x)`."""
+        k, n = self.k, self.n
+        y = torch.empty(*x.shape[:-1], n, dtype=x.dtype, device=x.device)
+        check(self.fn(self.w_ptr, x.data_ptr(), y.data_ptr(), x.numel() // k, n, k, self.w_stride, k, n, self.gate,
+                      self.code, _stream(x)))
+        return y
 
 
 def rope_append(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
