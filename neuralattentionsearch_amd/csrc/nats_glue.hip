@@ -16,6 +16,8 @@
 //   * matrix-vector products: the nn.Linear projections of a one-token step (hf/llama_nats_chunk.py:185-187 q / k / v,
 //     :290 o_proj, and the gate / up / down projections of the HF Llama MLP), fp32 accumulation over k, one
 //     rounding to the dtype at the end, as the library GEMM does; the order of the fp32 sum differs from the library's.
+#include <type_traits>
+
 #include "nats_common.h"
 
 namespace nats {
@@ -243,16 +245,20 @@ __global__ __launch_bounds__(kMatvecWaves * kWave) void matvec_kernel(MatvecArgs
     }
   };
   int p = lane;
-  for (; p + (kMatvecUnroll - 1) * kWave < pieces; p += kMatvecUnroll * kWave) {
-    uint4 wv[kMatvecUnroll][NW];
+  // batches of kMatvecUnroll pieces per weight row, then one of half that, then single pieces
+  auto batch = [&](auto n_const) {
+    constexpr int N = decltype(n_const)::value;
+    uint4 wv[N][NW];
 #pragma unroll
-    for (int u = 0; u < kMatvecUnroll; ++u)
+    for (int u = 0; u < N; ++u)
 #pragma unroll
-      for (int j = 0; j < NW; ++j)
-        wv[u][j] = stream_load16(wrow[j] + (int64_t)(p + u * kWave) * 16);
+      for (int j = 0; j < NW; ++j) wv[u][j] = stream_load16(wrow[j] + (int64_t)(p + u * kWave) * 16);
 #pragma unroll
-    for (int u = 0; u < kMatvecUnroll; ++u) step(p + u * kWave, wv[u]);
-  }
+    for (int u = 0; u < N; ++u) step(p + u * kWave, wv[u]);
+    p += N * kWave;
+  };
+  while (p + (kMatvecUnroll - 1) * kWave < pieces) batch(std::integral_constant<int, kMatvecUnroll>{});
+  if (p + (kMatvecUnroll / 2 - 1) * kWave < pieces) batch(std::integral_constant<int, kMatvecUnroll / 2>{});
   for (; p < pieces; p += kWave) {
     uint4 wv[NW];
 #pragma unroll
