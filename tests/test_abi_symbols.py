@@ -100,3 +100,16 @@ def test_ops_reject_cpu_tensors():
     from neuralattentionsearch_amd import ops
     with pytest.raises(ValueError):
         ops.role_scan(torch.zeros(1, 1, 4, dtype=torch.uint8), 4, 2)
+
+
+def test_matvec_arguments_are_validated():
+    lib = _lib.load()
+    fake = ctypes.c_void_p(256)  # never dereferenced: validation fails first
+    assert lib.nats_matvec(None, fake, fake, 1, 8, 64, 64, 64, 8, 0, 0, None) == -1
+    assert lib.nats_matvec(fake, fake, fake, 5, 8, 64, 64, 64, 8, 0, 0, None) == -4  # at most four rows of x
+    assert b"rows" in lib.nats_last_error()
+    assert lib.nats_matvec(fake, fake, fake, 1, 8, 60, 64, 64, 8, 0, 0, None) == -2  # k not in 16-byte pieces (bf16)
+    assert lib.nats_matvec(fake, fake, fake, 1, 8, 64, 60, 64, 8, 0, 0, None) == -2  # weight rows not 16-byte aligned
+    assert lib.nats_matvec(fake, fake, fake, 1, 8, 64, 64, 64, 4, 0, 0, None) == -2  # y rows shorter than n_out
+    assert lib.nats_matvec(fake, ctypes.c_void_p(264), fake, 1, 8, 64, 64, 64, 8, 0, 0, None) == -2  # x not 16-byte aligned
+    assert lib.nats_matvec(fake, fake, fake, 1, 8, 64, 64, 64, 8, 0, 7, None) == -3  # dtype code
