@@ -268,9 +268,10 @@ def bench_segments(args, ops):
     others attend over the evicted cache plus their own tokens (the multi-segment path); every segment is followed
     by its eviction, as in the caller."""
     from neuralattentionsearch_amd.cache import NAtSChunkLayerCache
-    B, Hq, Hkv, L, D, C, W = 1, 32, 8, args.prefill_len, 128, 64, 256
-    n_seg = 4
-    seg = L // n_seg
+    B, Hq, Hkv, D, C, W = 1, 32, 8, 128, 64, 256
+    n_seg = args.segments
+    seg = args.segment_len if args.segment_len else args.prefill_len // n_seg
+    L = n_seg * seg
     dev = "cuda"
     g = torch.Generator(device=dev).manual_seed(0)
     q = (torch.randn(B, Hq, L, D, generator=g, device=dev) / math.sqrt(D)).bfloat16()
@@ -293,21 +294,29 @@ def bench_segments(args, ops):
             if i == 0:
                 ops.prefill_attention(qs, kc, vc, rs, C, W)
             else:
-                if count:  # visible (query, key) pairs of this segment, from the mask the kernel implements
-                    seen["pairs"] += int(cache.generate_mask(seg).sum().item())
+                if count:
                     seen["rows"].append(int(kc.shape[2]))
+                    if seen["pairs"] is not None and seg * kc.shape[2] * Hkv <= 2 ** 32:
+                        # visible (query, key) pairs of this segment, from the mask the kernel implements
+                        seen["pairs"] += int(cache.generate_mask(seg).sum().item())
+                    else:
+                        seen["pairs"] = None  # (the mask would not be worth materialising)
                 cache.segment_attention(qs)
             cache.post_update(seg)
 
     run(count=True)
-    first_pairs = int(ops.prefill_mask(parts[0][3], seg, C, W).sum().item())
-    flops = 4.0 * D * (Hq // Hkv) * (seen["pairs"] + first_pairs)
+    flops = None
+    if seen["pairs"] is not None and seg * seg * Hkv <= 2 ** 32:
+        first_pairs = int(ops.prefill_mask(parts[0][3], seg, C, W).sum().item())
+        flops = 4.0 * D * (Hq // Hkv) * (seen["pairs"] + first_pairs)
     wall, ev_mean, ev_min = time_gpu(run, max(3, args.steps // 4), 2)
     return {"ms": ev_mean, "ms_min": ev_min, "ms_wall": wall, "segments": n_seg, "segment_tokens": seg,
-            "key_rows_of_later_segments": seen["rows"], "algorithmic_tflop": flops / 1e12,
-            "tflops_visible_pairs": flops / (ev_mean * 1e-3) / 1e12,
-            "note": "per step: 4 x (cache update, attention, eviction); FLOPs counted on visible (query, key) pairs, "
-                    "not on visited tiles",
+            "tokens_per_s": L / (ev_mean * 1e-3),
+            "key_rows_of_later_segments": seen["rows"] if n_seg <= 8 else [min(seen["rows"]), max(seen["rows"])],
+            "algorithmic_tflop": None if flops is None else flops / 1e12,
+            "tflops_visible_pairs": None if flops is None else flops / (ev_mean * 1e-3) / 1e12,
+            "note": "per step: segments x (cache update, attention, eviction); FLOPs counted on visible (query, key) "
+                    "pairs, not on visited tiles",
             "shape": dict(B=B, Hq=Hq, Hkv=Hkv, L=L, D=D, C=C, W=W)}
 
 
@@ -429,6 +438,8 @@ def main():
     ap.add_argument("--prefill-len", type=int, default=32768)
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--no-compare", action="store_true", help="skip the dense comparators of the prefill leg")
+    ap.add_argument("--segments", type=int, default=4, help="segments of the `--only segments` leg")
+    ap.add_argument("--segment-len", type=int, default=0, help="tokens per segment (default: prefill length / segments)")
     ap.add_argument("--only", choices=["prefill", "decode", "evict", "copy", "evict_stream", "segments", "role_step", "llama"], default=None)
     ap.add_argument("--llama-prefill", type=int, default=16384)
     ap.add_argument("--llama-decode", type=int, default=512)
