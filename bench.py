@@ -405,6 +405,20 @@ def cpu_baseline(args):
                    f"L=8192 {samples[8192]:.2f}s, L=16384 {samples[16384]:.2f}s; value = L=16384 time x (32768/16384)^2 x 8 groups (extrapolated, "
                    f"the [1,32,32768,32768] bool mask does not fit a host)"),
     }
+    # the same on one core, from the L = 8192 sample
+    torch.set_num_threads(1)
+    L = 8192
+    g = torch.Generator().manual_seed(0)
+    q = (torch.randn(1, 4, L, D, generator=g) / math.sqrt(D)).bfloat16()
+    k = (torch.randn(1, 1, L, D, generator=g) / math.sqrt(D)).bfloat16()
+    v = (torch.randn(1, 1, L, D, generator=g) / math.sqrt(D)).bfloat16()
+    roles = draw_roles(0, 1, 1, L // C, (0.05, 0.15, 0.80))
+    t0 = time.perf_counter()
+    orc.masked_attention(q, k, v, orc.prefill_mask(roles, L, C, W))
+    t1 = time.perf_counter() - t0
+    torch.set_num_threads(use)
+    out["one_core"] = {"value": t1 * (32768 / L) ** 2 * 8 * 1e3, "unit": "ms", "cores": 1,
+                       "sample": f"the L=8192 sample on one thread ({t1:.2f}s) x (32768/8192)^2 x 8 groups"}
     # decode: a 2-sequence slice of the batch, scaled linearly to batch 32
     Bs = 2
     q, k, v, valid, n_rows, _ = decode_inputs(Bs, 32, 8, D, C, W, 65536, 0, "cpu")
