@@ -1,6 +1,6 @@
 """Benchmark of the NAtS sparse-attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-cpu] [--only prefill|decode|evict|evict_stream|segments|role_step|llama]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-cpu] [--only prefill|decode|evict|evict_stream|segments|role_step|matvec|llama]
 
 One step = one pass of a kernel family over one batch of synthetic input that is already resident in HBM:
 
@@ -339,6 +339,38 @@ def bench_role_step(args, ops):
             "shape": dict(B=B, L=L, dim=dim, Hkv=Hkv, C=C, W=W)}
 
 
+def bench_matvec(args, ops):
+    """The one-token projections of the Llama-3-8B shape through the matrix-vector kernel and through the library,
+    one row of x; the weights rotate through about 1.5 GB of copies so that no launch finds them in a cache."""
+    shapes = [("qkv", 6144, 4096, False), ("o", 4096, 4096, False), ("gate_up+silu", 14336, 4096, True),
+              ("down", 4096, 14336, False), ("lm_head", 128256, 4096, False)]
+    dev = "cuda"
+    out = {}
+    for name, n, k, gate in shapes:
+        rows_w = 2 * n if gate else n
+        copies = max(2, int(1.5e9 // (rows_w * k * 2)))
+        ws = [(torch.randn(rows_w, k, device=dev) * 0.02).bfloat16() for _ in range(copies)]
+        x = torch.randn(1, 1, k, device=dev).bfloat16()
+        turn = [0]
+
+        def ours():
+            turn[0] = (turn[0] + 1) % copies
+            return ops.matvec(x, ws[turn[0]], gate=gate)
+
+        def library():
+            turn[0] = (turn[0] + 1) % copies
+            y = torch.nn.functional.linear(x, ws[turn[0]])
+            return ops.silu_mul(y) if gate else y
+
+        _, t_ours, _ = time_gpu(ours, args.steps, 10)
+        _, t_lib, _ = time_gpu(library, args.steps, 10)
+        nbytes = rows_w * k * 2
+        out[name] = {"n_out": n, "k": k, "us": t_ours * 1e3, "gbs": nbytes / (t_ours * 1e-3) / 1e9,
+                     "frac_of_hbm_peak": nbytes / (t_ours * 1e-3) / 1e9 / PEAK_HBM_GBS, "library_us": t_lib * 1e3}
+        del ws
+    return out
+
+
 def bench_llama(args):
     """End to end at the Llama-3-8B shape with random weights: one prefill, then greedy decode steps with
     eviction live in all 32 layers."""
@@ -454,7 +486,7 @@ def main():
     ap.add_argument("--no-compare", action="store_true", help="skip the dense comparators of the prefill leg")
     ap.add_argument("--segments", type=int, default=4, help="segments of the `--only segments` leg")
     ap.add_argument("--segment-len", type=int, default=0, help="tokens per segment (default: prefill length / segments)")
-    ap.add_argument("--only", choices=["prefill", "decode", "evict", "copy", "evict_stream", "segments", "role_step", "llama"], default=None)
+    ap.add_argument("--only", choices=["prefill", "decode", "evict", "copy", "evict_stream", "segments", "role_step", "matvec", "llama"], default=None)
     ap.add_argument("--llama-prefill", type=int, default=16384)
     ap.add_argument("--llama-decode", type=int, default=512)
     args = ap.parse_args()
@@ -487,10 +519,12 @@ def main():
         res["segments"] = bench_segments(args, ops)
     if args.only == "role_step":  # not part of the default run
         res["role_step"] = bench_role_step(args, ops)
+    if args.only == "matvec":  # not part of the default run
+        res["matvec"] = bench_matvec(args, ops)
     if args.only == "llama":  # not part of the default run
         res["llama_e2e"] = bench_llama(args)
     torch.cuda.synchronize()
-    cpu = None if args.skip_cpu or args.only in ("evict_stream", "segments", "role_step", "llama") else cpu_baseline(args)
+    cpu = None if args.skip_cpu or args.only in ("evict_stream", "segments", "role_step", "matvec", "llama") else cpu_baseline(args)
 
     pre = res.get("prefill")
     line = {
