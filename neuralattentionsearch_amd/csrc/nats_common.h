@@ -34,6 +34,7 @@ inline int ilog2(int64_t x) {
 
 constexpr int kWave = 64;
 constexpr int kTile = 64;  // prefill tile edge (queries and keys)
+constexpr int kGranule = 16;  // key rows whose limits are also summarised on their own (a quarter tile)
 constexpr int32_t kLimGlobal = 0x7fffffff;
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -71,8 +72,9 @@ struct KeyLimArgs {
   int64_t valid_s_b, valid_s_h;
   const int64_t* size_global;
   const int64_t* size_local;
-  int32_t* tok_lim;  // [streams, N] out
+  int32_t* tok_lim;  // [streams, N] out, followed by one entry that holds -1 (the limit of a row nobody sees)
   int2* tile_lim;    // [streams, Tk] out {max, min}
+  int2* gran_lim;    // [streams, Tk * 4] out {max, min} of every 16 rows
   int Hkv, S, N, Tk, c_shift, C, W;
   int base, gmin, tail, seen, fill_last;
 };
@@ -82,6 +84,7 @@ struct PrefillWorkspace {
   int32_t* first_global;
   int32_t* tok_lim;
   int2* tile_lim;
+  int2* gran_lim;
   size_t bytes;
 };
 

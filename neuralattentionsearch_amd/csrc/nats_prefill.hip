@@ -21,8 +21,9 @@ struct PrefillArgs {
   const void* k;
   const void* v;
   void* o;
-  const int32_t* tok_lim;  // [B*Hkv, N]
+  const int32_t* tok_lim;  // [B*Hkv, N], then one entry holding -1
   const int2* tile_lim;    // [B*Hkv, Tk] {max, min}
+  const int2* gran_lim;    // [B*Hkv, Tk * 4] {max, min} of every 16 key rows
   int64_t qs_b, qs_h, qs_l;
   int64_t ks_b, ks_h, ks_l;
   int64_t vs_b, vs_h, vs_l;
@@ -183,14 +184,24 @@ struct PrefillSmem {
   uint16_t k[4][kTile * D];  // tile j of the visit list in k[j & 3]
   uint16_t v[4][kTile * D];
   int limk[8][kTile];        // row limits of tile j in limk[j & 7]
+  int posk[8][kTile];        // packed tiles: region token of every key row (a row is visible up to limk and from posk on)
   int4 vlist[kWin];  // visited key tiles of the current window: {tile, max limit, min limit, -}
+                     // packed tiles: the four 16-row granules of the tile ({id | mask flag, id, id, id}, -1 = none)
   int vcount;
 };
+constexpr int kGranPerTile = kTile / kGranule;
+constexpr int kPackedMaskFlag = 1 << 30;  // on the first granule id of a packed tile: some score of the tile is masked
 
 // kUniform: the wavefronts are the q heads of ONE query tile (GQA groups of 4 and more), so every tile of
 // the visit list is visited by every wavefront and the tile loop has no per-wavefront branches.
-template <int D, bool kUniform>
+// kPacked (with kUniform, for chunks shorter than a tile): a tile is assembled from four 16-row granules taken
+// from anywhere in the key rows.  Granules no query of the tile sees are left out, granules every query sees
+// without a mask are packed among themselves and the rest (diagonal, partly visible, the remainder of the
+// first kind, padding) into tiles that go through the element mask.  The softmax does not care about the order
+// of the keys, so nothing else changes; without it a tile with one visible 16- or 32-row chunk costs a whole tile.
+template <int D, bool kUniform, bool kPacked = false>
 __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(PrefillArgs a) {
+  static_assert(!kPacked || kUniform, "packed tiles are built for one query tile per workgroup");
   constexpr int OCT = D / 8;                          // 16-byte chunks per row
   constexpr int DMA_PER_WAVE = OCT / kPrefillWaves;   // 1 KiB global->LDS transfers per wavefront and tensor
   constexpr int DSTEPS = D / 16;
@@ -280,8 +291,10 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
   for (int j = 0; j < DMA_PER_WAVE; ++j) {
     const int q = (wave * DMA_PER_WAVE + j) * kWave + lane;  // chunk slot in the LDS tile
     const int row = q / OCT, pos = q % OCT;
-    koff[j] = int(row * a.ks_l + (pos ^ (row % OCT)) * 8);
-    voff[j] = int(row * a.vs_l + (pos ^ ((row & 3) << 1)) * 8);
+    // (packed tiles: this wavefront's 8 rows of a tile lie in one granule; the offset counts from its first row)
+    const int srow = kPacked ? row % kGranule : row;
+    koff[j] = int(srow * a.ks_l + (pos ^ (row % OCT)) * 8);
+    voff[j] = int(srow * a.vs_l + (pos ^ ((row & 3) << 1)) * 8);
   }
   auto issue_rows = [&](const uint16_t* base, int64_t stride, const int (&off)[DMA_PER_WAVE], uint16_t* dst, int kt,
                         bool is_v) {
@@ -315,6 +328,49 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
                                        (uint32_t __attribute__((address_space(3)))*)(&sm.limk[slot][0]), 4, 0, 0);
   };
   auto issue_v = [&](int kt, int buf) { issue_rows(vp, a.vs_l, voff, sm.v[buf], kt, true); };
+  // packed tiles: the wavefront's 8 rows of the tile come from granule (wave / 2) of the list entry; a missing
+  // granule (padding) repeats granule 0, whose rows the limit -1 masks
+  auto issue_rows_p = [&](const uint16_t* base, int64_t stride, const int (&off)[DMA_PER_WAVE], uint16_t* dst, int gid,
+                          bool is_v) {
+    if (gid < 0) gid = 0;
+    if ((gid + 1) * kGranule <= a.N) {
+      const uint16_t* tb = base + (int64_t)gid * kGranule * stride;  // uniform
+#pragma unroll
+      for (int j = 0; j < DMA_PER_WAVE; ++j) {
+        const int inst = wave * DMA_PER_WAVE + j;
+        __builtin_amdgcn_global_load_lds(tb + (int)off[j], (uint32_t __attribute__((address_space(3)))*)(dst + inst * kWave * 8), 16, 0, 0);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < DMA_PER_WAVE; ++j) {
+        const int inst = wave * DMA_PER_WAVE + j;  // uniform
+        const int q = inst * kWave + lane;
+        const int row = q / OCT, pos = q % OCT;
+        const int n = min(gid * kGranule + row % kGranule, a.N - 1);
+        const int chunk = is_v ? pos ^ ((row & 3) << 1) : pos ^ (row % OCT);
+        __builtin_amdgcn_global_load_lds(base + (int64_t)n * stride + chunk * 8,
+                                         (uint32_t __attribute__((address_space(3)))*)(dst + inst * kWave * 8), 16, 0, 0);
+      }
+    }
+  };
+  auto granule_of = [&](int id0, int id1, int id2, int id3, int which) {
+    return which == 0 ? (id0 & ~kPackedMaskFlag) : which == 1 ? id1 : which == 2 ? id2 : id3;
+  };
+  auto issue_k_p = [&](int id0, int id1, int id2, int id3, int buf, int slot) {
+    issue_rows_p(kp, a.ks_l, koff, sm.k[buf], granule_of(id0, id1, id2, id3, wave >> 1), false);
+    if ((id0 & kPackedMaskFlag) && wave == 0) {
+      // limits and region tokens of the 64 rows, for the element mask (asynchronous like the tile itself)
+      const int gid = granule_of(id0, id1, id2, id3, lane >> 4);
+      const int row = gid * kGranule + (lane & (kGranule - 1));
+      const bool real = gid >= 0 && row < a.N;
+      const int32_t* src = real ? lim + row : a.tok_lim + (int64_t)a.B * a.Hkv * a.N;  // (the entry that holds -1)
+      __builtin_amdgcn_global_load_lds(src, (uint32_t __attribute__((address_space(3)))*)(&sm.limk[slot][0]), 4, 0, 0);
+      sm.posk[slot][lane] = real ? row - a.base : 0x7fffffff;
+    }
+  };
+  auto issue_v_p = [&](int id0, int id1, int id2, int id3, int buf) {
+    issue_rows_p(vp, a.vs_l, voff, sm.v[buf], granule_of(id0, id1, id2, id3, wave >> 1), true);
+  };
 
   auto k_frag = [&](const uint16_t* Kt, int kb, int s) {
     const int row = kb * 32 + l32;
@@ -369,6 +425,26 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
         for (int e = 0; e < 4; ++e) {
           int key = kt * kTile + kk + e - a.base;  // region token of the key row (negative: older row)
           bool vis = key <= qtok && qtok <= lv[e];
+          if (!vis) sv[kb][g4 * 4 + e] = -INFINITY;
+        }
+      }
+    }
+  };
+  // packed tile: every key row carries its own region token
+  auto mask_scores_p = [&](int slot, f32x16 (&sv)[2]) {
+    const int qtok = q0 + l32;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+      for (int g4 = 0; g4 < 4; ++g4) {
+        const int kk = kb * 32 + g4 * 8 + hl * 4;
+        const int4 lm = *reinterpret_cast<const int4*>(&sm.limk[slot][kk]);
+        const int4 ps = *reinterpret_cast<const int4*>(&sm.posk[slot][kk]);
+        const int lv[4] = {lm.x, lm.y, lm.z, lm.w};
+        const int pv[4] = {ps.x, ps.y, ps.z, ps.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const bool vis = pv[e] <= qtok && qtok <= lv[e];
           if (!vis) sv[kb][g4 * 4 + e] = -INFINITY;
         }
       }
@@ -482,9 +558,66 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
 #pragma unroll
     for (int i = 0; i < 16; ++i) sacc[kb][i] = 0.f;
 
-  for (int w0 = 0; w0 <= kt_end_group; w0 += kWin) {
+  // (packed tiles: the window counts granules, and leaves room for the one tile the packing can add)
+  const int g_end_group = (a.base + rlast_group) / kGranule;
+  const int win_last = kPacked ? g_end_group : kt_end_group;
+  constexpr int kWinStep = kPacked ? (kWin - 1) * kGranPerTile : kWin;
+  for (int w0 = 0; w0 <= win_last; w0 += kWinStep) {
     // ---- visit list of this window: wavefront 0 compacts the tiles some query tile of the group sees ----
-    if (wave == 0) {
+    if (kPacked && wave == 0) {
+      // granules seen without a mask and granules that need one, each kind in its own list (staged in the tile
+      // buffers, which are idle here), then four ids per tile
+      int* plain_ids = reinterpret_cast<int*>(&sm.k[0][0]);
+      int* mask_ids = reinterpret_cast<int*>(&sm.v[0][0]);
+      const int2* gl = a.gran_lim + (int64_t)ks * a.Tk * kGranPerTile;
+      const int g_hi = min(w0 + kWinStep - 1, g_end_group);
+      int n_plain = 0, n_mask = 0;
+      for (int gb = w0; gb <= g_hi; gb += 16 * kWave) {
+        int2 vals[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+          const int g = gb + u * kWave + lane;
+          vals[u] = g <= g_hi ? gl[g] : make_int2(-1, -1);
+        }
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+          const int g = gb + u * kWave + lane;
+          const bool vis = g <= g_hi && vals[u].x >= r0_group;
+          const int last_pos = g * kGranule + kGranule - 1 - a.base;
+          const bool plain = vis && vals[u].y >= rlast_group && last_pos <= r0_group && (g + 1) * kGranule <= a.N;
+          const bool masked = vis && !plain;
+          const uint64_t bp = __ballot(plain), bm = __ballot(masked);
+          const uint64_t below = (uint64_t(1) << lane) - 1;
+          if (plain) plain_ids[n_plain + __builtin_popcountll(bp & below)] = g;
+          if (masked) mask_ids[n_mask + __builtin_popcountll(bm & below)] = g;
+          n_plain += __builtin_popcountll(bp);
+          n_mask += __builtin_popcountll(bm);
+        }
+      }
+      wave_lds_sync();
+      const int n_pt = n_plain / kGranPerTile;
+      const int left = n_plain - n_pt * kGranPerTile;  // these join the masked kind
+      if (lane < left) mask_ids[n_mask + lane] = plain_ids[n_pt * kGranPerTile + lane];
+      n_mask += left;
+      wave_lds_sync();
+      const int n_mt = (n_mask + kGranPerTile - 1) / kGranPerTile;
+      for (int i = lane; i < n_pt + n_mt; i += kWave) {
+        int4 d;
+        if (i < n_pt) {
+          const int* p = plain_ids + i * kGranPerTile;
+          d = make_int4(p[0], p[1], p[2], p[3]);
+        } else {
+          const int o = (i - n_pt) * kGranPerTile;
+          d.x = mask_ids[o] | kPackedMaskFlag;
+          d.y = o + 1 < n_mask ? mask_ids[o + 1] : -1;
+          d.z = o + 2 < n_mask ? mask_ids[o + 2] : -1;
+          d.w = o + 3 < n_mask ? mask_ids[o + 3] : -1;
+        }
+        sm.vlist[i] = d;
+      }
+      if (lane == 0) sm.vcount = n_pt + n_mt;
+    }
+    if (!kPacked && wave == 0) {
       int2 vals[kWin / kWave];
 #pragma unroll
       for (int j = 0; j < kWin / kWave; ++j) {
@@ -522,20 +655,38 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
       // One step handles two tiles of the list (2s, 2s + 1) between two workgroup barriers.  At its start the
       // K tiles 2s + 1, 2s + 2 and the V tiles 2s, 2s + 1 are in LDS and the scores of tile 2s in registers; the
       // step puts K tiles 2s + 3, 2s + 4 and V tiles 2s + 2, 2s + 3 in flight.
+      // (packed tiles: kt, emax, emin, e3 are the four granule ids, kt with the mask flag)
       struct Entry {
-        int kt, emax, emin;
+        int kt, emax, emin, e3;
       };
       auto read_entry = [&](int j) {
-        Entry r = {0, 0, 0};
+        Entry r = {0, 0, 0, 0};
         if (j < n_vis) {
           int kt, emax, emin;
           entry(j, kt, emax, emin);
           r.kt = kt; r.emax = emax; r.emin = emin;
+          if (kPacked) r.e3 = __builtin_amdgcn_readfirstlane(sm.vlist[j].w);
         }
         return r;
       };
-      auto load_k = [&](int j, const Entry& e) { if (j < n_vis) issue_k(e.kt, j & 3, j & 7, group_needs_lim(e.kt, e.emin)); };
-      auto load_v = [&](int j, const Entry& e) { if (j < n_vis) issue_v(e.kt, j & 3); };
+      auto load_k = [&](int j, const Entry& e) {
+        if (j < n_vis) {
+          if (kPacked) {
+            issue_k_p(e.kt, e.emax, e.emin, e.e3, j & 3, j & 7);
+          } else {
+            issue_k(e.kt, j & 3, j & 7, group_needs_lim(e.kt, e.emin));
+          }
+        }
+      };
+      auto load_v = [&](int j, const Entry& e) {
+        if (j < n_vis) {
+          if (kPacked) {
+            issue_v_p(e.kt, e.emax, e.emin, e.e3, j & 3);
+          } else {
+            issue_v(e.kt, j & 3);
+          }
+        }
+      };
       // tile t: its scores (in sacc) become probabilities while the scores of tile t + 1 are computed, then O += P V
       auto process_tile = [&](int t, const Entry& ec, const Entry& en) {
         const bool vis_c = visits(ec.kt, ec.emax);
@@ -545,8 +696,15 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
         if (vis_c) {
           f32x16 sv[2] = {sacc[0], sacc[1]};
           // no masked score: every key row is at or before the first query and visible to the last one
-          const bool full = ec.kt * kTile + kTile - 1 - a.base <= my_r0 && ec.emin >= my_rlast;
-          if (!full) mask_scores(ec.kt, t & 7, sv);
+          const bool full = kPacked ? !(ec.kt & kPackedMaskFlag)
+                                    : (ec.kt * kTile + kTile - 1 - a.base <= my_r0 && ec.emin >= my_rlast);
+          if (!full) {
+            if (kPacked) {
+              mask_scores_p(t & 7, sv);
+            } else {
+              mask_scores(ec.kt, t & 7, sv);
+            }
+          }
           const float mx = row_max(sv);
           if (__ballot(mx > m_run + kRescaleSlack)) rescale(mx);
           if (kUniform) {
@@ -1241,19 +1399,19 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_stream_kernel(P
   }
 }
 
-template <int D, bool kUniform>
+template <int D, bool kUniform, bool kPacked = false>
 static int launch_prefill_mfma(const PrefillArgs& a, int64_t n_wg, hipStream_t st) {
   static bool configured[kMaxDevices] = {};  // per instantiation; the attribute is set once per device
   const size_t smem = sizeof(PrefillSmem<D>);
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail(NATS_ERR_LAUNCH, "prefill: no current device");
   if (!configured[dev]) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_mfma_kernel<D, kUniform>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_mfma_kernel<D, kUniform, kPacked>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return fail(NATS_ERR_LAUNCH, "hipFuncSetAttribute(%zu bytes of LDS): %s", smem, hipGetErrorString(e));
     configured[dev] = true;
   }
-  hipLaunchKernelGGL((prefill_mfma_kernel<D, kUniform>), dim3((unsigned)n_wg), dim3(kPrefillWaves * kWave), smem, st, a);
+  hipLaunchKernelGGL((prefill_mfma_kernel<D, kUniform, kPacked>), dim3((unsigned)n_wg), dim3(kPrefillWaves * kWave), smem, st, a);
   NATS_CHECK_LAUNCH("prefill_mfma_kernel");
   return NATS_OK;
 }
@@ -1406,6 +1564,11 @@ bool use_stream_kernel() {
   return e && e[0] == '1';
 }
 
+bool use_packed_tiles() {
+  const char* e = getenv("NATS_PREFILL_PACKED");
+  return !(e && e[0] == '0');
+}
+
 // the schedule workspace behind the key-limit workspace, if the caller's buffer has room for it
 StreamSched sched_in_workspace(void* workspace, size_t workspace_bytes, size_t base_bytes, int64_t B, int64_t H_q,
                                int64_t H_kv, int64_t n_qt, int64_t N, int dtype) {
@@ -1424,7 +1587,7 @@ int launch_segment(const char* who, const SegmentShape& g, const void* q, const 
                    hipStream_t st) {
   PrefillArgs a{};
   a.q = q; a.k = k; a.v = v; a.o = o;
-  a.tok_lim = w.tok_lim; a.tile_lim = w.tile_lim;
+  a.tok_lim = w.tok_lim; a.tile_lim = w.tile_lim; a.gran_lim = w.gran_lim;
   a.qs_b = q_strides[0]; a.qs_h = q_strides[1]; a.qs_l = q_strides[2];
   a.ks_b = k_strides[0]; a.ks_h = k_strides[1]; a.ks_l = k_strides[2];
   a.vs_b = v_strides[0]; a.vs_h = v_strides[1]; a.vs_l = v_strides[2];
@@ -1462,6 +1625,10 @@ int launch_segment(const char* who, const SegmentShape& g, const void* q, const 
   a.xcd_mode = ((g.B * g.H_kv) % 8 == 0) ? 1 : 0;
   int64_t n_wg = g.B * g.H_kv * a.n_hg * a.n_qg;
   NATS_REQUIRE(n_wg < (int64_t(1) << 31), NATS_ERR_BAD_SHAPE, "%s: grid too large", who);
+  // chunks shorter than a tile: tiles are packed from the 16-row granules that are visible (NATS_PREFILL_PACKED=0
+  // in the environment keeps whole tiles, for comparison)
+  if (hpw == 4 && g.C < kTile && use_packed_tiles())
+    return g.D == 64 ? launch_prefill_mfma<64, true, true>(a, n_wg, st) : launch_prefill_mfma<128, true, true>(a, n_wg, st);
   if (hpw == 4 && sw.bytes != 0 && use_stream_kernel())
     return g.D == 64 ? launch_prefill_stream<64>(a, sw, st) : launch_prefill_stream<128>(a, sw, st);
   if (hpw == 4) return g.D == 64 ? launch_prefill_mfma<64, true>(a, n_wg, st) : launch_prefill_mfma<128, true>(a, n_wg, st);

@@ -174,11 +174,19 @@ __global__ __launch_bounds__(256) void key_lim_kernel(KeyLimArgs a) {
   }
   int32_t mx = lim, mn = row < a.N ? lim : kLimGlobal;
 #pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) {
+  for (int off = kGranule / 2; off >= 1; off >>= 1) {
+    mx = max(mx, __shfl_xor(mx, off));
+    mn = min(mn, __shfl_xor(mn, off));
+  }
+  if ((lane & (kGranule - 1)) == 0)
+    a.gran_lim[((int64_t)stream * a.Tk + tile) * (kTile / kGranule) + lane / kGranule] = make_int2(mx, mn);
+#pragma unroll
+  for (int off = 32; off >= kGranule; off >>= 1) {
     mx = max(mx, __shfl_xor(mx, off));
     mn = min(mn, __shfl_xor(mn, off));
   }
   if (lane == 0) a.tile_lim[(int64_t)stream * a.Tk + tile] = make_int2(mx, mn);
+  if (stream == 0 && tile == 0 && lane == 0) a.tok_lim[(int64_t)gridDim.y * a.N] = -1;
 }
 
 // token-level mask from the per-row limits: query i of the segment is region token r = r_begin + i
@@ -233,9 +241,11 @@ PrefillWorkspace carve_prefill_workspace(void* ws, int64_t n_streams, int64_t S,
   w.first_global = reinterpret_cast<int32_t*>(p + off);
   off += up((size_t)n_streams * sizeof(int32_t));
   w.tok_lim = reinterpret_cast<int32_t*>(p + off);
-  off += up((size_t)(n_streams * N) * sizeof(int32_t));
+  off += up((size_t)(n_streams * N + 1) * sizeof(int32_t));
   w.tile_lim = reinterpret_cast<int2*>(p + off);
   off += up((size_t)(n_streams * Tk) * sizeof(int2));
+  w.gran_lim = reinterpret_cast<int2*>(p + off);
+  off += up((size_t)(n_streams * Tk * (kTile / kGranule)) * sizeof(int2));
   w.bytes = off;
   return w;
 }
@@ -250,6 +260,7 @@ int prepare_key_limits(const uint8_t* roles, int64_t B, int64_t H_kv, int64_t S,
   a.first_global = w.first_global;
   a.tok_lim = w.tok_lim;
   a.tile_lim = w.tile_lim;
+  a.gran_lim = w.gran_lim;
   a.Hkv = (int)H_kv; a.S = (int)S; a.N = (int)N; a.Tk = (int)((N + kTile - 1) / kTile);
   a.c_shift = ilog2(C); a.C = (int)C; a.W = (int)W;
   if (past) {

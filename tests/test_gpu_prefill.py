@@ -95,26 +95,26 @@ def test_strided_inputs_and_drop_in_signature():
     assert np.array_equal(m.cpu().numpy(), mask)
 
 
-def test_cfg2_full_size_sampled_rows():
-    """L = 32768, Llama-3-8B head shape: full-size run checked on sampled query rows against a direct
-    per-row evaluation of the mask predicate, and on the all-global case against dense causal attention."""
+def check_sampled_rows(B, Hq, Hkv, L, D, C, W, n_samples=96, p=(0.05, 0.15, 0.8)):
+    """A run too large for the oracle's dense mask, checked on sampled query rows against a direct per-row
+    evaluation of the mask predicate."""
     from neuralattentionsearch_amd import ops
-    say("prefill cfg2 full size")
-    B, Hq, Hkv, L, D, C, W = 1, 32, 8, 32768, 128, 64, 256
     g = torch.Generator().manual_seed(0)
     q = (torch.randn(B, Hq, L, D, generator=g) / math.sqrt(D)).bfloat16()
     k = (torch.randn(B, Hkv, L, D, generator=g) / math.sqrt(D)).bfloat16()
     v = (torch.randn(B, Hkv, L, D, generator=g) / math.sqrt(D)).bfloat16()
-    S = L // C
-    roles = draw_roles(1, B, Hkv, S, p=(0.05, 0.15, 0.8))
+    S = -(-L // C)
+    roles = draw_roles(1, B, Hkv, S, p=p)
+    if L % C:
+        roles[:, :, -1] = 0
     out = ops.prefill_attention(q.cuda(), k.cuda(), v.cuda(), to_dev(roles), C, W).cpu().float()
     assert torch.isfinite(out).all()
     gidx = orc.next_global_index(roles == 0)
     rng = np.random.default_rng(7)
     worst = 0.0
-    for _ in range(96):
+    for i in range(n_samples):
         hq = int(rng.integers(Hq))
-        m = int(rng.integers(L)) if _ % 4 else L - 1 - int(rng.integers(64))
+        m = int(rng.integers(L)) if i % 4 else L - 1 - int(rng.integers(64))
         hkv = hq // (Hq // Hkv)
         mc = m // C
         n = np.arange(m + 1)
@@ -127,6 +127,89 @@ def test_cfg2_full_size_sampled_rows():
         want = torch.softmax(s, -1) @ v[0, hkv, idx].float()
         worst = max(worst, (out[0, hq, m] - want).abs().max().item())
     assert worst <= 2e-2, worst
+
+
+def test_cfg2_full_size_sampled_rows():
+    """L = 32768, Llama-3-8B head shape, chunk 64."""
+    say("prefill cfg2 full size")
+    check_sampled_rows(1, 32, 8, 32768, 128, 64, 256)
+
+
+@pytest.mark.parametrize("Hq,Hkv,L,C,W", [(32, 8, 32768, 32, 256),   # the chunk size of the reference's Llama adapter
+                                          (4, 1, 70016, 16, 64),      # 4376 granules: two windows of the tile list
+                                          (8, 2, 40000, 8, 16)])      # chunks shorter than a granule
+def test_packed_tiles_full_size_sampled_rows(Hq, Hkv, L, C, W):
+    """Chunks shorter than a 64-row tile: the kernel packs tiles from visible 16-row granules."""
+    say("prefill packed, sampled rows", Hq, Hkv, L, C, W)
+    check_sampled_rows(1, Hq, Hkv, L, 128, C, W, n_samples=64)
+
+
+@pytest.fixture
+def packed_tiles(monkeypatch):
+    def switch(on: bool):
+        monkeypatch.setenv("NATS_PREFILL_PACKED", "1" if on else "0")
+    yield switch
+    monkeypatch.delenv("NATS_PREFILL_PACKED", raising=False)
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,L,D,C,W,p", [
+    (1, 32, 8, 2048, 128, 32, 256, (0.05, 0.15, 0.8)),
+    (2, 8, 2, 1000, 128, 16, 64, (0.2, 0.3, 0.5)),     # ragged last query tile and last granule
+    (1, 16, 2, 777, 128, 8, 16, (0.2, 0.3, 0.5)),      # GQA group of 8, chunks of half a granule
+    (2, 8, 2, 2048, 64, 32, 128, (0.1, 0.1, 0.8)),     # head_dim 64
+    (1, 8, 2, 3000, 128, 1, 64, (0.1, 0.2, 0.7)),      # per-token roles
+    (1, 8, 2, 1500, 128, 16, 64, (0.0, 0.0, 1.0)),     # sliding window only
+    (1, 8, 2, 1500, 128, 16, 64, (1.0, 0.0, 0.0)),     # dense: every granule is visible
+])
+def test_packed_tiles_agree_with_whole_tiles(packed_tiles, B, Hq, Hkv, L, D, C, W, p):
+    """The same scores reach the softmax in another order: the two kernels agree to rounding."""
+    from neuralattentionsearch_amd import ops
+    say("prefill packed vs whole tiles", B, Hq, Hkv, L, D, C, W, p)
+    g = torch.Generator().manual_seed(L + C)
+    q = torch.randn(B, Hq, L, D, generator=g).bfloat16().cuda()
+    k = torch.randn(B, Hkv, L, D, generator=g).bfloat16().cuda()
+    v = torch.randn(B, Hkv, L, D, generator=g).bfloat16().cuda()
+    roles = draw_roles(L, B, Hkv, -(-L // C), p=p)
+    if L % C:
+        roles[:, :, -1] = 0
+    roles = to_dev(roles)
+    packed_tiles(False)
+    whole = ops.prefill_attention(q, k, v, roles, C, W).float()
+    packed_tiles(True)
+    packed = ops.prefill_attention(q, k, v, roles, C, W).float()
+    assert torch.isfinite(packed).all()
+    assert (packed - whole).abs().max().item() <= 2e-2
+
+
+def test_packed_tiles_on_segments_over_a_filled_cache(packed_tiles):
+    """Rows an earlier segment left in the cache (ring, kept globals and locals, stale rows) as granules."""
+    from neuralattentionsearch_amd import ops
+    from neuralattentionsearch_amd.cache import NAtSChunkLayerCache
+    say("prefill packed, segments over a filled cache")
+    B, Hq, Hkv, D, C, W = 1, 8, 2, 128, 16, 64
+    outs = []
+    for on in (False, True):
+        packed_tiles(on)
+        gg = torch.Generator().manual_seed(3)
+        cache = NAtSChunkLayerCache(B, Hkv, W, chunk_size=C, device="cuda")
+        res = []
+        for n, seed in ((700, 1), (333, 2), (150, 3), (1000, 4)):
+            q = torch.randn(B, Hq, n, D, generator=gg).bfloat16().cuda()
+            k = torch.randn(B, Hkv, n, D, generator=gg).bfloat16().cuda()
+            v = torch.randn(B, Hkv, n, D, generator=gg).bfloat16().cuda()
+            S = math.ceil((cache.chunk_fill_size + n) / C)
+            roles = draw_roles(seed, B, Hkv, S, p=(0.2, 0.3, 0.5))
+            if (cache.chunk_fill_size + n) % C:
+                roles[:, :, -1] = 0
+            tsi = orc.one_hot_roles(roles).bfloat16().cuda()
+            first = cache.get_seq_length() == 0
+            kk, vv = cache.update(k, v, tsi)
+            res.append((ops.prefill_attention(q, kk, vv, to_dev(roles), C, W) if first else cache.segment_attention(q)).float())
+            cache.post_update(n)
+        outs.append(res)
+    for x, y in zip(*outs):
+        assert torch.isfinite(y).all()
+        assert (x - y).abs().max().item() <= 2e-2
 
 
 # ---- the persistent kernel (opt in: NATS_PREFILL_STREAM=1) -------------------------------------------------
