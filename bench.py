@@ -105,7 +105,7 @@ def time_gpu(fn, steps: int, warmup: int):
 
 # --------------------------------------------------------------------------------------------------
 def bench_prefill(args, ops):
-    B, Hq, Hkv, L, D, C, W = 1, 32, 8, args.prefill_len, 128, 64, 256
+    B, Hq, Hkv, L, D, C, W = 1, 32, 8, args.prefill_len, 128, args.chunk_size, 256
     n_rep = Hq // Hkv
     dev = "cuda"
     g = torch.Generator(device=dev).manual_seed(0)
@@ -482,6 +482,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--prefill-len", type=int, default=32768)
+    ap.add_argument("--chunk-size", type=int, default=64, help="chunk size of the prefill leg (the headline uses 64)")
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--no-compare", action="store_true", help="skip the dense comparators of the prefill leg")
     ap.add_argument("--segments", type=int, default=4, help="segments of the `--only segments` leg")
@@ -535,13 +536,13 @@ def main():
         "ms_per_step": pre["ms"] if pre else None,
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": f"prefill B=1 Hq=32 Hkv=8 D=128 L={args.prefill_len} chunk 64 window 256, roles 5/15/80 "
+        "config": {"workload": f"prefill B=1 Hq=32 Hkv=8 D=128 L={args.prefill_len} chunk {args.chunk_size} window 256, roles 5/15/80 "
                                "(global/local/sliding); decode and compaction ride along under their own keys"},
     }
     if pre:
         line["roofline"] = {"bound": "mfma", "achieved": pre["tflops_visited"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                             "frac": pre["tflops_visited"] / PEAK_BF16_TFLOPS,
-                            "traffic": MEASURED_TRAFFIC["prefill"] if args.prefill_len == 32768 else None,
+                            "traffic": MEASURED_TRAFFIC["prefill"] if args.prefill_len == 32768 and args.chunk_size == 64 else None,
                             "kernel": "prefill_mfma_kernel<128, true>"}
     if "decode" in res:
         d = res["decode"]
