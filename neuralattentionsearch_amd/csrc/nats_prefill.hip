@@ -195,13 +195,13 @@ constexpr int kPackedMaskFlag = 1 << 30;  // on the first granule id of a packed
 // kUniform: the wavefronts are the q heads of ONE query tile (GQA groups of 4 and more), so every tile of
 // the visit list is visited by every wavefront and the tile loop has no per-wavefront branches.
 // kPacked (with kUniform, for chunks shorter than a tile): a tile is assembled from four 16-row granules taken
-// from anywhere in the key rows.  Granules no query of the tile sees are left out, granules every query sees
-// without a mask are packed among themselves and the rest (diagonal, partly visible, the remainder of the
+// from anywhere in the key rows.  Granules no query of the workgroup sees are left out, granules every query of
+// the workgroup sees without a mask are packed among themselves and the rest (diagonal, partly visible, the remainder of the
 // first kind, padding) into tiles that go through the element mask.  The softmax does not care about the order
 // of the keys, so nothing else changes; without it a tile with one visible 16- or 32-row chunk costs a whole tile.
 template <int D, bool kUniform, bool kPacked = false>
 __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(PrefillArgs a) {
-  static_assert(!kPacked || kUniform, "packed tiles are built for one query tile per workgroup");
+  static_assert(!kPacked || kUniform, "packed tiles are walked by every wavefront of the workgroup");
   constexpr int OCT = D / 8;                          // 16-byte chunks per row
   constexpr int DMA_PER_WAVE = OCT / kPrefillWaves;   // 1 KiB global->LDS transfers per wavefront and tensor
   constexpr int DSTEPS = D / 16;
@@ -1627,7 +1627,9 @@ int launch_segment(const char* who, const SegmentShape& g, const void* q, const 
   NATS_REQUIRE(n_wg < (int64_t(1) << 31), NATS_ERR_BAD_SHAPE, "%s: grid too large", who);
   // chunks shorter than a tile: tiles are packed from the 16-row granules that are visible (NATS_PREFILL_PACKED=0
   // in the environment keeps whole tiles, for comparison)
-  if (hpw == 4 && g.C < kTile && use_packed_tiles())
+  // (GQA groups of 1 and 2: the workgroup's 2 or 4 query tiles form one group for the packing, every wavefront
+  // walks the whole list and the element mask sorts out what its own rows see)
+  if (g.C < kTile && use_packed_tiles())
     return g.D == 64 ? launch_prefill_mfma<64, true, true>(a, n_wg, st) : launch_prefill_mfma<128, true, true>(a, n_wg, st);
   if (hpw == 4 && sw.bytes != 0 && use_stream_kernel())
     return g.D == 64 ? launch_prefill_stream<64>(a, sw, st) : launch_prefill_stream<128>(a, sw, st);

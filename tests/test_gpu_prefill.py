@@ -43,6 +43,7 @@ def test_fp32_ragged_lengths_and_chunk_sizes(L, C, W, D):
 @pytest.mark.parametrize("n_rep", [1, 2, 4, 8])
 def test_bf16_gqa_group_sizes(n_rep):
     run_case(1, 2 * n_rep, 2, 1024, 128, 64, 256, torch.bfloat16, seed=n_rep)
+    run_case(1, 2 * n_rep, 2, 1100, 128, 16, 64, torch.bfloat16, seed=n_rep)  # packed tiles
 
 
 @pytest.mark.parametrize("L,C,W,D", [(1000, 64, 256, 128), (777, 32, 64, 128), (512, 16, 64, 64), (2048, 64, 128, 64),
@@ -160,6 +161,8 @@ def packed_tiles(monkeypatch):
     (1, 8, 2, 3000, 128, 1, 64, (0.1, 0.2, 0.7)),      # per-token roles
     (1, 8, 2, 1500, 128, 16, 64, (0.0, 0.0, 1.0)),     # sliding window only
     (1, 8, 2, 1500, 128, 16, 64, (1.0, 0.0, 0.0)),     # dense: every granule is visible
+    (2, 4, 4, 1500, 128, 32, 128, (0.1, 0.2, 0.7)),    # one q head per kv head: four query tiles per workgroup
+    (1, 8, 4, 2000, 64, 8, 16, (0.1, 0.2, 0.7)),       # groups of 2, head_dim 64
 ])
 def test_packed_tiles_agree_with_whole_tiles(packed_tiles, B, Hq, Hkv, L, D, C, W, p):
     """The same scores reach the softmax in another order: the two kernels agree to rounding."""
