@@ -262,6 +262,8 @@ struct ApplyArgs {
   int elem_bytes;
   int rs;                    // rows per slice
   int n_slices;
+  int chunks_per_wg;         // out-of-place only: destination chunks per workgroup
+  int64_t n_chunks;          // out-of-place only: destination chunks per head
 };
 
 // A tensor seen as units of type U: row `r` of head `head` starts at base + r * row_stride, holds upr units.
@@ -420,11 +422,11 @@ __global__ __launch_bounds__(256) void evict_apply_inplace_kernel(ApplyArgs a) {
   }
 }
 
-// Out of place, first prefill: destination chunk blockIdx.x of head blockIdx.y.
+// Out of place, first prefill: destination chunks [blockIdx.x * chunks_per_wg, +chunks_per_wg) of head blockIdx.y
+// (several chunks per workgroup when a chunk is shorter than 32 rows, so that a workgroup moves 16 KiB).
 __global__ __launch_bounds__(256) void evict_apply_first_kernel(ApplyArgs a) {
   const nats_evict_params& p = a.p;
   const int tid = threadIdx.x;
-  const int64_t ci = blockIdx.x;
   const int head = blockIdx.y;
   const int which = blockIdx.z;
   const int b = head / (int)p.H_kv, h = head % (int)p.H_kv;
@@ -443,6 +445,8 @@ __global__ __launch_bounds__(256) void evict_apply_first_kernel(ApplyArgs a) {
   const int count = res.all_local ? 0 : hp.count;
   const bool tail_move = !res.all_local && partial && res.max_keep < S - 1;
 
+  const int64_t ci_end = min((int64_t)(blockIdx.x + 1) * a.chunks_per_wg, a.n_chunks);
+  for (int64_t ci = (int64_t)blockIdx.x * a.chunks_per_wg; ci < ci_end; ++ci) {
   // where the rows of this destination chunk come from: a source chunk of the raw prefill tensor
   // (-1 = zeros); the untouched part of [W zeros | K | pad] keeps its own rows
   int64_t src_chunk;
@@ -514,6 +518,7 @@ __global__ __launch_bounds__(256) void evict_apply_first_kernel(ApplyArgs a) {
       a.size_local[head] = sl_new;
     }
   }
+  }  // chunks of this workgroup
 }
 
 static int check_params(const char* who, const nats_evict_params* p) {
@@ -640,7 +645,9 @@ extern "C" int nats_evict_apply_first(const void* src_k, const void* src_v, void
   a.ss_b = src_strides[0]; a.ss_h = src_strides[1]; a.ss_r = src_strides[2];
   a.vs_b = valid_strides[0]; a.vs_h = valid_strides[1];
   a.elem_bytes = elem_bytes; a.rs = 0; a.n_slices = 0;
-  dim3 grid((unsigned)(params->n_alloc / params->C), (unsigned)(params->B * params->H_kv), pos ? 3u : 2u);
+  a.n_chunks = params->n_alloc / params->C;
+  a.chunks_per_wg = params->C >= 32 ? 1 : (int)(64 / params->C);
+  dim3 grid((unsigned)((a.n_chunks + a.chunks_per_wg - 1) / a.chunks_per_wg), (unsigned)(params->B * params->H_kv), pos ? 3u : 2u);
   hipLaunchKernelGGL(evict_apply_first_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream), a);
   NATS_CHECK_LAUNCH("evict_apply_first_kernel");
   return NATS_OK;
