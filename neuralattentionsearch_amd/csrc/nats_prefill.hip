@@ -359,13 +359,18 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
   auto issue_k_p = [&](int id0, int id1, int id2, int id3, int buf, int slot) {
     issue_rows_p(kp, a.ks_l, koff, sm.k[buf], granule_of(id0, id1, id2, id3, wave >> 1), false);
     if ((id0 & kPackedMaskFlag) && wave == 0) {
-      // limits and region tokens of the 64 rows, for the element mask (asynchronous like the tile itself)
-      const int gid = granule_of(id0, id1, id2, id3, lane >> 4);
-      const int row = gid * kGranule + (lane & (kGranule - 1));
+      // limits and region tokens of the 64 rows, for the element mask (asynchronous like the tile itself).
+      // (The lane id is taken afresh so that nothing derived from it has to live across the tile loop.)
+      int ln = lane;
+#if defined(__HIP_DEVICE_COMPILE__)
+      asm volatile("" : "+v"(ln));
+#endif
+      const int gid = granule_of(id0, id1, id2, id3, ln >> 4);
+      const int row = gid * kGranule + (ln & (kGranule - 1));
       const bool real = gid >= 0 && row < a.N;
       const int32_t* src = real ? lim + row : a.tok_lim + (int64_t)a.B * a.Hkv * a.N;  // (the entry that holds -1)
       __builtin_amdgcn_global_load_lds(src, (uint32_t __attribute__((address_space(3)))*)(&sm.limk[slot][0]), 4, 0, 0);
-      sm.posk[slot][lane] = real ? row - a.base : 0x7fffffff;
+      sm.posk[slot][ln] = real ? row - a.base : 0x7fffffff;
     }
   };
   auto issue_v_p = [&](int id0, int id1, int id2, int id3, int buf) {
