@@ -375,7 +375,7 @@ def bench_llama(args):
     """End to end at the Llama-3-8B shape with random weights: one prefill, then greedy decode steps with
     eviction live in all 32 layers."""
     from neuralattentionsearch_amd.llama import NAtSLlamaConfig, NAtSLlamaForCausalLM
-    cfg = NAtSLlamaConfig.llama3_8b()
+    cfg = NAtSLlamaConfig.llama3_8b(fused_role_step=True)
     model = NAtSLlamaForCausalLM.random_init(cfg, seed=0)
     g = torch.Generator().manual_seed(0)
     ids = torch.randint(0, cfg.vocab_size, (1, args.llama_prefill), generator=g).cuda()

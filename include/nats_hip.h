@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define NATS_ABI_VERSION 4
+#define NATS_ABI_VERSION 5
 
 typedef enum {
   NATS_OK = 0,
@@ -300,6 +300,17 @@ int nats_silu_mul(const void* gate_up, void* out, int64_t rows, int64_t inter, i
  */
 int nats_matvec(const void* w, const void* x, void* y, int64_t x_rows, int64_t n_out, int64_t k, int64_t w_stride,
                 int64_t x_stride, int64_t y_stride, int gate, int dtype, void* stream);
+
+/* Rotary embedding of q and k of a multi-token segment (transformers' apply_rotary_pos_emb as called at
+ * hf/llama_nats_chunk.py:227: q * cos + rotate_half(q) * sin, every product and the sum rounded to the dtype):
+ *   q_out [B, H_q, x_len, D] and k_out [B, H_kv, x_len, D] contiguous
+ *   q [B, H_q, x_len, D], k [B, H_kv, x_len, D]: strides (b, h, l), last dimension contiguous (the transposed views of
+ *   a [B, x_len, heads, D] projection are taken as they are); cos / sin [B, x_len, D]: strides (b, l)
+ *   D a multiple of 32 bytes, every row 16-byte aligned
+ */
+int nats_rope_qk(const void* q, const void* k, const void* cos, const void* sin, void* q_out, void* k_out, int64_t B,
+                 int64_t H_q, int64_t H_kv, int64_t x_len, int64_t D, const int64_t* q_strides, const int64_t* k_strides,
+                 const int64_t* cos_strides, int dtype, void* stream);
 
 /* Rotary embedding of q and k (transformers' apply_rotary_pos_emb, hf/llama_nats_chunk.py:227) and the row
  * write of NAtSChunkLayerCache.update (components/cache/nats_chunk_layer_cache.py:243-256) in one launch:

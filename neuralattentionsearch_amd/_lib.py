@@ -19,7 +19,7 @@ c_i64p = ctypes.POINTER(ctypes.c_int64)
 NATS_DTYPE_BF16 = 0
 NATS_DTYPE_F32 = 1
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 
 class EvictParams(ctypes.Structure):
@@ -73,6 +73,7 @@ SIGNATURES = {
                                          ctypes.c_int, c_p]),
     "nats_silu_mul": (ctypes.c_int, [c_p, c_p, c_i64, c_i64, ctypes.c_int, c_p]),
     "nats_matvec": (ctypes.c_int, [c_p, c_p, c_p] + [c_i64] * 6 + [ctypes.c_int, ctypes.c_int, c_p]),
+    "nats_rope_qk": (ctypes.c_int, [c_p] * 6 + [c_i64] * 5 + [c_i64p] * 3 + [ctypes.c_int, c_p]),
     "nats_rope_append": (ctypes.c_int, [c_p] * 10 + [c_i64] * 8 + [c_i64p] * 6 + [ctypes.c_int, c_p]),
 }
 

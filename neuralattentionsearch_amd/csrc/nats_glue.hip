@@ -152,17 +152,21 @@ __global__ __launch_bounds__(kNormThreads) void add_rms_norm_kernel(AddNormArgs 
   }
 }
 
-template <bool kBf16>
+// VEC consecutive columns per thread (16-byte loads and stores when the rows allow it, else 1)
+template <bool kBf16, int VEC>
 __global__ __launch_bounds__(256) void silu_mul_kernel(const void* __restrict__ gate_up, void* __restrict__ out, int64_t rows,
                                                         int inter) {
+  const int per_row = inter / VEC;
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= rows * inter) return;
-  const int64_t r = i / inter;
-  const int c = (int)(i - r * inter);
-  const float g = g_load<kBf16>(gate_up, r * 2 * inter + c);
-  const float u = g_load<kBf16>(gate_up, r * 2 * inter + inter + c);
-  const float s = g_round<kBf16>(g / (1.f + expf(-g)));
-  g_store<kBf16>(out, i, s * u);
+  if (i >= rows * per_row) return;
+  const int64_t r = i / per_row;
+  const int c = (int)(i - r * per_row) * VEC;
+  float g[VEC], u[VEC], y[VEC];
+  load_vec<kBf16, VEC>(gate_up, r * 2 * inter + c, g);
+  load_vec<kBf16, VEC>(gate_up, r * 2 * inter + inter + c, u);
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) y[e] = g_round<kBf16>(g[e] / (1.f + expf(-g[e]))) * u[e];
+  store_vec<kBf16, VEC>(out, r * inter + c, y);
 }
 
 // ---- y[r, n] = sum_k x[r, k] * w[n, k] for a few rows of x (the projections of a one-token step) --------------
@@ -338,6 +342,81 @@ __global__ void rope_append_kernel(RopeAppendArgs a) {
   }
 }
 
+// ---- rotary embedding of q and k of a multi-token segment (no cache write) -------------------------------------
+// One thread rotates VEC consecutive dims of the first half of a head vector and their partners in the second
+// half (16-byte loads and stores); a block of 256 threads takes 256 / (D / (2 VEC)) head vectors, ordered
+// (b, l, head) as the projection output lies in memory.  Same rounding points as rope_append_kernel.
+struct RopeQkArgs {
+  const void *q, *k, *cos, *sin;
+  void *q_out, *k_out;
+  int64_t qs[3], ks[3];  // strides (b, h, l) of q, k; last dim contiguous
+  int64_t cs[2];         // strides (b, l) of cos / sin
+  int Hq, Hkv, x_len, D;
+  int64_t n_vec;         // head vectors in all: B * x_len * (Hq + Hkv)
+};
+
+template <bool kBf16>
+__global__ __launch_bounds__(256) void rope_qk_kernel(RopeQkArgs a) {
+#pragma clang fp contract(off)
+  constexpr int VEC = kBf16 ? 8 : 4;
+  const int tpv = a.D / (2 * VEC);  // threads per head vector
+  const int64_t vec = (int64_t)blockIdx.x * (256 / tpv) + threadIdx.x / tpv;
+  if (threadIdx.x >= (256 / tpv) * tpv || vec >= a.n_vec) return;
+  const int d = (threadIdx.x % tpv) * VEC;
+  const int half = a.D / 2;
+  const int H = a.Hq + a.Hkv;
+  const int hh = (int)(vec % H);
+  const int64_t bl = vec / H;
+  const int l = (int)(bl % a.x_len), b = (int)(bl / a.x_len);
+  const bool is_q = hh < a.Hq;
+  const int h = is_q ? hh : hh - a.Hq;
+  const void* src = is_q ? a.q : a.k;
+  const int64_t* st = is_q ? a.qs : a.ks;
+  const int64_t s0 = b * st[0] + h * st[1] + l * st[2];
+  const int64_t c0 = b * a.cs[0] + l * a.cs[1];
+  float lo[VEC], hi[VEC], c_lo[VEC], c_hi[VEC], s_lo[VEC], s_hi[VEC], y_lo[VEC], y_hi[VEC];
+  if (kBf16) {
+    float t8[8];
+    load_vec<true, 8>(src, s0 + d, t8);
+    for (int e = 0; e < VEC; ++e) lo[e] = t8[e];
+    load_vec<true, 8>(src, s0 + d + half, t8);
+    for (int e = 0; e < VEC; ++e) hi[e] = t8[e];
+    load_vec<true, 8>(a.cos, c0 + d, t8);
+    for (int e = 0; e < VEC; ++e) c_lo[e] = t8[e];
+    load_vec<true, 8>(a.cos, c0 + d + half, t8);
+    for (int e = 0; e < VEC; ++e) c_hi[e] = t8[e];
+    load_vec<true, 8>(a.sin, c0 + d, t8);
+    for (int e = 0; e < VEC; ++e) s_lo[e] = t8[e];
+    load_vec<true, 8>(a.sin, c0 + d + half, t8);
+    for (int e = 0; e < VEC; ++e) s_hi[e] = t8[e];
+  } else {
+    const auto ld4 = [](const void* p, int64_t i, float (&v)[VEC]) {
+      const float4 r = *reinterpret_cast<const float4*>(static_cast<const float*>(p) + i);
+      v[0] = r.x; v[1] = r.y; v[2] = r.z; v[3] = r.w;
+    };
+    ld4(src, s0 + d, lo); ld4(src, s0 + d + half, hi);
+    ld4(a.cos, c0 + d, c_lo); ld4(a.cos, c0 + d + half, c_hi);
+    ld4(a.sin, c0 + d, s_lo); ld4(a.sin, c0 + d + half, s_hi);
+  }
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) {
+    y_lo[e] = g_round<kBf16>(lo[e] * c_lo[e]) + g_round<kBf16>(-hi[e] * s_lo[e]);
+    y_hi[e] = g_round<kBf16>(hi[e] * c_hi[e]) + g_round<kBf16>(lo[e] * s_hi[e]);
+  }
+  void* dst = is_q ? a.q_out : a.k_out;
+  const int64_t o0 = (((int64_t)b * (is_q ? a.Hq : a.Hkv) + h) * a.x_len + l) * a.D;
+  if (kBf16) {
+    float t8[8];
+    for (int e = 0; e < VEC; ++e) t8[e] = y_lo[e];
+    store_vec<true, 8>(dst, o0 + d, t8);
+    for (int e = 0; e < VEC; ++e) t8[e] = y_hi[e];
+    store_vec<true, 8>(dst, o0 + d + half, t8);
+  } else {
+    *reinterpret_cast<float4*>(static_cast<float*>(dst) + o0 + d) = make_float4(y_lo[0], y_lo[1], y_lo[2], y_lo[3]);
+    *reinterpret_cast<float4*>(static_cast<float*>(dst) + o0 + d + half) = make_float4(y_hi[0], y_hi[1], y_hi[2], y_hi[3]);
+  }
+}
+
 }  // namespace nats
 
 using namespace nats;
@@ -378,11 +457,21 @@ extern "C" int nats_silu_mul(const void* gate_up, void* out, int64_t rows, int64
                "nats_silu_mul: rows=%lld inter=%lld", (long long)rows, (long long)inter);
   NATS_REQUIRE(dtype == NATS_DTYPE_BF16 || dtype == NATS_DTYPE_F32, NATS_ERR_BAD_DTYPE, "nats_silu_mul: dtype %d", dtype);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  const unsigned blocks = (unsigned)((rows * inter + 255) / 256);
+  const bool wide = inter % 8 == 0 && ((reinterpret_cast<uintptr_t>(gate_up) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+  const int64_t n_threads = wide ? rows * (inter / 8) : rows * inter;
+  const unsigned blocks = (unsigned)((n_threads + 255) / 256);
   if (dtype == NATS_DTYPE_BF16) {
-    hipLaunchKernelGGL(silu_mul_kernel<true>, dim3(blocks), dim3(256), 0, st, gate_up, out, rows, (int)inter);
+    if (wide) {
+      hipLaunchKernelGGL((silu_mul_kernel<true, 8>), dim3(blocks), dim3(256), 0, st, gate_up, out, rows, (int)inter);
+    } else {
+      hipLaunchKernelGGL((silu_mul_kernel<true, 1>), dim3(blocks), dim3(256), 0, st, gate_up, out, rows, (int)inter);
+    }
   } else {
-    hipLaunchKernelGGL(silu_mul_kernel<false>, dim3(blocks), dim3(256), 0, st, gate_up, out, rows, (int)inter);
+    if (wide) {
+      hipLaunchKernelGGL((silu_mul_kernel<false, 8>), dim3(blocks), dim3(256), 0, st, gate_up, out, rows, (int)inter);
+    } else {
+      hipLaunchKernelGGL((silu_mul_kernel<false, 1>), dim3(blocks), dim3(256), 0, st, gate_up, out, rows, (int)inter);
+    }
   }
   NATS_CHECK_LAUNCH("silu_mul_kernel");
   return NATS_OK;
@@ -476,5 +565,43 @@ extern "C" int nats_rope_append(const void* q, const void* k, const void* v, con
     hipLaunchKernelGGL(rope_append_kernel<false>, grid, dim3(threads), 0, st, a);
   }
   NATS_CHECK_LAUNCH("rope_append_kernel");
+  return NATS_OK;
+}
+
+extern "C" int nats_rope_qk(const void* q, const void* k, const void* cos, const void* sin, void* q_out, void* k_out, int64_t B,
+                            int64_t H_q, int64_t H_kv, int64_t x_len, int64_t D, const int64_t* q_strides,
+                            const int64_t* k_strides, const int64_t* cos_strides, int dtype, void* stream) {
+  NATS_REQUIRE(q && k && cos && sin && q_out && k_out && q_strides && k_strides && cos_strides, NATS_ERR_NULL_POINTER,
+               "nats_rope_qk: NULL pointer");
+  NATS_REQUIRE(dtype == NATS_DTYPE_BF16 || dtype == NATS_DTYPE_F32, NATS_ERR_BAD_DTYPE, "nats_rope_qk: dtype %d", dtype);
+  const int64_t vec = dtype == NATS_DTYPE_BF16 ? 8 : 4;
+  NATS_REQUIRE(B > 0 && H_q > 0 && H_kv > 0 && x_len > 0 && B * x_len * (H_q + H_kv) < (int64_t(1) << 40), NATS_ERR_BAD_SHAPE,
+               "nats_rope_qk: B=%lld H_q=%lld H_kv=%lld x_len=%lld", (long long)B, (long long)H_q, (long long)H_kv,
+               (long long)x_len);
+  NATS_REQUIRE(D > 0 && D % (2 * vec) == 0 && D <= 512, NATS_ERR_UNSUPPORTED, "nats_rope_qk: head_dim %lld", (long long)D);
+  bool aligned = ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(cos) |
+                   reinterpret_cast<uintptr_t>(sin) | reinterpret_cast<uintptr_t>(q_out) | reinterpret_cast<uintptr_t>(k_out)) & 15) == 0;
+  for (int i = 0; i < 3; ++i) aligned = aligned && q_strides[i] % vec == 0 && k_strides[i] % vec == 0;
+  for (int i = 0; i < 2; ++i) aligned = aligned && cos_strides[i] % vec == 0;
+  NATS_REQUIRE(aligned, NATS_ERR_BAD_SHAPE, "nats_rope_qk: rows must be 16-byte aligned");
+  RopeQkArgs a{};
+  a.q = q; a.k = k; a.cos = cos; a.sin = sin; a.q_out = q_out; a.k_out = k_out;
+  for (int i = 0; i < 3; ++i) {
+    a.qs[i] = q_strides[i]; a.ks[i] = k_strides[i];
+  }
+  a.cs[0] = cos_strides[0]; a.cs[1] = cos_strides[1];
+  a.Hq = (int)H_q; a.Hkv = (int)H_kv; a.x_len = (int)x_len; a.D = (int)D;
+  a.n_vec = B * x_len * (H_q + H_kv);
+  const int tpv = (int)(D / (2 * vec));
+  const int64_t per_block = 256 / tpv;
+  const int64_t blocks = (a.n_vec + per_block - 1) / per_block;
+  NATS_REQUIRE(blocks < (int64_t(1) << 31), NATS_ERR_BAD_SHAPE, "nats_rope_qk: grid too large");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == NATS_DTYPE_BF16) {
+    hipLaunchKernelGGL(rope_qk_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, st, a);
+  } else {
+    hipLaunchKernelGGL(rope_qk_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, st, a);
+  }
+  NATS_CHECK_LAUNCH("rope_qk_kernel");
   return NATS_OK;
 }

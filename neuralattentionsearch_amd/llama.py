@@ -10,10 +10,11 @@ Differences from BaseNAtSChunkAttentionLayer that this twin has and that are kep
 logit (:206-214 takes the plain maximum) and `position_ids[0, 0] == 0` decides between the prefill kernel
 and the cached paths (:194, :238-270).
 
-One-token steps take a shorter route through the same arithmetic (`fused_decode`): q / k / v and gate / up are
-one GEMM each over merged weights (the separate `*_proj.weight` parameters are views of them), the residual add,
-RMSNorm and the running chunk statistic are one kernel, the rotary embedding and the cache append another, the
-SiLU gate a third, so that a decoder layer is about a dozen launches.
+With `fused_decode` (the default) the same arithmetic takes a shorter route: q / k / v and gate / up are one
+projection each over merged weights (the separate `*_proj.weight` parameters are views of them), the residual add
+and RMSNorm (and, for the token of an open chunk, the running chunk statistic) are one kernel, the rotary
+embedding another (fused with the cache append for a one-token step), the SiLU gate a third; one-token steps run
+their projections through the matrix-vector kernel, so that a decoder layer is about a dozen launches.
 
 Weights are random-initialised (there is no checkpoint loader here); `NAtSLlamaConfig.llama3_8b()` gives the
 Llama-3-8B shape.
@@ -45,7 +46,7 @@ class NAtSLlamaConfig:
     local_seq_max_length: int = 256  # sliding window, in tokens
     chunk_merge_method: str = "mean"
     fused_role_step: bool = False  # pooling + role projection + argmax in one kernel instead of torch ops
-    fused_decode: bool = True      # one-token steps: fused norm / rotary + append / gate kernels, merged projections
+    fused_decode: bool = True      # fused norm / rotary / gate kernels and merged projections (one-token steps and segments)
 
     @property
     def head_dim(self) -> int:
@@ -204,14 +205,19 @@ class NAtSLlamaAttention(nn.Module):
         return step_linear(out.transpose(1, 2).reshape(bsz, 1, -1), self.o_proj)
 
     def forward(self, hidden_states: torch.Tensor, position_embeddings, start_pos: int, past_key_value: NAtSCache,
-                fused_decode: bool = False, statistic_done: bool = False):
+                fused_decode: bool = False, statistic_done: bool = False, fused_segment: bool = False):
         bsz, q_len, _ = hidden_states.shape
         C, idx = self.chunk_size, self.layer_idx
         if fused_decode:
             return self._decode_one(hidden_states, position_embeddings, start_pos, past_key_value, statistic_done)
-        q = self.q_proj(hidden_states).view(bsz, q_len, self.num_heads, self.head_dim).transpose(1, 2)
-        k = self.k_proj(hidden_states).view(bsz, q_len, self.num_key_value_heads, self.head_dim).transpose(1, 2)
-        v = self.v_proj(hidden_states).view(bsz, q_len, self.num_key_value_heads, self.head_dim).transpose(1, 2)
+        if fused_segment and self.fused_ok():  # one GEMM over the merged matrix; q / k / v are views of its output
+            Hq, Hkv, D = self.num_heads, self.num_key_value_heads, self.head_dim
+            qkv = nn.functional.linear(hidden_states, self.qkv_weight).view(bsz, q_len, Hq + 2 * Hkv, D).transpose(1, 2)
+            q, k, v = qkv[:, :Hq], qkv[:, Hq:Hq + Hkv], qkv[:, Hq + Hkv:]
+        else:
+            q = self.q_proj(hidden_states).view(bsz, q_len, self.num_heads, self.head_dim).transpose(1, 2)
+            k = self.k_proj(hidden_states).view(bsz, q_len, self.num_key_value_heads, self.head_dim).transpose(1, 2)
+            v = self.v_proj(hidden_states).view(bsz, q_len, self.num_key_value_heads, self.head_dim).transpose(1, 2)
 
         pre_fill = past_key_value.get_nats_chunk_fill_size(idx)
         is_pre_filling = start_pos == 0
@@ -238,7 +244,10 @@ class NAtSLlamaAttention(nn.Module):
             roles, tsi = ops.roles_from_logits(logit, 0.0, force_first_global=start_pos < C, force_last_global=pad != 0)
 
         cos, sin = position_embeddings
-        q, k = apply_rotary_pos_emb(q, k, cos, sin)
+        if fused_segment and ops.rope_qk_ok(q, k, cos, sin):
+            q, k = ops.rope_qk(q, k, cos, sin)
+        else:
+            q, k = apply_rotary_pos_emb(q, k, cos, sin)
         keys, values = past_key_value.update(k, v, idx, cache_kwargs={"token_states_info": tsi})
         layer = past_key_value.cache_model[idx]
         scale = 1.0 / math.sqrt(self.head_dim)
@@ -265,6 +274,14 @@ class NAtSLlamaDecoderLayer(nn.Module):
     def forward(self, x, position_embeddings, start_pos: int, cache: NAtSCache):
         x = x + self.self_attn(self.input_layernorm(x), position_embeddings, start_pos, cache)
         return x + self.mlp(self.post_attention_layernorm(x))
+
+    def segment_step(self, x, delta, position_embeddings, start_pos: int, cache: NAtSCache):
+        """A multi-token segment with the fused norm, rotary and gate kernels and the merged projections; `x` and
+        `delta` as in `decode_step`."""
+        h = ops.add_rms_norm(x, delta, self.input_layernorm.weight, self.input_layernorm.eps)
+        att = self.self_attn(h, position_embeddings, start_pos, cache, fused_segment=True)
+        h = ops.add_rms_norm(x, att, self.post_attention_layernorm.weight, self.post_attention_layernorm.eps)
+        return self.mlp.forward_fused(h)
 
     def decode_step(self, x, delta, position_embeddings, start_pos: int, cache: NAtSCache):
         """One token.  `x` [B, 1, dim] is the residual stream, updated in place; `delta` is the branch output of the
@@ -335,6 +352,16 @@ class NAtSLlamaForCausalLM(nn.Module):
             for layer in self.layers:
                 delta = layer.decode_step(x, delta, position_embeddings, start_pos, cache)
             return step_linear(ops.add_rms_norm(x, delta, self.norm.weight, self.norm.eps), self.lm_head)[:, 0]
+        if self.config.fused_decode and q_len > 1 and x.shape[-1] <= ops.NORM_MAX_DIM:
+            x = x.contiguous()
+            delta = None
+            for layer in self.layers:
+                delta = layer.segment_step(x, delta, position_embeddings, start_pos, cache)
+            if all_logits:
+                return self.lm_head(ops.add_rms_norm(x, delta, self.norm.weight, self.norm.eps))
+            last = x[:, -1:].contiguous()
+            return step_linear(ops.add_rms_norm(last, delta[:, -1:].contiguous(), self.norm.weight, self.norm.eps),
+                               self.lm_head)[:, 0]
         for layer in self.layers:
             x = layer(x, position_embeddings, start_pos, cache)
         x = self.norm(x if all_logits else x[:, -1:])

@@ -411,6 +411,7 @@ def evict_apply_first(src_k, src_v, cache_k, cache_v, valid, pos, roles, size_gl
 # decode-step glue of the HF-shaped caller
 # ------------------------------------------------------------------------------------------------
 CARRY_NONE, CARRY_MEAN_FIRST, CARRY_MEAN_ADD, CARRY_MAX_FIRST, CARRY_MAX_MERGE = 0, 1, 2, 3, 4
+NORM_MAX_DIM = 8192  # widest row add_rms_norm takes
 
 
 def add_rms_norm(x: torch.Tensor, delta: torch.Tensor | None, weight: torch.Tensor, eps: float,
@@ -508,6 +509,32 @@ class MatvecPlan:
         check(self.fn(self.w_ptr, x.data_ptr(), y.data_ptr(), x.numel() // k, n, k, self.w_stride, k, n, self.gate,
                       self.code, _stream(x)))
         return y
+
+
+def rope_qk_ok(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> bool:
+    """Whether `rope_qk` takes these tensors (16-byte rows everywhere)."""
+    e = 16 // q.element_size()
+    ts = (q, k, cos, sin)
+    return (q.dtype in (torch.bfloat16, torch.float32) and all(t.is_cuda and t.dtype == q.dtype and t.stride(-1) == 1 for t in ts)
+            and q.shape[-1] % (2 * e) == 0 and all(t.data_ptr() % 16 == 0 for t in ts)
+            and all(st % e == 0 for t in (q, k) for st in t.stride()[:3]) and all(st % e == 0 for st in cos.stride()[:2])
+            and sin.stride() == cos.stride())
+
+
+def rope_qk(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor):
+    """apply_rotary_pos_emb for a multi-token segment in one launch: q [B, H_q, L, D], k [B, H_kv, L, D] (any strides,
+    last dimension contiguous), cos / sin [B, L, D].  Returns contiguous (q_rot, k_rot)."""
+    _require_cuda(q, k, cos, sin)
+    B, Hq, L, D = q.shape
+    Hkv = k.shape[1]
+    if k.shape != (B, Hkv, L, D) or cos.shape != (B, L, D) or sin.shape != cos.shape or not rope_qk_ok(q, k, cos, sin):
+        raise ValueError("rope_qk: q [B, H_q, L, D], k [B, H_kv, L, D], cos / sin [B, L, D] of one dtype with 16-byte rows")
+    q_out = torch.empty(B, Hq, L, D, dtype=q.dtype, device=q.device)
+    k_out = torch.empty(B, Hkv, L, D, dtype=q.dtype, device=q.device)
+    check(_lib.load().nats_rope_qk(_ptr(q), _ptr(k), _ptr(cos), _ptr(sin), _ptr(q_out), _ptr(k_out), B, Hq, Hkv, L, D,
+                                   i64_array(q.stride()[:3]), i64_array(k.stride()[:3]), i64_array(cos.stride()[:2]),
+                                   _dtype_code(q), _stream(q)))
+    return q_out, k_out
 
 
 def rope_append(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,

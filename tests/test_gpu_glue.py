@@ -213,3 +213,24 @@ def test_fused_projection_weights_are_views():
     assert (a.qkv_weight[a.q_proj.weight.shape[0]:a.q_proj.weight.shape[0] + a.k_proj.weight.shape[0]] == 0.5).all()
     model = model.float()  # the parameters are re-created: the merged matrix is rebuilt on the next use
     assert not model.layers[0].self_attn.fused_ok()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("B,Hq,Hkv,L,D", [(2, 8, 2, 37, 64), (1, 32, 8, 300, 128), (2, 4, 4, 5, 32)])
+def test_rope_qk(dtype, B, Hq, Hkv, L, D):
+    """The segment form of the rotary embedding on the strided views of a merged projection: bit for bit what
+    apply_rotary_pos_emb computes."""
+    from neuralattentionsearch_amd import ops
+    from neuralattentionsearch_amd.attention import apply_rotary_pos_emb
+    from neuralattentionsearch_amd.llama import rotary_tables
+    say("rope_qk", dtype, B, Hq, Hkv, L, D)
+    g = torch.Generator().manual_seed(L)
+    qkv = torch.randn(B, L, Hq + 2 * Hkv, D, generator=g).to(dtype).cuda().transpose(1, 2)
+    q, k = qkv[:, :Hq], qkv[:, Hq:Hq + Hkv]
+    pos = torch.arange(11, 11 + L, device="cuda")[None].expand(B, -1)
+    cos, sin = rotary_tables(pos, D, 10000.0, dtype)
+    assert ops.rope_qk_ok(q, k, cos, sin)
+    q_rot, k_rot = ops.rope_qk(q, k, cos, sin)
+    q_want, k_want = apply_rotary_pos_emb(q, k, cos, sin)
+    assert q_rot.is_contiguous() and k_rot.is_contiguous()
+    assert torch.equal(q_rot, q_want) and torch.equal(k_rot, k_want)
