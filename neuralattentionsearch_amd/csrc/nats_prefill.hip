@@ -42,7 +42,31 @@ struct PrefillArgs {
   // persistent kernel only: the flat tile lists of the schedule
   const int32_t* entries;
   const int2* bounds;  // [workgroups] {first entry, end entry}
+  // few query tiles over many key rows: n_split workgroups share the tile list of one (kv stream, head group,
+  // query group) and leave partial results, which prefill_split_merge_kernel combines
+  int n_split;      // 1: no split
+  float* part_acc;  // [workgroup, split, wavefront, 32 rows, D]
+  float* part_ml;   // [workgroup, split, wavefront, 32 rows, 2] running maximum (base-2 exponent) and row sum
 };
+
+// workgroup index -> (kv stream, head group, rank of the query group; heavy query groups come first)
+__device__ __forceinline__ void map_workgroup(const PrefillArgs& a, int bid, int& ks, int& hg, int& rank) {
+  if (a.xcd_mode) {
+    int x = bid & 7;
+    int j = bid >> 3;
+    int n_x = (a.B * a.Hkv / 8) * a.n_hg;
+    int sl = j % n_x;
+    rank = j / n_x;
+    ks = x + 8 * (sl / a.n_hg);
+    hg = sl % a.n_hg;
+  } else {
+    int ns = a.B * a.Hkv * a.n_hg;
+    int sidx = bid % ns;
+    rank = bid / ns;
+    ks = sidx / a.n_hg;
+    hg = sidx % a.n_hg;
+  }
+}
 
 // ---------------------------------------------------------------------------------------------------
 // fp32 / generic kernel: 64 lanes = 64 query rows, key sub-tiles of 32 rows staged in LDS as fp32.
@@ -166,6 +190,7 @@ __global__ __launch_bounds__(64) void prefill_simple_kernel(PrefillArgs a) {
 // ---------------------------------------------------------------------------------------------------
 constexpr float kRescaleSlack = 8.0f;
 constexpr int kPrefillWaves = 8;
+constexpr int kMaxSplit = 32;  // workgroups that may share one tile list
 constexpr int kMaxDevices = 64;
 
 // both halves of the wavefront get max / sum over lane and lane ^ 32 (one cross-half swap, no LDS round trip)
@@ -222,22 +247,13 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
 
   // ---- which (kv stream, head group, query group) -------------------------------------------------
   int bid = blockIdx.x;
-  int ks, hg, rank;
-  if (a.xcd_mode) {
-    int x = bid & 7;
-    int j = bid >> 3;
-    int n_x = (a.B * a.Hkv / 8) * a.n_hg;
-    int sl = j % n_x;
-    rank = j / n_x;
-    ks = x + 8 * (sl / a.n_hg);
-    hg = sl % a.n_hg;
-  } else {
-    int ns = a.B * a.Hkv * a.n_hg;
-    int sidx = bid % ns;
-    rank = bid / ns;
-    ks = sidx / a.n_hg;
-    hg = sidx % a.n_hg;
+  int split = 0;  // which share of the tile list (n_split > 1)
+  if (a.n_split > 1) {
+    split = bid % a.n_split;
+    bid /= a.n_split;
   }
+  int ks, hg, rank;
+  map_workgroup(a, bid, ks, hg, rank);
   const int qg = a.n_qg - 1 - rank;  // heavy query groups first
   const int b = ks / a.Hkv, hkv = ks % a.Hkv;
   const int hq = hkv * a.n_rep + hg * a.hpw + (sub % a.hpw);
@@ -641,14 +657,20 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
       if (lane == 0) sm.vcount = count;
     }
     __syncthreads();
-    const int n_vis = __builtin_amdgcn_readfirstlane(sm.vcount);
+    int n_vis = __builtin_amdgcn_readfirstlane(sm.vcount);
+    int j0 = 0;  // first list entry of this workgroup's share
+    if (a.n_split > 1) {
+      const int per = (n_vis + a.n_split - 1) / a.n_split;
+      j0 = split * per;
+      n_vis = max(0, min(per, n_vis - j0));
+    }
     if (n_vis > 0) {
       // The list entries are the same for every lane: they are kept in scalar registers.
       // Tile j of the list: the matrix pipe computes the scores of tile j+1 while the vector ALU turns those of
       // tile j into probabilities; then O += P V for tile j.  Buffers: K tile j in k[j & 3], V tile j in
       // v[j & 3], row limits of tile j in limk[j & 7].
       auto entry = [&](int j, int& kt, int& emax, int& emin) {
-        const int4 e = sm.vlist[j];
+        const int4 e = sm.vlist[j0 + j];
         kt = __builtin_amdgcn_readfirstlane(e.x);
         emax = __builtin_amdgcn_readfirstlane(e.y);
         emin = __builtin_amdgcn_readfirstlane(e.z);
@@ -670,7 +692,7 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
           int kt, emax, emin;
           entry(j, kt, emax, emin);
           r.kt = kt; r.emax = emax; r.emin = emin;
-          if (kPacked) r.e3 = __builtin_amdgcn_readfirstlane(sm.vlist[j].w);
+          if (kPacked) r.e3 = __builtin_amdgcn_readfirstlane(sm.vlist[j0 + j].w);
         }
         return r;
       };
@@ -747,7 +769,27 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
         __builtin_amdgcn_s_waitcnt(0);  // the tiles in flight have landed in LDS
         __syncthreads();                // ... for every wavefront, and the tiles of this step are no longer read
       }
+    } else if (w0 + kWinStep <= win_last) {
+      __syncthreads();  // (nobody may still be reading this window's count when wavefront 0 starts the next list)
     }
+  }
+
+  // ---- a share of the tile list: the unnormalised sums, the running maximum and the row sum leave as they are ----
+  if (a.n_split > 1) {
+    const float l = half_swap_sum(l_run);
+    const int64_t slot = ((int64_t)bid * a.n_split + split) * kPrefillWaves + wave;
+    float* pa = a.part_acc + (slot * kHalf + l32) * D;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+      for (int g4 = 0; g4 < 4; ++g4) {
+        const int d = dt * 32 + g4 * 8 + hl * 4;
+        *reinterpret_cast<float4*>(pa + d) =
+            make_float4(oacc[dt][g4 * 4 + 0], oacc[dt][g4 * 4 + 1], oacc[dt][g4 * 4 + 2], oacc[dt][g4 * 4 + 3]);
+      }
+    }
+    if (hl == 0) *reinterpret_cast<float2*>(a.part_ml + (slot * kHalf + l32) * 2) = make_float2(m_run, l);
+    return;
   }
 
   // ---- epilogue: O rows go through LDS so that every row leaves as whole 16-byte pieces ----------------
@@ -786,6 +828,65 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
         *reinterpret_cast<uint4*>(op + (int64_t)(qtok - a.r_begin) * a.os_l + piece * 8) = val;
       }
     }
+  }
+}
+
+// Combines the partial results of the n_split workgroups that shared one tile list: grid = (the workgroups of the
+// unsplit launch, slices of their 8 x 32 x D / 4 outputs), one thread per (wavefront, row, 4 dims).
+template <int D>
+__global__ __launch_bounds__(256) void prefill_split_merge_kernel(PrefillArgs a) {
+  constexpr int kHalf = kTile / 2;
+  constexpr int Q4 = D / 4;
+  const int bid = blockIdx.x;
+  int ks, hg, rank;
+  map_workgroup(a, bid, ks, hg, rank);
+  const int qg = a.n_qg - 1 - rank;
+  const int b = ks / a.Hkv, hkv = ks % a.Hkv;
+  const int qt_lo = a.qt_first + qg * a.qpw;
+  const int qt_hi = min(qt_lo + a.qpw - 1, a.qt_last);
+  {
+    const int item = blockIdx.y * 256 + threadIdx.x;
+    if (item >= kPrefillWaves * kHalf * Q4) return;
+    const int wave = item / (kHalf * Q4);
+    const int row = (item / Q4) % kHalf;
+    const int d = (item % Q4) * 4;
+    const int sub = wave & 3, half = wave >> 2;
+    const int my_qt = qt_lo + sub / a.hpw;
+    const int qtok = my_qt * kTile + half * kHalf + row;
+    if (my_qt > qt_hi || qtok < a.r_begin || qtok >= a.r_end) return;
+    const int hq = hkv * a.n_rep + hg * a.hpw + (sub % a.hpw);
+    const int64_t first = ((int64_t)bid * a.n_split * kPrefillWaves + wave) * kHalf + row;  // split 0
+    const int64_t step = (int64_t)kPrefillWaves * kHalf;                                       // to the next split
+    // the (maximum, sum) pairs of all partials first, then the accumulators eight at a time
+    float2 ml[kMaxSplit];
+#pragma unroll
+    for (int sp = 0; sp < kMaxSplit; ++sp)
+      ml[sp] = sp < a.n_split ? *reinterpret_cast<const float2*>(a.part_ml + (first + sp * step) * 2) : make_float2(-INFINITY, 0.f);
+    float M = -INFINITY;
+#pragma unroll
+    for (int sp = 0; sp < kMaxSplit; ++sp) M = fmaxf(M, ml[sp].x);
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    float lsum = 0.f;
+#pragma unroll
+    for (int s0 = 0; s0 < kMaxSplit; s0 += 8) {
+      if (s0 >= a.n_split) break;
+      float4 p[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        p[u] = s0 + u < a.n_split ? *reinterpret_cast<const float4*>(a.part_acc + (first + (s0 + u) * step) * D + d)
+                                  : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const float m = ml[s0 + u].x;
+        const float w = m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m - M);
+        acc.x = fmaf(p[u].x, w, acc.x); acc.y = fmaf(p[u].y, w, acc.y); acc.z = fmaf(p[u].z, w, acc.z); acc.w = fmaf(p[u].w, w, acc.w);
+        lsum = fmaf(ml[s0 + u].y, w, lsum);
+      }
+    }
+    const float inv = 1.f / lsum;
+    const bf16x4 ob = {(__bf16)(acc.x * inv), (__bf16)(acc.y * inv), (__bf16)(acc.z * inv), (__bf16)(acc.w * inv)};
+    uint16_t* op = static_cast<uint16_t*>(a.o) + b * a.os_b + hq * a.os_h + (int64_t)(qtok - a.r_begin) * a.os_l + d;
+    *reinterpret_cast<uint2*>(op) = __builtin_bit_cast(uint2, ob);
   }
 }
 
@@ -1482,6 +1583,24 @@ static int device_cu_count() {
   return cached[dev];
 }
 
+// Few query tiles over many key rows (a short segment over a long cache): how many workgroups share one tile list,
+// so that the launch still fills the device.  1 = no split.
+static bool use_split() {
+  const char* e = getenv("NATS_PREFILL_SPLIT");
+  return !(e && e[0] == '0');
+}
+static int choose_split(int64_t n_wg, int64_t Tk) {
+  const int n_cu = device_cu_count();
+  if (!use_split() || n_cu <= 0 || n_wg * 2 > n_cu) return 1;
+  int64_t n = n_cu / n_wg;
+  if (n > kMaxSplit) n = kMaxSplit;
+  if (n > Tk / 4) n = Tk / 4;  // at least four key tiles per share
+  return n < 2 ? 1 : (int)n;
+}
+static size_t split_partial_bytes(int64_t n_wg, int n_split, int64_t D) {
+  return n_split <= 1 ? 0 : (size_t)n_wg * n_split * kPrefillWaves * (kTile / 2) * (D + 2) * sizeof(float);
+}
+
 template <int D>
 static int launch_prefill_stream(PrefillArgs a, const StreamSched& sw, hipStream_t st) {
   int n_wg = device_cu_count();
@@ -1589,7 +1708,7 @@ StreamSched sched_in_workspace(void* workspace, size_t workspace_bytes, size_t b
 int launch_segment(const char* who, const SegmentShape& g, const void* q, const void* k, const void* v, void* o,
                    const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
                    const int64_t* o_strides, float sm_scale, int dtype, const PrefillWorkspace& w, const StreamSched& sw,
-                   hipStream_t st) {
+                   void* extra, size_t extra_bytes, hipStream_t st) {
   PrefillArgs a{};
   a.q = q; a.k = k; a.v = v; a.o = o;
   a.tok_lim = w.tok_lim; a.tile_lim = w.tile_lim; a.gran_lim = w.gran_lim;
@@ -1630,6 +1749,34 @@ int launch_segment(const char* who, const SegmentShape& g, const void* q, const 
   a.xcd_mode = ((g.B * g.H_kv) % 8 == 0) ? 1 : 0;
   int64_t n_wg = g.B * g.H_kv * a.n_hg * a.n_qg;
   NATS_REQUIRE(n_wg < (int64_t(1) << 31), NATS_ERR_BAD_SHAPE, "%s: grid too large", who);
+  const bool packed = g.C < kTile && use_packed_tiles();
+  const bool persistent = hpw == 4 && !packed && sw.bytes != 0 && use_stream_kernel();
+  a.n_split = 1;
+  if ((hpw == 4 || packed) && !persistent) {  // the kernels in which every wavefront walks the whole tile list
+    const int ns = choose_split(n_wg, a.Tk);
+    if (ns > 1 && extra && extra_bytes >= split_partial_bytes(n_wg, ns, g.D)) {
+      a.n_split = ns;
+      a.part_acc = static_cast<float*>(extra);
+      a.part_ml = a.part_acc + (size_t)n_wg * ns * kPrefillWaves * (kTile / 2) * g.D;
+    }
+  }
+  if (a.n_split > 1) {
+    const int64_t n_launch = n_wg * a.n_split;
+    int rc;
+    if (packed) {
+      rc = g.D == 64 ? launch_prefill_mfma<64, true, true>(a, n_launch, st) : launch_prefill_mfma<128, true, true>(a, n_launch, st);
+    } else {
+      rc = g.D == 64 ? launch_prefill_mfma<64, true>(a, n_launch, st) : launch_prefill_mfma<128, true>(a, n_launch, st);
+    }
+    if (rc) return rc;
+    if (g.D == 64) {
+      hipLaunchKernelGGL((prefill_split_merge_kernel<64>), dim3((unsigned)n_wg, kPrefillWaves * (kTile / 2) * 16 / 256), dim3(256), 0, st, a);
+    } else {
+      hipLaunchKernelGGL((prefill_split_merge_kernel<128>), dim3((unsigned)n_wg, kPrefillWaves * (kTile / 2) * 32 / 256), dim3(256), 0, st, a);
+    }
+    NATS_CHECK_LAUNCH("prefill_split_merge_kernel");
+    return NATS_OK;
+  }
   // chunks shorter than a tile: tiles are packed from the 16-row granules that are visible (NATS_PREFILL_PACKED=0
   // in the environment keeps whole tiles, for comparison)
   // (GQA groups of 1 and 2: the workgroup's 2 or 4 query tiles form one group for the packing, every wavefront
@@ -1654,7 +1801,17 @@ extern "C" size_t nats_prefill_sched_workspace_bytes(int64_t B, int64_t H_q, int
   if (B <= 0 || H_q <= 0 || H_kv <= 0 || n_queries <= 0 || n_rows < n_queries) return 0;
   // a segment over a filled cache starts anywhere inside a 64-token tile of its region
   const int64_t n_qt = n_rows == n_queries ? (n_queries + kTile - 1) / kTile : (n_queries + kTile - 2) / kTile + 1;
-  return carve_stream_sched(nullptr, B, H_q, H_kv, n_qt, (n_rows + kTile - 1) / kTile).bytes;
+  const int64_t Tk = (n_rows + kTile - 1) / kTile;
+  const size_t sched = carve_stream_sched(nullptr, B, H_q, H_kv, n_qt, Tk).bytes;
+  // the partial results of a split launch use the same region (a launch is either split or persistent)
+  const int64_t n_rep = H_q / H_kv;
+  const int64_t hpw = n_rep >= 4 ? 4 : (n_rep > 0 ? n_rep : 1);
+  // (a split launch never has more workgroups than the device has CUs, whatever the exact number of query tiles
+  // turns out to be: room for that many partial results whenever a launch of this size may be split)
+  const int64_t n_qg_min = (n_qt > 1 ? n_qt - 1 : 1) + 4 / hpw - 1;
+  const int64_t n_wg_min = B * H_kv * (n_rep / hpw > 0 ? n_rep / hpw : 1) * (n_qg_min / (4 / hpw));
+  const size_t split = choose_split(n_wg_min, Tk) > 1 ? split_partial_bytes(device_cu_count(), 2, 128) / 2 : 0;
+  return sched > split ? sched : split;
 }
 
 extern "C" size_t nats_prefill_past_workspace_bytes(int64_t B, int64_t H_kv, int64_t n_rows, int64_t S) {
@@ -1678,7 +1835,8 @@ extern "C" int nats_prefill_fwd(const void* q, const void* k, const void* v, con
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (int rc = prepare_key_limits(roles, B, H_kv, S, L, C, W, nullptr, w, st)) return rc;
   const StreamSched sw = sched_in_workspace(workspace, workspace_bytes, w.bytes, B, H_q, H_kv, (L + kTile - 1) / kTile, L, dtype);
-  return launch_segment(who, g, q, k, v, o, q_strides, k_strides, v_strides, o_strides, sm_scale, dtype, w, sw, st);
+  return launch_segment(who, g, q, k, v, o, q_strides, k_strides, v_strides, o_strides, sm_scale, dtype, w, sw,
+                        static_cast<char*>(workspace) + w.bytes, workspace_bytes - w.bytes, st);
 }
 
 extern "C" int nats_prefill_past_fwd(const void* q, const void* cache_k, const void* cache_v, const uint8_t* valid,
@@ -1708,5 +1866,6 @@ extern "C" int nats_prefill_past_fwd(const void* q, const void* cache_k, const v
   if (int rc = prepare_key_limits(roles, B, H_kv, S, N, C, W, &pv, w, st)) return rc;
   const int64_t n_qt = (state->old_fill + x_len - 1) / kTile - state->old_fill / kTile + 1;
   const StreamSched sw = sched_in_workspace(workspace, workspace_bytes, w.bytes, B, H_q, H_kv, n_qt, N, dtype);
-  return launch_segment(who, g, q, cache_k, cache_v, o, q_strides, k_strides, v_strides, o_strides, sm_scale, dtype, w, sw, st);
+  return launch_segment(who, g, q, cache_k, cache_v, o, q_strides, k_strides, v_strides, o_strides, sm_scale, dtype, w, sw,
+                        static_cast<char*>(workspace) + w.bytes, workspace_bytes - w.bytes, st);
 }

@@ -146,6 +146,57 @@ def test_packed_tiles_full_size_sampled_rows(Hq, Hkv, L, C, W):
 
 
 @pytest.fixture
+def split_lists(monkeypatch):
+    def switch(on: bool):
+        monkeypatch.setenv("NATS_PREFILL_SPLIT", "1" if on else "0")
+    yield switch
+    monkeypatch.delenv("NATS_PREFILL_SPLIT", raising=False)
+
+
+@pytest.mark.parametrize("C,W,lens", [(64, 256, (6000, 64, 200, 1, 700)), (16, 64, (5000, 100, 33, 900)),
+                                      (64, 128, (40000, 128))])
+def test_short_segments_over_a_long_cache_split_their_tile_lists(split_lists, C, W, lens):
+    """Few query tiles over many key rows: several workgroups share one tile list and a merge kernel combines their
+    partial results.  Same outputs as one workgroup per list, to rounding."""
+    from neuralattentionsearch_amd import ops
+    from neuralattentionsearch_amd.cache import NAtSChunkLayerCache
+    say("prefill split lists", C, W, lens)
+    B, Hq, Hkv, D = 1, 8, 2, 128
+    outs = []
+    for on in (False, True):
+        split_lists(on)
+        gg = torch.Generator().manual_seed(11)
+        cache = NAtSChunkLayerCache(B, Hkv, W, chunk_size=C, device="cuda")
+        res = []
+        for si, n in enumerate(lens):
+            q = torch.randn(B, Hq, n, D, generator=gg).bfloat16().cuda()
+            k = torch.randn(B, Hkv, n, D, generator=gg).bfloat16().cuda()
+            v = torch.randn(B, Hkv, n, D, generator=gg).bfloat16().cuda()
+            total = cache.chunk_fill_size + n
+            first = cache.get_seq_length() == 0
+            if total < C:
+                roles = np.zeros((B, Hkv, 1), dtype=np.uint8)
+            else:
+                roles = draw_roles(si, B, Hkv, math.ceil(total / C), p=(0.3, 0.3, 0.4), first_global=first)
+                if total % C:
+                    roles[:, :, -1] = 0
+            tsi = orc.one_hot_roles(roles).bfloat16().cuda()
+            kk, vv = cache.update(k, v, tsi)
+            if first:
+                o = ops.prefill_attention(q, kk, vv, to_dev(roles), C, W)
+            elif n > 1:
+                o = cache.segment_attention(q)
+            else:
+                o = ops.decode_attention(q, kk, vv, cache.valid_tokens, kk.shape[2])
+            res.append(o.float())
+            cache.post_update(n)
+        outs.append(res)
+    for x, y in zip(*outs):
+        assert torch.isfinite(y).all()
+        assert (x - y).abs().max().item() <= 2e-2
+
+
+@pytest.fixture
 def packed_tiles(monkeypatch):
     def switch(on: bool):
         monkeypatch.setenv("NATS_PREFILL_PACKED", "1" if on else "0")
@@ -221,8 +272,12 @@ def stream_kernel(monkeypatch):
     """Selects the persistent prefill kernel for the calls made through the returned switch."""
     def switch(on: bool):
         monkeypatch.setenv("NATS_PREFILL_STREAM", "1" if on else "0")
+        # (the two kernels are bit-identical when one workgroup walks a whole tile list; small launches would
+        # otherwise share a list among several workgroups and merge partial results)
+        monkeypatch.setenv("NATS_PREFILL_SPLIT", "0")
     yield switch
     monkeypatch.delenv("NATS_PREFILL_STREAM", raising=False)
+    monkeypatch.delenv("NATS_PREFILL_SPLIT", raising=False)
 
 
 @pytest.mark.parametrize("B,Hq,Hkv,L,D,C,W,p", [
