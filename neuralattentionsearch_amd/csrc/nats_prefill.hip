@@ -1749,7 +1749,10 @@ int launch_segment(const char* who, const SegmentShape& g, const void* q, const 
   a.xcd_mode = ((g.B * g.H_kv) % 8 == 0) ? 1 : 0;
   int64_t n_wg = g.B * g.H_kv * a.n_hg * a.n_qg;
   NATS_REQUIRE(n_wg < (int64_t(1) << 31), NATS_ERR_BAD_SHAPE, "%s: grid too large", who);
-  const bool packed = g.C < kTile && use_packed_tiles();
+  // Packed tiles for chunks shorter than a tile, and for GQA groups of 1 and 2 at any chunk size: there the
+  // workgroup's four or two query tiles walk one list together, which costs the same as every wavefront skipping
+  // on its own between shared barriers and lets small launches share their lists among workgroups.
+  const bool packed = (g.C < kTile || hpw < 4) && use_packed_tiles();
   const bool persistent = hpw == 4 && !packed && sw.bytes != 0 && use_stream_kernel();
   a.n_split = 1;
   if ((hpw == 4 || packed) && !persistent) {  // the kernels in which every wavefront walks the whole tile list
@@ -1781,7 +1784,7 @@ int launch_segment(const char* who, const SegmentShape& g, const void* q, const 
   // in the environment keeps whole tiles, for comparison)
   // (GQA groups of 1 and 2: the workgroup's 2 or 4 query tiles form one group for the packing, every wavefront
   // walks the whole list and the element mask sorts out what its own rows see)
-  if (g.C < kTile && use_packed_tiles())
+  if (packed)
     return g.D == 64 ? launch_prefill_mfma<64, true, true>(a, n_wg, st) : launch_prefill_mfma<128, true, true>(a, n_wg, st);
   if (hpw == 4 && sw.bytes != 0 && use_stream_kernel())
     return g.D == 64 ? launch_prefill_stream<64>(a, sw, st) : launch_prefill_stream<128>(a, sw, st);
