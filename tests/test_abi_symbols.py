@@ -113,3 +113,15 @@ def test_matvec_arguments_are_validated():
     assert lib.nats_matvec(fake, fake, fake, 1, 8, 64, 64, 64, 4, 0, 0, None) == -2  # y rows shorter than n_out
     assert lib.nats_matvec(fake, ctypes.c_void_p(264), fake, 1, 8, 64, 64, 64, 8, 0, 0, None) == -2  # x not 16-byte aligned
     assert lib.nats_matvec(fake, fake, fake, 1, 8, 64, 64, 64, 8, 0, 7, None) == -3  # dtype code
+
+
+def test_rope_qk_arguments_are_validated():
+    lib = _lib.load()
+    fake = ctypes.c_void_p(256)
+    st3, st2 = _lib.i64_array([4096, 128, 512]), _lib.i64_array([4096, 128])
+    assert lib.nats_rope_qk(None, fake, fake, fake, fake, fake, 1, 4, 2, 8, 128, st3, st3, st2, 0, None) == -1
+    assert lib.nats_rope_qk(fake, fake, fake, fake, fake, fake, 1, 4, 2, 8, 24, st3, st3, st2, 0, None) == -4  # D % 16
+    assert lib.nats_rope_qk(fake, fake, fake, fake, fake, fake, 1, 4, 2, 0, 128, st3, st3, st2, 0, None) == -2  # no tokens
+    odd = _lib.i64_array([4096, 124, 512])
+    assert lib.nats_rope_qk(fake, fake, fake, fake, fake, fake, 1, 4, 2, 8, 128, odd, st3, st2, 0, None) == -2  # 16-byte rows
+    assert lib.nats_rope_qk(fake, fake, fake, fake, fake, fake, 1, 4, 2, 8, 128, st3, st3, st2, 9, None) == -3  # dtype
