@@ -1,8 +1,12 @@
 // Role-masked, chunked flash-attention prefill for gfx950.
 //
-// Two kernels share one tile-skip map:
-//   prefill_mfma_kernel   bf16, QK^T and PV on v_mfma_f32_32x32x16_bf16, fp32 online softmax
-//   prefill_simple_kernel fp32 (or bf16) FMA kernel, one query row per lane; the fp32 parity path
+// Kernels (they share the per-row limits and the tile / granule summaries of the key-limit stage):
+//   prefill_mfma_kernel        bf16, QK^T and PV on v_mfma_f32_32x32x16_bf16, fp32 online softmax; walks whole 64-row
+//                              key tiles, or (kPacked) tiles assembled from the visible 16-row granules; with
+//                              n_split > 1 several workgroups share one tile list and leave partial results
+//   prefill_split_merge_kernel combines those partial results
+//   prefill_stream_kernel      persistent form of the first (one workgroup per CU, precomputed visit lists; opt in)
+//   prefill_simple_kernel      fp32 (or bf16) FMA kernel, one query row per lane; the fp32 parity path
 //
 // Mask semantics (components/masks/utils.py:89-94, components/cache/nats_chunk_layer_cache.py:462-511, 603-616):
 // the queries are tokens [r_begin, r_end) of the open-chunk region, which starts at key row `base`; every key
