@@ -252,7 +252,9 @@ class NAtSLlamaAttention(nn.Module):
         layer = past_key_value.cache_model[idx]
         scale = 1.0 / math.sqrt(self.head_dim)
         if is_pre_filling:
-            out = ops.prefill_attention(q, keys, values, roles, C, self.local_seq_max_length, scale)
+            # (written as [B, L, H, D], the layout o_proj reads, through the strided view the kernel takes)
+            out = torch.empty(bsz, q_len, self.num_heads, self.head_dim, dtype=q.dtype, device=q.device).transpose(1, 2)
+            ops.prefill_attention(q, keys, values, roles, C, self.local_seq_max_length, scale, out=out)
         elif q_len > 1:
             out = layer.segment_attention(q, scale)
         else:
