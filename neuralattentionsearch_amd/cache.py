@@ -332,8 +332,10 @@ class NAtSCache:
     """Container of per-layer caches (src/nats/components/cache/dyn_cache.py:66-195)."""
 
     def __init__(self, sliding_window_size: int, chunk_size: int = 1, track_positions: bool = False):
-        if chunk_size == 1:
-            raise NotImplementedError("the per-token cache (chunk_size == 1) is not built; use chunk_size > 1")
+        # chunk_size == 1 (per-token roles): served by the chunk state machine with one-token chunks.  Visibility
+        # and surviving tokens are those of the per-token rules (global / local until the next global / sliding
+        # window); rows are dropped at every token, where the reference's separate per-token class
+        # (nats_layer_cache.py) defers the physical update by 16 tokens and keeps its own row order.
         self.cache_model: list[NAtSChunkLayerCache] = []
         self.sliding_window_size = sliding_window_size
         self.chunk_size = chunk_size
@@ -353,7 +355,7 @@ class NAtSCache:
         return self.cache_model[layer_idx].generate_mask(x_len)
 
     def get_nats_chunk_fill_size(self, layer_idx: int = 0):
-        if len(self.cache_model) <= layer_idx or self.chunk_size == 1:
+        if len(self.cache_model) <= layer_idx:
             return 0
         return self.cache_model[layer_idx].chunk_fill_size
 

@@ -27,8 +27,11 @@ How each function is pinned (see tests/test_oracle_*.py):
                                  open chunk, and the invariant that any split of a stream into calls gives
                                  the statistics of one call (dyn_cache.py:98-171, chunk_utils.py:13-62)
 
-Functions with parity unpinned: none of the above; the per-token cache (chunk_size == 1,
-components/cache/nats_layer_cache.py) is not restated here.
+Functions with parity unpinned: none of the above.  The reference's per-token cache class (chunk_size == 1,
+components/cache/nats_layer_cache.py: 16-token deferred eviction, its own row order) is not restated here; per-token
+roles are covered as ChunkCacheOracle with C = 1, which gives the visibility and the surviving tokens of the
+per-token rules but not that class's cache layout (parity unpinned for the layout: the class cannot be imported
+in the reference's own checkout, so no vectors of it exist).
 """
 from __future__ import annotations
 

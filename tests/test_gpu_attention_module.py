@@ -31,6 +31,12 @@ def test_module_segments_over_a_filled_cache(lens, C, W):
     run_module(lens, C, W)
 
 
+@pytest.mark.parametrize("lens,W", [([40] + [1] * 30, 16), ([70, 45, 1, 1, 33, 1, 90], 32)])
+def test_module_with_per_token_roles(lens, W):
+    """chunk_size == 1: a role per token, served by the same state machine with one-token chunks."""
+    run_module(lens, 1, W)
+
+
 def run_module(lens, C, W):
     from neuralattentionsearch_amd.attention import LlamaNAtSChunkAttentionLayer, apply_rotary_pos_emb
     from neuralattentionsearch_amd.cache import NAtSCache

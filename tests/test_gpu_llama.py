@@ -102,6 +102,14 @@ def test_small_fp32_model_layer_by_layer():
     run(cfg, torch.float32, [100, 37] + [1] * 40 + [50, 1, 1], tol=2e-5)
 
 
+def test_per_token_roles_layer_by_layer():
+    """chunk_size == 1: a role per token (the per-token adapters of the reference), one-token chunks in the cache."""
+    from neuralattentionsearch_amd.llama import NAtSLlamaConfig
+    cfg = NAtSLlamaConfig(vocab_size=1000, hidden_size=512, intermediate_size=1024, num_hidden_layers=2,
+                          num_attention_heads=8, num_key_value_heads=2, chunk_size=1, local_seq_max_length=16)
+    run(cfg, torch.float32, [60, 21] + [1] * 24, tol=2e-5)
+
+
 def test_llama_head_shape_bf16_layer_by_layer():
     """32 q heads / 8 kv heads / head_dim 128, chunk 64, window 256, two layers."""
     from neuralattentionsearch_amd.llama import NAtSLlamaConfig
