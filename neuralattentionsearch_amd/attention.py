@@ -172,7 +172,7 @@ class BaseNAtSChunkAttentionLayer(BaseNAtSAttentionLayer):
         layer = cache.cache_model[self.layer_id]
         if x_len == 1 and layer.get_seq_length() > 0:
             output = ops.decode_attention(xq, keys, values, layer.valid_tokens, keys.shape[2], self.sm_scale,
-                                          row_end=layer.size_global_kv + layer.size_local_kv,
+                                          row_end=layer.row_end(),
                                           tail_start=layer.n_ctx_data - (layer.chunk_fill_size - 1))
         elif layer.get_seq_length() == 0:
             roles = ops.roles_from_one_hot(kwargs["token_states_info"])

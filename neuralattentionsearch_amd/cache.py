@@ -335,7 +335,8 @@ class NAtSCache:
         # chunk_size == 1 (per-token roles): served by the chunk state machine with one-token chunks.  Visibility
         # and surviving tokens are those of the per-token rules (global / local until the next global / sliding
         # window); rows are dropped at every token, where the reference's separate per-token class
-        # (nats_layer_cache.py) defers the physical update by 16 tokens and keeps its own row order.
+        # (nats_layer_cache.py) defers the update by 16 tokens, keeps the tokens of the pending block visible until
+        # then (:300-310, :544-554) and has its own row order.
         self.cache_model: list[NAtSChunkLayerCache] = []
         self.sliding_window_size = sliding_window_size
         self.chunk_size = chunk_size

@@ -259,7 +259,7 @@ class NAtSLlamaAttention(nn.Module):
             out = layer.segment_attention(q, scale)
         else:
             out = ops.decode_attention(q, keys, values, layer.valid_tokens, keys.shape[2], scale,
-                                       row_end=layer.size_global_kv + layer.size_local_kv,
+                                       row_end=layer.row_end(),
                                        tail_start=layer.n_ctx_data - (layer.chunk_fill_size - 1))
         past_key_value.post_update(layer_idx=idx, x_len=q_len)
         return self.o_proj(out.transpose(1, 2).reshape(bsz, q_len, -1))
@@ -348,13 +348,14 @@ class NAtSLlamaForCausalLM(nn.Module):
         x = self.embed_tokens(input_ids)
         pos = torch.arange(start_pos, start_pos + q_len, device=input_ids.device)[None].expand(bsz, -1)
         position_embeddings = rotary_tables(pos, self.config.head_dim, self.config.rope_theta, x.dtype)
-        if self.config.fused_decode and q_len == 1 and start_pos > 0 and len(cache.cache_model) == len(self.layers):
+        fused = self.config.fused_decode and x.shape[-1] <= ops.NORM_MAX_DIM
+        if fused and q_len == 1 and start_pos > 0 and len(cache.cache_model) == len(self.layers):
             x = x.contiguous()
             delta = None
             for layer in self.layers:
                 delta = layer.decode_step(x, delta, position_embeddings, start_pos, cache)
             return step_linear(ops.add_rms_norm(x, delta, self.norm.weight, self.norm.eps), self.lm_head)[:, 0]
-        if self.config.fused_decode and q_len > 1 and x.shape[-1] <= ops.NORM_MAX_DIM:
+        if fused and q_len > 1:
             x = x.contiguous()
             delta = None
             for layer in self.layers:

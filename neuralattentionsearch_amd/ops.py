@@ -52,7 +52,10 @@ def _require_cuda(*ts):
 
 
 def workspace(device, key: str, nbytes: int) -> torch.Tensor:
-    """A per-(device, purpose) scratch buffer that only ever grows."""
+    """A per-(device, purpose) scratch buffer that only ever grows.
+
+    Calls of one purpose share the buffer, so they must be ordered on the device: issue them on one stream (or
+    order the streams with events).  Two streams that run, say, two prefills side by side would race on it."""
     k = (str(device), key)
     buf = _workspaces.get(k)
     if buf is None or buf.numel() < nbytes:
@@ -322,10 +325,14 @@ def decode_attention(q: torch.Tensor, cache_k: torch.Tensor, cache_v: torch.Tens
     hold nothing valid (size_global_kv + size_local_kv and the start of the open chunk); they are skipped."""
     _require_cuda(q, cache_k, cache_v, valid)
     lib = _lib.load()
+    if q.dim() != 4 or cache_k.dim() != 4 or valid.dim() != 3:
+        raise ValueError("decode_attention takes q [B, H_q, 1, D], cache_k / cache_v [B, H_kv, rows, D], valid [B, H_kv, rows]")
     B, Hq, one, D = q.shape
     if one != 1:
         raise ValueError("decode_attention takes exactly one query token per sequence")
     Hkv = cache_k.shape[1]
+    if cache_k.shape[0] != B or cache_k.shape[3] != D or tuple(valid.shape[:2]) != (B, Hkv) or Hkv == 0 or Hq % Hkv:
+        raise ValueError(f"shape mismatch: q {tuple(q.shape)}, cache {tuple(cache_k.shape)}, valid {tuple(valid.shape)}")
     if cache_k.shape != cache_v.shape or cache_k.stride() != cache_v.stride():
         raise ValueError("cache_k and cache_v must share shape and strides")
     if cache_k.shape[2] < n_rows or valid.shape[2] < n_rows:
@@ -495,7 +502,8 @@ class MatvecPlan:
 
     def current(self, weight: torch.Tensor) -> bool:
         """Whether the plan still describes `weight` (same storage, dtype and shape)."""
-        return weight.data_ptr() == self.w_ptr and weight.dtype == self.dtype and weight.shape[1] == self.k
+        return (weight.data_ptr() == self.w_ptr and weight.dtype == self.dtype and weight.shape[1] == self.k
+                and weight.shape[0] == (2 * self.n if self.gate else self.n) and weight.stride(0) == self.w_stride)
 
     def takes(self, x: torch.Tensor) -> bool:
         k = self.k

@@ -30,8 +30,9 @@ How each function is pinned (see tests/test_oracle_*.py):
 Functions with parity unpinned: none of the above.  The reference's per-token cache class (chunk_size == 1,
 components/cache/nats_layer_cache.py: 16-token deferred eviction, its own row order) is not restated here; per-token
 roles are covered as ChunkCacheOracle with C = 1, which gives the visibility and the surviving tokens of the
-per-token rules but not that class's cache layout (parity unpinned for the layout: the class cannot be imported
-in the reference's own checkout, so no vectors of it exist).
+per-token rules but not that class's cache layout, nor the extra tokens it leaves visible between two deferred
+evictions (parity unpinned for both: the class cannot be imported in the reference's own checkout, so no vectors of
+it exist).
 """
 from __future__ import annotations
 
