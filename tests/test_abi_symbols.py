@@ -95,6 +95,18 @@ def test_evict_params_are_validated():
     assert rc == -2
 
 
+def test_missing_library_raises_instead_of_falling_back(monkeypatch, tmp_path):
+    """Without the built shared object every operator raises: there is no CPU or PyTorch path behind them."""
+    import torch
+    from neuralattentionsearch_amd import ops
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libnats_hip.so"))
+    with pytest.raises(ImportError, match="no CPU or PyTorch fallback"):
+        _lib.load()
+    with pytest.raises(ImportError):
+        ops.matvec_ok(torch.zeros(1, 8), torch.zeros(8, 8)) or ops.MatvecPlan(torch.zeros(8, 8))
+
+
 def test_ops_reject_cpu_tensors():
     import torch
     from neuralattentionsearch_amd import ops
