@@ -169,6 +169,7 @@ __global__ __launch_bounds__(256) void decode_split_mfma_kernel(DecodeArgs a) {
 
     const int b = ks / a.Hkv, hkv = ks % a.Hkv;
     const int hq0 = hkv * a.n_rep + grp * NREP;
+    const int nr = min(NREP, a.n_rep - grp * NREP);  // q heads of this group (the last group may hold fewer)
     const uint16_t* kp = static_cast<const uint16_t*>(a.k) + b * a.ks_b + hkv * a.ks_h;
     const uint16_t* vp = static_cast<const uint16_t*>(a.v) + b * a.ks_b + hkv * a.ks_h;
     const uint8_t* valp = a.valid + b * a.vs_b + hkv * a.vs_h;
@@ -177,14 +178,14 @@ __global__ __launch_bounds__(256) void decode_split_mfma_kernel(DecodeArgs a) {
     const int e = a.row_end ? (int)min((long long)a.row_end[ks], (long long)ts) : a.n_rows;
     const int nA = (e + kDecTile - 1) / kDecTile;
 
-    // Q as the B operand: column = q head of the group (zero beyond NREP), k = 8 dims per lane group
+    // Q as the B operand: column = q head of the group (zero beyond nr), k = 8 dims per lane group
     bf16x8 qreg[STEPS];
     {
-      const uint16_t* qp = static_cast<const uint16_t*>(a.q) + ((int64_t)b * a.Hq + hq0 + (l16 < NREP ? l16 : 0)) * D;
+      const uint16_t* qp = static_cast<const uint16_t*>(a.q) + ((int64_t)b * a.Hq + hq0 + (l16 < nr ? l16 : 0)) * D;
 #pragma unroll
       for (int s = 0; s < STEPS; ++s) {
         uint4 raw = *reinterpret_cast<const uint4*>(qp + s * 32 + lg * 8);
-        if (l16 >= NREP) raw = make_uint4(0, 0, 0, 0);
+        if (l16 >= nr) raw = make_uint4(0, 0, 0, 0);
         qreg[s] = __builtin_bit_cast(bf16x8, raw);
       }
     }
@@ -192,7 +193,7 @@ __global__ __launch_bounds__(256) void decode_split_mfma_kernel(DecodeArgs a) {
     f32x4 oacc[DB];  // O^T block db: lane holds dims db*16 + lg*4 + i of q head l16
 #pragma unroll
     for (int db = 0; db < DB; ++db) oacc[db] = f32x4{0.f, 0.f, 0.f, 0.f};
-    float m_run = -INFINITY, l_run = 0.f;  // of q head l16 (meaningful for l16 < NREP)
+    float m_run = -INFINITY, l_run = 0.f;  // of q head l16 (meaningful for l16 < nr)
 
     uint4 kreg[2][STEPS];
 
@@ -280,7 +281,7 @@ __global__ __launch_bounds__(256) void decode_split_mfma_kernel(DecodeArgs a) {
         mx = fmaxf(mx, __shfl_xor(mx, 32)) * c;  // vm != 0, so the maximum is finite
         // raise the running maximum only when it is exceeded by more than the slack (probabilities stay
         // below 2^slack otherwise); the accumulators are rescaled only then
-        if (__ballot(l16 < NREP && mx > m_run + kDecodeRescaleSlack)) {
+        if (__ballot(l16 < nr && mx > m_run + kDecodeRescaleSlack)) {
           float m_new = fmaxf(m_run, mx);
           float alpha = m_run == -INFINITY ? 0.f : exp2_guard(m_run - m_new);
           l_run *= alpha;
@@ -330,18 +331,18 @@ __global__ __launch_bounds__(256) void decode_split_mfma_kernel(DecodeArgs a) {
     l_run += __shfl_xor(l_run, 16);
     l_run += __shfl_xor(l_run, 32);
     float* wacc_mine = reinterpret_cast<float*>(&sm.v[wave][0][0]);  // [NREP][D], this wavefront's tiles are consumed
-    if (l16 < NREP) {
+    if (l16 < nr) {
 #pragma unroll
       for (int db = 0; db < DB; ++db)
 #pragma unroll
         for (int i = 0; i < 4; ++i) wacc_mine[l16 * D + db * 16 + lg * 4 + i] = oacc[db][i];
     }
-    if (lane < NREP) {
+    if (lane < nr) {
       sm.wm[wave][lane] = m_run;
       sm.wl[wave][lane] = l_run;
     }
     __syncthreads();
-    for (int idx = tid; idx < NREP * D; idx += 256) {
+    for (int idx = tid; idx < nr * D; idx += 256) {
       int h = idx / D, d = idx % D;
       float M = fmaxf(fmaxf(sm.wm[0][h], sm.wm[1][h]), fmaxf(sm.wm[2][h], sm.wm[3][h]));
       float sum = 0.f, lsum = 0.f;
@@ -643,38 +644,54 @@ extern "C" int nats_decode_fwd(const void* q, const void* cache_k, const void* c
     return NATS_OK;
   }
 
-  NATS_REQUIRE(B * H_kv <= kMaxBalancedHeads, NATS_ERR_UNSUPPORTED,
-               "nats_decode_fwd: %lld (batch, kv head) streams, the bf16 kernel schedules at most %d", (long long)(B * H_kv),
+  NATS_REQUIRE(H_kv <= kMaxBalancedHeads, NATS_ERR_UNSUPPORTED,
+               "nats_decode_fwd: %lld kv heads, the bf16 kernel schedules at most %d per sequence", (long long)H_kv,
                kMaxBalancedHeads);
-  a.n_wg = decode_balanced_workgroups(B, H_kv, n_rows);
-  a.head_table = static_cast<int2*>(workspace);
-  a.ws_acc = reinterpret_cast<float*>(static_cast<char*>(workspace) + align256((size_t)(B * H_kv) * sizeof(int2)));
-  a.ws_ml = a.ws_acc + ((size_t)a.n_wg + (size_t)(B * H_kv)) * (size_t)a.n_rep * D;
-  int n_rep = a.n_rep;
-  int nrep_k = (n_rep % 8 == 0) ? 8 : (n_rep % 4 == 0) ? 4 : (n_rep % 2 == 0) ? 2 : 1;
-  int groups = n_rep / nrep_k;
-  int rc;
-  if (D == 128) {
-    switch (nrep_k) {
-      case 8: rc = launch_mfma<128, 8>(a, groups, st); break;
-      case 4: rc = launch_mfma<128, 4>(a, groups, st); break;
-      case 2: rc = launch_mfma<128, 2>(a, groups, st); break;
-      default: rc = launch_mfma<128, 1>(a, groups, st); break;
+  // One launch pair schedules at most kMaxBalancedHeads (b, kv head) streams (their prefix sums live in LDS); a
+  // larger batch goes in groups of whole sequences, one after the other on the stream, over the same workspace.
+  const int64_t b_step = kMaxBalancedHeads / H_kv;
+  const int n_rep = a.n_rep;
+  // q heads of a kv head share the key / value rows of one pass, up to eight at a time (columns of the MFMA);
+  // a group size that is no power of two runs the next wider kernel with its spare columns zero
+  const int nrep_k = n_rep >= 5 ? 8 : n_rep >= 3 ? 4 : n_rep;
+  const int groups = (n_rep + nrep_k - 1) / nrep_k;
+  for (int64_t b0 = 0; b0 < B; b0 += b_step) {
+    const int64_t nb = B - b0 < b_step ? B - b0 : b_step;
+    DecodeArgs c = a;
+    c.B = (int)nb;
+    c.q = static_cast<const uint16_t*>(q) + b0 * H_q * D;
+    c.k = static_cast<const uint16_t*>(cache_k) + b0 * a.ks_b;
+    c.v = static_cast<const uint16_t*>(cache_v) + b0 * a.ks_b;
+    c.valid = valid + b0 * a.vs_b;
+    c.row_end = a.row_end ? a.row_end + b0 * H_kv : nullptr;
+    c.o = static_cast<uint16_t*>(o) + b0 * H_q * D;
+    c.n_wg = decode_balanced_workgroups(nb, H_kv, n_rows);
+    c.head_table = static_cast<int2*>(workspace);
+    c.ws_acc = reinterpret_cast<float*>(static_cast<char*>(workspace) + align256((size_t)(nb * H_kv) * sizeof(int2)));
+    c.ws_ml = c.ws_acc + ((size_t)c.n_wg + (size_t)(nb * H_kv)) * (size_t)n_rep * D;
+    int rc;
+    if (D == 128) {
+      switch (nrep_k) {
+        case 8: rc = launch_mfma<128, 8>(c, groups, st); break;
+        case 4: rc = launch_mfma<128, 4>(c, groups, st); break;
+        case 2: rc = launch_mfma<128, 2>(c, groups, st); break;
+        default: rc = launch_mfma<128, 1>(c, groups, st); break;
+      }
+    } else {
+      switch (nrep_k) {
+        case 8: rc = launch_mfma<64, 8>(c, groups, st); break;
+        case 4: rc = launch_mfma<64, 4>(c, groups, st); break;
+        case 2: rc = launch_mfma<64, 2>(c, groups, st); break;
+        default: rc = launch_mfma<64, 1>(c, groups, st); break;
+      }
     }
-  } else {
-    switch (nrep_k) {
-      case 8: rc = launch_mfma<64, 8>(a, groups, st); break;
-      case 4: rc = launch_mfma<64, 4>(a, groups, st); break;
-      case 2: rc = launch_mfma<64, 2>(a, groups, st); break;
-      default: rc = launch_mfma<64, 1>(a, groups, st); break;
-    }
+    if (rc) return rc;
+    NATS_CHECK_LAUNCH("decode_split_mfma_kernel");
+    // (a head has at most one partial per workgroup plus one)
+    const size_t merge_smem = ((size_t)c.n_wg + 2 + 8) * sizeof(float);
+    hipLaunchKernelGGL(decode_merge_balanced_kernel, dim3((unsigned)(nb * H_q)), dim3((unsigned)D), merge_smem, st, c.ws_acc,
+                       c.ws_ml, c.head_table, static_cast<uint16_t*>(c.o), (int)H_q, (int)H_kv, (int)D);
+    NATS_CHECK_LAUNCH("decode_merge_balanced_kernel");
   }
-  if (rc) return rc;
-  NATS_CHECK_LAUNCH("decode_split_mfma_kernel");
-  // (a head has at most one partial per workgroup plus one)
-  const size_t merge_smem = ((size_t)a.n_wg + 2 + 8) * sizeof(float);
-  hipLaunchKernelGGL(decode_merge_balanced_kernel, dim3((unsigned)(B * H_q)), dim3((unsigned)D), merge_smem, st, a.ws_acc, a.ws_ml,
-                     a.head_table, static_cast<uint16_t*>(o), (int)H_q, (int)H_kv, (int)D);
-  NATS_CHECK_LAUNCH("decode_merge_balanced_kernel");
   return NATS_OK;
 }

@@ -1743,9 +1743,7 @@ int launch_segment(const char* who, const SegmentShape& g, const void* q, const 
 
   // bf16: pack the q heads of one kv head into one workgroup (up to 4), fill the rest with query tiles
   int n_rep = a.n_rep;
-  int hpw = n_rep >= 4 ? 4 : n_rep;
-  NATS_REQUIRE(n_rep % hpw == 0 && (4 % hpw) == 0, NATS_ERR_UNSUPPORTED,
-               "%s: GQA group size %d (supported: 1, 2, 4 and multiples of 4)", who, n_rep);
+  int hpw = n_rep % 4 == 0 ? 4 : n_rep % 2 == 0 ? 2 : 1;  // (a group of 3, 5, 6, 7 ... goes in parts of 1 or 2 heads)
   a.hpw = hpw;
   a.qpw = 4 / hpw;
   a.n_hg = n_rep / hpw;
@@ -1812,7 +1810,7 @@ extern "C" size_t nats_prefill_sched_workspace_bytes(int64_t B, int64_t H_q, int
   const size_t sched = carve_stream_sched(nullptr, B, H_q, H_kv, n_qt, Tk).bytes;
   // the partial results of a split launch use the same region (a launch is either split or persistent)
   const int64_t n_rep = H_q / H_kv;
-  const int64_t hpw = n_rep >= 4 ? 4 : (n_rep > 0 ? n_rep : 1);
+  const int64_t hpw = n_rep % 4 == 0 ? 4 : n_rep % 2 == 0 ? 2 : 1;  // as in launch_segment
   // (a split launch never has more workgroups than the device has CUs, whatever the exact number of query tiles
   // turns out to be: room for that many partial results whenever a launch of this size may be split)
   const int64_t n_qg_min = (n_qt > 1 ? n_qt - 1 : 1) + 4 / hpw - 1;

@@ -59,7 +59,7 @@ def run_case(B, Hq, Hkv, D, W, C, n_max_chunks, dtype, seed=0, frac=(0.1, 1.0), 
     assert err2 <= TOL[dtype], f"max abs err with hint {err2}"
 
 
-@pytest.mark.parametrize("n_rep", [1, 2, 4, 8])
+@pytest.mark.parametrize("n_rep", [1, 2, 3, 4, 5, 6, 7, 8, 12, 16])
 @pytest.mark.parametrize("D", [64, 128])
 def test_bf16_group_sizes(n_rep, D):
     run_case(2, 2 * n_rep, 2, D, 128, 64, 20, torch.bfloat16, seed=n_rep + D)
@@ -72,6 +72,12 @@ def test_bf16_chunk_sizes_and_open_chunk(C, W, fill):
 
 def test_bf16_single_sequence_long_cache():
     run_case(1, 32, 8, 128, 256, 64, 300, torch.bfloat16, seed=9, frac=(0.2, 1.0), fill=13)
+
+
+def test_bf16_more_streams_than_one_launch_schedules():
+    """More than 1024 (batch, kv head) streams: the library takes the batch in groups of whole sequences."""
+    run_case(300, 8, 4, 64, 16, 8, 6, torch.bfloat16, seed=21, fill=3)   # 1200 streams: 256 + 44 sequences
+    run_case(129, 16, 8, 128, 64, 16, 4, torch.bfloat16, seed=22)       # 1032 streams: 128 + 1 sequences
 
 
 def test_bf16_nothing_but_the_new_token():

@@ -40,7 +40,7 @@ def test_fp32_ragged_lengths_and_chunk_sizes(L, C, W, D):
     run_case(2, 4, 2, L, D, C, W, torch.float32, seed=L)
 
 
-@pytest.mark.parametrize("n_rep", [1, 2, 4, 8])
+@pytest.mark.parametrize("n_rep", [1, 2, 3, 4, 6, 7, 8, 12])
 def test_bf16_gqa_group_sizes(n_rep):
     run_case(1, 2 * n_rep, 2, 1024, 128, 64, 256, torch.bfloat16, seed=n_rep)
     run_case(1, 2 * n_rep, 2, 1100, 128, 16, 64, torch.bfloat16, seed=n_rep)  # packed tiles
