@@ -157,94 +157,101 @@ __global__ __launch_bounds__(256) void decode_split_mfma_kernel(DecodeArgs a) {
   int ks = sm.first_head;  // b * Hkv + hkv
   const float c = a.scale * 1.4426950408889634f;
 
-  while (pos < pos_end) {
-    const int p0 = sm.tile_prefix[ks], p1 = sm.tile_prefix[ks + 1];
-    if (p1 == p0) {  // a head without tiles
-      ++ks;
-      continue;
+  const int nr = min(NREP, a.n_rep - grp * NREP);  // q heads of this group (the last group may hold fewer)
+
+  // ---- state of the head being walked (set by begin_head) ----------------------------------------------
+  const uint16_t* kp = nullptr;
+  const uint16_t* vp = nullptr;
+  const uint8_t* valp = nullptr;
+  int e = 0, nA = 0;    // rows [0, e) and [ts, n_rows) are walked; nA = tiles of the first range
+  int t = 0, t_end = 0; // this wavefront's next tile and the end of the workgroup's tiles, within the head
+  int slot = 0;         // where the head's partial result goes
+  int cur = 0;          // LDS buffer of tile t
+  uint32_t vm = 0, vb_next = 0;
+  bf16x8 qreg[STEPS];   // Q as the B operand: column = q head of the group (zero beyond nr), k = 8 dims per lane group
+  uint4 kreg[2][STEPS];
+
+  // Rows are walked in 32-row tiles over [0, e) and [ts, n_rows); [e, ts) is the dead region between this
+  // head's own end and the open chunk (nothing there is valid), skipped without a look when hinted.
+  auto tile_row0 = [&](int tt) -> int { return tt < nA ? tt * kDecTile : ts + (tt - nA) * kDecTile; };
+  auto tile_row1 = [&](int tt) -> int {
+    return tt < nA ? min(tt * kDecTile + kDecTile, e) : min(ts + (tt - nA + 1) * kDecTile, a.n_rows);
+  };
+  auto load_valid = [&](int tt) -> uint32_t {
+    uint32_t vb = 0;
+    if (tt < t_end) {
+      int r0 = tile_row0(tt), r1 = tile_row1(tt);
+      if (lane < kDecTile && r0 + lane < r1) vb = valp[r0 + lane];
     }
-    const int seg_end = min(pos_end, p1);
-    const int t_begin = pos - p0, t_end = seg_end - p0;  // tiles of this head
-    const int slot = sm.slot_prefix[ks] + (wg - p0 / tpw);
-
-    const int b = ks / a.Hkv, hkv = ks % a.Hkv;
-    const int hq0 = hkv * a.n_rep + grp * NREP;
-    const int nr = min(NREP, a.n_rep - grp * NREP);  // q heads of this group (the last group may hold fewer)
-    const uint16_t* kp = static_cast<const uint16_t*>(a.k) + b * a.ks_b + hkv * a.ks_h;
-    const uint16_t* vp = static_cast<const uint16_t*>(a.v) + b * a.ks_b + hkv * a.ks_h;
-    const uint8_t* valp = a.valid + b * a.vs_b + hkv * a.vs_h;
-    // Rows are walked in 32-row tiles over [0, e) and [ts, n_rows); [e, ts) is the dead region between this
-    // head's own end and the open chunk (nothing there is valid), skipped without a look when hinted.
-    const int e = a.row_end ? (int)min((long long)a.row_end[ks], (long long)ts) : a.n_rows;
-    const int nA = (e + kDecTile - 1) / kDecTile;
-
-    // Q as the B operand: column = q head of the group (zero beyond nr), k = 8 dims per lane group
-    bf16x8 qreg[STEPS];
-    {
-      const uint16_t* qp = static_cast<const uint16_t*>(a.q) + ((int64_t)b * a.Hq + hq0 + (l16 < nr ? l16 : 0)) * D;
+    return vb;
+  };
+  auto issue_k = [&](int r0, uint32_t m) {
+    const int fv = __builtin_ctz(m);
+#pragma unroll
+    for (int g = 0; g < 2; ++g) {
+      int kl = g * 16 + l16;
+      int row = ((m >> kl) & 1) ? kl : fv;
+      const uint16_t* rp = kp + (int64_t)(r0 + row) * a.ks_r + lg * 8;
 #pragma unroll
       for (int s = 0; s < STEPS; ++s) {
-        uint4 raw = *reinterpret_cast<const uint4*>(qp + s * 32 + lg * 8);
-        if (l16 >= nr) raw = make_uint4(0, 0, 0, 0);
-        qreg[s] = __builtin_bit_cast(bf16x8, raw);
+        const u32x4 w = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(rp + s * 32));
+        kreg[g][s] = make_uint4(w.x, w.y, w.z, w.w);
       }
     }
-
-    f32x4 oacc[DB];  // O^T block db: lane holds dims db*16 + lg*4 + i of q head l16
+  };
+  auto issue_v = [&](int r0, uint32_t m, int buf) {
+    const int fv = __builtin_ctz(m);
 #pragma unroll
-    for (int db = 0; db < DB; ++db) oacc[db] = f32x4{0.f, 0.f, 0.f, 0.f};
-    float m_run = -INFINITY, l_run = 0.f;  // of q head l16 (meaningful for l16 < nr)
-
-    uint4 kreg[2][STEPS];
-
-    auto tile_row0 = [&](int t) -> int { return t < nA ? t * kDecTile : ts + (t - nA) * kDecTile; };
-    auto tile_row1 = [&](int t) -> int {
-      return t < nA ? min(t * kDecTile + kDecTile, e) : min(ts + (t - nA + 1) * kDecTile, a.n_rows);
-    };
-    auto load_valid = [&](int t) -> uint32_t {
-      uint32_t vb = 0;
-      if (t < t_end) {
-        int r0 = tile_row0(t), r1 = tile_row1(t);
-        if (lane < kDecTile && r0 + lane < r1) vb = valp[r0 + lane];
-      }
-      return vb;
-    };
-    auto issue_k = [&](int r0, uint32_t vm) {
-      const int fv = __builtin_ctz(vm);
+    for (int j = 0; j < NDMA; ++j) {
+      const int q = j * kWave + lane;  // chunk slot in the LDS tile
+      const int row = q / OCT, cpos = q % OCT;
+      const int src_row = ((m >> row) & 1) ? row : fv;
+      const int chunk = cpos ^ ((row & 3) << 1);
+      __builtin_amdgcn_global_load_lds(vp + (int64_t)(r0 + src_row) * a.ks_r + chunk * 8,
+                                       (uint32_t __attribute__((address_space(3)))*)(&sm.v[wave][buf][j * kWave * 8]), 16, 0,
+                                       kAuxStream);
+    }
+  };
+  // Moves on to the head that holds tile `pos` of the list (`ks` is that head or an empty one before it): its
+  // pointers and ranges, Q, and the requests for this wavefront's first tile, into LDS buffer `buf`.  Returns the
+  // end of the workgroup's tiles in that head, as a list position.
+  auto begin_head = [&](int buf) -> int {
+    while (sm.tile_prefix[ks + 1] == sm.tile_prefix[ks]) ++ks;  // heads without tiles (pos < total: one with tiles follows)
+    const int p0 = sm.tile_prefix[ks], p1 = sm.tile_prefix[ks + 1];
+    const int seg_end = min(pos_end, p1);
+    t_end = seg_end - p0;
+    slot = sm.slot_prefix[ks] + (wg - p0 / tpw);
+    const int b = ks / a.Hkv, hkv = ks % a.Hkv;
+    const int hq0 = hkv * a.n_rep + grp * NREP;
+    kp = static_cast<const uint16_t*>(a.k) + b * a.ks_b + hkv * a.ks_h;
+    vp = static_cast<const uint16_t*>(a.v) + b * a.ks_b + hkv * a.ks_h;
+    valp = a.valid + b * a.vs_b + hkv * a.vs_h;
+    e = a.row_end ? (int)min((long long)a.row_end[ks], (long long)ts) : a.n_rows;
+    nA = (e + kDecTile - 1) / kDecTile;
+    const uint16_t* qp = static_cast<const uint16_t*>(a.q) + ((int64_t)b * a.Hq + hq0 + (l16 < nr ? l16 : 0)) * D;
 #pragma unroll
-      for (int g = 0; g < 2; ++g) {
-        int kl = g * 16 + l16;
-        int row = ((vm >> kl) & 1) ? kl : fv;
-        const uint16_t* rp = kp + (int64_t)(r0 + row) * a.ks_r + lg * 8;
-#pragma unroll
-        for (int s = 0; s < STEPS; ++s) {
-          const u32x4 w = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(rp + s * 32));
-          kreg[g][s] = make_uint4(w.x, w.y, w.z, w.w);
-        }
-      }
-    };
-    auto issue_v = [&](int r0, uint32_t vm, int buf) {
-      const int fv = __builtin_ctz(vm);
-#pragma unroll
-      for (int j = 0; j < NDMA; ++j) {
-        const int q = j * kWave + lane;  // chunk slot in the LDS tile
-        const int row = q / OCT, cpos = q % OCT;
-        const int src_row = ((vm >> row) & 1) ? row : fv;
-        const int chunk = cpos ^ ((row & 3) << 1);
-        __builtin_amdgcn_global_load_lds(vp + (int64_t)(r0 + src_row) * a.ks_r + chunk * 8,
-                                         (uint32_t __attribute__((address_space(3)))*)(&sm.v[wave][buf][j * kWave * 8]), 16, 0,
-                                         kAuxStream);
-      }
-    };
-
-    int t = t_begin + wave;
-    int cur = 0;
-    uint32_t vm = (uint32_t)__ballot(load_valid(t) != 0);
+    for (int s = 0; s < STEPS; ++s) {
+      uint4 raw = *reinterpret_cast<const uint4*>(qp + s * 32 + lg * 8);
+      if (l16 >= nr) raw = make_uint4(0, 0, 0, 0);
+      qreg[s] = __builtin_bit_cast(bf16x8, raw);
+    }
+    t = pos - p0 + wave;
+    cur = buf;
+    vm = (uint32_t)__ballot(load_valid(t) != 0);
     if (vm) {
       issue_k(tile_row0(t), vm);
       issue_v(tile_row0(t), vm, cur);
     }
-    uint32_t vb_next = load_valid(t + 4);
+    vb_next = load_valid(t + 4);
+    return seg_end;
+  };
+
+  int seg_end = begin_head(0);
+  for (;;) {
+    f32x4 oacc[DB];  // O^T block db: lane holds dims db*16 + lg*4 + i of q head l16
+#pragma unroll
+    for (int db = 0; db < DB; ++db) oacc[db] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.f;  // of q head l16 (meaningful for l16 < nr)
 
     while (t < t_end) {
       __builtin_amdgcn_s_waitcnt(0);  // K(t) in registers, V(t) in LDS, valid bytes of the next tile loaded
@@ -328,9 +335,12 @@ __global__ __launch_bounds__(256) void decode_split_mfma_kernel(DecodeArgs a) {
     __builtin_amdgcn_s_waitcnt(0);
 
     // ---- merge the wavefronts of the workgroup, emit this head's partial ------------------------------
+    // The accumulators are staged in the wavefront's LDS buffer 0 (its tiles are consumed); the first tile of the
+    // workgroup's next head, if there is one, is requested into buffer 1 before the merge, which hides most of its
+    // trip from memory.
     l_run += __shfl_xor(l_run, 16);
     l_run += __shfl_xor(l_run, 32);
-    float* wacc_mine = reinterpret_cast<float*>(&sm.v[wave][0][0]);  // [NREP][D], this wavefront's tiles are consumed
+    float* wacc_mine = reinterpret_cast<float*>(&sm.v[wave][0][0]);  // [NREP][D]
     if (l16 < nr) {
 #pragma unroll
       for (int db = 0; db < DB; ++db)
@@ -340,6 +350,13 @@ __global__ __launch_bounds__(256) void decode_split_mfma_kernel(DecodeArgs a) {
     if (lane < nr) {
       sm.wm[wave][lane] = m_run;
       sm.wl[wave][lane] = l_run;
+    }
+    const int slot_done = slot;
+    pos = seg_end;
+    const bool more = pos < pos_end;  // (the same for every wavefront of the workgroup)
+    if (more) {
+      ++ks;
+      seg_end = begin_head(1);
     }
     __syncthreads();
     for (int idx = tid; idx < nr * D; idx += 256) {
@@ -354,16 +371,15 @@ __global__ __launch_bounds__(256) void decode_split_mfma_kernel(DecodeArgs a) {
           lsum += sm.wl[w][h] * f;
         }
       }
-      const int64_t prt = (int64_t)slot * a.n_rep + grp * NREP + h;  // partial of (slot, q head in the kv group)
+      const int64_t prt = (int64_t)slot_done * a.n_rep + grp * NREP + h;  // partial of (slot, q head in the kv group)
       a.ws_acc[prt * D + d] = sum;
       if (d == 0) {
         a.ws_ml[prt * 2 + 0] = M;
         a.ws_ml[prt * 2 + 1] = lsum;
       }
     }
-    __syncthreads();  // wacc / wm / wl are reused by the next head
-    pos = seg_end;
-    ++ks;
+    if (!more) break;
+    __syncthreads();  // the staged accumulators, wm and wl are reused by the next head
   }
 }
 
