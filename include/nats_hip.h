@@ -196,7 +196,9 @@ int nats_prefill_past_mask(const uint8_t* valid, const int64_t* size_global, con
  *           hold nothing valid (the cache's size_global_kv + size_local_kv and the start of the open chunk,
  *           components/cache/nats_chunk_layer_cache.py:644-656) and are skipped without reading valid
  *   workspace: nats_decode_workspace_bytes(...) bytes
- * D in {64, 128}; dtype bf16 (MFMA) or f32 (fp32 FMA kernel, ignores the hint).
+ * D in {64, 128}; H_q % H_kv == 0 (any group size); dtype bf16 (MFMA) or f32 (fp32 FMA kernel, ignores the hint).
+ * bf16: a batch of more than 1024 (b, kv head) streams is taken in groups of whole sequences, launched one after
+ * the other on `stream`.
  */
 size_t nats_decode_workspace_bytes(int64_t B, int64_t H_q, int64_t H_kv, int64_t D, int64_t n_rows);
 
