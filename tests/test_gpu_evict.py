@@ -201,3 +201,38 @@ def test_cfg4_bulk_eviction_properties():
             assert int(valid[b, h, W:].sum()) == int(sg[b, h] - W + sl[b, h])
     assert int(valid.sum()) == int((sg - W + sl).sum() + (roles[:, :, S - W // C:] == 2).sum() * C)
     assert not hip.cache_k[:, :, hip.n_ctx_data:].any()
+
+
+def test_cfg4_streamed_eviction_equals_bulk():
+    """The same 16 x 8 x 65536-token stream appended chunk by chunk (1024 x update(64) + post_update(64)) leaves
+    the sizes, the surviving tokens and their rows that one bulk post_update(65536) leaves."""
+    from neuralattentionsearch_amd.cache import NAtSChunkLayerCache
+    say("evict cfg4 streamed against bulk")
+    B, H, L, D, C, W = 16, 8, 65536, 128, 64, 512
+    S = L // C
+    rng = np.random.default_rng(1)
+    roles = rng.choice(3, size=(B, H, S), p=(0.10, 0.15, 0.75)).astype(np.uint8)
+    roles[:, :, 0] = 0
+    g = torch.Generator(device="cuda").manual_seed(1)
+    k = torch.randn(B, H, L, D, generator=g, device="cuda", dtype=torch.bfloat16)
+    v = torch.randn(B, H, L, D, generator=g, device="cuda", dtype=torch.bfloat16)
+    tsi = one_hot_roles(roles, dtype=torch.bfloat16).cuda()
+    bulk = NAtSChunkLayerCache(B, H, W, chunk_size=C, device="cuda", track_positions=True)
+    bulk.update(k, v, tsi)
+    bulk.post_update(L)
+    stream = NAtSChunkLayerCache(B, H, W, chunk_size=C, device="cuda", track_positions=True)
+    for s in range(S):
+        stream.update(k[:, :, s * C:(s + 1) * C], v[:, :, s * C:(s + 1) * C], tsi[:, :, s:s + 1])
+        stream.post_update(C)
+    assert torch.equal(stream.size_global_kv, bulk.size_global_kv)
+    assert torch.equal(stream.size_local_kv, bulk.size_local_kv)
+    assert stream.n_ctx_data == bulk.n_ctx_data and stream.sliding_queue_tail == bulk.sliding_queue_tail
+    n = bulk.n_ctx_data
+    vs, vb = stream.valid_tokens[:, :, :n], bulk.valid_tokens[:, :, :n]
+    assert torch.equal(vs, vb)
+    ps, pb = stream.token_positions[:, :, :n], bulk.token_positions[:, :, :n]
+    assert torch.equal(torch.where(vs, ps, -1), torch.where(vb, pb, -1))
+    m = vs.unsqueeze(-1)
+    assert torch.equal(stream.cache_k[:, :, :n] * m, bulk.cache_k[:, :, :n] * m)
+    assert torch.equal(stream.cache_v[:, :, :n] * m, bulk.cache_v[:, :, :n] * m)
+
