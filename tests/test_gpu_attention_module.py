@@ -97,3 +97,39 @@ def run_module(lens, C, W):
             assert np.array_equal(layer.valid_tokens.cpu().numpy(), st.valid), step
             assert np.array_equal(layer.size_global_kv.cpu().numpy(), st.size_global), step
             seen += n
+
+
+def test_container_surface_the_reference_callers_use():
+    """NAtSCache through the calls and attributes the reference's callers rely on (components/cache/dyn_cache.py:66-195;
+    attributes read by hf/llama.py:235-252 and experiments/efficiency/eval_efficiency.py:350-352)."""
+    from neuralattentionsearch_amd.cache import NAtSCache
+    say("container surface")
+    B, H, D, C, W, L = 2, 2, 64, 8, 16, 40
+    cache = NAtSCache(sliding_window_size=W, chunk_size=C)
+    assert cache.get_seq_length(0) == 0 and cache.get_nats_chunk_fill_size(0) == 0
+    assert cache.get_nats_cached_x_in_chunk(0) is None
+    g = torch.Generator().manual_seed(5)
+    k = torch.randn(B, H, L, D, generator=g).bfloat16().cuda()
+    v = torch.randn(B, H, L, D, generator=g).bfloat16().cuda()
+    roles = np.array([[[0, 2, 1, 0, 2], [0, 1, 1, 2, 2]]] * B, dtype=np.uint8)
+    tsi = orc.one_hot_roles(roles, dtype=torch.bfloat16).cuda()
+    keys, values = cache.update(k, v, 0, cache_kwargs={"token_states_info": tsi})
+    assert keys.shape == k.shape and torch.equal(keys, k) and torch.equal(values, v)  # the first call hands back the raw K, V
+    mask = cache.generate_mask(0, L)
+    assert mask.dtype == torch.bool and tuple(mask.shape) == (B, H, L, L)
+    cache.post_update(layer_idx=0, x_len=L)
+    layer = cache.cache_model[0]
+    assert cache.get_seq_length(0) == L and layer.get_seq_length() == L
+    assert cache.get_nats_chunk_fill_size(0) == 0 == layer.chunk_fill_size
+    assert layer._tokens_info is tsi
+    # head 0: global chunks 0 and 3, nothing local after the last global; head 1: global chunk 0, local chunks 1 and 2
+    assert layer.size_global_kv.tolist() == [[W + 2 * C, W + C]] * B
+    assert layer.size_local_kv.tolist() == [[0, 2 * C]] * B
+    assert layer.n_ctx_data == W + 3 * C and layer.sliding_queue_tail == (min(L // C, W // C) * C) % W
+    assert layer.valid_tokens.dtype == torch.bool and layer.valid_tokens.shape[:2] == (B, H)
+    assert layer.cache_k.shape == layer.cache_v.shape == (B, H, layer.valid_tokens.shape[2], D)
+    # ring: the last W / C = 2 chunks, valid where sliding window (head 0: chunk 4; head 1: chunks 3 and 4)
+    assert layer.valid_tokens[0, 0, :W].tolist() == [False] * C + [True] * C
+    assert layer.valid_tokens[0, 1, :W].tolist() == [True] * W
+    cache.reset_cache()
+    assert cache.cache_model == [] and cache.get_seq_length(0) == 0
