@@ -37,7 +37,7 @@ def test_module_with_per_token_roles(lens, W):
     run_module(lens, 1, W)
 
 
-def run_module(lens, C, W):
+def run_module(lens, C, W, executor=None):
     from neuralattentionsearch_amd.attention import LlamaNAtSChunkAttentionLayer, apply_rotary_pos_emb
     from neuralattentionsearch_amd.cache import NAtSCache
     say("attention module", lens, C, W)
@@ -48,6 +48,7 @@ def run_module(lens, C, W):
                                        chunk_size=C).cuda().eval()
     with torch.no_grad():
         mod.proj_layer.weight.mul_(8.0)  # spread the role logits
+    mod.executor = executor
     logits_seen = []
     mod.proj_layer.register_forward_hook(lambda m, i, o: logits_seen.append(o.detach().float().cpu()))
     cache = NAtSCache(sliding_window_size=W, chunk_size=C)
@@ -97,6 +98,14 @@ def run_module(lens, C, W):
             assert np.array_equal(layer.valid_tokens.cpu().numpy(), st.valid), step
             assert np.array_equal(layer.size_global_kv.cpu().numpy(), st.size_global), step
             seen += n
+
+
+def test_module_with_post_update_on_an_executor():
+    """post_update submitted to a thread pool, as the reference's modules do when `executor` is set
+    (nats_attention.py:189-192)."""
+    from concurrent.futures import ThreadPoolExecutor
+    with ThreadPoolExecutor(max_workers=1) as pool:
+        run_module([50, 1, 1, 1, 20, 1, 1], 8, 16, executor=pool)
 
 
 def test_container_surface_the_reference_callers_use():
