@@ -300,6 +300,9 @@ class NAtSLlamaDecoderLayer(nn.Module):
                 carry = torch.empty_like(x)
                 mode = ops.CARRY_MAX_FIRST if is_max else ops.CARRY_MEAN_FIRST
             else:
+                if carry.shape[1] != 1:  # (max statistic of a first partial chunk: the reference keeps its raw rows)
+                    carry = carry.max(1, keepdim=True)[0]
+                carry = carry.contiguous()
                 mode = ops.CARRY_MAX_MERGE if is_max else ops.CARRY_MEAN_ADD
         h = ops.add_rms_norm(x, delta, self.input_layernorm.weight, self.input_layernorm.eps, carry, mode, C)
         if mode != ops.CARRY_NONE:

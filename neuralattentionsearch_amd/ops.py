@@ -111,6 +111,11 @@ def role_step(x: torch.Tensor, weight: torch.Tensor, chunk_size: int, window: in
         x = x.contiguous()
     weight = weight.contiguous()
     if carry_in is not None:
+        if carry_in.dim() == 3 and carry_in.shape[1] != 1:
+            # the reference keeps the raw rows of a first partial chunk as its max statistic (dyn_cache.py:111-112)
+            if not merge_max:
+                raise ValueError(f"carry_in must be [B, 1, dim] or [B, dim], got {tuple(carry_in.shape)}")
+            carry_in = carry_in.max(1)[0]
         carry_in = carry_in.reshape(B, dim).contiguous()
     total = pre_fill + L
     S = 0 if total < C else math.ceil(total / C)

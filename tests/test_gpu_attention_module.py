@@ -142,3 +142,38 @@ def test_container_surface_the_reference_callers_use():
     assert layer.valid_tokens[0, 1, :W].tolist() == [True] * W
     cache.reset_cache()
     assert cache.cache_model == [] and cache.get_seq_length(0) == 0
+
+
+@pytest.mark.parametrize("method", ["mean", "max"])
+def test_container_chunk_statistics_follow_the_oracle(method):
+    """The running and per-chunk statistics of the hidden states (dyn_cache.py:98-171) that the role projection
+    reads, over a stream cut into ragged segments, against the oracle's restatement."""
+    from neuralattentionsearch_amd.cache import ChunkMergeType, NAtSCache, NAtSChunkLayerCache
+    say("container statistics", method)
+    B, dim, C, W = 2, 96, 8, 16
+    mm = method == "max"
+    kind = ChunkMergeType.MAX if mm else ChunkMergeType.MEAN
+    cache = NAtSCache(sliding_window_size=W, chunk_size=C)
+    cache.cache_model.append(NAtSChunkLayerCache(B, 1, W, 0, C, device="cuda"))
+    layer = cache.cache_model[0]
+    weight = torch.zeros(3, dim)
+    g = torch.Generator().manual_seed(11)
+    fill, carry = 0, None
+    for n in (5, 2, 20, 1, 1, 9, 64, 3, 5, 1):
+        x = torch.randn(B, n, dim, generator=g)
+        pooled_o, _, carry_o, pad_o = orc.pooled_role_logits(x, weight, C, pre_fill=fill, carry_in=carry, merge_max=mm)
+        layer.chunk_fill_size = fill
+        if fill + n < C:
+            cache.update_nats_cached_x_in_chunk(x.cuda(), 0, kind)
+            assert pooled_o is None
+        else:
+            pooled, pad = cache.update_nats_cached_x_across_chunk(x.cuda(), fill, 0, kind)
+            assert pad == pad_o and pooled.shape == pooled_o.shape
+            torch.testing.assert_close(pooled.cpu(), pooled_o, rtol=1e-6, atol=1e-6)
+        got = cache.get_nats_cached_x_in_chunk(0)
+        assert (got is None) == (carry_o is None)
+        if got is not None:
+            if mm:  # (the reference keeps the raw rows of a first partial chunk; their maximum is the statistic)
+                got = got.max(1, keepdim=True)[0]
+            torch.testing.assert_close(got.cpu(), carry_o, rtol=1e-6, atol=1e-6)
+        fill, carry = (fill + n) % C, carry_o

@@ -110,6 +110,16 @@ def test_per_token_roles_layer_by_layer():
     run(cfg, torch.float32, [60, 21] + [1] * 24, tol=2e-5)
 
 
+def test_max_statistic_after_a_short_first_segment():
+    """chunk_merge_method "max": a first segment shorter than a chunk leaves its raw rows as the running statistic
+    (dyn_cache.py:111-112); the one-token steps and segments after it must take that form in."""
+    from neuralattentionsearch_amd.llama import NAtSLlamaConfig
+    cfg = NAtSLlamaConfig(vocab_size=1000, hidden_size=512, intermediate_size=1024, num_hidden_layers=2,
+                          num_attention_heads=8, num_key_value_heads=2, chunk_size=8, local_seq_max_length=16,
+                          chunk_merge_method="max")
+    run(cfg, torch.float32, [3, 1, 1, 2] + [1] * 20 + [19, 1, 1, 30, 1], tol=2e-5, seed=2)
+
+
 def test_llama_head_shape_bf16_layer_by_layer():
     """32 q heads / 8 kv heads / head_dim 128, chunk 64, window 256, two layers."""
     from neuralattentionsearch_amd.llama import NAtSLlamaConfig
@@ -141,14 +151,15 @@ def test_generate_is_deterministic_and_matches_stepwise_forward():
     assert min(l.n_ctx_data for l in cache_a.cache_model) < 45 + 29 + 16
 
 
-def test_fused_role_step_gives_the_same_generation():
+@pytest.mark.parametrize("method,prompt", [("mean", 45), ("max", 45), ("max", 3), ("mean", 3)])
+def test_fused_role_step_gives_the_same_generation(method, prompt):
     """The harness with the fused role-step kernel against the same model with torch pooling + projection (fp32:
     the two differ in summation order only, which the seeded logits' gaps absorb)."""
     from neuralattentionsearch_amd.llama import NAtSLlamaConfig, NAtSLlamaForCausalLM
-    say("llama fused role step")
+    say("llama fused role step", method, prompt)
     kw = dict(vocab_size=777, hidden_size=512, intermediate_size=512, num_hidden_layers=2, num_attention_heads=8,
-              num_key_value_heads=4, chunk_size=8, local_seq_max_length=16)
-    ids = torch.randint(0, 777, (2, 45), generator=torch.Generator().manual_seed(1)).cuda()
+              num_key_value_heads=4, chunk_size=8, local_seq_max_length=16, chunk_merge_method=method)
+    ids = torch.randint(0, 777, (2, prompt), generator=torch.Generator().manual_seed(1)).cuda()
     outs, kept = [], []
     for fused in (False, True):
         model = NAtSLlamaForCausalLM.random_init(NAtSLlamaConfig(fused_role_step=fused, **kw), dtype=torch.float32, seed=3, std=0.08)
