@@ -193,8 +193,10 @@ class NAtSChunkLayerCache:
         self._note_roles(token_states_info, roles)
         if self._buf_k is None and self._pending is None:
             self._pending = (key_states, value_states)
-            if self.chunk_fill_size < self.chunk_size:
-                self._materialize_pending()  # nothing will be evicted by the coming post_update
+            if self.chunk_fill_size < self.chunk_size or x_len == 1:
+                # nothing will be evicted by the coming post_update, or (one token that is a whole chunk:
+                # chunk_size == 1) it takes the one-token form, which works in place
+                self._materialize_pending()
             return key_states, value_states
         self._materialize_pending()
         start = self.n_ctx_data
@@ -304,7 +306,7 @@ class NAtSChunkLayerCache:
                 self._allocate(rows, like, zero=False)  # the apply kernel writes all rows
                 params.n_alloc = rows
                 k_raw, v_raw = src
-                if k_raw.stride(-1) != 1 or k_raw.stride() != v_raw.stride():
+                if k_raw.stride(-1) != 1 or ops.strides_differ(k_raw, v_raw):
                     k_raw, v_raw = k_raw.contiguous(), v_raw.contiguous()
                 ops.evict_apply_first(k_raw, v_raw, self._buf_k, self._buf_v, self._buf_valid, self._buf_pos, roles,
                                       self.size_global_kv, self.size_local_kv, params, ws, result)

@@ -37,6 +37,11 @@ def _ptr(t: torch.Tensor | None):
     return None if t is None else t.data_ptr()
 
 
+def strides_differ(a: torch.Tensor, b: torch.Tensor, dims: int | None = None) -> bool:
+    """Whether two tensors of one shape are laid out differently (a dimension of size 1 may carry any stride)."""
+    return any(sa != sb for sa, sb, n in list(zip(a.stride(), b.stride(), a.shape))[:dims] if n != 1)
+
+
 def _dtype_code(t: torch.Tensor) -> int:
     if t.dtype == torch.bfloat16:
         return NATS_DTYPE_BF16
@@ -338,7 +343,7 @@ def decode_attention(q: torch.Tensor, cache_k: torch.Tensor, cache_v: torch.Tens
     Hkv = cache_k.shape[1]
     if cache_k.shape[0] != B or cache_k.shape[3] != D or tuple(valid.shape[:2]) != (B, Hkv) or Hkv == 0 or Hq % Hkv:
         raise ValueError(f"shape mismatch: q {tuple(q.shape)}, cache {tuple(cache_k.shape)}, valid {tuple(valid.shape)}")
-    if cache_k.shape != cache_v.shape or cache_k.stride() != cache_v.stride():
+    if cache_k.shape != cache_v.shape or strides_differ(cache_k, cache_v):
         raise ValueError("cache_k and cache_v must share shape and strides")
     if cache_k.shape[2] < n_rows or valid.shape[2] < n_rows:
         raise ValueError(f"n_rows={n_rows} exceeds the cache ({cache_k.shape[2]} rows) or valid ({valid.shape[2]})")
@@ -392,10 +397,10 @@ def read_result(result: torch.Tensor) -> EvictResult:
 def evict_apply_inplace(cache_k, cache_v, valid, pos, roles, size_global, size_local, params: EvictParams, ws, result):
     _require_cuda(cache_k, cache_v, valid, roles)
     lib = _lib.load()
-    if cache_k.stride() != cache_v.stride() or cache_k.dtype != cache_v.dtype:
+    if cache_k.shape != cache_v.shape or strides_differ(cache_k, cache_v) or cache_k.dtype != cache_v.dtype:
         raise ValueError("cache_k and cache_v must share dtype and strides")
     v8 = valid.view(torch.uint8) if valid.dtype == torch.bool else valid
-    if pos is not None and (pos.dtype != torch.int32 or pos.stride()[:2] != v8.stride()[:2]):
+    if pos is not None and (pos.dtype != torch.int32 or pos.shape != v8.shape or strides_differ(pos, v8, 2)):
         raise ValueError("pos must be int32 with the strides of valid")
     check(lib.nats_evict_apply_inplace(_ptr(cache_k), _ptr(cache_v), _ptr(v8), _ptr(pos), _ptr(roles), _ptr(size_global),
                                        _ptr(size_local), ctypes.byref(params), i64_array(cache_k.stride()[:3]),
@@ -407,10 +412,10 @@ def evict_apply_first(src_k, src_v, cache_k, cache_v, valid, pos, roles, size_gl
                       ws, result):
     _require_cuda(src_k, src_v, cache_k, cache_v, valid, roles)
     lib = _lib.load()
-    if src_k.stride() != src_v.stride() or cache_k.stride() != cache_v.stride():
+    if src_k.shape != src_v.shape or strides_differ(src_k, src_v) or strides_differ(cache_k, cache_v):
         raise ValueError("K and V must share strides")
     v8 = valid.view(torch.uint8) if valid.dtype == torch.bool else valid
-    if pos is not None and (pos.dtype != torch.int32 or pos.stride()[:2] != v8.stride()[:2]):
+    if pos is not None and (pos.dtype != torch.int32 or pos.shape != v8.shape or strides_differ(pos, v8, 2)):
         raise ValueError("pos must be int32 with the strides of valid")
     check(lib.nats_evict_apply_first(_ptr(src_k), _ptr(src_v), _ptr(cache_k), _ptr(cache_v), _ptr(v8), _ptr(pos),
                                      _ptr(roles), _ptr(size_global), _ptr(size_local), ctypes.byref(params),
@@ -564,12 +569,12 @@ def rope_append(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cos: torch.Te
     ts = (q, k, v, cos, sin, cache_k, cache_v)
     if any(t.dtype != q.dtype for t in ts) or any(t.stride(-1) != 1 for t in ts):
         raise ValueError("rope_append: one dtype and a contiguous last dimension everywhere")
-    if cache_v.stride() != cache_k.stride() or cache_k.shape[:2] != (B, Hkv) or cache_k.shape[3] != D:
+    if cache_v.shape != cache_k.shape or strides_differ(cache_v, cache_k) or cache_k.shape[:2] != (B, Hkv) or cache_k.shape[3] != D:
         raise ValueError("rope_append: cache_k / cache_v must be [B, H_kv, rows, D] with equal strides")
-    if sin.stride() != cos.stride():
+    if strides_differ(sin, cos):
         sin = sin.contiguous()
         cos = cos.contiguous()
-    if valid.dtype != torch.uint8 or valid.stride(-1) != 1 or (pos is not None and (pos.stride() != valid.stride()
+    if valid.dtype != torch.uint8 or valid.stride(-1) != 1 or (pos is not None and (pos.shape != valid.shape or strides_differ(pos, valid)
                                                                                    or pos.dtype != torch.int32)):
         raise ValueError("rope_append: valid must be uint8 rows (pos: int32 of the same layout)")
     q_out = torch.empty(B, Hq, x_len, D, dtype=q.dtype, device=q.device)

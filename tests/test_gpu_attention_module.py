@@ -20,7 +20,7 @@ def rope_tables(B, start, n, D, device):
     return emb.cos()[None].expand(B, -1, -1), emb.sin()[None].expand(B, -1, -1)
 
 
-@pytest.mark.parametrize("L,C,W,steps", [(100, 16, 32, 40), (64, 16, 32, 20), (5, 8, 16, 30)])
+@pytest.mark.parametrize("L,C,W,steps", [(100, 16, 32, 40), (64, 16, 32, 20), (5, 8, 16, 30), (1, 8, 16, 30)])
 def test_module_prefill_and_decode(L, C, W, steps):
     run_module([L] + [1] * steps, C, W)
 
@@ -31,7 +31,8 @@ def test_module_segments_over_a_filled_cache(lens, C, W):
     run_module(lens, C, W)
 
 
-@pytest.mark.parametrize("lens,W", [([40] + [1] * 30, 16), ([70, 45, 1, 1, 33, 1, 90], 32)])
+@pytest.mark.parametrize("lens,W", [([40] + [1] * 30, 16), ([70, 45, 1, 1, 33, 1, 90], 32),
+                                    ([1, 1, 1, 12, 1, 1, 30, 1], 16)])  # (a first segment of one token is a whole chunk)
 def test_module_with_per_token_roles(lens, W):
     """chunk_size == 1: a role per token, served by the same state machine with one-token chunks."""
     run_module(lens, 1, W)
