@@ -35,7 +35,7 @@ class LayerProbe:
         self.att = args[0].detach()
 
 
-def run(cfg, dtype, lens, tol, B=2, seed=0, std=0.05):
+def run(cfg, dtype, lens, tol, B=2, seed=0, std=0.05, need_all_roles=True):
     from neuralattentionsearch_amd.attention import apply_rotary_pos_emb
     from neuralattentionsearch_amd.llama import NAtSLlamaForCausalLM
     model = NAtSLlamaForCausalLM.random_init(cfg, dtype=dtype, seed=seed, std=std)
@@ -91,7 +91,8 @@ def run(cfg, dtype, lens, tol, B=2, seed=0, std=0.05):
             assert np.array_equal(lc.size_global_kv.cpu().numpy(), st.size_global), (step, li)
             assert np.array_equal(lc.size_local_kv.cpu().numpy(), st.size_local), (step, li)
         seen += n
-    assert (role_counts > 0).all(), role_counts  # the run exercised all three roles
+    if need_all_roles:
+        assert (role_counts > 0).all(), role_counts  # the run exercised all three roles
     return model, cache
 
 
