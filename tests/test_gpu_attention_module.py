@@ -178,3 +178,13 @@ def test_container_chunk_statistics_follow_the_oracle(method):
                 got = got.max(1, keepdim=True)[0]
             torch.testing.assert_close(got.cpu(), carry_o, rtol=1e-6, atol=1e-6)
         fill, carry = (fill + n) % C, carry_o
+
+
+def test_module_on_a_side_stream():
+    """Every kernel goes to torch's current stream: the same run under a stream of the caller's own."""
+    say("attention module on a side stream")
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run_module([40, 1, 1, 1, 20, 1, 1, 9], 8, 16)
+    side.synchronize()
