@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define NATS_ABI_VERSION 5
+#define NATS_ABI_VERSION 6
 
 typedef enum {
   NATS_OK = 0,
@@ -206,6 +206,23 @@ int nats_decode_fwd(const void* q, const void* cache_k, const void* cache_v, con
                     const int64_t* row_end, int64_t tail_start, void* o, int64_t B, int64_t H_q, int64_t H_kv, int64_t D,
                     int64_t n_rows, const int64_t* kv_strides, const int64_t* valid_strides, float sm_scale, int dtype,
                     void* workspace, size_t workspace_bytes, void* stream);
+
+/* nats_decode_fwd for callers that cannot allocate device memory or bring a workspace: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid the allocator.  It has no counterpart in the reference.
+ * Same arguments, same kernels and bit-identical results; the partial results of the split kernels live in a
+ * static device array of NATS_DECODE_STATIC_SCRATCH_BYTES that every GPU the library runs on holds until the
+ * process ends.  The call allocates and frees nothing.  A shape whose nats_decode_workspace_bytes(...) exceeds
+ * that size is rejected with NATS_ERR_WORKSPACE (take nats_decode_fwd then).  All calls on one GPU share the
+ * array: calls that overlap in time on one GPU (two streams, two threads) race on it; order them on one stream.
+ */
+#define NATS_DECODE_STATIC_SCRATCH_BYTES (8u << 20)
+
+size_t nats_decode_static_scratch_bytes(void);
+
+int nats_decode_fwd_static(const void* q, const void* cache_k, const void* cache_v, const uint8_t* valid,
+                           const int64_t* row_end, int64_t tail_start, void* o, int64_t B, int64_t H_q, int64_t H_kv,
+                           int64_t D, int64_t n_rows, const int64_t* kv_strides, const int64_t* valid_strides,
+                           float sm_scale, int dtype, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
  * KV eviction + compaction: NAtSChunkLayerCache._post_update from its ring insert to its

@@ -19,7 +19,7 @@ c_i64p = ctypes.POINTER(ctypes.c_int64)
 NATS_DTYPE_BF16 = 0
 NATS_DTYPE_F32 = 1
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 
 class EvictParams(ctypes.Structure):
@@ -63,6 +63,9 @@ SIGNATURES = {
     "nats_decode_workspace_bytes": (ctypes.c_size_t, [c_i64] * 5),
     "nats_decode_fwd": (ctypes.c_int, [c_p, c_p, c_p, c_p, c_p, c_i64, c_p, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64p,
                                        c_i64p, ctypes.c_float, ctypes.c_int, c_p, ctypes.c_size_t, c_p]),
+    "nats_decode_static_scratch_bytes": (ctypes.c_size_t, []),
+    "nats_decode_fwd_static": (ctypes.c_int, [c_p, c_p, c_p, c_p, c_p, c_i64, c_p, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64p,
+                                              c_i64p, ctypes.c_float, ctypes.c_int, c_p]),
     "nats_evict_workspace_bytes": (ctypes.c_size_t, [c_i64] * 3),
     "nats_evict_plan": (ctypes.c_int, [c_p, c_p, c_p, ctypes.POINTER(EvictParams), c_p, ctypes.c_size_t, c_p, c_p]),
     "nats_evict_apply_inplace": (ctypes.c_int, [c_p, c_p, c_p, c_p, c_p, c_p, c_p, ctypes.POINTER(EvictParams), c_i64p,

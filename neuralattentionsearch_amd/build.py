@@ -17,6 +17,20 @@ HIPCC_FLAGS = [
 ]
 
 
+# The packed-fp32 switch is a feature of the gfx950 target; hipcc hands -Xclang options to its x86 host pass as well,
+# which answers with this line (three times per file) and ignores the option there.  Only that exact line is dropped.
+_HOST_PASS_NOTE = "'-packed-fp32-ops' is not a recognized feature for this target (ignoring feature)"
+
+
+def _run_hipcc(cmd):
+    proc = subprocess.run(cmd, stderr=subprocess.PIPE, text=True)
+    rest = [ln for ln in proc.stderr.splitlines() if ln.strip() != _HOST_PASS_NOTE]
+    if rest:
+        print("\n".join(rest), file=sys.stderr, flush=True)
+    if proc.returncode:
+        raise subprocess.CalledProcessError(proc.returncode, cmd)
+
+
 def build(verbose: bool = True) -> str:
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     objs = []
@@ -25,7 +39,7 @@ def build(verbose: bool = True) -> str:
         cmd = [hipcc, *HIPCC_FLAGS, "-I", INCLUDE, "-I", CSRC, "-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
-        subprocess.run(cmd, check=True)
+        _run_hipcc(cmd)
         objs.append(obj)
     cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", "-Wl,-z,defs", *objs, "-o", LIB_PATH]
     if verbose:

@@ -13,6 +13,8 @@
 
 #include "nats_common.h"
 
+#include <mutex>
+
 namespace nats {
 
 struct DecodeArgs {
@@ -551,15 +553,14 @@ static void decode_split_geometry(int64_t B, int64_t H_kv, int64_t n_rows, int* 
 
 // workgroups of the balanced bf16 schedule: two per compute unit, fewer when there is little to do
 static int decode_balanced_workgroups(int64_t B, int64_t H_kv, int64_t n_rows) {
-  static int n_cu = 0;
-  if (n_cu == 0) {
-    int dev = 0, v = 0;
-    if (hipGetDevice(&dev) == hipSuccess &&
-        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) {
-      n_cu = v;
-    } else {
-      n_cu = 256;
+  static int n_cu_of[64] = {};  // compute units of every device, asked for once each
+  int dev = 0, n_cu = 256;
+  if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64) {
+    if (n_cu_of[dev] == 0) {
+      int v = 0;
+      n_cu_of[dev] = (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) ? v : 256;
     }
+    n_cu = n_cu_of[dev];
   }
   int64_t upper = B * H_kv * ((n_rows + kDecTile - 1) / kDecTile + 1);  // tiles, at most
   int64_t want = (upper + 7) / 8;                                        // at least 8 tiles per workgroup
@@ -600,10 +601,13 @@ extern "C" size_t nats_decode_workspace_bytes(int64_t B, int64_t H_q, int64_t H_
   return split_layout > balanced_layout ? split_layout : balanced_layout;
 }
 
-extern "C" int nats_decode_fwd(const void* q, const void* cache_k, const void* cache_v, const uint8_t* valid,
-                               const int64_t* row_end, int64_t tail_start, void* o, int64_t B, int64_t H_q, int64_t H_kv,
-                               int64_t D, int64_t n_rows, const int64_t* kv_strides, const int64_t* valid_strides,
-                               float sm_scale, int dtype, void* workspace, size_t workspace_bytes, void* stream) {
+// `workspace` is caller memory (nats_decode_fwd) or the library's static scratch array (nats_decode_fwd_static);
+// `max_bytes` != 0 names the fixed size of the latter, for the error text.
+static int decode_fwd_impl(const void* q, const void* cache_k, const void* cache_v, const uint8_t* valid,
+                           const int64_t* row_end, int64_t tail_start, void* o, int64_t B, int64_t H_q, int64_t H_kv,
+                           int64_t D, int64_t n_rows, const int64_t* kv_strides, const int64_t* valid_strides,
+                           float sm_scale, int dtype, void* workspace, size_t workspace_bytes, size_t max_bytes,
+                           void* stream) {
   NATS_REQUIRE(q && cache_k && cache_v && valid && o && workspace, NATS_ERR_NULL_POINTER,
                "nats_decode_fwd: NULL pointer argument");
   NATS_REQUIRE(kv_strides && valid_strides, NATS_ERR_NULL_POINTER, "nats_decode_fwd: NULL stride array");
@@ -621,6 +625,10 @@ extern "C" int nats_decode_fwd(const void* q, const void* cache_k, const void* c
   NATS_REQUIRE(row_end == nullptr || (tail_start >= 0 && tail_start <= n_rows), NATS_ERR_BAD_SHAPE,
                "nats_decode_fwd: tail_start=%lld outside [0, n_rows=%lld]", (long long)tail_start, (long long)n_rows);
   size_t need = nats_decode_workspace_bytes(B, H_q, H_kv, D, n_rows);
+  NATS_REQUIRE(max_bytes == 0 || need <= max_bytes, NATS_ERR_WORKSPACE,
+               "nats_decode_fwd_static: this shape needs %zu bytes of scratch, the static array holds %zu; use "
+               "nats_decode_fwd with a caller workspace",
+               need, max_bytes);
   NATS_REQUIRE(workspace_bytes >= need, NATS_ERR_WORKSPACE, "nats_decode_fwd: workspace %zu bytes < %zu", workspace_bytes,
                need);
   if (dtype == NATS_DTYPE_BF16) {
@@ -710,4 +718,54 @@ extern "C" int nats_decode_fwd(const void* q, const void* cache_k, const void* c
     NATS_CHECK_LAUNCH("decode_merge_balanced_kernel");
   }
   return NATS_OK;
+}
+
+extern "C" int nats_decode_fwd(const void* q, const void* cache_k, const void* cache_v, const uint8_t* valid,
+                               const int64_t* row_end, int64_t tail_start, void* o, int64_t B, int64_t H_q, int64_t H_kv,
+                               int64_t D, int64_t n_rows, const int64_t* kv_strides, const int64_t* valid_strides,
+                               float sm_scale, int dtype, void* workspace, size_t workspace_bytes, void* stream) {
+  return decode_fwd_impl(q, cache_k, cache_v, valid, row_end, tail_start, o, B, H_q, H_kv, D, n_rows, kv_strides,
+                         valid_strides, sm_scale, dtype, workspace, workspace_bytes, 0, stream);
+}
+
+// ---------------------------------------------------------------------------------------------------
+// The same op for callers that cannot allocate: the partial results live in a static device array.
+// ---------------------------------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[NATS_DECODE_STATIC_SCRATCH_BYTES];
+
+// Every device holds its own copy of `scratch` at its own address; in host code the array's name is only a
+// handle for hipGetSymbolAddress, never a device address.  Looked up once per device, with that device current.
+static int static_scratch_of_current_device(void** out) {
+  static std::mutex mu;
+  static void* ptr_of[64] = {};
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= 64)
+    return fail(NATS_ERR_LAUNCH, "nats_decode_fwd_static: no current device (%s)", hipGetErrorString(e));
+  std::lock_guard<std::mutex> lock(mu);
+  if (ptr_of[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr)
+      return fail(NATS_ERR_LAUNCH, "nats_decode_fwd_static: hipGetSymbolAddress(scratch) on device %d: %s", dev,
+                  hipGetErrorString(e));
+    ptr_of[dev] = p;
+  }
+  *out = ptr_of[dev];
+  return NATS_OK;
+}
+
+extern "C" size_t nats_decode_static_scratch_bytes(void) { return NATS_DECODE_STATIC_SCRATCH_BYTES; }
+
+extern "C" int nats_decode_fwd_static(const void* q, const void* cache_k, const void* cache_v, const uint8_t* valid,
+                                      const int64_t* row_end, int64_t tail_start, void* o, int64_t B, int64_t H_q,
+                                      int64_t H_kv, int64_t D, int64_t n_rows, const int64_t* kv_strides,
+                                      const int64_t* valid_strides, float sm_scale, int dtype, void* stream) {
+  void* ws = nullptr;
+  if (int rc = static_scratch_of_current_device(&ws)) return rc;
+  // Nothing in the scratch has to start at zero: the split kernels write every partial sum, maximum, row sum and
+  // head-table entry that the merge kernels of the same call read.
+  return decode_fwd_impl(q, cache_k, cache_v, valid, row_end, tail_start, o, B, H_q, H_kv, D, n_rows, kv_strides,
+                         valid_strides, sm_scale, dtype, ws, NATS_DECODE_STATIC_SCRATCH_BYTES,
+                         NATS_DECODE_STATIC_SCRATCH_BYTES, stream);
 }
