@@ -19,7 +19,7 @@ How each function is pinned (see tests/test_oracle_*.py):
 * masked_attention ............. torch SDPA with a bool mask is the library routine itself
 * ChunkCacheOracle.update / generate_mask / post_update
                                  golden vectors written by the reference's NAtSChunkLayerCache on CPU
-                                 (tests/golden/make_golden.py), 21 scenarios / 228 calls, compared on
+                                 (tests/golden/make_golden.py), 24 scenarios / 270 calls (chunk sizes 1 to 4), compared on
                                  every byte of cache_k, cache_v, valid_tokens, sizes and scalars
 * decode_attention ............. equals masked_attention restricted to the valid rows (gather, then dense
                                  softmax); checked against torch SDPA
@@ -27,12 +27,17 @@ How each function is pinned (see tests/test_oracle_*.py):
                                  open chunk, and the invariant that any split of a stream into calls gives
                                  the statistics of one call (dyn_cache.py:98-171, chunk_utils.py:13-62)
 
-Functions with parity unpinned: none of the above.  The reference's per-token cache class (chunk_size == 1,
-components/cache/nats_layer_cache.py: 16-token deferred eviction, its own row order) is not restated here; per-token
-roles are covered as ChunkCacheOracle with C = 1, which gives the visibility and the surviving tokens of the
-per-token rules but not that class's cache layout, nor the extra tokens it leaves visible between two deferred
-evictions (parity unpinned for both: the class cannot be imported in the reference's own checkout, so no vectors of
-it exist).
+* TokenCacheOracle.update / generate_mask / post_update (the per-token class, chunk_size == 1)
+                                 golden vectors written by the reference's NAtSLayerCache on CPU
+                                 (tests/golden/make_golden_token.py), 25 scenarios / 893 calls: every mask and,
+                                 after every post_update, every byte of cache_k, cache_v, valid_tokens, the sizes
+                                 and the scalars (deferred 16-token eviction, ring insert, all-sliding and
+                                 all-local blocks, multi-token segments over pending tokens, first segments
+                                 shorter than the window and than the update chunk, update chunks of 4 and 8)
+
+Functions with parity unpinned: none of the above.  Not restated: the branch of the per-token class for
+update_chunk_size == 1 (cache/nats_layer_cache.py:328-367), which the container never constructs
+(dyn_cache.py:183-185 leaves the default of 16); TokenCacheOracle refuses U == 1.
 """
 from __future__ import annotations
 
@@ -525,6 +530,235 @@ class ChunkCacheOracle:
         """Stream positions of the rows a decode step would attend to, in cache order."""
         n = self.n_ctx_data
         return self.pos_k[b, h, :n][self.valid[b, h, :n]]
+
+
+# ----------------------------------------------------------------------------------------------
+# the per-token layer cache (chunk_size == 1) as an explicit state machine
+# ----------------------------------------------------------------------------------------------
+@dataclass
+class TokenCacheOracle:
+    """State of one layer of the reference's per-token cache, NAtSLayerCache
+    (cache/nats_layer_cache.py:20-80): a role per token, rows appended at once, eviction deferred until
+    `U` (update_chunk_size, 16 as the container builds it) tokens are pending.
+
+    Row layout of cache_k[b, h] between calls:
+        [0, W)                      ring of the last W tokens that went through an eviction; `tail` is the slot
+                                    written last; a slot is valid iff its token was sliding-window (its row is
+                                    copied whatever the role)
+        [W, size_global)            global tokens, stream order
+        [size_global, +size_local)  local tokens newer than the last global token
+        [.., P)                     stale rows of shorter heads (and the still-valid rows of pending blocks whose
+                                    tokens were all sliding-window, which the reference leaves where they were)
+        [P, P + fill)               the pending block, valid, P + fill = n_ctx_data
+    Rows at and beyond n_ctx_data keep whatever they held (nothing is zeroed).
+    `pos_k` shadows cache_k with the stream position of the token each row holds (-1 = none)."""
+    B: int
+    H: int
+    W: int
+    U: int = 16
+    size_global: np.ndarray = field(init=False)
+    size_local: np.ndarray = field(init=False)
+    n_ctx_data: int = field(init=False)
+    gmin: int = field(init=False)
+    tail: int = 0
+    fill: int = 0
+    fill_last: int = 0
+    seen: int = 0
+    cache_k: torch.Tensor | None = None
+    cache_v: torch.Tensor | None = None
+    pos_k: np.ndarray | None = None
+    valid: np.ndarray | None = None
+    block: np.ndarray | None = None       # roles of the pending block, [B, H, fill] (:209-219, _tokens_info)
+    mask_roles: np.ndarray | None = None  # the block as of the last multi-token update (:229-231)
+
+    def __post_init__(self):
+        if self.W < self.U:  # :77-78
+            raise NotImplementedError("The sliding window size must be greater or equal to the update chunk size!")
+        if self.U == 1:
+            raise NotImplementedError("the one-step branch of update_chunk_size == 1 (:328-367) is not restated")
+        self.size_global = np.full((self.B, self.H), self.W, dtype=np.int64)
+        self.size_local = np.zeros((self.B, self.H), dtype=np.int64)
+        self.n_ctx_data = self.W
+        self.gmin = self.W
+        self._in_chunk = np.zeros((self.B, self.H, self.U), dtype=np.uint8)
+
+    # -- append (:167-286) ------------------------------------------------------------------------
+    def update(self, k: torch.Tensor, v: torch.Tensor, roles: np.ndarray):
+        """roles uint8 [B, H, x_len], one per new token.  Returns the K, V the attention of this call runs over."""
+        B, H, x_len, D = k.shape
+        if x_len == 0:  # :204-205
+            return self.cache_k[:, :, :self.n_ctx_data], self.cache_v[:, :, :self.n_ctx_data]
+        roles = np.asarray(roles, dtype=np.uint8)
+        assert roles.shape == (B, H, x_len)
+        self.fill += x_len
+        if self.fill > self.U:  # :209-215
+            self.block = np.concatenate([self._in_chunk[:, :, :self.fill_last], roles], axis=2)
+        else:  # :217-219
+            self._in_chunk[:, :, self.fill_last:self.fill] = roles
+            self.block = self._in_chunk[:, :, :self.fill].copy()
+        if x_len > 1:  # :229-231
+            self.mask_roles = self.block.copy()
+        if self.cache_k is None:  # :236-259
+            pad = (-x_len) % self.U
+            rows = self.W + x_len + pad
+            self.cache_k = torch.zeros(B, H, rows, D, dtype=k.dtype)
+            self.cache_v = torch.zeros(B, H, rows, D, dtype=v.dtype)
+            self.cache_k[:, :, self.W:self.W + x_len] = k
+            self.cache_v[:, :, self.W:self.W + x_len] = v
+            self.valid = np.zeros((B, H, rows), dtype=bool)
+            self.valid[:, :, self.W:self.W + x_len] = True
+            self.pos_k = np.full((B, H, rows), -1, dtype=np.int64)
+            self.pos_k[:, :, self.W:self.W + x_len] = np.arange(self.seen, self.seen + x_len)
+            return k, v
+        start = self.n_ctx_data  # :265-286
+        end = start + x_len
+        need = math.ceil(end / self.U) * self.U
+        have = self.cache_k.shape[2]
+        if need > have:
+            grow = need - have
+            self.cache_k = torch.cat([self.cache_k, torch.zeros(B, H, grow, D, dtype=self.cache_k.dtype)], 2)
+            self.cache_v = torch.cat([self.cache_v, torch.zeros(B, H, grow, D, dtype=self.cache_v.dtype)], 2)
+            self.valid = np.concatenate([self.valid, np.zeros((B, H, grow), dtype=bool)], 2)
+            self.pos_k = np.concatenate([self.pos_k, np.full((B, H, grow), -1, dtype=np.int64)], 2)
+        self.cache_k[:, :, start:end] = k.to(self.cache_k.dtype)
+        self.cache_v[:, :, start:end] = v.to(self.cache_v.dtype)
+        self.valid[:, :, start:end] = True
+        self.pos_k[:, :, start:end] = np.arange(self.seen, self.seen + x_len)
+        return self.cache_k[:, :, :end], self.cache_v[:, :, :end]
+
+    # -- masks ------------------------------------------------------------------------------------
+    def _block_mask(self, start: int):
+        """:519-542.  Rows = block tokens [start, fill), columns = block tokens [0, fill)."""
+        roles = self.mask_roles
+        fill = roles.shape[-1]
+        g = next_global_index(roles == ROLE_GLOBAL)
+        any_sw = bool((roles == ROLE_SW).any())
+        m = np.arange(start, fill)[:, None]
+        n = np.arange(fill)[None, :]
+        out = np.zeros((self.B, self.H, fill - start, fill), dtype=bool)
+        for b in range(self.B):
+            for h in range(self.H):
+                r = roles[b, h]
+                is_g = (r == ROLE_GLOBAL) | (np.arange(fill) == fill - 1)
+                vis = (g[b, h][None, :] >= m) | is_g[None, :]  # masks/utils.py:92
+                if any_sw:
+                    vis = np.where((r == ROLE_SW)[None, :], (m - n) <= self.W, vis)  # :527-536
+                out[b, h] = vis & (n <= m)  # :538
+        return out, g
+
+    def generate_mask(self, x_len: int) -> np.ndarray:
+        """:155-162, :469-517.  Bool [B, H, x_len, n_ctx_data + x_len] (or [.., x_len, x_len] from empty)."""
+        if x_len == 1:
+            if self.seen == 0:  # :550-551
+                return np.ones((1, 1, 1, 1), dtype=bool)
+            return self.valid[:, :, None, :self.n_ctx_data + 1].copy()  # :553
+        start = self.fill - x_len  # :159
+        new_mask, g = self._block_mask(start)
+        if self.seen == 0 or self.valid.shape[-1] == 0:  # :484-488
+            return new_mask
+        W = self.W
+        P = self.n_ctx_data - self.fill_last  # :490, first row of the pending block
+        cached = np.repeat(self.valid[:, :, None, :P], x_len, axis=2).copy()
+        i = np.arange(x_len)[:, None]  # the query's index within this call, not within the block
+        if self.seen < W:  # :612-619: the columns of the tokens seen so far are overwritten, valid or not
+            j = np.arange(self.seen)[None, :]
+            cached[:, :, :, :self.seen] = ((i + j) < W)[None, None]
+        else:  # :621-647: slot tail + 1 is the oldest and is seen by the first query only
+            age = (np.arange(W) + W - 1 - self.tail) % W
+            ok = (age[None, :] >= i) & (i < W)
+            cached[:, :, :, :W] &= ok[None, None]
+        gmin = self.gmin  # :502-516: cached local tokens live until the first global token of the block
+        for b in range(self.B):
+            for h in range(self.H):
+                lo = self.size_global[b, h] - gmin
+                hi = self.size_global[b, h] + self.size_local[b, h] - gmin
+                col_local = (np.arange(x_len) <= g[b, h, 0])
+                for c in range(gmin, P):
+                    t = c - gmin
+                    if t >= hi:
+                        cached[b, h, :, c] = False
+                    elif t >= lo:
+                        cached[b, h, :, c] = col_local
+                    else:
+                        cached[b, h, :, c] = True
+        return np.concatenate([cached, new_mask], axis=-1)
+
+    # -- evict + compact (:292-418) ---------------------------------------------------------------
+    def _ring_insert(self):
+        """:424-458.  The last min(fill, W) tokens of the pending block enter the ring, rows copied whatever the
+        role, valid only if sliding-window."""
+        W, n = self.W, self.n_ctx_data
+        x_sw = min(self.fill, W)
+        if self.fill == self.seen:
+            slots = np.arange(x_sw)
+            self.tail = x_sw - 1
+        else:
+            slots = (np.arange(x_sw) + self.tail + 1) % W
+            self.tail = (self.tail + x_sw) % W
+        self.valid[:, :, slots] = self.block[:, :, -x_sw:] == ROLE_SW
+        self.cache_k[:, :, slots] = self.cache_k[:, :, n - x_sw:n].clone()
+        self.cache_v[:, :, slots] = self.cache_v[:, :, n - x_sw:n].clone()
+        self.pos_k[:, :, slots] = self.pos_k[:, :, n - x_sw:n].copy()
+
+    def post_update(self, x_len: int):
+        B, H, W, U = self.B, self.H, self.W, self.U
+        self.seen += x_len
+        if x_len == 0:
+            return
+        self.n_ctx_data += x_len
+        if self.fill < U:  # :300-310: the eviction is deferred, one ring slot is switched off
+            slot = self.fill if self.seen < U else (self.fill + self.tail + 1) % W
+            self.valid[:, :, slot] = False
+            self.fill_last = self.fill
+            return
+        block = self.block
+        fill = self.fill
+        assert block.shape[-1] == fill
+        if (block == ROLE_SW).all():  # :316-327: rows and n_ctx_data stay as they are
+            self._ring_insert()
+            self.fill = self.fill_last = 0
+            return
+        self._ring_insert()
+        if not (block == ROLE_LOCAL).all():  # :651-770 + cache_update.py:25-76 (chunk_size 1)
+            P = self.n_ctx_data - fill  # :759
+            moves = []
+            new_sizes = {}
+            for b in range(B):
+                for h in range(H):
+                    r = block[b, h]
+                    sg, sl = int(self.size_global[b, h]), int(self.size_local[b, h])
+                    glob = [s for s in range(fill) if r[s] == ROLE_GLOBAL]
+                    last_g = glob[-1] if glob else -1
+                    later_local = [s for s in range(fill) if s > last_g and r[s] == ROLE_LOCAL]
+                    dec_local = (last_g + sl if last_g > -1 else 0) + (fill - max(last_g, 0) - len(later_local))  # :723-729
+                    keep = sorted(glob + later_local)
+                    base = sg + sl if last_g == -1 else sg  # :748-749
+                    for rank, s in enumerate(keep):
+                        moves.append((b, h, P + s, base + rank))
+                    new_sizes[(b, h)] = (sg + len(glob), sl - dec_local)
+            stash = [(self.cache_k[b, h, s].clone(), self.cache_v[b, h, s].clone(), self.pos_k[b, h, s])
+                     for (b, h, s, _) in moves]
+            for (b, h, _, d), (kk, vv, pp) in zip(moves, stash):
+                self.cache_k[b, h, d] = kk
+                self.cache_v[b, h, d] = vv
+                self.pos_k[b, h, d] = pp
+            for (b, h), (sg, sl) in new_sizes.items():
+                self.size_global[b, h] = sg
+                self.size_local[b, h] = sl
+        self.size_local += fill  # :393
+        assert not (self.size_local < 0).any()
+        self.n_ctx_data = int((self.size_global + self.size_local).max())  # :394
+        old_gmin = self.gmin  # :565 uses the minimum from before this call
+        if self.n_ctx_data != old_gmin:
+            idx = np.arange(old_gmin, self.n_ctx_data)
+            end = (self.size_global + self.size_local)[:, :, None]
+            self.valid[:, :, old_gmin:self.n_ctx_data] = idx[None, None, :] < end
+        self.gmin = int(self.size_global.min())
+        if self.seen == x_len:  # :404-408
+            n = self.n_ctx_data
+            self.cache_k, self.cache_v = self.cache_k[:, :, :n], self.cache_v[:, :, :n]
+            self.valid, self.pos_k = self.valid[:, :, :n], self.pos_k[:, :, :n]
+        self.fill = self.fill_last = 0
 
 
 def kept_token_fraction(cache: ChunkCacheOracle) -> float:

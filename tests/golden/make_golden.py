@@ -93,6 +93,12 @@ def scenarios():
                     segs=[(30, "rand"), (11, "rand"), (7, "rand"), (1, "rand"), (1, "rand"), (13, "rand")]))
     out.append(dict(name="multiseg_first_lt_w_c2_w8", B=1, H=2, D=2, C=2, W=8, p=mix,
                     segs=[(4, "rand"), (6, "rand"), (12, "rand")]))
+    # one-token chunks through the chunk class (the container never builds this, the class accepts it)
+    out.append(dict(name="chunk1_prefill_decode_w4", B=2, H=2, D=2, C=1, W=4, p=mix, segs=[(19, "rand")] + [(1, "rand")] * 20))
+    out.append(dict(name="chunk1_multiseg_w8", B=1, H=3, D=2, C=1, W=8, p=mix,
+                    segs=[(24, "rand"), (9, "rand"), (1, "rand"), (1, "rand"), (13, "rand"), (3, "rand")]))
+    out.append(dict(name="chunk1_first_lt_w", B=1, H=2, D=2, C=1, W=8, p=(0.15, 0.25, 0.6),
+                    segs=[(3, "rand"), (4, "rand")] + [(1, "rand")] * 12 + [(10, "rand")]))
     return out
 
 
