@@ -158,6 +158,9 @@ typedef struct {
   int64_t tail;       /* sliding_queue_tail */
   int64_t seen;       /* _seen_tokens (not yet counting the segment) */
   int64_t fill_last;  /* chunk_fill_size_last */
+  int64_t update_chunk; /* 0: the chunked cache (NAtSChunkLayerCache).  U > 0: the per-token cache (NAtSLayerCache,
+                           components/cache/nats_layer_cache.py:469-517, 603-649) with update chunk size U; C must be 1,
+                           old_fill < U counts the pending tokens and `tail` is the ring slot written last */
 } nats_past_state;
 
 /*   q [B, H_q, x_len, D], o like q; cache_k / cache_v [B, H_kv, >= n_ctx_data + x_len, D]
@@ -243,6 +246,13 @@ typedef struct {
   int64_t tail;        /* sliding_queue_tail before this call */
   int64_t first;       /* 1 if these are the first tokens the layer has seen (_seen_tokens == x_len) */
   int64_t n_alloc;     /* rows allocated in cache_k / cache_v / valid (in place) or in the new cache (out of place) */
+  int64_t update_chunk; /* 0: the chunked cache.  U > 0: the per-token cache NAtSLayerCache._post_update
+                           (components/cache/nats_layer_cache.py:292-418, 424-458, 556-574, 651-770) once U tokens
+                           are pending: C = 1, S = fill = the pending block with one role per token, n_ctx_data = the
+                           first row of that block, tail = the ring slot written last, first = 1 if the block holds
+                           every token seen so far.  Ring rows are copied whatever the role (valid only if
+                           sliding-window), rows at and beyond the new n_ctx_data keep their contents, and a block of
+                           sliding-window tokens only leaves n_ctx_data where it is. */
 } nats_evict_params;
 
 typedef struct {

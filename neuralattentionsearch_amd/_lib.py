@@ -25,7 +25,8 @@ ABI_VERSION = 6
 class EvictParams(ctypes.Structure):
     """nats_evict_params"""
     _fields_ = [(n, c_i64) for n in
-                ("B", "H_kv", "D", "C", "W", "S", "x_len", "fill", "n_ctx_data", "gmin", "tail", "first", "n_alloc")]
+                ("B", "H_kv", "D", "C", "W", "S", "x_len", "fill", "n_ctx_data", "gmin", "tail", "first", "n_alloc",
+                 "update_chunk")]
 
 
 class EvictResult(ctypes.Structure):
@@ -36,7 +37,7 @@ class EvictResult(ctypes.Structure):
 
 class PastState(ctypes.Structure):
     """nats_past_state"""
-    _fields_ = [(n, c_i64) for n in ("n_ctx_data", "old_fill", "gmin", "tail", "seen", "fill_last")]
+    _fields_ = [(n, c_i64) for n in ("n_ctx_data", "old_fill", "gmin", "tail", "seen", "fill_last", "update_chunk")]
 
 
 # every symbol include/nats_hip.h declares: name -> (restype, argtypes)

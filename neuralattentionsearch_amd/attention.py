@@ -104,6 +104,7 @@ class BaseNAtSAttentionLayer(AttentionLayer):
         one_hot_values[0] = 1.0
         self.one_hot_values = one_hot_values
         self.executor = None
+        self._cache_is_till_updating = None
 
     def prepare_x_values(self, x, bsz: int, seqlen: int, pos_emb, start_pos: int = 0, cache: NAtSCache | None = None):
         xq, xk, xv = self.wq(x), self.wk(x), self.wv(x)
@@ -128,7 +129,46 @@ class BaseNAtSAttentionLayer(AttentionLayer):
         return one_hot
 
     def prepare_kv(self, xq, xk, xv, start_pos: int = 0, cache: NAtSCache | None = None, kwargs: dict | None = None):
+        if self._cache_is_till_updating is not None:  # nats_attention.py:122-123
+            self._cache_is_till_updating.result()
+            self._cache_is_till_updating = None
         return cache.update(key_states=xk, value_states=xv, layer_idx=self.layer_id, cache_kwargs=kwargs)
+
+    def _post_update(self, cache: NAtSCache, x_len: int):
+        """Eviction after the attention (nats_attention.py:189-195).  With an executor the job is handed to its
+        thread together with the caller's stream: torch's current stream is a per-thread setting, and the eviction
+        kernels must follow the attention kernel on the stream that ran it."""
+        if self.executor is None:
+            cache.post_update(layer_idx=self.layer_id, x_len=x_len)
+            return
+        stream = torch.cuda.current_stream()
+
+        def job():
+            with torch.cuda.stream(stream):
+                cache.post_update(layer_idx=self.layer_id, x_len=x_len)
+
+        self._cache_is_till_updating = self.executor.submit(job)
+
+    def multi_head_attention(self, xq, keys, values, mask=None, cache: NAtSCache | None = None,
+                             is_first_module: bool = True, kwargs: dict | None = None):
+        """Inference branch of nats_attention.py:136-195 / nats_chunk_attention.py:97-157 on the kernels: the mask
+        the reference takes from cache.generate_mask is evaluated inside them, from the cache's own window."""
+        assert "token_states_info" in kwargs, "Token States Infor is required for multi head attention!"
+        x_len = xq.shape[-2]
+        layer = cache.cache_model[self.layer_id]
+        if x_len == 1 and layer.get_seq_length() > 0:
+            row_end, tail_start = layer.decode_hint()
+            output = ops.decode_attention(xq, keys, values, layer.valid_tokens, keys.shape[2], self.sm_scale,
+                                          row_end=row_end, tail_start=tail_start)
+        elif layer.get_seq_length() == 0:
+            roles = ops.roles_from_one_hot(kwargs["token_states_info"])
+            output = ops.prefill_attention(xq, keys, values, roles, layer.chunk_size, layer.sliding_window_size,
+                                           self.sm_scale)
+        else:
+            output = layer.segment_attention(xq, self.sm_scale)
+        self._post_update(cache, x_len)
+        return output
+
 
 
 class BaseNAtSChunkAttentionLayer(BaseNAtSAttentionLayer):
@@ -165,27 +205,14 @@ class BaseNAtSChunkAttentionLayer(BaseNAtSAttentionLayer):
         return super()._sample_for_token_info_values_inference(x_pooled, start_pos, sink_token_end=self.chunk_size,
                                                                force_last_global=pad_size != 0)
 
-    def multi_head_attention(self, xq, keys, values, mask=None, cache: NAtSCache | None = None,
-                             is_first_module: bool = True, kwargs: dict | None = None):
-        assert "token_states_info" in kwargs, "Token States Infor is required for multi head attention!"
-        x_len = xq.shape[-2]
-        layer = cache.cache_model[self.layer_id]
-        if x_len == 1 and layer.get_seq_length() > 0:
-            output = ops.decode_attention(xq, keys, values, layer.valid_tokens, keys.shape[2], self.sm_scale,
-                                          row_end=layer.row_end(),
-                                          tail_start=layer.n_ctx_data - (layer.chunk_fill_size - 1))
-        elif layer.get_seq_length() == 0:
-            roles = ops.roles_from_one_hot(kwargs["token_states_info"])
-            output = ops.prefill_attention(xq, keys, values, roles, self.chunk_size, self.local_seq_max_length,
-                                           self.sm_scale)
-        else:
-            output = layer.segment_attention(xq, self.sm_scale)
-        if self.executor is not None:
-            self._cache_is_till_updating = self.executor.submit(cache.post_update, layer_idx=self.layer_id, x_len=x_len)
-            self._cache_is_till_updating.result()
-        else:
-            cache.post_update(layer_idx=self.layer_id, x_len=x_len)
-        return output
+
+
+class GPTNAtSAttentionLayer(BaseNAtSAttentionLayer):
+    """Per-token roles (chunk_size == 1), nats_attention.py:198-199."""
+
+
+class LlamaNAtSAttentionLayer(BaseNAtSAttentionLayer):
+    """Per-token roles (chunk_size == 1), nats_attention.py:202-203."""
 
 
 class GPTNAtSChunkAttentionLayer(BaseNAtSChunkAttentionLayer):

@@ -273,6 +273,11 @@ class NAtSChunkLayerCache:
             self._row_end = self.size_global_kv + self.size_local_kv
         return self._row_end
 
+    def decode_hint(self):
+        """(row_end, tail_start) for `ops.decode_attention` after the update of a one-token step: rows
+        [row_end[b, h], tail_start) hold nothing valid; the open chunk starts at tail_start."""
+        return self.row_end(), self.n_ctx_data - (self.chunk_fill_size - 1)
+
     # -- evict + compact (nats_chunk_layer_cache.py:258-389) -------------------------------------
     def post_update(self, x_len: int):
         C, W = self.chunk_size, self.sliding_window_size
@@ -330,16 +335,223 @@ class NAtSChunkLayerCache:
             self._rows = math.ceil(self.n_ctx_data / C) * C
 
 
+class NAtSLayerCache(NAtSChunkLayerCache):
+    """One layer's cache with a role per token (chunk_size == 1), the reference's NAtSLayerCache
+    (src/nats/components/cache/nats_layer_cache.py:20-808): rows are appended at once, the eviction is deferred
+    until `update_chunk_size` tokens are pending and then handles the whole pending block.  Row layout of
+    cache_k[b, h] between forward calls:
+
+        [0, W)                        ring of the last W evicted-or-kept tokens, `sliding_queue_tail` = the slot
+                                      written last; rows are copied whatever the role, valid only if sliding window
+        [W, size_global)              global tokens, stream order
+        [size_global, +size_local)    local tokens newer than the last global token
+        [.., P)                       stale rows of shorter heads (and the rows of earlier all-sliding-window blocks)
+        [P, n_ctx_data)               the pending block
+
+    Storage (capacity buffer, deferred first prefill) and the kernels are those of the chunked class with one-token
+    chunks; the state machine is this class's own."""
+
+    def __init__(self, bsz: int, n_msks: int, sliding_window_size: int, layer_id: int = 0, update_chunk_size: int = 16,
+                 device: torch.device | str = "cuda", track_positions: bool = False):
+        if sliding_window_size < update_chunk_size:  # nats_layer_cache.py:77-78
+            raise NotImplementedError("The sliding window size must be greater or equal to the update chunk size!")
+        if update_chunk_size < 2:
+            raise NotImplementedError("update_chunk_size == 1 (the one-step branch, nats_layer_cache.py:328-367) is not "
+                                      "built; the container always uses 16")
+        self.update_chunk_size = update_chunk_size
+        super().__init__(bsz, n_msks, sliding_window_size, layer_id=layer_id, chunk_size=1, device=device,
+                         track_positions=track_positions)
+
+    def reset_cache(self):
+        super().reset_cache()
+        self._in_chunk = None   # uint8 [B, H, U]: roles of the pending tokens (:196-200, :218)
+        self._block = None      # roles of the whole pending block as of the last update (_tokens_info, :209-219)
+        self._mask_roles = None  # the block as of the last multi-token update (:229-231)
+        self._live_end = self.sliding_window_size  # n_ctx_data after the last eviction that moved rows
+
+    # -- append (nats_layer_cache.py:167-286) ------------------------------------------------------
+    def _pad_rows(self, n: int) -> int:
+        U = self.update_chunk_size
+        return math.ceil(n / U) * U
+
+    def _materialize_pending(self):
+        """[W zeros | K | pad to the update chunk] (:236-258) if the first prefill is still raw."""
+        if self._pending is None:
+            return
+        k, v = self._pending
+        self._pending = None
+        W, x_len = self.sliding_window_size, k.shape[2]
+        self._allocate(W + self._pad_rows(x_len), k)
+        self._buf_k[:, :, W:W + x_len] = k
+        self._buf_v[:, :, W:W + x_len] = v
+        self._buf_valid[:, :, W:W + x_len] = 1
+        if self._buf_pos is not None:
+            self._buf_pos[:, :, W:W + x_len] = torch.arange(x_len, dtype=torch.int32, device=k.device)
+
+    def _grow(self, rows: int):
+        super()._grow(self._pad_rows(rows))
+
+    def _note_roles(self, token_states_info, roles):
+        """Roles of the new tokens join the pending block."""
+        U = self.update_chunk_size
+        if roles is None:
+            roles = ops.roles_from_one_hot(token_states_info)
+        x_len = roles.shape[-1]
+        self._tokens_info = token_states_info
+        if self._in_chunk is None:
+            self._in_chunk = torch.zeros(self.bsz, self.n_msks, U, dtype=torch.uint8, device=self.device)
+        fill, last = self.chunk_fill_size, self.chunk_fill_size_last
+        if fill > U:
+            self._block = torch.cat([self._in_chunk[:, :, :last], roles], dim=2).contiguous()
+        else:
+            self._in_chunk[:, :, last:fill] = roles
+            self._block = self._in_chunk[:, :, :fill].contiguous()
+        self._roles = self._block
+        if x_len > 1:
+            self._mask_roles = self._block
+
+    def update(self, key_states: torch.Tensor, value_states: torch.Tensor, token_states_info: torch.Tensor | None,
+               roles: torch.Tensor | None = None):
+        """token_states_info [B, H, x_len, 3] (or `roles` uint8 [B, H, x_len]): one role per new token."""
+        if not key_states.is_cuda:
+            raise ValueError("NAtSLayerCache.update takes GPU tensors")
+        x_len = key_states.shape[2]
+        if x_len == 0:
+            return self.cache_k[:, :, :self.n_ctx_data], self.cache_v[:, :, :self.n_ctx_data]
+        if token_states_info is None and roles is None:
+            raise ValueError("the per-token cache needs the role of every new token")
+        self.chunk_fill_size += x_len
+        self._note_roles(token_states_info, roles)
+        if self._buf_k is None and self._pending is None:
+            self._pending = (key_states, value_states)
+            if self.chunk_fill_size < self.update_chunk_size:
+                self._materialize_pending()  # nothing will be evicted by the coming post_update
+            return key_states, value_states
+        self._materialize_pending()
+        start = self.n_ctx_data
+        end = start + x_len
+        self._grow(end)
+        self._buf_k[:, :, start:end] = key_states.to(self._buf_k.dtype)
+        self._buf_v[:, :, start:end] = value_states.to(self._buf_v.dtype)
+        self._buf_valid[:, :, start:end] = 1
+        if self._buf_pos is not None:
+            self._buf_pos[:, :, start:end] = torch.arange(self._seen_tokens, self._seen_tokens + x_len,
+                                                          dtype=torch.int32, device=self.device)
+        return self._buf_k[:, :, :end], self._buf_v[:, :, :end]
+
+    def append_rotated(self, q, key_states, value_states, cos, sin, token_states_info=None, roles=None):
+        """`update` for a cache that already holds rows, with the rotary embedding of q and k applied on the way."""
+        if self._buf_k is None and self._pending is None:
+            raise ValueError("append_rotated needs a cache that holds rows; the first segment goes through update")
+        if token_states_info is None and roles is None:
+            raise ValueError("the per-token cache needs the role of every new token")
+        x_len = key_states.shape[2]
+        self.chunk_fill_size += x_len
+        self._note_roles(token_states_info, roles)
+        self._materialize_pending()
+        start = self.n_ctx_data
+        end = start + x_len
+        self._grow(end)
+        q_rot = ops.rope_append(q, key_states, value_states, cos, sin, self._buf_k, self._buf_v, self._buf_valid,
+                                self._buf_pos, start, self._seen_tokens)
+        return q_rot, self._buf_k[:, :, :end], self._buf_v[:, :, :end]
+
+    # -- masks (nats_layer_cache.py:155-162, 469-554) ------------------------------------------------
+    def generate_mask(self, x_len: int):
+        """Debug / parity output; the attention kernels never call it."""
+        if x_len == 1:
+            if self._seen_tokens == 0:
+                return torch.ones(1, 1, 1, 1, dtype=torch.bool, device=self.device)
+            return self.valid_tokens[:, :, :self.n_ctx_data + 1].unsqueeze(-2)
+        if self._mask_roles is None:
+            raise ValueError("generate_mask needs the roles handed to update")
+        if self._seen_tokens == 0:
+            return ops.prefill_mask(self._mask_roles, x_len, 1, self.sliding_window_size)
+        self._materialize_pending()
+        return ops.prefill_past_mask(self._buf_valid, self.size_global_kv, self.size_local_kv, self._mask_roles, x_len, 1,
+                                     self.sliding_window_size, self.past_state(x_len))
+
+    def past_state(self, x_len: int):
+        return ops.past_state(self.n_ctx_data, self.chunk_fill_size - x_len, self._n_global_min, self.sliding_queue_tail,
+                              self._seen_tokens, self.chunk_fill_size_last, self.update_chunk_size)
+
+    def segment_roles(self):
+        return self._mask_roles
+
+    def decode_hint(self):
+        """(row_end, tail_start) for `ops.decode_attention` after the update of a one-token step: rows
+        [row_end[b, h], tail_start) hold nothing valid.  Pending blocks start where the last eviction that moved rows
+        left n_ctx_data (blocks of sliding-window tokens stay where they were, still valid)."""
+        return self.row_end(), min(self._live_end, self.n_ctx_data)
+
+    # -- evict + compact (nats_layer_cache.py:292-418) ---------------------------------------------
+    def post_update(self, x_len: int):
+        W, U = self.sliding_window_size, self.update_chunk_size
+        self._seen_tokens += x_len
+        if x_len == 0:
+            return
+        fill = self.chunk_fill_size
+        block_start = self.n_ctx_data - (fill - x_len)  # first row of the pending block
+        self.n_ctx_data += x_len
+        if fill < U:
+            # the eviction is deferred; the ring slot the next token would take is switched off (:300-310)
+            slot = fill if self._seen_tokens < U else (fill + self.sliding_queue_tail + 1) % W
+            self._materialize_pending()
+            self._buf_valid[:, :, slot] = 0
+            self.chunk_fill_size_last = fill
+            return
+        first_ring = fill == self._seen_tokens   # the block holds every token seen so far (:439)
+        first_call = self._seen_tokens == x_len  # (:404)
+        roles = self._block
+        src = self._pending
+        like = src[0] if src is not None else self._buf_k
+        D = like.shape[3]
+        params = ops.evict_params(self.bsz, self.n_msks, D, 1, W, fill, x_len, fill, block_start, self._n_global_min,
+                                  self.sliding_queue_tail, first_ring, max(self._rows, 1), U)
+        ws, result = ops.evict_plan(roles, self.size_global_kv, self.size_local_kv, params)
+        self._row_end = None
+        if src is not None:
+            res = ops.read_result(result)
+            if res.all_sw:  # the reference keeps the untruncated cache here (:316-327)
+                self._materialize_pending()
+                src = None
+            else:
+                rows = int(res.n_ctx_data)
+                self._pending = None
+                self._allocate(rows, like, zero=False)  # the apply kernel writes all rows
+                params.n_alloc = rows
+                k_raw, v_raw = src
+                if k_raw.stride(-1) != 1 or ops.strides_differ(k_raw, v_raw):
+                    k_raw, v_raw = k_raw.contiguous(), v_raw.contiguous()
+                ops.evict_apply_first(k_raw, v_raw, self._buf_k, self._buf_v, self._buf_valid, self._buf_pos, roles,
+                                      self.size_global_kv, self.size_local_kv, params, ws, result)
+        if src is None:
+            params.n_alloc = self._rows
+            ops.evict_apply_inplace(self._buf_k, self._buf_v, self._buf_valid, self._buf_pos, roles, self.size_global_kv,
+                                    self.size_local_kv, params, ws, result)
+            res = ops.read_result(result)
+        n_ring = min(fill, W)  # :437-445
+        self.sliding_queue_tail = n_ring - 1 if first_ring else (self.sliding_queue_tail + n_ring) % W
+        self.chunk_fill_size = 0
+        self.chunk_fill_size_last = 0
+        self.last_evict_result = res
+        self._block = self._roles = None
+        if res.all_sw:
+            return  # n_ctx_data stays: the block's rows remain where they are, valid
+        self.n_ctx_data = int(res.n_ctx_data)
+        self._live_end = self.n_ctx_data
+        self._n_global_min = int(res.gmin)
+        if first_call:
+            self._rows = self.n_ctx_data
+
+
 class NAtSCache:
     """Container of per-layer caches (src/nats/components/cache/dyn_cache.py:66-195)."""
 
     def __init__(self, sliding_window_size: int, chunk_size: int = 1, track_positions: bool = False):
-        # chunk_size == 1 (per-token roles): served by the chunk state machine with one-token chunks.  Visibility
-        # and surviving tokens are those of the per-token rules (global / local until the next global / sliding
-        # window); rows are dropped at every token, where the reference's separate per-token class
-        # (nats_layer_cache.py) defers the update by 16 tokens, keeps the tokens of the pending block visible until
-        # then (:300-310, :544-554) and has its own row order.
-        self.cache_model: list[NAtSChunkLayerCache] = []
+        # chunk_size == 1 (per-token roles) builds NAtSLayerCache layers, any other size NAtSChunkLayerCache layers
+        # (dyn_cache.py:180-190)
+        self.cache_model: list[NAtSChunkLayerCache | NAtSLayerCache] = []
         self.sliding_window_size = sliding_window_size
         self.chunk_size = chunk_size
         self.cached_x: list[torch.Tensor | None] = []
@@ -358,7 +570,7 @@ class NAtSCache:
         return self.cache_model[layer_idx].generate_mask(x_len)
 
     def get_nats_chunk_fill_size(self, layer_idx: int = 0):
-        if len(self.cache_model) <= layer_idx:
+        if len(self.cache_model) <= layer_idx or self.chunk_size == 1:  # dyn_cache.py:87-91
             return 0
         return self.cache_model[layer_idx].chunk_fill_size
 
@@ -420,9 +632,14 @@ class NAtSCache:
     def update(self, key_states, value_states, layer_idx: int, cache_kwargs: dict[str, Any] | None = None):
         if len(self.cache_model) <= layer_idx:
             bsz, n_kv_heads = key_states.shape[:2]
-            self.cache_model.append(NAtSChunkLayerCache(bsz, n_kv_heads, self.sliding_window_size, layer_id=layer_idx,
-                                                        chunk_size=self.chunk_size, device=key_states.device,
-                                                        track_positions=self.track_positions))
+            if self.chunk_size == 1:
+                new_cache = NAtSLayerCache(bsz, n_kv_heads, self.sliding_window_size, layer_id=layer_idx,
+                                           device=key_states.device, track_positions=self.track_positions)
+            else:
+                new_cache = NAtSChunkLayerCache(bsz, n_kv_heads, self.sliding_window_size, layer_id=layer_idx,
+                                                chunk_size=self.chunk_size, device=key_states.device,
+                                                track_positions=self.track_positions)
+            self.cache_model.append(new_cache)
         return self.cache_model[layer_idx].update(key_states, value_states, **(cache_kwargs or {}))
 
     def post_update(self, layer_idx: int, x_len=1, **kwargs):

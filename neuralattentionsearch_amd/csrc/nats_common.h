@@ -63,6 +63,8 @@ struct PastView {
   const int64_t* size_local;   // [B * H_kv]
   int64_t base;                // first cache row of the open-chunk region = n_ctx_data - old_fill
   int64_t gmin, tail, seen, fill_last;
+  int64_t old_fill;   // region tokens cached before the segment
+  int token_mode;     // the per-token cache (one role per token, `tail` = ring slot written last)
 };
 
 struct KeyLimArgs {
@@ -77,6 +79,7 @@ struct KeyLimArgs {
   int2* gran_lim;    // [streams, Tk * 4] out {max, min} of every 16 rows
   int Hkv, S, N, Tk, c_shift, C, W;
   int base, gmin, tail, seen, fill_last;
+  int old_fill, token_mode;
 };
 
 struct PrefillWorkspace {

@@ -1,4 +1,4 @@
-// KV eviction + compaction of the chunked NAtS layer cache (HBM-bound byte moves, bit exact).
+// KV eviction + compaction of the NAtS layer caches (HBM-bound byte moves, bit exact).
 //
 // Follows NAtSChunkLayerCache._post_update (components/cache/nats_chunk_layer_cache.py:270-371), its
 // helpers move_sliding_window_tokens_to_head (:391-437), get_updated_cache_info (:715-868),
@@ -8,6 +8,13 @@
 //                (globals + locals after the last global) and gives each one its destination rank by a
 //                wave-wide prefix sum (stream compaction of slot ids); one more workgroup folds the heads
 //                into the global decisions and scalars.
+// The per-token cache (params.update_chunk != 0; NAtSLayerCache._post_update, components/cache/nats_layer_cache.py:
+// 292-418, with move_sliding_window_tokens_to_head :424-458, get_updated_cache_info :651-770 and mask_invalid_tokens
+// :556-574) runs through the same kernels with one-token chunks: its sizes follow the same arithmetic; what differs
+// is the ring (rows copied whatever the role, the slot after `tail` written first), that rows beyond the new
+// n_ctx_data keep their contents, that a block of sliding-window tokens leaves n_ctx_data alone, and that a block
+// completed by a one-token step takes the general path.
+//
 // apply kernels: move chunk-granular row blocks.  In place, a workgroup owns one row slice of every chunk
 //                of one (b, kv head, tensor) and processes the ordered move list in batches, reading a
 //                whole batch before writing it; because destinations never pass sources this equals
@@ -86,7 +93,7 @@ __global__ __launch_bounds__(256) void evict_plan_heads_kernel(const uint8_t* __
   const uint8_t* r = roles + (int64_t)head * S;
   const long long sg = size_global[head], sl = size_local[head];
   HeadPlan hp;
-  if (p.x_len == 1) {
+  if (p.x_len == 1 && !p.update_chunk) {
     // one completed chunk is scattered for every head (:289-330)
     int r0 = r[0], rl = r[S - 1];
     bool is_g = r0 == NATS_ROLE_GLOBAL;
@@ -212,12 +219,12 @@ __global__ __launch_bounds__(256) void evict_plan_finalize_kernel(const int64_t*
     const PlanAgg t = agg[0];
     nats_evict_result res;
     res.all_sw = t.all_sw;
-    res.all_local = (p.x_len != 1) && t.all_local && !t.all_sw;
+    res.all_local = (p.x_len != 1 || p.update_chunk) && t.all_local && !t.all_sw;
     res.max_keep = t.max_keep;
     res.max_end = t.max_end;
     res.reserved = 0;
-    if (res.all_sw) {  // :283-288
-      res.n_ctx_data = t.max_tot_old + partial;
+    if (res.all_sw) {  // :283-288; the per-token cache keeps the block where it is (nats_layer_cache.py:316-327)
+      res.n_ctx_data = p.update_chunk ? p.n_ctx_data + p.fill : t.max_tot_old + partial;
       res.gmin = p.gmin;
       res.moved_rows = 0;
     } else if (res.all_local) {  // :747-749, then :356-358, :371
@@ -227,7 +234,7 @@ __global__ __launch_bounds__(256) void evict_plan_finalize_kernel(const int64_t*
     } else {
       res.n_ctx_data = t.max_tot_new + partial;
       res.gmin = t.min_sg_new;
-      bool tail_move = p.x_len != 1 && partial && t.max_keep < S - 1;  // :840
+      bool tail_move = (p.x_len != 1 || p.update_chunk) && partial && t.max_keep < S - 1;  // :840
       res.moved_rows = (t.sum_keep + (tail_move ? n_heads : 0)) * (long long)C;
     }
     *result = res;
@@ -306,14 +313,16 @@ __device__ void apply_inplace_body(const ApplyArgs& a, TensorView<U> t, int head
   };
 
   // 1. ring insert (:391-437)
+  const bool token = p.update_chunk != 0;
   const int n_ring = n_done < wc ? n_done : wc;
-  const int start_chunk = p.first ? 0 : (int)(p.tail / p.C);
+  // the chunked cache's tail is the next slot to write, the per-token cache's the slot written last
+  const int start_chunk = p.first ? 0 : token ? (int)((p.tail + 1) % p.W) : (int)(p.tail / p.C);
   for (int j = wave; j < n_ring; j += 4) {
     int slot = n_done - n_ring + j;
     bool is_sw = r[slot] == NATS_ROLE_SW;
     int rc = (start_chunk + j) % wc;
     for (int u = lane; u < units; u += kWave) {
-      U val = is_sw ? *unit_ptr(off + slot, u) : zero_unit<U>();
+      U val = (is_sw || token) ? *unit_ptr(off + slot, u) : zero_unit<U>();  // (nats_layer_cache.py:451-454 copies all)
       *unit_ptr(rc, u) = val;
     }
     if (owns_valid && lane < a.rs) {
@@ -326,7 +335,7 @@ __device__ void apply_inplace_body(const ApplyArgs& a, TensorView<U> t, int head
   // 2. ordered chunk moves, each batch read completely before it is written
   int n_moves;
   bool tail_move = false;
-  if (p.x_len == 1) {
+  if (p.x_len == 1 && !token) {
     n_moves = 1;
   } else if (res.all_local) {
     n_moves = 0;
@@ -374,8 +383,8 @@ __device__ void apply_inplace_body(const ApplyArgs& a, TensorView<U> t, int head
   }
   __syncthreads();
 
-  // 3. rows >= n_ctx_data are zeroed (:360-362)
-  const int64_t n_chunks_alloc = p.n_alloc / C;
+  // 3. rows >= n_ctx_data are zeroed (:360-362); the per-token cache leaves them as they are
+  const int64_t n_chunks_alloc = token ? 0 : p.n_alloc / C;
   for (int64_t ci = res.n_ctx_data / C + wave; ci < n_chunks_alloc; ci += 4) {
     for (int u = lane; u < units; u += kWave) {
       int64_t row = ci * C + row0 + u / t.upr;
@@ -450,11 +459,13 @@ __global__ __launch_bounds__(256) void evict_apply_first_kernel(ApplyArgs a) {
   // where the rows of this destination chunk come from: a source chunk of the raw prefill tensor
   // (-1 = zeros); the untouched part of [W zeros | K | pad] keeps its own rows
   int64_t src_chunk;
+  bool ring_sw = false;  // a ring chunk whose tokens are sliding-window (valid)
   if (ci < wc) {
     src_chunk = -1;
     if (ci < n_ring) {
       int slot = n_done - n_ring + (int)ci;
-      if (r[slot] == NATS_ROLE_SW) src_chunk = slot;
+      ring_sw = r[slot] == NATS_ROLE_SW;
+      if (ring_sw || p.update_chunk) src_chunk = slot;  // the per-token cache copies the row whatever the role
     }
   } else {
     int64_t rel = ci - hp.dst_base;
@@ -500,7 +511,7 @@ __global__ __launch_bounds__(256) void evict_apply_first_kernel(ApplyArgs a) {
       int64_t i = ci * C + row;
       uint8_t v;
       if (i < p.W) {
-        v = (ci < n_ring && src_chunk >= 0) ? 1 : 0;
+        v = ring_sw ? 1 : 0;
       } else {
         v = (i - p.W) < L ? 1 : 0;  // what update() left behind (:229-236)
         if (res.n_ctx_data != p.gmin && i >= p.gmin) {
@@ -532,7 +543,10 @@ static int check_params(const char* who, const nats_evict_params* p) {
   int64_t n_done = p->fill / p->C, partial = p->fill % p->C;
   NATS_REQUIRE(p->S == n_done + (partial ? 1 : 0), NATS_ERR_BAD_SHAPE, "%s: S=%lld role slots for fill=%lld, chunk %lld", who,
                (long long)p->S, (long long)p->fill, (long long)p->C);
-  NATS_REQUIRE(p->x_len != 1 || p->S == 1, NATS_ERR_BAD_SHAPE, "%s: a one-token step completes exactly one chunk", who);
+  NATS_REQUIRE(p->update_chunk >= 0 && (p->update_chunk == 0 || (p->C == 1 && p->fill >= p->update_chunk && p->update_chunk <= p->W)),
+               NATS_ERR_BAD_SHAPE, "%s: update_chunk=%lld needs chunk size 1, a window and a pending block of at least that many tokens",
+               who, (long long)p->update_chunk);
+  NATS_REQUIRE(p->x_len != 1 || p->S == 1 || p->update_chunk, NATS_ERR_BAD_SHAPE, "%s: a one-token step completes exactly one chunk", who);
   NATS_REQUIRE(p->n_ctx_data >= p->W && p->gmin >= p->W && p->tail >= 0 && p->tail < p->W && p->tail % p->C == 0,
                NATS_ERR_BAD_SHAPE, "%s: n_ctx_data=%lld gmin=%lld tail=%lld", who, (long long)p->n_ctx_data,
                (long long)p->gmin, (long long)p->tail);
@@ -590,8 +604,10 @@ extern "C" int nats_evict_apply_inplace(void* cache_k, void* cache_v, uint8_t* v
                NATS_ERR_NULL_POINTER, "nats_evict_apply_inplace: NULL pointer argument");
   NATS_REQUIRE(kv_strides && valid_strides, NATS_ERR_NULL_POINTER, "nats_evict_apply_inplace: NULL stride array");
   if (int rc = check_params("nats_evict_apply_inplace", params)) return rc;
-  NATS_REQUIRE(params->n_alloc % params->C == 0 && params->n_alloc >= params->n_ctx_data - (params->fill - params->x_len) + params->fill,
-               NATS_ERR_BAD_SHAPE, "nats_evict_apply_inplace: n_alloc=%lld", (long long)params->n_alloc);
+  // rows up to the end of the open-chunk region (the per-token cache hands over the first row of its pending block)
+  const int64_t region0 = params->update_chunk ? params->n_ctx_data : params->n_ctx_data - (params->fill - params->x_len);
+  NATS_REQUIRE(params->n_alloc % params->C == 0 && params->n_alloc >= region0 + params->fill, NATS_ERR_BAD_SHAPE,
+               "nats_evict_apply_inplace: n_alloc=%lld", (long long)params->n_alloc);
   ApplyArgs a;
   if (int rc = slice_geometry("nats_evict_apply_inplace", params, elem_bytes, &a.rs, &a.n_slices)) return rc;
   NATS_REQUIRE((kv_strides[0] * elem_bytes) % 16 == 0 && (kv_strides[1] * elem_bytes) % 16 == 0 &&

@@ -1866,7 +1866,7 @@ extern "C" int nats_prefill_past_fwd(const void* q, const void* cache_k, const v
   PrefillWorkspace w = carve_prefill_workspace(workspace, B * H_kv, S, N);
   NATS_REQUIRE(workspace_bytes >= w.bytes, NATS_ERR_WORKSPACE, "%s: workspace %zu bytes < %zu", who, workspace_bytes, w.bytes);
   PastView pv{valid, valid_strides[0], valid_strides[1], size_global, size_local, base,
-              state->gmin, state->tail, state->seen, state->fill_last};
+              state->gmin, state->tail, state->seen, state->fill_last, state->old_fill, state->update_chunk != 0};
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (int rc = prepare_key_limits(roles, B, H_kv, S, N, C, W, &pv, w, st)) return rc;
   const int64_t n_qt = (state->old_fill + x_len - 1) / kTile - state->old_fill / kTile + 1;

@@ -140,7 +140,33 @@ __global__ __launch_bounds__(256) void key_lim_kernel(KeyLimArgs a) {
       const int b = stream / a.Hkv, h = stream % a.Hkv;
       const bool val = a.valid[b * a.valid_s_b + h * a.valid_s_h + row] != 0;
       const int C = a.C;
-      if (row < a.W) {
+      if (a.token_mode) {
+        // The per-token cache (components/cache/nats_layer_cache.py:469-517, 603-649).  Its limits count the
+        // queries of this call (i = r - old_fill), hence the + old_fill.
+        if (row < a.W) {
+          if (a.seen < a.W) {
+            // ring not yet full: the columns of the tokens seen so far are overwritten with an age test, valid
+            // or not (:612-619); the others keep valid_tokens
+            lim = row < a.seen ? a.W - 1 - row + a.old_fill : (val ? kLimGlobal : -1);
+          } else {
+            // slot tail + 1 holds the oldest token, seen by the first query only (:621-647)
+            lim = val ? (row + a.W - 1 - a.tail) % a.W + a.old_fill : -1;
+          }
+        } else if (row < a.gmin) {
+          lim = val ? kLimGlobal : -1;
+        } else {
+          // rows [gmin, base): global rows always, local rows up to the first global token of the block,
+          // nothing beyond a head's own rows (:502-516)
+          const int64_t sg = a.size_global[stream], sl = a.size_local[stream];
+          if (row >= sg + sl) {
+            lim = -1;
+          } else if (row >= sg) {
+            lim = a.first_global[stream] + a.old_fill;
+          } else {
+            lim = kLimGlobal;
+          }
+        }
+      } else if (row < a.W) {
         const int s = row >> a.c_shift;
         if (!val) {
           lim = -1;
@@ -268,6 +294,7 @@ int prepare_key_limits(const uint8_t* roles, int64_t B, int64_t H_kv, int64_t S,
     a.size_global = past->size_global; a.size_local = past->size_local;
     a.base = (int)past->base; a.gmin = (int)past->gmin; a.tail = (int)past->tail; a.seen = (int)past->seen;
     a.fill_last = (int)past->fill_last;
+    a.old_fill = (int)past->old_fill; a.token_mode = past->token_mode;
   }
   return launch_key_lim(a, n_streams, past != nullptr, st);
 }
@@ -364,8 +391,12 @@ extern "C" int nats_prefill_tile_map(const uint8_t* roles, int64_t B, int64_t H_
 int nats::check_past_state(const char* who, const nats_past_state* ps, int64_t x_len, int64_t C, int64_t W) {
   NATS_REQUIRE(ps, NATS_ERR_NULL_POINTER, "%s: NULL past state", who);
   NATS_REQUIRE(x_len > 0, NATS_ERR_BAD_SHAPE, "%s: x_len=%lld", who, (long long)x_len);
-  NATS_REQUIRE(ps->old_fill >= 0 && ps->old_fill < C, NATS_ERR_BAD_SHAPE, "%s: old_fill=%lld outside [0, %lld)", who,
-               (long long)ps->old_fill, (long long)C);
+  NATS_REQUIRE(ps->update_chunk >= 0 && (ps->update_chunk == 0 || (C == 1 && ps->update_chunk <= W)), NATS_ERR_BAD_SHAPE,
+               "%s: update_chunk=%lld needs chunk size 1 and a window of at least that many tokens", who,
+               (long long)ps->update_chunk);
+  const int64_t fill_cap = ps->update_chunk ? ps->update_chunk : C;  // pending tokens stay below one (update) chunk
+  NATS_REQUIRE(ps->old_fill >= 0 && ps->old_fill < fill_cap, NATS_ERR_BAD_SHAPE, "%s: old_fill=%lld outside [0, %lld)", who,
+               (long long)ps->old_fill, (long long)fill_cap);
   NATS_REQUIRE(ps->n_ctx_data >= W + ps->old_fill && ps->n_ctx_data + x_len < (int64_t(1) << 30), NATS_ERR_BAD_SHAPE,
                "%s: n_ctx_data=%lld with window %lld and %lld open-chunk tokens", who, (long long)ps->n_ctx_data,
                (long long)W, (long long)ps->old_fill);
@@ -373,7 +404,7 @@ int nats::check_past_state(const char* who, const nats_past_state* ps, int64_t x
                "%s: gmin=%lld outside [W, first open-chunk row]", who, (long long)ps->gmin);
   NATS_REQUIRE(ps->tail >= 0 && (W == 0 ? ps->tail == 0 : ps->tail < W), NATS_ERR_BAD_SHAPE, "%s: tail=%lld", who,
                (long long)ps->tail);
-  NATS_REQUIRE(ps->seen >= 0 && ps->fill_last >= 0 && ps->fill_last < C, NATS_ERR_BAD_SHAPE, "%s: seen=%lld fill_last=%lld",
+  NATS_REQUIRE(ps->seen >= 0 && ps->fill_last >= 0 && ps->fill_last < fill_cap, NATS_ERR_BAD_SHAPE, "%s: seen=%lld fill_last=%lld",
                who, (long long)ps->seen, (long long)ps->fill_last);
   return NATS_OK;
 }
@@ -395,7 +426,7 @@ extern "C" int nats_prefill_past_mask(const uint8_t* valid, const int64_t* size_
   NATS_REQUIRE(workspace_bytes >= w.bytes, NATS_ERR_WORKSPACE, "nats_prefill_past_mask: workspace %zu bytes < %zu",
                workspace_bytes, w.bytes);
   PastView pv{valid, valid_strides[0], valid_strides[1], size_global, size_local, ps->n_ctx_data - ps->old_fill,
-              ps->gmin, ps->tail, ps->seen, ps->fill_last};
+              ps->gmin, ps->tail, ps->seen, ps->fill_last, ps->old_fill, ps->update_chunk != 0};
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (int rc = prepare_key_limits(roles, B, H_kv, S, N, C, W, &pv, w, st)) return rc;
   return launch_mask_rows(w, B * H_kv, N, x_len, pv.base, ps->old_fill, mask, st);

@@ -198,9 +198,9 @@ class NAtSLlamaAttention(nn.Module):
         layer = past_key_value.cache_model[idx]
         cos, sin = position_embeddings
         q, keys, values = layer.append_rotated(q, k, v, cos, sin, tsi, roles)
+        row_end, tail_start = layer.decode_hint()
         out = ops.decode_attention(q, keys, values, layer.valid_tokens, keys.shape[2], 1.0 / math.sqrt(D),
-                                   row_end=layer.row_end(),
-                                   tail_start=layer.n_ctx_data - (layer.chunk_fill_size - 1))
+                                   row_end=row_end, tail_start=tail_start)
         past_key_value.post_update(layer_idx=idx, x_len=1)
         return step_linear(out.transpose(1, 2).reshape(bsz, 1, -1), self.o_proj)
 
@@ -258,9 +258,9 @@ class NAtSLlamaAttention(nn.Module):
         elif q_len > 1:
             out = layer.segment_attention(q, scale)
         else:
-            out = ops.decode_attention(q, keys, values, layer.valid_tokens, keys.shape[2], scale,
-                                       row_end=layer.row_end(),
-                                       tail_start=layer.n_ctx_data - (layer.chunk_fill_size - 1))
+            row_end, tail_start = layer.decode_hint()
+            out = ops.decode_attention(q, keys, values, layer.valid_tokens, keys.shape[2], scale, row_end=row_end,
+                                       tail_start=tail_start)
         past_key_value.post_update(layer_idx=idx, x_len=q_len)
         return self.o_proj(out.transpose(1, 2).reshape(bsz, q_len, -1))
 

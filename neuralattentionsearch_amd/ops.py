@@ -57,11 +57,14 @@ def _require_cuda(*ts):
 
 
 def workspace(device, key: str, nbytes: int) -> torch.Tensor:
-    """A per-(device, purpose) scratch buffer that only ever grows.
+    """A scratch buffer per (device, current stream, purpose) that only ever grows.
 
-    Calls of one purpose share the buffer, so they must be ordered on the device: issue them on one stream (or
-    order the streams with events).  Two streams that run, say, two prefills side by side would race on it."""
-    k = (str(device), key)
+    Calls of one purpose on one stream share the buffer, which the stream orders; calls on different streams (two
+    prefills side by side, a worker thread under the caller's stream) get buffers of their own."""
+    device = torch.device(device)
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    handle = _raw_stream(idx) if _raw_stream is not None else torch.cuda.current_stream(device).cuda_stream
+    k = (idx, int(handle or 0), key)
     buf = _workspaces.get(k)
     if buf is None or buf.numel() < nbytes:
         buf = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
@@ -221,8 +224,10 @@ def prefill_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, roles: 
     return out
 
 
-def past_state(n_ctx_data: int, old_fill: int, gmin: int, tail: int, seen: int, fill_last: int) -> PastState:
-    return PastState(int(n_ctx_data), int(old_fill), int(gmin), int(tail), int(seen), int(fill_last))
+def past_state(n_ctx_data: int, old_fill: int, gmin: int, tail: int, seen: int, fill_last: int,
+               update_chunk: int = 0) -> PastState:
+    """`update_chunk` = U > 0 describes the per-token cache (one role per token, eviction every U tokens)."""
+    return PastState(int(n_ctx_data), int(old_fill), int(gmin), int(tail), int(seen), int(fill_last), int(update_chunk))
 
 
 def _check_past(valid, size_global, size_local, roles, B, Hkv, x_len, C, state: PastState):
@@ -372,8 +377,8 @@ def decode_attention(q: torch.Tensor, cache_k: torch.Tensor, cache_v: torch.Tens
 # ------------------------------------------------------------------------------------------------
 # eviction + compaction
 # ------------------------------------------------------------------------------------------------
-def evict_params(B, H_kv, D, C, W, S, x_len, fill, n_ctx_data, gmin, tail, first, n_alloc) -> EvictParams:
-    return EvictParams(B, H_kv, D, C, W, S, x_len, fill, n_ctx_data, gmin, tail, int(first), n_alloc)
+def evict_params(B, H_kv, D, C, W, S, x_len, fill, n_ctx_data, gmin, tail, first, n_alloc, update_chunk=0) -> EvictParams:
+    return EvictParams(B, H_kv, D, C, W, S, x_len, fill, n_ctx_data, gmin, tail, int(first), n_alloc, int(update_chunk))
 
 
 def evict_plan(roles: torch.Tensor, size_global: torch.Tensor, size_local: torch.Tensor, params: EvictParams):

@@ -29,7 +29,8 @@ def test_library_exports_every_declared_symbol():
 
 
 def test_struct_sizes_match_header():
-    assert ctypes.sizeof(_lib.EvictParams) == 13 * 8
+    assert ctypes.sizeof(_lib.EvictParams) == 14 * 8
+    assert ctypes.sizeof(_lib.PastState) == 7 * 8
     assert ctypes.sizeof(_lib.EvictResult) == 64
 
 
@@ -73,11 +74,11 @@ def test_past_state_is_validated():
     st = _lib.i64_array([8, 8, 8])
     args = lambda ps, ws=1 << 24: (fake, fake, fake, fake, fake, fake, fake, fake, 1, 4, 2, 100, 128, 16, 32,
                                    ctypes.byref(ps), st, st, st, st, st, 1.0, 0, fake, ws, None)
-    ok = _lib.PastState(320, 5, 64, 16, 400, 5)
+    ok = _lib.PastState(320, 5, 64, 16, 400, 5, 0)
     assert lib.nats_prefill_past_fwd(*args(ok, 8)) == -5  # everything valid but the workspace
-    assert lib.nats_prefill_past_fwd(*args(_lib.PastState(320, 16, 64, 16, 400, 5))) == -2  # old_fill >= C
-    assert lib.nats_prefill_past_fwd(*args(_lib.PastState(320, 5, 16, 16, 400, 5))) == -2  # gmin < W
-    assert lib.nats_prefill_past_fwd(*args(_lib.PastState(320, 5, 64, 32, 400, 5))) == -2  # tail >= W
+    assert lib.nats_prefill_past_fwd(*args(_lib.PastState(320, 16, 64, 16, 400, 5, 0))) == -2  # old_fill >= C
+    assert lib.nats_prefill_past_fwd(*args(_lib.PastState(320, 5, 16, 16, 400, 5, 0))) == -2  # gmin < W
+    assert lib.nats_prefill_past_fwd(*args(_lib.PastState(320, 5, 64, 32, 400, 5, 0))) == -2  # tail >= W
     assert lib.nats_prefill_past_fwd(*args(_lib.PastState(20, 5, 64, 16, 400, 5))) == -2  # n_ctx_data < W + old_fill
     assert b"n_ctx_data" in lib.nats_last_error()
     need = lib.nats_prefill_past_workspace_bytes(1, 2, 420, 7)

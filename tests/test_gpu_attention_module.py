@@ -32,9 +32,9 @@ def test_module_segments_over_a_filled_cache(lens, C, W):
 
 
 @pytest.mark.parametrize("lens,W", [([40] + [1] * 30, 16), ([70, 45, 1, 1, 33, 1, 90], 32),
-                                    ([1, 1, 1, 12, 1, 1, 30, 1], 16)])  # (a first segment of one token is a whole chunk)
+                                    ([1, 1, 1, 12, 1, 1, 30, 1], 16), ([5] + [1] * 14 + [40, 3, 1, 1, 20], 16)])
 def test_module_with_per_token_roles(lens, W):
-    """chunk_size == 1: a role per token, served by the same state machine with one-token chunks."""
+    """chunk_size == 1: a role per token, the per-token cache class with its eviction deferred by 16 tokens."""
     run_module(lens, 1, W)
 
 
@@ -53,7 +53,8 @@ def run_module(lens, C, W, executor=None):
     logits_seen = []
     mod.proj_layer.register_forward_hook(lambda m, i, o: logits_seen.append(o.detach().float().cpu()))
     cache = NAtSCache(sliding_window_size=W, chunk_size=C)
-    st = orc.ChunkCacheOracle(B=B, H=Hkv, W=W, C=C)
+    # (chunk_size == 1 builds the per-token class with its deferred eviction, as the reference's container does)
+    st = orc.TokenCacheOracle(B=B, H=Hkv, W=W) if C == 1 else orc.ChunkCacheOracle(B=B, H=Hkv, W=W, C=C)
 
     def qkv(x, start):
         n = x.shape[1]
@@ -71,6 +72,8 @@ def run_module(lens, C, W, executor=None):
             q, k, v, pos = qkv(x, seen)
             logits_seen.clear()
             out = mod(x, pos, None, start_pos=seen, cache=cache)
+            if mod._cache_is_till_updating is not None:  # an executor runs the eviction; the next call waits for it
+                mod._cache_is_till_updating.result()
             # oracle side, fed with the module's own logits
             total = fill + n
             if total < C:
@@ -187,4 +190,17 @@ def test_module_on_a_side_stream():
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
         run_module([40, 1, 1, 1, 20, 1, 1, 9], 8, 16)
+    side.synchronize()
+
+
+def test_module_with_an_executor_under_a_side_stream():
+    """The eviction runs on the executor's thread, where torch's current stream would be the default one: the module
+    hands the caller's stream over, so the eviction kernels follow the attention kernel that still reads the rows."""
+    from concurrent.futures import ThreadPoolExecutor
+    say("attention module: executor under a side stream")
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with ThreadPoolExecutor(max_workers=1) as pool, torch.cuda.stream(side):
+        run_module([300, 1, 1, 1, 120, 1, 1, 9, 200], 8, 16, executor=pool)
+        run_module([200] + [1] * 20 + [90], 1, 16, executor=pool)
     side.synchronize()

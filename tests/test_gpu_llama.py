@@ -46,7 +46,9 @@ def run(cfg, dtype, lens, tol, B=2, seed=0, std=0.05, need_all_roles=True):
     cache = model.new_cache()
     C, W = cfg.chunk_size, cfg.local_seq_max_length
     Hq, Hkv, D = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
-    states = [orc.ChunkCacheOracle(B=B, H=Hkv, W=W, C=C) for _ in model.layers]
+    # (chunk_size == 1 builds the per-token class with its deferred eviction, as the reference's container does)
+    states = [orc.TokenCacheOracle(B=B, H=Hkv, W=W) if C == 1 else orc.ChunkCacheOracle(B=B, H=Hkv, W=W, C=C)
+              for _ in model.layers]
     fills = [0] * len(model.layers)
     g = torch.Generator().manual_seed(seed)
     seen = 0
@@ -104,7 +106,7 @@ def test_small_fp32_model_layer_by_layer():
 
 
 def test_per_token_roles_layer_by_layer():
-    """chunk_size == 1: a role per token (the per-token adapters of the reference), one-token chunks in the cache."""
+    """chunk_size == 1: a role per token (the per-token adapters of the reference), the per-token cache class."""
     from neuralattentionsearch_amd.llama import NAtSLlamaConfig
     cfg = NAtSLlamaConfig(vocab_size=1000, hidden_size=512, intermediate_size=1024, num_hidden_layers=2,
                           num_attention_heads=8, num_key_value_heads=2, chunk_size=1, local_seq_max_length=16)

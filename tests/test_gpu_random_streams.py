@@ -35,7 +35,9 @@ def test_random_streams_through_the_attention_module(seed):
     rng = np.random.default_rng(1000 + seed)
     C = int(rng.choice([1, 2, 4, 8, 16, 32, 64]))
     W = C * int(rng.integers(1, 6))
-    lens = draw_stream(rng, C, int(rng.integers(2, 7)))
+    if C == 1:
+        W = 16 * W  # the per-token class wants a window of at least its update chunk size
+    lens = draw_stream(rng, 16 if C == 1 else C, int(rng.integers(2, 7)))
     say("random module stream", seed, C, W, lens)
     run_module(lens, C, W)
 
@@ -49,10 +51,12 @@ def test_random_configurations_of_the_harness(seed):
     D = int(rng.choice([64, 128]))
     C = int(rng.choice([1, 4, 8, 16, 64]))
     W = C * int(rng.integers(1, 5))
+    if C == 1:
+        W = 16 * W
     cfg = NAtSLlamaConfig(vocab_size=500, hidden_size=Hq * D, intermediate_size=256, num_hidden_layers=2,
                           num_attention_heads=Hq, num_key_value_heads=Hkv, chunk_size=C, local_seq_max_length=W,
                           chunk_merge_method=str(rng.choice(["mean", "max"])), fused_decode=bool(rng.integers(0, 2)))
-    lens = draw_stream(rng, C, int(rng.integers(3, 6)))
+    lens = draw_stream(rng, 16 if C == 1 else C, int(rng.integers(3, 6)))
     say("random harness configuration", seed, cfg, lens)
     # (weights scaled so that q, k, v keep the scale of the 512-wide model the fixed cases use)
     run_harness(cfg, torch.float32, lens, tol=5e-5, B=int(rng.integers(1, 3)), seed=seed, std=0.05 * (512.0 / (Hq * D)) ** 0.5,
