@@ -298,6 +298,17 @@ def prefill_past_attention(q: torch.Tensor, cache_k: torch.Tensor, cache_v: torc
     return out
 
 
+def _roles_from_kernel_arguments(end_seqs_idx: torch.Tensor, sliding_tokens: torch.Tensor) -> torch.Tensor:
+    """A slot is global iff end_seqs_idx[n] == n (nats_flashattn_fwd.py:110), sliding window iff its flag is set."""
+    slots = torch.arange(end_seqs_idx.shape[-1], device=end_seqs_idx.device)
+    is_global = end_seqs_idx == slots
+    is_sw = sliding_tokens > 0
+    return torch.where(is_global, ROLE_GLOBAL, torch.where(is_sw, ROLE_SW, ROLE_LOCAL)).to(torch.uint8)
+
+
+PER_TOKEN_UPDATE_CHUNK = 16  # update_chunk_size of the per-token cache as NAtSCache builds it (dyn_cache.py:183-185)
+
+
 def nats_prefill(q, k, v, end_seqs_idx, sliding_tokens, sm_scale, nats_chunk_size: int = 1, global_kv_size=None,
                  local_kv_size=None, valid_sw_tokens=None, n_ctx_data=None, sw_token_tails=None, n_rep: int = 1,
                  n_tokens_in_first_chunk: int = 0, local_seq_max_length: int = 4, return_masks: bool = False,
@@ -306,23 +317,46 @@ def nats_prefill(q, k, v, end_seqs_idx, sliding_tokens, sm_scale, nats_chunk_siz
     names and meaning, returns (o, mask or None)).
 
     end_seqs_idx [B, H_kv, S] int64 is the next-global index computed with the last slot forced global;
-    sliding_tokens [B, H_kv, S] is option 2 of token_states_info.  A slot is global iff
-    end_seqs_idx[n] == n (nats_flashattn_fwd.py:110)."""
-    if global_kv_size is not None:
-        # the reference's only caller of this form (hf/llama.py:237-252) unpacks four results from a function
-        # that returns two; the working path for such a segment is generate_mask + SDPA, which
-        # prefill_past_attention stands in for
-        raise NotImplementedError("the HAS_PAST_INFO form is not mirrored: use prefill_past_attention, the "
-                                  "replacement of generate_mask + SDPA for a segment over an existing cache")
+    sliding_tokens [B, H_kv, S] is option 2 of token_states_info.
+
+    With `global_kv_size` the call is a segment over a cache that earlier segments filled (the HAS_PAST_INFO form,
+    nats_flashattn_fwd.py:622-627, 476-571, called as in the reference's own smoke :925-956): k / v are the cache
+    views `cache.update` returned, [B, H_kv, n_ctx_data + L_q, D]; global_kv_size / local_kv_size are the cache's
+    size tensors; valid_sw_tokens [B, H_kv, W / C] = valid_tokens[..., :W:C]; n_ctx_data and sw_token_tails its
+    n_ctx_data and sliding_queue_tail before the eviction of this segment; n_tokens_in_first_chunk the tokens of
+    the open chunk cached before the segment.  The result is SDPA(q, k, v, cache.generate_mask(L_q)), the path
+    this kernel form is checked against there, for a cache in the state those arguments describe: valid_tokens is
+    rebuilt from them (ring bits, a head's own rows, the open chunk), the window is taken as full
+    (_seen_tokens >= W; the arguments do not carry it), and nats_chunk_size == 1 means the per-token cache class
+    (`sliding_queue_tail` = the slot written last)."""
     if q.shape[1] // k.shape[1] != n_rep:
         raise ValueError(f"n_rep={n_rep} does not match {q.shape[1]} q heads / {k.shape[1]} kv heads")
-    S = end_seqs_idx.shape[-1]
-    slots = torch.arange(S, device=end_seqs_idx.device)
-    is_global = end_seqs_idx == slots
-    is_sw = sliding_tokens > 0
-    roles = torch.where(is_global, ROLE_GLOBAL, torch.where(is_sw, ROLE_SW, ROLE_LOCAL)).to(torch.uint8)
-    o = prefill_attention(q, k, v, roles, nats_chunk_size, local_seq_max_length, sm_scale)
-    mask = prefill_mask(roles, q.shape[2], nats_chunk_size, local_seq_max_length) if return_masks else None
+    roles = _roles_from_kernel_arguments(end_seqs_idx, sliding_tokens)
+    C, W = int(nats_chunk_size), int(local_seq_max_length)
+    if global_kv_size is None:
+        o = prefill_attention(q, k, v, roles, C, W, sm_scale)
+        mask = prefill_mask(roles, q.shape[2], C, W) if return_masks else None
+        return o, mask
+    if local_kv_size is None or valid_sw_tokens is None or n_ctx_data is None or sw_token_tails is None:
+        raise ValueError("the form over an existing cache needs local_kv_size, valid_sw_tokens, n_ctx_data and sw_token_tails")
+    B, Hkv, x_len = k.shape[0], k.shape[1], q.shape[2]
+    n_ctx, tail, old_fill = int(n_ctx_data), int(sw_token_tails), int(n_tokens_in_first_chunk)
+    if k.shape[2] != n_ctx + x_len:
+        raise ValueError(f"k / v must hold n_ctx_data + L_q = {n_ctx + x_len} rows, got {k.shape[2]}")
+    if C > 1 and n_ctx % C != old_fill:
+        raise ValueError(f"n_ctx_data={n_ctx} does not end {old_fill} tokens into a chunk of {C}")
+    if tuple(valid_sw_tokens.shape) != (B, Hkv, W // C):
+        raise ValueError(f"valid_sw_tokens must be [B, H_kv, W / C], got {tuple(valid_sw_tokens.shape)}")
+    sg = global_kv_size.to(torch.int64).contiguous()
+    sl = local_kv_size.to(torch.int64).contiguous()
+    rows = torch.arange(n_ctx, device=q.device)
+    valid = rows < (sg + sl).unsqueeze(-1)                                       # a head's own global and local rows
+    valid[:, :, :W] = valid_sw_tokens.bool().repeat_interleave(C, dim=-1)       # ring slots
+    valid[:, :, n_ctx - old_fill:] = True                                        # the open chunk
+    state = past_state(n_ctx, old_fill, int(sg.min()), tail, W, old_fill,
+                       PER_TOKEN_UPDATE_CHUNK if C == 1 else 0)
+    o = prefill_past_attention(q, k, v, valid, sg, sl, roles, C, W, state, sm_scale)
+    mask = prefill_past_mask(valid, sg, sl, roles, x_len, C, W, state) if return_masks else None
     return o, mask
 
 
