@@ -545,8 +545,16 @@ class NAtSLayerCache(NAtSChunkLayerCache):
             self._rows = self.n_ctx_data
 
 
-class NAtSCache:
-    """Container of per-layer caches (src/nats/components/cache/dyn_cache.py:66-195)."""
+try:  # the reference's container is a transformers cache (dyn_cache.py:66): HF models take it as past_key_values
+    from transformers.cache_utils import DynamicCache as _CacheBase
+except Exception:  # transformers absent or unusable: a plain class with the same surface
+    _CacheBase = object
+
+
+class NAtSCache(_CacheBase):
+    """Container of per-layer caches (src/nats/components/cache/dyn_cache.py:66-195).  A subclass of
+    transformers' DynamicCache where that library is importable; like the reference it does not run the base
+    class's __init__ and answers every call its callers make itself."""
 
     def __init__(self, sliding_window_size: int, chunk_size: int = 1, track_positions: bool = False):
         # chunk_size == 1 (per-token roles) builds NAtSLayerCache layers, any other size NAtSChunkLayerCache layers
@@ -560,6 +568,12 @@ class NAtSCache:
     def reset_cache(self):
         self.cache_model = []
         self.cached_x = []
+
+    def __len__(self):
+        return len(self.cache_model)
+
+    def get_max_cache_shape(self, layer_idx: int = 0):
+        return -1  # no fixed maximum: rows are evicted, capacity grows on demand
 
     def get_seq_length(self, layer_idx: int = 0) -> int:
         if len(self.cache_model) <= layer_idx:

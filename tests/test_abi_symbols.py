@@ -138,3 +138,17 @@ def test_rope_qk_arguments_are_validated():
     odd = _lib.i64_array([4096, 124, 512])
     assert lib.nats_rope_qk(fake, fake, fake, fake, fake, fake, 1, 4, 2, 8, 128, odd, st3, st2, 0, None) == -2  # 16-byte rows
     assert lib.nats_rope_qk(fake, fake, fake, fake, fake, fake, 1, 4, 2, 8, 128, st3, st3, st2, 9, None) == -3  # dtype
+
+
+def test_container_is_a_transformers_cache():
+    """The reference's NAtSCache subclasses DynamicCache (components/cache/dyn_cache.py:66) and is handed to HF models
+    as past_key_values; its constructor and the calls made before any update work without a GPU."""
+    cache_utils = pytest.importorskip("transformers.cache_utils")
+    from neuralattentionsearch_amd.cache import NAtSCache
+    cache = NAtSCache(256, 64)
+    assert isinstance(cache, cache_utils.Cache) and isinstance(cache, cache_utils.DynamicCache)
+    assert cache.get_seq_length() == 0 and cache.get_seq_length(3) == 0 and len(cache) == 0
+    assert cache.get_nats_chunk_fill_size(0) == 0 and cache.get_nats_cached_x_in_chunk(0) is None
+    assert cache.sliding_window_size == 256 and cache.chunk_size == 64
+    cache.reset_cache()
+    assert cache.cache_model == []

@@ -35,7 +35,9 @@ def test_prefill_decode_and_segment_agree(Hq, Hkv, L, C, W, tail):
     roles[:, :, 0] = 0
     g = torch.Generator(device="cuda").manual_seed(L + C)
     N = L + tail
-    q = torch.randn(B, Hq, N, D, generator=g, device="cuda", dtype=torch.bfloat16)
+    # scores with a standard deviation of 4 nats: every row's output is carried by a few keys and is of the size of
+    # v, so that a missing or an extra key shows against the tolerance
+    q = (torch.randn(B, Hq, N, D, generator=g, device="cuda") * 4.0).bfloat16()
     k = torch.randn(B, Hkv, N, D, generator=g, device="cuda", dtype=torch.bfloat16)
     v = torch.randn(B, Hkv, N, D, generator=g, device="cuda", dtype=torch.bfloat16)
     scale = 1.0 / math.sqrt(D)
@@ -62,9 +64,9 @@ def test_prefill_decode_and_segment_agree(Hq, Hkv, L, C, W, tail):
         t = L + i
         closes = (cache.chunk_fill_size + 1) >= C
         keys, values = cache.update(k[:, :, t:t + 1], v[:, :, t:t + 1], None, roles=one_global if closes else None)
+        row_end, tail_start = cache.decode_hint()
         out_b.append(ops.decode_attention(q[:, :, t:t + 1], keys, values, cache.valid_tokens, keys.shape[2], scale,
-                                          row_end=cache.row_end(),
-                                          tail_start=cache.n_ctx_data - (cache.chunk_fill_size - 1)))
+                                          row_end=row_end, tail_start=tail_start))
         cache.post_update(1)
     out_b = torch.cat(out_b, dim=2).float()
 
@@ -73,8 +75,10 @@ def test_prefill_decode_and_segment_agree(Hq, Hkv, L, C, W, tail):
     cache.update(k[:, :, L:], v[:, :, L:], None, roles=torch.zeros(B, Hkv, n_tail_slots, dtype=torch.uint8, device="cuda"))
     out_c = cache.segment_attention(q[:, :, L:], scale).float()
 
-    err_ab = (out_a - out_b).abs().max().item()
-    err_ac = (out_a - out_c).abs().max().item()
     assert torch.isfinite(out_a).all() and torch.isfinite(out_b).all() and torch.isfinite(out_c).all()
-    assert err_ab <= TOL, f"prefill rows vs token-by-token decode: {err_ab}"
-    assert err_ac <= TOL, f"prefill rows vs one segment over the cache: {err_ac}"
+    rms = out_a.pow(2).mean(-1, keepdim=True).sqrt()
+    assert rms.min().item() > 0.05, rms.min().item()
+    bound = TOL * torch.maximum(rms, out_a.abs()) + 2e-3  # (both sides are rounded to bf16: an element may differ by its ulp)
+    err_ab, err_ac = (out_a - out_b).abs(), (out_a - out_c).abs()
+    assert not (err_ab > bound).any(), f"prefill rows vs token-by-token decode: {err_ab.max().item()}"
+    assert not (err_ac > bound).any(), f"prefill rows vs one segment over the cache: {err_ac.max().item()}"

@@ -98,12 +98,14 @@ def test_strided_inputs_and_drop_in_signature():
 
 def check_sampled_rows(B, Hq, Hkv, L, D, C, W, n_samples=96, p=(0.05, 0.15, 0.8)):
     """A run too large for the oracle's dense mask, checked on sampled query rows against a direct per-row
-    evaluation of the mask predicate."""
+    evaluation of the mask predicate.  Scores are peaked (standard deviation 4 nats), so a row's output is carried by
+    a few keys and is of the size of v: a dropped tile, granule or key shows, and the error is held against the
+    row's own magnitude."""
     from neuralattentionsearch_amd import ops
     g = torch.Generator().manual_seed(0)
-    q = (torch.randn(B, Hq, L, D, generator=g) / math.sqrt(D)).bfloat16()
-    k = (torch.randn(B, Hkv, L, D, generator=g) / math.sqrt(D)).bfloat16()
-    v = (torch.randn(B, Hkv, L, D, generator=g) / math.sqrt(D)).bfloat16()
+    q = (torch.randn(B, Hq, L, D, generator=g) * 2.0).bfloat16()
+    k = (torch.randn(B, Hkv, L, D, generator=g) * 2.0).bfloat16()
+    v = torch.randn(B, Hkv, L, D, generator=g).bfloat16()
     S = -(-L // C)
     roles = draw_roles(1, B, Hkv, S, p=p)
     if L % C:
@@ -112,7 +114,7 @@ def check_sampled_rows(B, Hq, Hkv, L, D, C, W, n_samples=96, p=(0.05, 0.15, 0.8)
     assert torch.isfinite(out).all()
     gidx = orc.next_global_index(roles == 0)
     rng = np.random.default_rng(7)
-    worst = 0.0
+    worst, smallest = 0.0, float("inf")
     for i in range(n_samples):
         hq = int(rng.integers(Hq))
         m = int(rng.integers(L)) if i % 4 else L - 1 - int(rng.integers(64))
@@ -126,8 +128,11 @@ def check_sampled_rows(B, Hq, Hkv, L, D, C, W, n_samples=96, p=(0.05, 0.15, 0.8)
         idx = torch.from_numpy(n[vis])
         s = (q[0, hq, m].float() @ k[0, hkv, idx].float().T) / math.sqrt(D)
         want = torch.softmax(s, -1) @ v[0, hkv, idx].float()
-        worst = max(worst, (out[0, hq, m] - want).abs().max().item())
-    assert worst <= 2e-2, worst
+        rms = want.pow(2).mean().sqrt().item()
+        err = (out[0, hq, m] - want).abs().max().item()
+        assert err <= 2e-2 * rms + 2e-3, (hq, m, err, rms)
+        worst, smallest = max(worst, err), min(smallest, rms)
+    assert smallest > 0.05, smallest  # the rows checked are far from zero
 
 
 def test_cfg2_full_size_sampled_rows():
@@ -341,3 +346,115 @@ def test_persistent_kernel_on_a_segment_over_a_filled_cache(stream_kernel):
         outs.append(res)
     for x, y in zip(*outs):
         assert torch.equal(x, y)
+
+
+# ---- running maxima that keep rising: the rescaling branch of every variant ------------------------------------
+def rising_inputs(B, Hq, Hkv, L, D, step_rows, step_nats, seed):
+    """q, k, v whose scores grow by `step_nats` every `step_rows` keys (a common direction u: q carries sqrt(D) u,
+    key n carries (n // step_rows) * step_nats * u), on top of unit noise.  Every later block of keys beats the
+    running maximum of the earlier ones by more than the slack within which the kernels leave it alone, so their
+    accumulators are rescaled with 0 < alpha < 1 again and again."""
+    g = torch.Generator().manual_seed(seed)
+    u = torch.nn.functional.normalize(torch.randn(D, generator=g), dim=0)
+    q = torch.randn(B, Hq, L, D, generator=g) * 0.5 + math.sqrt(D) * u
+    level = (torch.arange(L) // step_rows).float() * step_nats
+    k = torch.randn(B, Hkv, L, D, generator=g) * 0.5 + level[None, None, :, None] * u
+    v = torch.randn(B, Hkv, L, D, generator=g)
+    return q.bfloat16(), k.bfloat16(), v.bfloat16()
+
+
+def check_rising(B, Hq, Hkv, L, D, C, W, p, step_rows=48, step_nats=7.0, seed=0):
+    from neuralattentionsearch_amd import ops
+    q, k, v = rising_inputs(B, Hq, Hkv, L, D, step_rows, step_nats, seed)
+    roles = draw_roles(seed + 1, B, Hkv, -(-L // C), p=p)
+    if L % C:
+        roles[:, :, -1] = 0
+    want = orc.masked_attention(q.float(), k.float(), v.float(), orc.prefill_mask(roles, L, C, W))
+    got = ops.prefill_attention(q.cuda(), k.cuda(), v.cuda(), to_dev(roles), C, W).cpu().float()
+    assert torch.isfinite(got).all()
+    rms = want.pow(2).mean(-1, keepdim=True).sqrt()
+    bad = ((got - want).abs() > 2e-2 * torch.maximum(rms, want.abs()) + 2e-3)
+    assert not bad.any(), (int(bad.sum()), (got - want).abs().max().item())
+
+
+@pytest.mark.parametrize("Hq,Hkv,L,D,C,W,p", [
+    (8, 2, 1500, 128, 64, 256, (1.0, 0.0, 0.0)),   # whole tiles, dense
+    (8, 2, 1500, 128, 64, 128, (0.2, 0.3, 0.5)),   # whole tiles, mixed roles
+    (8, 2, 1300, 64, 64, 128, (0.3, 0.3, 0.4)),    # head_dim 64
+    (8, 2, 1500, 128, 16, 64, (0.3, 0.3, 0.4)),    # packed tiles
+    (4, 4, 1200, 128, 64, 128, (0.3, 0.3, 0.4)),   # one q head per kv head (packed form, four query tiles a workgroup)
+    (4, 2, 1200, 128, 8, 32, (0.3, 0.3, 0.4)),     # groups of two
+    (6, 2, 900, 128, 64, 128, (0.4, 0.3, 0.3)),    # a group of three: the per-wavefront form
+])
+def test_rising_scores_rescale_the_accumulators(Hq, Hkv, L, D, C, W, p):
+    say("prefill rising scores", Hq, Hkv, L, D, C, W, p)
+    check_rising(1, Hq, Hkv, L, D, C, W, p)
+
+
+def test_rising_scores_in_the_persistent_kernel(stream_kernel):
+    say("prefill rising scores, persistent kernel")
+    stream_kernel(True)
+    check_rising(1, 8, 2, 1500, 128, 64, 256, (0.5, 0.2, 0.3))
+
+
+def test_rising_scores_in_split_lists_and_the_decode_kernel(split_lists):
+    """A short segment over a long cache (several workgroups share a tile list, partial results merged) and one-token
+    steps over the same rows (split over workgroups, merged): both with scores that rise along the rows."""
+    from neuralattentionsearch_amd import ops
+    from neuralattentionsearch_amd.cache import NAtSChunkLayerCache
+    say("prefill split lists + decode, rising scores")
+    split_lists(True)
+    B, Hq, Hkv, D, C, W = 1, 8, 2, 128, 64, 256
+    n1, n2 = 6016, 64
+    q, k, v = rising_inputs(B, Hq, Hkv, n1 + n2 + 1, D, 40, 6.0, seed=5)
+    roles1 = np.zeros((B, Hkv, n1 // C), dtype=np.uint8)  # all global: every row stays in the cache
+    roles2 = np.zeros((B, Hkv, 1), dtype=np.uint8)
+    cache = NAtSChunkLayerCache(B, Hkv, W, chunk_size=C, device="cuda")
+    st = orc.ChunkCacheOracle(B=B, H=Hkv, W=W, C=C)
+    for roles, lo, hi in ((roles1, 0, n1), (roles2, n1, n1 + n2), (roles2, n1 + n2, n1 + n2 + 1)):
+        n = hi - lo
+        ko, vo = st.update(k[:, :, lo:hi], v[:, :, lo:hi], roles)
+        kk, vv = cache.update(k[:, :, lo:hi].cuda(), v[:, :, lo:hi].cuda(), orc.one_hot_roles(roles).bfloat16().cuda())
+        if lo:
+            qq = q[:, :, lo:hi]
+            if n > 1:
+                want = orc.masked_attention(qq.float(), ko.float(), vo.float(), st.generate_mask(n))
+                got = cache.segment_attention(qq.cuda())
+            else:
+                want = orc.decode_attention(qq, ko, vo, torch.from_numpy(st.valid), st.n_ctx_data + 1).float()
+                got = ops.decode_attention(qq.cuda(), kk, vv, cache.valid_tokens, kk.shape[2])
+            got = got.float().cpu()
+            rms = want.pow(2).mean(-1, keepdim=True).sqrt()
+            assert not ((got - want).abs() > 2e-2 * torch.maximum(rms, want.abs()) + 2e-3).any(), (n, (got - want).abs().max().item())
+        st.post_update(n)
+        cache.post_update(n)
+
+
+def test_two_prefills_on_two_streams_equal_the_serial_results():
+    """Scratch buffers are kept per stream: launches that run side by side on two streams do not share key limits."""
+    from neuralattentionsearch_amd import ops
+    say("prefill on two streams at once")
+    B, Hq, Hkv, D, C, W = 1, 8, 2, 128, 64, 128
+    cases = []
+    for i, L in enumerate((6000, 4100)):
+        g = torch.Generator().manual_seed(20 + i)
+        q = (torch.randn(B, Hq, L, D, generator=g) * 2).bfloat16().cuda()
+        k = (torch.randn(B, Hkv, L, D, generator=g) * 2).bfloat16().cuda()
+        v = torch.randn(B, Hkv, L, D, generator=g).bfloat16().cuda()
+        roles = to_dev(draw_roles(30 + i, B, Hkv, -(-L // C), p=(0.3, 0.3, 0.4)))
+        cases.append((q, k, v, roles))
+    serial = [ops.prefill_attention(q, k, v, r, C, W) for q, k, v, r in cases]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    for rep in range(3):
+        outs = []
+        for st, (q, k, v, r) in zip(streams, cases):
+            st.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(st):
+                for _ in range(4):  # several launches each, so that the two streams overlap
+                    o = ops.prefill_attention(q, k, v, r, C, W)
+                outs.append(o)
+        for st in streams:
+            st.synchronize()
+        for o, want in zip(outs, serial):
+            assert torch.equal(o, want), rep
