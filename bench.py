@@ -1,12 +1,14 @@
 """Benchmark of the NAtS sparse-attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-cpu] [--only prefill|decode|evict|evict_stream|segments|role_step|matvec|llama]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-cpu] [--no-llama] [--only prefill|decode|evict|evict_stream|segments|role_step|matvec|llama]
 
 One step = one pass of a kernel family over one batch of synthetic input that is already resident in HBM:
 
 * prefill  role-masked chunked flash attention at the Llama-3-8B head shape, L = 32768 (the headline)
 * decode   one query token per sequence over the ragged, evicted KV cache (batch 32, context 65536)
 * evict    bulk eviction + compaction of a 16 x 8 x 65536 x 128 cache after its prefill
+* llama_e2e  the three together inside a random-weight Llama-3-8B-shape model: a 16384-token prefill, then 512 greedy
+           one-token steps with eviction live in all 32 layers (seconds for the prefill, ms per token)
 
 Prints ONE JSON line.  `value` is the prefill time in ms; decode tokens/s, GB/s and the compaction GB/s
 ride along in the same line, each with its roofline fraction, next to a CPU baseline (the oracle, timed
@@ -488,6 +490,7 @@ def main():
     ap.add_argument("--segments", type=int, default=4, help="segments of the `--only segments` leg")
     ap.add_argument("--segment-len", type=int, default=0, help="tokens per segment (default: prefill length / segments)")
     ap.add_argument("--only", choices=["prefill", "decode", "evict", "copy", "evict_stream", "segments", "role_step", "matvec", "llama"], default=None)
+    ap.add_argument("--no-llama", action="store_true", help="skip the end-to-end Llama-3-8B-shape leg of the default run")
     ap.add_argument("--llama-prefill", type=int, default=16384)
     ap.add_argument("--llama-decode", type=int, default=512)
     args = ap.parse_args()
@@ -522,8 +525,6 @@ def main():
         res["role_step"] = bench_role_step(args, ops)
     if args.only == "matvec":  # not part of the default run
         res["matvec"] = bench_matvec(args, ops)
-    if args.only == "llama":  # not part of the default run
-        res["llama_e2e"] = bench_llama(args)
     torch.cuda.synchronize()
     cpu = None if args.skip_cpu or args.only in ("evict_stream", "segments", "role_step", "matvec", "llama") else cpu_baseline(args)
 
@@ -555,6 +556,10 @@ def main():
                                   "frac": e["frac_of_hbm_peak"], "traffic": MEASURED_TRAFFIC["evict"],
                                   "kernel": "evict_plan_* + evict_apply_first_kernel (whole post_update)"}
     line["cpu_baseline"] = cpu
+    if args.only in (None, "llama") and not args.no_llama:
+        # the end-to-end workload: last, so that the kernel legs above are timed on a GPU that holds nothing else
+        torch.cuda.empty_cache()
+        res["llama_e2e"] = bench_llama(args)
     line.update(res)
     print(json.dumps(line))
 

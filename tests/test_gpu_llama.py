@@ -171,3 +171,58 @@ def test_fused_role_step_gives_the_same_generation(method, prompt):
         kept.append([l.valid_tokens.sum().item() for l in cache.cache_model])
     assert torch.equal(outs[0], outs[1])
     assert kept[0] == kept[1]
+
+
+def test_full_size_llama3_8b_shape_prefill_16384_and_512_steps():
+    """The end-to-end workload at its full size (32 layers, d_model 4096, 32 / 8 heads, FFN 14336, vocabulary 128256,
+    bf16; 16384 prompt tokens, 512 greedy steps with eviction live), where no oracle run is affordable: properties
+    that hold at any size.  Finite logits; the same tokens from a second run; the same tokens with the role step as
+    torch ops instead of the fused kernel (roles are the argmax of logits that differ in summation order only; the
+    comparison allows the few near-ties of 8 heads x 33 layers x 260 chunks to flip, by bounding how the kept rows
+    differ rather than demanding equal tokens); and in every layer the valid rows are exactly the rows the sizes
+    describe: ring slots flagged valid + global rows + local rows + the open chunk."""
+    from neuralattentionsearch_amd.llama import NAtSLlamaConfig, NAtSLlamaForCausalLM
+    say("llama full size: init")
+    cfg = NAtSLlamaConfig.llama3_8b(fused_role_step=True)
+    model = NAtSLlamaForCausalLM.random_init(cfg, seed=0)
+    W, C, H = cfg.local_seq_max_length, cfg.chunk_size, cfg.num_key_value_heads
+    prompt, steps = 16384, 512
+    ids = torch.randint(0, cfg.vocab_size, (1, prompt), generator=torch.Generator().manual_seed(0)).cuda()
+
+    def check_layers(cache, seen):
+        for li, lc in enumerate(cache.cache_model):
+            assert lc.get_seq_length() == seen
+            n = lc.n_ctx_data
+            valid = lc.valid_tokens[:, :, :n]
+            rows = lc.size_global_kv - W + lc.size_local_kv  # [B, H]
+            want = rows.sum().item() + valid[:, :, :W].sum().item() + lc.chunk_fill_size * H
+            assert valid.sum().item() == want, (li, valid.sum().item(), want)
+            assert n == int((lc.size_global_kv + lc.size_local_kv).max()) + lc.chunk_fill_size, li
+            assert (lc.size_global_kv % C == 0).all() and (lc.size_local_kv % C == 0).all() and (lc.size_local_kv >= 0).all()
+            # a head's own rows are valid, the rows between its end and the open chunk are not
+            per_head = valid[:, :, W:n - lc.chunk_fill_size].sum(-1)
+            assert torch.equal(per_head, rows), li
+
+    say("llama full size: run 1")
+    toks_a, cache_a = model.generate(ids, steps)
+    assert toks_a.shape == (1, steps)
+    logits = model(toks_a[:, -1:], prompt + steps - 1, cache_a)
+    assert torch.isfinite(logits).all() and logits.shape == (1, cfg.vocab_size)
+    check_layers(cache_a, prompt + steps)
+    kept_a = [int(lc.valid_tokens[:, :, :lc.n_ctx_data].sum()) for lc in cache_a.cache_model]
+    assert max(kept_a) < H * (prompt + steps), "nothing was evicted"
+    del cache_a
+    say("llama full size: run 2 (same tokens)")
+    toks_b, cache_b = model.generate(ids, steps)
+    assert torch.equal(toks_a, toks_b)
+    del cache_b
+    say("llama full size: role step as torch ops")
+    for layer in model.layers:
+        layer.self_attn.fused_role_step = False
+    toks_c, cache_c = model.generate(ids, steps)
+    check_layers(cache_c, prompt + steps - 1)
+    kept_c = [int(lc.valid_tokens[:, :, :lc.n_ctx_data].sum()) for lc in cache_c.cache_model]
+    agree = (toks_a == toks_c).float().mean().item()
+    say("llama full size: token agreement fused / unfused role step", agree, "kept", sum(kept_a), sum(kept_c))
+    # layer 0 sees the same hidden states in both runs: its roles agree except at near-ties of bf16 logits
+    assert abs(kept_a[0] - kept_c[0]) <= 0.02 * kept_c[0] + 2 * C * H, (kept_a[0], kept_c[0])
