@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define NATS_ABI_VERSION 6
+#define NATS_ABI_VERSION 7
 
 typedef enum {
   NATS_OK = 0,
@@ -246,6 +246,8 @@ typedef struct {
   int64_t tail;        /* sliding_queue_tail before this call */
   int64_t first;       /* 1 if these are the first tokens the layer has seen (_seen_tokens == x_len) */
   int64_t n_alloc;     /* rows allocated in cache_k / cache_v / valid (in place) or in the new cache (out of place) */
+  int64_t seq;         /* any number the caller chooses; it comes back in nats_evict_result.seq and, its low 32 bits, in
+                          the nats_evict_brief a host may poll (which gives every call a new one) */
   int64_t update_chunk; /* 0: the chunked cache.  U > 0: the per-token cache NAtSLayerCache._post_update
                            (components/cache/nats_layer_cache.py:292-418, 424-458, 556-574, 651-770) once U tokens
                            are pending: C = 1, S = fill = the pending block with one role per token, n_ctx_data = the
@@ -263,17 +265,30 @@ typedef struct {
   int64_t max_keep;    /* largest number of kept chunks over (b, h) */
   int64_t max_end;     /* largest (kept + destination base) over (b, h), in chunks */
   int64_t moved_rows;  /* rows copied by the compaction (both tensors counted once), for bandwidth accounting */
-  int64_t reserved;
+  int64_t seq;         /* params->seq of the call that wrote this result */
 } nats_evict_result;
+
+/* What a host that does not want to synchronise with the stream polls for: 16 bytes that the plan step writes with
+ * one store, meant for pinned host memory.  Whoever reads its own params->seq (its low 32 bits) in `seq` has the rest. */
+typedef struct {
+  int32_t seq;         /* low 32 bits of params->seq of the call that wrote this */
+  int32_t flags;       /* bit 0: all_sw, bit 1: all_local */
+  int32_t n_ctx_data;  /* after the call */
+  int32_t gmin;        /* after the call */
+} nats_evict_brief;
 
 size_t nats_evict_workspace_bytes(int64_t B, int64_t H_kv, int64_t S);
 
 /* Step 1, always: roles -> per-head plan in `workspace`, new sizes and the scalars in `result`.
  *   size_global / size_local [B, H_kv] int64, read here, rewritten by the apply step
+ *   workspace: nats_evict_workspace_bytes(...) bytes (contents need not be kept between calls)
+ *   result_mirror: NULL, or 16 bytes (16-byte aligned) that receive the short form of the result in one store, meant
+ *              for pinned host memory: a host that sees its own params->seq there has n_ctx_data, gmin and the two
+ *              flags without synchronising with the stream
  */
 int nats_evict_plan(const uint8_t* roles, const int64_t* size_global, const int64_t* size_local,
                     const nats_evict_params* params, void* workspace, size_t workspace_bytes, nats_evict_result* result,
-                    void* stream);
+                    nats_evict_brief* result_mirror, void* stream);
 
 /* Step 2a, in place: ring insert, ordered chunk moves (all sources of a batch are read before any of its
  * destinations is written, which equals the reference's gather-clone-then-scatter), zero fill of rows
@@ -299,6 +314,17 @@ int nats_evict_apply_first(const void* src_k, const void* src_v, void* cache_k, 
                            const nats_evict_params* params, const int64_t* src_strides, const int64_t* kv_strides,
                            const int64_t* valid_strides, int elem_bytes, const void* workspace,
                            const nats_evict_result* result, void* stream);
+
+/* The row write of the cache update for a cache that already holds rows (NAtSChunkLayerCache.update,
+ * components/cache/nats_chunk_layer_cache.py:243-256; NAtSLayerCache.update, nats_layer_cache.py:279-284) in one launch:
+ *   cache_k / cache_v[b, h, row0 + l] = k / v[b, h, l],  valid[b, h, row0 + l] = 1,  pos[b, h, row0 + l] = pos0 + l
+ *   k / v [B, H_kv, x_len, D]: strides (b, h, l);  cache_k / cache_v [B, H_kv, n_alloc, D]: strides (b, h, row)
+ *   valid / pos [B, H_kv, n_alloc]: strides (b, h);  pos may be NULL;  rows and strides multiples of 16 bytes
+ */
+int nats_cache_append(const void* k, const void* v, void* cache_k, void* cache_v, uint8_t* valid, int32_t* pos, int64_t B,
+                      int64_t H_kv, int64_t x_len, int64_t D, int64_t row0, int64_t n_alloc, int64_t pos0,
+                      const int64_t* k_strides, const int64_t* v_strides, const int64_t* cache_strides,
+                      const int64_t* valid_strides, int elem_bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
  * Decode-step glue of the HF-shaped caller (models/transformer/hf/llama_nats_chunk.py:171-292 inside a Llama

@@ -19,20 +19,20 @@ c_i64p = ctypes.POINTER(ctypes.c_int64)
 NATS_DTYPE_BF16 = 0
 NATS_DTYPE_F32 = 1
 
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 
 class EvictParams(ctypes.Structure):
     """nats_evict_params"""
     _fields_ = [(n, c_i64) for n in
                 ("B", "H_kv", "D", "C", "W", "S", "x_len", "fill", "n_ctx_data", "gmin", "tail", "first", "n_alloc",
-                 "update_chunk")]
+                 "seq", "update_chunk")]
 
 
 class EvictResult(ctypes.Structure):
     """nats_evict_result (64 bytes)"""
     _fields_ = [(n, c_i64) for n in
-                ("n_ctx_data", "gmin", "all_sw", "all_local", "max_keep", "max_end", "moved_rows", "reserved")]
+                ("n_ctx_data", "gmin", "all_sw", "all_local", "max_keep", "max_end", "moved_rows", "seq")]
 
 
 class PastState(ctypes.Structure):
@@ -68,11 +68,12 @@ SIGNATURES = {
     "nats_decode_fwd_static": (ctypes.c_int, [c_p, c_p, c_p, c_p, c_p, c_i64, c_p, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64p,
                                               c_i64p, ctypes.c_float, ctypes.c_int, c_p]),
     "nats_evict_workspace_bytes": (ctypes.c_size_t, [c_i64] * 3),
-    "nats_evict_plan": (ctypes.c_int, [c_p, c_p, c_p, ctypes.POINTER(EvictParams), c_p, ctypes.c_size_t, c_p, c_p]),
+    "nats_evict_plan": (ctypes.c_int, [c_p, c_p, c_p, ctypes.POINTER(EvictParams), c_p, ctypes.c_size_t, c_p, c_p, c_p]),
     "nats_evict_apply_inplace": (ctypes.c_int, [c_p, c_p, c_p, c_p, c_p, c_p, c_p, ctypes.POINTER(EvictParams), c_i64p,
                                                 c_i64p, ctypes.c_int, c_p, c_p, c_p]),
     "nats_evict_apply_first": (ctypes.c_int, [c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, ctypes.POINTER(EvictParams),
                                               c_i64p, c_i64p, c_i64p, ctypes.c_int, c_p, c_p, c_p]),
+    "nats_cache_append": (ctypes.c_int, [c_p] * 6 + [c_i64] * 7 + [c_i64p] * 4 + [ctypes.c_int, c_p]),
     "nats_add_rms_norm": (ctypes.c_int, [c_p, c_p, c_p, c_p, c_p, c_i64, c_i64, ctypes.c_float, ctypes.c_int, c_i64,
                                          ctypes.c_int, c_p]),
     "nats_silu_mul": (ctypes.c_int, [c_p, c_p, c_i64, c_i64, ctypes.c_int, c_p]),

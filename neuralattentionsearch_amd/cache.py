@@ -9,8 +9,10 @@ monkey-patches can use them unchanged.  What differs is how the state is kept:
   views of the logical rows, whose number equals the reference's ``cache_k.shape[2]`` at every step;
 * the first prefill is not copied into ``[W zeros | K | pad]``: the raw K / V handed to ``update`` are kept
   until ``post_update`` gathers the surviving rows straight into a right-sized cache;
-* ``post_update`` issues two kernels (plan, apply) and reads one 64-byte struct back, instead of the
-  reference's gather / scatter ops with six device-to-host synchronisations.
+* ``post_update`` issues two kernels (plan, apply) instead of the reference's gather / scatter ops with six
+  device-to-host synchronisations; the plan kernel leaves its 64-byte result (new n_ctx_data, minimum global size)
+  in pinned host memory as well, and the host picks it up when it next needs those numbers (the next update of that
+  layer, an attribute read), without a stream synchronisation.
 """
 from __future__ import annotations
 
@@ -69,28 +71,136 @@ class NAtSChunkLayerCache:
         self.n_chunks_per_sw = sliding_window_size // chunk_size
         self.device = device
         self.track_positions = track_positions
-        self.size_local_kv = torch.zeros(bsz, n_msks, device=device, dtype=torch.long)
-        self.size_global_kv = torch.full([bsz, n_msks], sliding_window_size, device=device, dtype=torch.long)
+        # (the two size tensors are halves of one, so that a reset is one small copy)
+        self._sizes = torch.empty(2, bsz, n_msks, device=device, dtype=torch.long)
+        self._sizes_init = torch.zeros(2, bsz, n_msks, device=device, dtype=torch.long)
+        self._sizes_init[0] = sliding_window_size
+        self.size_global_kv, self.size_local_kv = self._sizes[0], self._sizes[1]
         self._row_end = None  # size_global_kv + size_local_kv, kept between evictions
+        self._evict = None    # ops.EvictBuffers, made by the first eviction
+        self._await = None    # (sequence number, first) of an eviction whose scalars the host has not picked up yet
+        self._redo = None     # what a first eviction launched on a guessed capacity needs if the guess was too small
+        self._kept_share = None  # logical rows after the last first eviction / rows of the uncompacted cache
         self.reset_cache()
 
     # -- state ----------------------------------------------------------------------------------
     def reset_cache(self):
-        self.size_local_kv.zero_()
-        self.size_global_kv.fill_(self.sliding_window_size)
+        self._await = self._redo = None  # (a result still on its way belongs to the state that is dropped here)
+        torch.add(self._sizes_init, 0, out=self._sizes)  # (a kernel; a tensor copy would go through the runtime's copy path)
         self._row_end = None
         self.sliding_queue_tail = 0
         self.chunk_fill_size = 0
         self.chunk_fill_size_last = 0
-        self.n_ctx_data = self.sliding_window_size
-        self._n_global_min = self.sliding_window_size
+        self._n_ctx = self.sliding_window_size
+        self._gmin = self.sliding_window_size
         self._seen_tokens = 0
         self._tokens_info = None
         self._roles = None
         self._buf_k = self._buf_v = self._buf_valid = self._buf_pos = None
-        self._rows = 0
+        self._n_rows = 0
         self._pending = None  # raw (K, V) of a first prefill not yet compacted
-        self.last_evict_result = None
+        self._last_result = None
+
+    # The scalars an eviction computes on the device (n_ctx_data, the minimum global size, through them the number of
+    # logical rows after a first update) reach the host lazily: `post_update` only notes that they are on their way.
+    def _resolve(self):
+        if self._await is None:
+            return
+        seq, first = self._await
+        self._await = None
+        res = self._evict.wait(seq)
+        redo, self._redo = self._redo, None
+        if redo is not None:
+            # a first eviction that was launched into a cache of guessed capacity
+            src, roles, params, ws, result, full = redo
+            if res.all_sw:
+                # the kernel left everything alone: the reference keeps the uncompacted cache here and works in place
+                self._buf_k = self._buf_v = self._buf_valid = self._buf_pos = None
+                self._n_rows = 0
+                self._pending = src
+                self._materialize_pending()
+                params.n_alloc = self._n_rows
+                ops.evict_apply_inplace(self._buf_k, self._buf_v, self._buf_valid, self._buf_pos, roles, self.size_global_kv,
+                                        self.size_local_kv, params, ws, result)
+            else:
+                rows = self._logical_rows(int(res.n_ctx_data))
+                self._kept_share = rows / full
+                if rows > self._buf_k.shape[2]:  # the guess was too small: once more, at the right size
+                    self._launch_first(src, roles, params, ws, result, rows)
+        self._take_result(res, first)
+
+    def _logical_rows(self, n_ctx: int) -> int:
+        """Rows the reference's cache tensors have after a first eviction that left n_ctx live rows (:373-380)."""
+        return math.ceil(n_ctx / self.chunk_size) * self.chunk_size
+
+    def _full_rows(self, x_len: int) -> int:
+        """Rows of [W zeros | K | pad] (:215-236)."""
+        return self.sliding_window_size + x_len + get_pad_size(x_len, self.chunk_size)
+
+    def _launch_first(self, src, roles, params, ws, result, rows: int):
+        """The out-of-place eviction of a first prefill into a fresh cache of `rows` rows."""
+        k_raw, v_raw = src
+        self._pending = None
+        self._allocate(rows, k_raw, zero=False)  # the apply kernel writes all rows
+        params.n_alloc = rows
+        if k_raw.stride(-1) != 1 or ops.strides_differ(k_raw, v_raw):
+            k_raw, v_raw = k_raw.contiguous(), v_raw.contiguous()
+        ops.evict_apply_first(k_raw, v_raw, self._buf_k, self._buf_v, self._buf_valid, self._buf_pos, roles,
+                              self.size_global_kv, self.size_local_kv, params, ws, result)
+
+    def _evict_first(self, src, roles, params, ws, result, first: bool):
+        """The eviction of a first prefill that is still raw K / V.  The size of the compacted cache is a result of
+        the plan kernel.  A cache that has been through a first eviction before (and was reset) allocates on the
+        share of rows it kept then, with some room, launches at once and checks the guess when the plan's numbers
+        arrive; otherwise the host waits for them.  Returns False if the eviction has to run in place instead."""
+        full = self._full_rows(src[0].shape[2])
+        if self._kept_share is not None:
+            C = self.chunk_size
+            cap = min(full, math.ceil((full * min(1.0, self._kept_share * 1.0625) + 2 * C) / C) * C)
+            self._launch_first(src, roles, params, ws, result, cap)
+            self._redo = (src, roles, params, ws, result, full)
+            self._await = (params.seq, first)
+            return True
+        res = self._evict.wait(params.seq)
+        if res.all_sw:  # the reference keeps the untruncated cache here (:283-288)
+            self._materialize_pending()
+            return False
+        rows = self._logical_rows(int(res.n_ctx_data))
+        self._kept_share = rows / full
+        self._launch_first(src, roles, params, ws, result, rows)
+        self._take_result(res, first)
+        return True
+
+    def _take_result(self, res, first: bool):
+        """nats_chunk_layer_cache.py:283-288, 358, 371-380 on the numbers of the plan kernel."""
+        self._last_result = res
+        self._n_ctx = int(res.n_ctx_data)
+        if res.all_sw:
+            return
+        self._gmin = int(res.gmin)
+        if first:
+            self._n_rows = math.ceil(self._n_ctx / self.chunk_size) * self.chunk_size
+
+    def _lazy(name):  # noqa: N805 -- a host scalar that a pending eviction result may still change
+        def get(self):
+            self._resolve()
+            return getattr(self, name)
+
+        def put(self, value):
+            self._resolve()
+            setattr(self, name, value)
+        return property(get, put)
+
+    n_ctx_data = _lazy("_n_ctx")
+    _n_global_min = _lazy("_gmin")
+    _rows = _lazy("_n_rows")
+    del _lazy
+
+    @property
+    def last_evict_result(self):
+        """All numbers of the last eviction's plan (nats_evict_result), read from device memory."""
+        self._resolve()
+        return None if self._last_result is None else self._evict.full_result()
 
     def get_seq_length(self):
         return self._seen_tokens
@@ -202,13 +312,22 @@ class NAtSChunkLayerCache:
         start = self.n_ctx_data
         end = start + x_len
         self._grow(math.ceil(end / self.chunk_size) * self.chunk_size)
+        self._write_rows(key_states, value_states, start, end)
+        return self._buf_k[:, :, :end], self._buf_v[:, :, :end]
+
+    def _write_rows(self, key_states, value_states, start: int, end: int):
+        """Rows [start, end) of the cache, their valid bytes and stream positions: one kernel where the layouts
+        allow 16-byte accesses, slice assignments otherwise."""
+        if ops.cache_append_ok(key_states, value_states, self._buf_k, self._buf_v):
+            ops.cache_append(key_states, value_states, self._buf_k, self._buf_v, self._buf_valid, self._buf_pos, start,
+                             self._seen_tokens)
+            return
         self._buf_k[:, :, start:end] = key_states.to(self._buf_k.dtype)
         self._buf_v[:, :, start:end] = value_states.to(self._buf_v.dtype)
         self._buf_valid[:, :, start:end] = 1
         if self._buf_pos is not None:
-            self._buf_pos[:, :, start:end] = torch.arange(self._seen_tokens, self._seen_tokens + x_len,
+            self._buf_pos[:, :, start:end] = torch.arange(self._seen_tokens, self._seen_tokens + end - start,
                                                           dtype=torch.int32, device=self.device)
-        return self._buf_k[:, :, :end], self._buf_v[:, :, :end]
 
     def append_rotated(self, q: torch.Tensor, key_states: torch.Tensor, value_states: torch.Tensor, cos: torch.Tensor,
                        sin: torch.Tensor, token_states_info: torch.Tensor | None = None,
@@ -297,42 +416,22 @@ class NAtSChunkLayerCache:
         src = self._pending
         like = src[0] if src is not None else self._buf_k
         D = like.shape[3]
+        if self._evict is None:
+            self._evict = ops.EvictBuffers(self.device)
         params = ops.evict_params(self.bsz, self.n_msks, D, C, W, S, x_len, fill, self.n_ctx_data, self._n_global_min,
                                   self.sliding_queue_tail, first, max(self._rows, C))
-        ws, result = ops.evict_plan(roles, self.size_global_kv, self.size_local_kv, params)
-        if src is not None:
-            res = ops.read_result(result)
-            if res.all_sw:  # the reference keeps the untruncated cache here (:283-288)
-                self._materialize_pending()
-                src = None
-            else:
-                rows = math.ceil(res.n_ctx_data / C) * C
-                self._pending = None
-                self._allocate(rows, like, zero=False)  # the apply kernel writes all rows
-                params.n_alloc = rows
-                k_raw, v_raw = src
-                if k_raw.stride(-1) != 1 or ops.strides_differ(k_raw, v_raw):
-                    k_raw, v_raw = k_raw.contiguous(), v_raw.contiguous()
-                ops.evict_apply_first(k_raw, v_raw, self._buf_k, self._buf_v, self._buf_valid, self._buf_pos, roles,
-                                      self.size_global_kv, self.size_local_kv, params, ws, result)
-        if src is None:
+        ws, result = ops.evict_plan(roles, self.size_global_kv, self.size_local_kv, params, self._evict)
+        if src is None or not self._evict_first(src, roles, params, ws, result, first):
             params.n_alloc = self._rows
             ops.evict_apply_inplace(self._buf_k, self._buf_v, self._buf_valid, self._buf_pos, roles, self.size_global_kv,
                                     self.size_local_kv, params, ws, result)
-            res = ops.read_result(result)
-        # host-side bookkeeping (nats_chunk_layer_cache.py:400-413, 280-288, 358, 371-380)
+            self._await = (params.seq, first)  # picked up when the host next needs n_ctx_data or the minimum global size
+        # host-side bookkeeping (nats_chunk_layer_cache.py:400-413)
         n_ring = min(n_done, self.n_chunks_per_sw)
         start = 0 if first else self.sliding_queue_tail
         self.sliding_queue_tail = (start + n_ring * C) % W
         self.chunk_fill_size = partial
         self.chunk_fill_size_last = partial
-        self.n_ctx_data = int(res.n_ctx_data)
-        self.last_evict_result = res
-        if res.all_sw:
-            return
-        self._n_global_min = int(res.gmin)
-        if first:
-            self._rows = math.ceil(self.n_ctx_data / C) * C
 
 
 class NAtSLayerCache(NAtSChunkLayerCache):
@@ -391,6 +490,12 @@ class NAtSLayerCache(NAtSChunkLayerCache):
     def _grow(self, rows: int):
         super()._grow(self._pad_rows(rows))
 
+    def _logical_rows(self, n_ctx: int) -> int:
+        return n_ctx  # the first eviction cuts the cache to its live rows (:404-408)
+
+    def _full_rows(self, x_len: int) -> int:
+        return self.sliding_window_size + self._pad_rows(x_len)
+
     def _note_roles(self, token_states_info, roles):
         """Roles of the new tokens join the pending block."""
         U = self.update_chunk_size
@@ -431,12 +536,7 @@ class NAtSLayerCache(NAtSChunkLayerCache):
         start = self.n_ctx_data
         end = start + x_len
         self._grow(end)
-        self._buf_k[:, :, start:end] = key_states.to(self._buf_k.dtype)
-        self._buf_v[:, :, start:end] = value_states.to(self._buf_v.dtype)
-        self._buf_valid[:, :, start:end] = 1
-        if self._buf_pos is not None:
-            self._buf_pos[:, :, start:end] = torch.arange(self._seen_tokens, self._seen_tokens + x_len,
-                                                          dtype=torch.int32, device=self.device)
+        self._write_rows(key_states, value_states, start, end)
         return self._buf_k[:, :, :end], self._buf_v[:, :, :end]
 
     def append_rotated(self, q, key_states, value_states, cos, sin, token_states_info=None, roles=None):
@@ -482,7 +582,20 @@ class NAtSLayerCache(NAtSChunkLayerCache):
         """(row_end, tail_start) for `ops.decode_attention` after the update of a one-token step: rows
         [row_end[b, h], tail_start) hold nothing valid.  Pending blocks start where the last eviction that moved rows
         left n_ctx_data (blocks of sliding-window tokens stay where they were, still valid)."""
+        self._resolve()
         return self.row_end(), min(self._live_end, self.n_ctx_data)
+
+    def _take_result(self, res, first: bool):
+        """nats_layer_cache.py:316-327, 394, 402-408 on the numbers of the plan kernel (`first`: the call held every
+        token seen so far, so the cache is cut to its live rows)."""
+        self._last_result = res
+        if res.all_sw:
+            return  # n_ctx_data stays: the block's rows remain where they are, valid
+        self._n_ctx = int(res.n_ctx_data)
+        self._live_end = self._n_ctx
+        self._gmin = int(res.gmin)
+        if first:
+            self._n_rows = self._n_ctx
 
     # -- evict + compact (nats_layer_cache.py:292-418) ---------------------------------------------
     def post_update(self, x_len: int):
@@ -506,43 +619,22 @@ class NAtSLayerCache(NAtSChunkLayerCache):
         src = self._pending
         like = src[0] if src is not None else self._buf_k
         D = like.shape[3]
+        if self._evict is None:
+            self._evict = ops.EvictBuffers(self.device)
         params = ops.evict_params(self.bsz, self.n_msks, D, 1, W, fill, x_len, fill, block_start, self._n_global_min,
-                                  self.sliding_queue_tail, first_ring, max(self._rows, 1), U)
-        ws, result = ops.evict_plan(roles, self.size_global_kv, self.size_local_kv, params)
+                                  self.sliding_queue_tail, first_ring, max(self._rows, 1), update_chunk=U)
+        ws, result = ops.evict_plan(roles, self.size_global_kv, self.size_local_kv, params, self._evict)
         self._row_end = None
-        if src is not None:
-            res = ops.read_result(result)
-            if res.all_sw:  # the reference keeps the untruncated cache here (:316-327)
-                self._materialize_pending()
-                src = None
-            else:
-                rows = int(res.n_ctx_data)
-                self._pending = None
-                self._allocate(rows, like, zero=False)  # the apply kernel writes all rows
-                params.n_alloc = rows
-                k_raw, v_raw = src
-                if k_raw.stride(-1) != 1 or ops.strides_differ(k_raw, v_raw):
-                    k_raw, v_raw = k_raw.contiguous(), v_raw.contiguous()
-                ops.evict_apply_first(k_raw, v_raw, self._buf_k, self._buf_v, self._buf_valid, self._buf_pos, roles,
-                                      self.size_global_kv, self.size_local_kv, params, ws, result)
-        if src is None:
+        if src is None or not self._evict_first(src, roles, params, ws, result, first_call):
             params.n_alloc = self._rows
             ops.evict_apply_inplace(self._buf_k, self._buf_v, self._buf_valid, self._buf_pos, roles, self.size_global_kv,
                                     self.size_local_kv, params, ws, result)
-            res = ops.read_result(result)
+            self._await = (params.seq, first_call)  # picked up when the host next needs n_ctx_data
         n_ring = min(fill, W)  # :437-445
         self.sliding_queue_tail = n_ring - 1 if first_ring else (self.sliding_queue_tail + n_ring) % W
         self.chunk_fill_size = 0
         self.chunk_fill_size_last = 0
-        self.last_evict_result = res
         self._block = self._roles = None
-        if res.all_sw:
-            return  # n_ctx_data stays: the block's rows remain where they are, valid
-        self.n_ctx_data = int(res.n_ctx_data)
-        self._live_end = self.n_ctx_data
-        self._n_global_min = int(res.gmin)
-        if first_call:
-            self._rows = self.n_ctx_data
 
 
 try:  # the reference's container is a transformers cache (dyn_cache.py:66): HF models take it as past_key_values

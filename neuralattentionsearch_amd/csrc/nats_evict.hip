@@ -22,6 +22,8 @@
 //                produced independently straight from the raw K / V of the prefill.
 #include "nats_common.h"
 
+#include <stddef.h>
+
 namespace nats {
 
 struct HeadPlan {
@@ -75,14 +77,10 @@ __device__ __forceinline__ void load_roles(const uint8_t* __restrict__ r, int S,
   }
 }
 
-__global__ __launch_bounds__(256) void evict_plan_heads_kernel(const uint8_t* __restrict__ roles,
-                                                               const int64_t* __restrict__ size_global,
-                                                               const int64_t* __restrict__ size_local,
-                                                               nats_evict_params p, char* __restrict__ ws) {
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+__device__ __forceinline__ void plan_one_head(const uint8_t* __restrict__ roles, const int64_t* __restrict__ size_global,
+                                              const int64_t* __restrict__ size_local, const nats_evict_params& p,
+                                              char* __restrict__ ws, int head, int lane) {
   const int n_heads = (int)(p.B * p.H_kv);
-  const int head = blockIdx.x * 4 + wave;
-  if (head >= n_heads) return;
   const int S = (int)p.S;
   const int C = (int)p.C;
   const int partial = (int)(p.fill % p.C);
@@ -161,6 +159,63 @@ __global__ __launch_bounds__(256) void evict_plan_heads_kernel(const uint8_t* __
   if (lane == 0) plans[head] = hp;
 }
 
+// The same plan for a head with few role slots, computed by one lane on its own (no wave-wide steps), so that a
+// workgroup plans 256 heads side by side.
+__device__ __forceinline__ void plan_one_head_serial(const uint8_t* __restrict__ roles, const int64_t* __restrict__ size_global,
+                                                     const int64_t* __restrict__ size_local, const nats_evict_params& p,
+                                                     char* __restrict__ ws, int head) {
+  const int n_heads = (int)(p.B * p.H_kv);
+  const int S = (int)p.S;
+  const int C = (int)p.C;
+  const int partial = (int)(p.fill % p.C);
+  const int n_done = (int)(p.fill / p.C);
+  const int S_eff = S - (partial ? 1 : 0);
+  HeadPlan* plans = reinterpret_cast<HeadPlan*>(ws + kPlanHeaderBytes);
+  int32_t* keep = reinterpret_cast<int32_t*>(ws + plan_lists_offset(n_heads)) + (int64_t)head * S;
+  const uint8_t* r = roles + (int64_t)head * S;
+  const long long sg = size_global[head], sl = size_local[head];
+  HeadPlan hp;
+  if (p.x_len == 1 && !p.update_chunk) {
+    int r0 = r[0], rl = r[S - 1];
+    bool is_g = r0 == NATS_ROLE_GLOBAL;
+    long long dst = is_g ? sg : sg + sl;
+    long long dec = (is_g ? sl / C + 1 : 0) + (rl == NATS_ROLE_SW ? 1 : 0);
+    hp.count = 1;
+    hp.dst_base = (int32_t)(dst / C);
+    hp.sg_new = sg + (is_g ? C : 0);
+    hp.sl_new = sl - dec * C + (long long)n_done * C;
+    hp.all_sw = r0 == NATS_ROLE_SW;
+    hp.all_local = 0;
+    keep[0] = 0;
+  } else {
+    int n_glob_all = 0, n_sw = 0, n_loc = 0, last_g = -1;
+    for (int s2 = 0; s2 < S; ++s2) {
+      const int role = r[s2];
+      n_glob_all += role == NATS_ROLE_GLOBAL;
+      n_sw += role == NATS_ROLE_SW;
+      n_loc += role == NATS_ROLE_LOCAL;
+      if (role == NATS_ROLE_GLOBAL && s2 < S_eff) last_g = s2;
+    }
+    int count = 0, later_local = 0;
+    for (int s2 = 0; s2 < S; ++s2) {
+      const int role = r[s2];
+      const bool la = role == NATS_ROLE_LOCAL && s2 > last_g;
+      later_local += la;
+      if (s2 < S_eff && (role == NATS_ROLE_GLOBAL || la)) keep[count++] = s2;
+    }
+    int n_glob = n_glob_all - (partial ? 1 : 0);
+    long long n_other = (long long)S - (last_g > 0 ? last_g : 0) - later_local - (partial ? 1 : 0);
+    long long dec_l = (last_g > -1 ? (long long)last_g * C + sl : 0) + n_other * C;
+    hp.count = count;
+    hp.dst_base = (int32_t)((last_g == -1 ? sg + sl : sg) / C);
+    hp.sg_new = sg + (long long)n_glob * C;
+    hp.sl_new = sl - dec_l + (long long)n_done * C;
+    hp.all_sw = n_sw == S;
+    hp.all_local = n_loc == S;
+  }
+  plans[head] = hp;
+}
+
 // plan, step 2: one workgroup folds the per-head plans into the global decisions and scalars.
 struct PlanAgg {
   int all_sw, all_local;
@@ -181,10 +236,10 @@ __device__ __forceinline__ void fold(PlanAgg& a, const PlanAgg& b) {
   a.sum_keep += b.sum_keep;
 }
 
-__global__ __launch_bounds__(256) void evict_plan_finalize_kernel(const int64_t* __restrict__ size_global,
-                                                                  const int64_t* __restrict__ size_local,
-                                                                  nats_evict_params p, char* __restrict__ ws,
-                                                                  nats_evict_result* __restrict__ result) {
+__device__ __forceinline__ void plan_finalize(const int64_t* __restrict__ size_global, const int64_t* __restrict__ size_local,
+                                              const nats_evict_params& p, char* __restrict__ ws,
+                                              nats_evict_result* __restrict__ result,
+                                              nats_evict_brief* __restrict__ result_mirror) {
   __shared__ PlanAgg agg[256];
   __shared__ int all_local_flag;
   const int tid = threadIdx.x;
@@ -222,7 +277,7 @@ __global__ __launch_bounds__(256) void evict_plan_finalize_kernel(const int64_t*
     res.all_local = (p.x_len != 1 || p.update_chunk) && t.all_local && !t.all_sw;
     res.max_keep = t.max_keep;
     res.max_end = t.max_end;
-    res.reserved = 0;
+    res.seq = p.seq;
     if (res.all_sw) {  // :283-288; the per-token cache keeps the block where it is (nats_layer_cache.py:316-327)
       res.n_ctx_data = p.update_chunk ? p.n_ctx_data + p.fill : t.max_tot_old + partial;
       res.gmin = p.gmin;
@@ -238,6 +293,16 @@ __global__ __launch_bounds__(256) void evict_plan_finalize_kernel(const int64_t*
       res.moved_rows = (t.sum_keep + (tail_move ? n_heads : 0)) * (long long)C;
     }
     *result = res;
+    if (result_mirror) {
+      // what a host may be polling for (pinned memory): one 16-byte store, so that whoever sees the sequence number
+      // sees the rest with it and no fence has to order several stores
+      nats_evict_brief m;
+      m.seq = (int32_t)p.seq;
+      m.flags = (int32_t)(res.all_sw | (res.all_local << 1));
+      m.n_ctx_data = (int32_t)res.n_ctx_data;
+      m.gmin = (int32_t)res.gmin;
+      *reinterpret_cast<uint4*>(result_mirror) = *reinterpret_cast<const uint4*>(&m);
+    }
     all_local_flag = (int)res.all_local;
   }
   __syncthreads();
@@ -248,6 +313,36 @@ __global__ __launch_bounds__(256) void evict_plan_finalize_kernel(const int64_t*
       plans[h].sl_new = size_local[h] + (long long)n_done * C;
     }
   }
+}
+
+// Few role slots per head (a chunk boundary while decoding or streaming): one workgroup, a lane per head, folds the
+// heads itself, so that nothing has to cross workgroups.
+__global__ __launch_bounds__(256) void evict_plan_small_kernel(const uint8_t* __restrict__ roles,
+                                                               const int64_t* __restrict__ size_global,
+                                                               const int64_t* __restrict__ size_local, nats_evict_params p,
+                                                               char* __restrict__ ws, nats_evict_result* __restrict__ result,
+                                                               nats_evict_brief* __restrict__ result_mirror) {
+  const int n_heads = (int)(p.B * p.H_kv);
+  for (int head = threadIdx.x; head < n_heads; head += 256) plan_one_head_serial(roles, size_global, size_local, p, ws, head);
+  __syncthreads();  // (global writes of this workgroup are visible to it after the barrier)
+  plan_finalize(size_global, size_local, p, ws, result, result_mirror);
+}
+
+// Many role bytes (a prefill): a wavefront per head over the whole device, then one workgroup folds the heads.
+__global__ __launch_bounds__(256) void evict_plan_heads_kernel(const uint8_t* __restrict__ roles,
+                                                               const int64_t* __restrict__ size_global,
+                                                               const int64_t* __restrict__ size_local, nats_evict_params p,
+                                                               char* __restrict__ ws) {
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int head = blockIdx.x * 4 + wave;
+  if (head < (int)(p.B * p.H_kv)) plan_one_head(roles, size_global, size_local, p, ws, head, lane);
+}
+
+__global__ __launch_bounds__(256) void evict_plan_finalize_kernel(const int64_t* __restrict__ size_global,
+                                                                  const int64_t* __restrict__ size_local, nats_evict_params p,
+                                                                  char* __restrict__ ws, nats_evict_result* __restrict__ result,
+                                                                  nats_evict_brief* __restrict__ result_mirror) {
+  plan_finalize(size_global, size_local, p, ws, result, result_mirror);
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -521,6 +616,8 @@ __global__ __launch_bounds__(256) void evict_apply_first_kernel(ApplyArgs a) {
             v = 1;
           }
         }
+        // rows of a cache that was allocated with room to spare, beyond what the reference's tensors hold
+        if (i >= (res.n_ctx_data + C - 1) / C * C) v = 0;
       }
       vrow[i] = v;
     }
@@ -530,6 +627,36 @@ __global__ __launch_bounds__(256) void evict_apply_first_kernel(ApplyArgs a) {
     }
   }
   }  // chunks of this workgroup
+}
+
+// Rows of new keys / values into the cache, 16 bytes per lane, with their valid bytes and stream positions.
+struct AppendArgs {
+  const void* src[2];
+  void* dst[2];
+  uint8_t* valid;
+  int32_t* pos;
+  int64_t ss[2][3];  // strides (b, h, l) of k and of v, in 16-byte units
+  int64_t ds[3];     // cache strides (b, h, row), in 16-byte units
+  int64_t vs_b, vs_h;
+  int64_t row0, pos0;
+  int x_len, upr, H_kv;
+};
+
+__global__ __launch_bounds__(256) void cache_append_kernel(AppendArgs a) {
+  const int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int head = blockIdx.y, which = blockIdx.z;
+  const int b = head / a.H_kv, h = head % a.H_kv;
+  const int64_t l = u / a.upr;
+  const int col = (int)(u % a.upr);
+  if (l >= a.x_len) return;
+  const uint4* src = static_cast<const uint4*>(a.src[which]) + b * a.ss[which][0] + h * a.ss[which][1] + l * a.ss[which][2] + col;
+  uint4* dst = static_cast<uint4*>(a.dst[which]) + b * a.ds[0] + h * a.ds[1] + (a.row0 + l) * a.ds[2] + col;
+  *dst = *src;
+  if (which == 0 && col == 0) {
+    const int64_t at = b * a.vs_b + h * a.vs_h + a.row0 + l;
+    a.valid[at] = 1;
+    if (a.pos) a.pos[at] = (int32_t)(a.pos0 + l);
+  }
 }
 
 static int check_params(const char* who, const nats_evict_params* p) {
@@ -565,7 +692,7 @@ extern "C" size_t nats_evict_workspace_bytes(int64_t B, int64_t H_kv, int64_t S)
 
 extern "C" int nats_evict_plan(const uint8_t* roles, const int64_t* size_global, const int64_t* size_local,
                                const nats_evict_params* params, void* workspace, size_t workspace_bytes,
-                               nats_evict_result* result, void* stream) {
+                               nats_evict_result* result, nats_evict_brief* result_mirror, void* stream) {
   NATS_REQUIRE(roles && size_global && size_local && workspace && result, NATS_ERR_NULL_POINTER,
                "nats_evict_plan: NULL pointer argument");
   if (int rc = check_params("nats_evict_plan", params)) return rc;
@@ -573,11 +700,17 @@ extern "C" int nats_evict_plan(const uint8_t* roles, const int64_t* size_global,
   NATS_REQUIRE(workspace_bytes >= need, NATS_ERR_WORKSPACE, "nats_evict_plan: workspace %zu bytes < %zu", workspace_bytes, need);
   hipStream_t st = static_cast<hipStream_t>(stream);
   const unsigned n_wg = (unsigned)((params->B * params->H_kv + 3) / 4);
+  if (params->S <= 32 && params->B * params->H_kv <= 4096) {
+    hipLaunchKernelGGL(evict_plan_small_kernel, dim3(1), dim3(256), 0, st, roles, size_global, size_local, *params,
+                       static_cast<char*>(workspace), result, result_mirror);
+    NATS_CHECK_LAUNCH("evict_plan_small_kernel");
+    return NATS_OK;
+  }
   hipLaunchKernelGGL(evict_plan_heads_kernel, dim3(n_wg), dim3(256), 0, st, roles, size_global, size_local, *params,
                      static_cast<char*>(workspace));
   NATS_CHECK_LAUNCH("evict_plan_heads_kernel");
   hipLaunchKernelGGL(evict_plan_finalize_kernel, dim3(1), dim3(256), 0, st, size_global, size_local, *params,
-                     static_cast<char*>(workspace), result);
+                     static_cast<char*>(workspace), result, result_mirror);
   NATS_CHECK_LAUNCH("evict_plan_finalize_kernel");
   return NATS_OK;
 }
@@ -666,5 +799,43 @@ extern "C" int nats_evict_apply_first(const void* src_k, const void* src_v, void
   dim3 grid((unsigned)((a.n_chunks + a.chunks_per_wg - 1) / a.chunks_per_wg), (unsigned)(params->B * params->H_kv), pos ? 3u : 2u);
   hipLaunchKernelGGL(evict_apply_first_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream), a);
   NATS_CHECK_LAUNCH("evict_apply_first_kernel");
+  return NATS_OK;
+}
+
+extern "C" int nats_cache_append(const void* k, const void* v, void* cache_k, void* cache_v, uint8_t* valid, int32_t* pos,
+                                 int64_t B, int64_t H_kv, int64_t x_len, int64_t D, int64_t row0, int64_t n_alloc, int64_t pos0,
+                                 const int64_t* k_strides, const int64_t* v_strides, const int64_t* cache_strides,
+                                 const int64_t* valid_strides, int elem_bytes, void* stream) {
+  const char* who = "nats_cache_append";
+  NATS_REQUIRE(k && v && cache_k && cache_v && valid, NATS_ERR_NULL_POINTER, "%s: NULL pointer argument", who);
+  NATS_REQUIRE(k_strides && v_strides && cache_strides && valid_strides, NATS_ERR_NULL_POINTER, "%s: NULL stride array", who);
+  NATS_REQUIRE(B > 0 && H_kv > 0 && x_len > 0 && D > 0 && B * H_kv <= 65535, NATS_ERR_BAD_SHAPE,
+               "%s: B=%lld H_kv=%lld x_len=%lld D=%lld", who, (long long)B, (long long)H_kv, (long long)x_len, (long long)D);
+  NATS_REQUIRE(row0 >= 0 && row0 + x_len <= n_alloc, NATS_ERR_BAD_SHAPE, "%s: rows [%lld, %lld) of %lld", who,
+               (long long)row0, (long long)(row0 + x_len), (long long)n_alloc);
+  NATS_REQUIRE(elem_bytes == 2 || elem_bytes == 4, NATS_ERR_BAD_DTYPE, "%s: element size %d", who, elem_bytes);
+  NATS_REQUIRE((D * elem_bytes) % 16 == 0, NATS_ERR_UNSUPPORTED, "%s: row of %lld bytes", who, (long long)(D * elem_bytes));
+  AppendArgs a;
+  for (int i = 0; i < 3; ++i) {
+    NATS_REQUIRE((k_strides[i] * elem_bytes) % 16 == 0 && (v_strides[i] * elem_bytes) % 16 == 0 &&
+                     (cache_strides[i] * elem_bytes) % 16 == 0,
+                 NATS_ERR_BAD_SHAPE, "%s: rows must be 16-byte aligned", who);
+    a.ss[0][i] = k_strides[i] * elem_bytes / 16;
+    a.ss[1][i] = v_strides[i] * elem_bytes / 16;
+    a.ds[i] = cache_strides[i] * elem_bytes / 16;
+  }
+  NATS_REQUIRE((reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) | reinterpret_cast<uintptr_t>(cache_k) |
+                reinterpret_cast<uintptr_t>(cache_v)) % 16 == 0,
+               NATS_ERR_BAD_SHAPE, "%s: tensors must be 16-byte aligned", who);
+  a.src[0] = k; a.src[1] = v; a.dst[0] = cache_k; a.dst[1] = cache_v;
+  a.valid = valid; a.pos = pos;
+  a.vs_b = valid_strides[0]; a.vs_h = valid_strides[1];
+  a.row0 = row0; a.pos0 = pos0;
+  a.x_len = (int)x_len; a.upr = (int)(D * elem_bytes / 16); a.H_kv = (int)H_kv;
+  const int64_t units = x_len * a.upr;
+  NATS_REQUIRE(units < (int64_t(1) << 38), NATS_ERR_BAD_SHAPE, "%s: too many rows", who);
+  dim3 grid((unsigned)((units + 255) / 256), (unsigned)(B * H_kv), 2u);
+  hipLaunchKernelGGL(cache_append_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream), a);
+  NATS_CHECK_LAUNCH("cache_append_kernel");
   return NATS_OK;
 }

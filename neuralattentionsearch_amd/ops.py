@@ -6,6 +6,7 @@ ops: CPU tensors are rejected.
 """
 from __future__ import annotations
 
+import collections
 import ctypes
 import math
 import weakref
@@ -14,6 +15,8 @@ import torch
 
 from . import _lib
 from ._lib import NATS_DTYPE_BF16, NATS_DTYPE_F32, EvictParams, EvictResult, PastState, check, i64_array
+
+EvictBrief = collections.namedtuple("EvictBrief", "n_ctx_data gmin all_sw all_local")  # nats_evict_brief without its seq
 
 ROLE_GLOBAL, ROLE_LOCAL, ROLE_SW = 0, 1, 2
 TILE = 64
@@ -91,6 +94,8 @@ def roles_from_logits(logits: torch.Tensor, global_bias: float = 0.1, force_firs
     check(lib.nats_roles_from_logits(_ptr(logits), _dtype_code(logits), B, S, H, float(global_bias),
                                      int(force_first_global), int(force_last_global), _ptr(roles), _ptr(one_hot),
                                      _stream(logits)))
+    if one_hot is not None:
+        one_hot.nats_roles = roles  # whoever receives only the one-hot tensor finds the compact form on it
     return roles, one_hot
 
 
@@ -139,12 +144,18 @@ def role_step(x: torch.Tensor, weight: torch.Tensor, chunk_size: int, window: in
                              int(merge_max), float(global_bias), int(force_first_global), i64_array(x.stride()[:2]),
                              _ptr(roles), _ptr(one_hot), _ptr(logits), _ptr(carry), _ptr(end_idx), _ptr(vis_lim),
                              _stream(x)))
+    if one_hot is not None:
+        one_hot.nats_roles = roles
     return {"roles": roles, "token_states_info": one_hot, "logits": logits, "carry": carry, "end_idx": end_idx,
             "vis_lim": vis_lim, "pad": pad}
 
 
 def roles_from_one_hot(token_states_info: torch.Tensor) -> torch.Tensor:
-    """[B, H_kv, S, 3] one-hot float -> uint8 roles (index of the 1)."""
+    """[B, H_kv, S, 3] one-hot float -> uint8 roles (index of the 1).  A tensor that `roles_from_logits` or
+    `role_step` produced carries its roles with it."""
+    roles = getattr(token_states_info, "nats_roles", None)
+    if roles is not None and roles.shape == token_states_info.shape[:-1] and roles.device == token_states_info.device:
+        return roles
     return token_states_info.argmax(-1).to(torch.uint8)
 
 
@@ -412,18 +423,68 @@ def decode_attention(q: torch.Tensor, cache_k: torch.Tensor, cache_v: torch.Tens
 # eviction + compaction
 # ------------------------------------------------------------------------------------------------
 def evict_params(B, H_kv, D, C, W, S, x_len, fill, n_ctx_data, gmin, tail, first, n_alloc, update_chunk=0) -> EvictParams:
-    return EvictParams(B, H_kv, D, C, W, S, x_len, fill, n_ctx_data, gmin, tail, int(first), n_alloc, int(update_chunk))
+    return EvictParams(B, H_kv, D, C, W, S, x_len, fill, n_ctx_data, gmin, tail, int(first), n_alloc, 0, int(update_chunk))
 
 
-def evict_plan(roles: torch.Tensor, size_global: torch.Tensor, size_local: torch.Tensor, params: EvictParams):
-    """Returns (workspace, result): the per-head plan (device) and the 64-byte result struct (device int64[8])."""
+class EvictBuffers:
+    """What the eviction calls of one cache keep between calls: the plan workspace, the 64-byte result in device
+    memory, which the apply kernels read, and 16 bytes of pinned host memory into which the plan kernel also writes
+    the numbers the host needs (n_ctx_data, minimum global size, two flags) with the call's sequence number: the
+    host polls for that number instead of synchronising with the stream."""
+
+    def __init__(self, device):
+        self.device = torch.device(device)
+        self.ws = None
+        self.result = torch.zeros(8, dtype=torch.int64, device=self.device)
+        self.mirror = torch.zeros(4, dtype=torch.int32).pin_memory()
+        self.mirror_np = self.mirror.numpy()
+        self.seq = 0
+
+    def workspace(self, nbytes: int) -> torch.Tensor:
+        if self.ws is None or self.ws.numel() < nbytes:
+            have = 0 if self.ws is None else self.ws.numel()
+            self.ws = torch.empty(max(int(nbytes), 2 * have, 4096), dtype=torch.uint8, device=self.device)
+        return self.ws
+
+    def next_seq(self) -> int:
+        self.seq = self.seq % 0x7fffffff + 1
+        return self.seq
+
+    def wait(self, seq: int) -> EvictBrief:
+        """The short result of the plan call numbered `seq`, as soon as its kernel has written it."""
+        m = self.mirror_np
+        for _ in range(200000):
+            if m[0] == seq:
+                break
+        else:  # (about a tenth of a second: something is slow; fall back to a synchronisation)
+            torch.cuda.synchronize(self.device)
+            if m[0] != seq:
+                raise RuntimeError(f"eviction plan {seq} never reported its result (mirror holds {int(m[0])})")
+        flags = int(m[1])
+        return EvictBrief(int(m[2]), int(m[3]), flags & 1, (flags >> 1) & 1)
+
+    def full_result(self) -> EvictResult:
+        """All eight numbers of the last plan call, copied from device memory (synchronises with the stream)."""
+        return read_result(self.result)
+
+
+def evict_plan(roles: torch.Tensor, size_global: torch.Tensor, size_local: torch.Tensor, params: EvictParams,
+               buffers: EvictBuffers | None = None):
+    """Returns (workspace, result): the per-head plan (device) and the 64-byte result struct (device int64[8]).
+    With `buffers` the call uses that cache's workspace, numbers itself (params.seq) and mirrors its result into
+    pinned host memory, where `buffers.wait(params.seq)` finds its short form without a stream synchronisation."""
     _require_cuda(roles, size_global, size_local)
     lib = _lib.load()
     nbytes = lib.nats_evict_workspace_bytes(params.B, params.H_kv, params.S)
-    ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=roles.device)
-    result = torch.empty(8, dtype=torch.int64, device=roles.device)
+    if buffers is None:
+        ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=roles.device)
+        result = torch.empty(8, dtype=torch.int64, device=roles.device)
+        mirror = None
+    else:
+        ws, result, mirror = buffers.workspace(nbytes), buffers.result, buffers.mirror
+        params.seq = buffers.next_seq()
     check(lib.nats_evict_plan(_ptr(roles), _ptr(size_global), _ptr(size_local), ctypes.byref(params), _ptr(ws), ws.numel(),
-                              _ptr(result), _stream(roles)))
+                              _ptr(result), _ptr(mirror), _stream(roles)))
     return ws, result
 
 
@@ -431,6 +492,28 @@ def read_result(result: torch.Tensor) -> EvictResult:
     """Copies the device result struct to the host (synchronises with the stream)."""
     host = result.cpu().tolist()
     return EvictResult(*host)
+
+
+def cache_append_ok(k: torch.Tensor, v: torch.Tensor, cache_k: torch.Tensor, cache_v: torch.Tensor) -> bool:
+    """Whether `cache_append` takes these tensors: one dtype, 16-byte rows and strides everywhere."""
+    e = 16 // cache_k.element_size()
+    ts = (k, v, cache_k, cache_v)
+    return (all(t.is_cuda and t.dtype == cache_k.dtype and t.stride(-1) == 1 and t.data_ptr() % 16 == 0 for t in ts)
+            and cache_k.shape[-1] % e == 0 and all(st % e == 0 for t in ts for st, n in zip(t.stride()[:3], t.shape[:3]) if n != 1)
+            and not strides_differ(cache_k, cache_v))
+
+
+def cache_append(k: torch.Tensor, v: torch.Tensor, cache_k: torch.Tensor, cache_v: torch.Tensor, valid: torch.Tensor,
+                 pos: torch.Tensor | None, row0: int, pos0: int = 0):
+    """k / v [B, H_kv, x_len, D] into rows [row0, row0 + x_len) of the cache, with their valid bytes (and stream
+    positions): the row write of the cache update in one launch."""
+    B, H, x_len, D = k.shape
+    e = 16 // cache_k.element_size()
+    fix = lambda t: tuple(st if n != 1 else e for st, n in zip(t.stride()[:3], t.shape[:3]))  # (a size-1 dimension may carry any stride)
+    check(_lib.load().nats_cache_append(_ptr(k), _ptr(v), _ptr(cache_k), _ptr(cache_v), _ptr(valid), _ptr(pos), B, H, x_len, D,
+                                        int(row0), min(cache_k.shape[2], valid.shape[2]), int(pos0), i64_array(fix(k)),
+                                        i64_array(fix(v)), i64_array(fix(cache_k)), i64_array(valid.stride()[:2]),
+                                        cache_k.element_size(), _stream(k)))
 
 
 def evict_apply_inplace(cache_k, cache_v, valid, pos, roles, size_global, size_local, params: EvictParams, ws, result):

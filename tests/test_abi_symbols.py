@@ -29,7 +29,7 @@ def test_library_exports_every_declared_symbol():
 
 
 def test_struct_sizes_match_header():
-    assert ctypes.sizeof(_lib.EvictParams) == 14 * 8
+    assert ctypes.sizeof(_lib.EvictParams) == 15 * 8
     assert ctypes.sizeof(_lib.PastState) == 7 * 8
     assert ctypes.sizeof(_lib.EvictResult) == 64
 
@@ -89,10 +89,10 @@ def test_evict_params_are_validated():
     lib = _lib.load()
     fake = ctypes.c_void_p(256)
     p = _lib.EvictParams(1, 2, 128, 64, 96, 1, 64, 64, 96, 96, 0, 1, 256)  # W % C != 0
-    rc = lib.nats_evict_plan(fake, fake, fake, ctypes.byref(p), fake, 1 << 20, fake, None)
+    rc = lib.nats_evict_plan(fake, fake, fake, ctypes.byref(p), fake, 1 << 20, fake, None, None)
     assert rc == -2
     p = _lib.EvictParams(1, 2, 128, 64, 128, 3, 64, 64, 128, 128, 0, 1, 256)  # S inconsistent with fill
-    rc = lib.nats_evict_plan(fake, fake, fake, ctypes.byref(p), fake, 1 << 20, fake, None)
+    rc = lib.nats_evict_plan(fake, fake, fake, ctypes.byref(p), fake, 1 << 20, fake, None, None)
     assert rc == -2
 
 

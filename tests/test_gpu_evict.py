@@ -236,3 +236,42 @@ def test_cfg4_streamed_eviction_equals_bulk():
     assert torch.equal(stream.cache_k[:, :, :n] * m, bulk.cache_k[:, :, :n] * m)
     assert torch.equal(stream.cache_v[:, :, :n] * m, bulk.cache_v[:, :, :n] * m)
 
+
+
+@pytest.mark.parametrize("C,W,per_token", [(64, 256, False), (16, 32, False), (1, 32, True)])
+def test_a_reset_cache_evicts_its_next_prefill_on_a_guessed_capacity(C, W, per_token):
+    """A cache object that is reset and fed a new prompt launches the first eviction into a cache sized from the share
+    of rows it kept last time, before the plan kernel's numbers have reached the host.  The state must be the oracle's
+    byte for byte whether the guess was right, too small (the eviction runs again at the right size), far too large
+    (spare rows: zeros, not valid) or moot (every chunk sliding-window: the reference works in place), and the
+    tokens appended afterwards must land in rows that look as the reference's zero padding does."""
+    from neuralattentionsearch_amd.cache import NAtSChunkLayerCache, NAtSLayerCache
+    from oracle.nats_oracle import TokenCacheOracle
+    B, H, D, dtype = 2, 3, 64, torch.bfloat16
+    hip = (NAtSLayerCache(B, H, W, device="cuda", track_positions=True) if per_token
+           else NAtSChunkLayerCache(B, H, W, chunk_size=C, device="cuda", track_positions=True))
+    g = torch.Generator().manual_seed(C + W)
+    rng = np.random.default_rng(C)
+    runs = [(40 * max(C, 16) + 3, (0.2, 0.3, 0.5)),     # no history yet: the host waits for the size
+            (40 * max(C, 16) + 3, (0.2, 0.3, 0.5)),     # the same share again: the guess holds
+            (30 * max(C, 16), (0.7, 0.2, 0.1)),         # far more rows kept: too small, runs again
+            (50 * max(C, 16) + 1, (0.02, 0.08, 0.9)),   # far fewer rows kept: spare rows
+            (6 * max(C, 16), (0.0, 0.0, 1.0)),          # sliding-window only: the uncompacted cache, in place
+            (20 * max(C, 16) + 5, (0.3, 0.3, 0.4))]
+    for ri, (L, p) in enumerate(runs):
+        hip.reset_cache()
+        st = TokenCacheOracle(B=B, H=H, W=W) if per_token else ChunkCacheOracle(B=B, H=H, W=W, C=C)
+        lens = [L] + [1] * (2 * max(C, 16) + 3) + [max(C, 16) + 7]
+        segs = [(n, rng.choice(3, size=(B, H, n), p=p).astype(np.uint8)) for n in lens] if per_token \
+            else role_stream(rng, B, H, C, lens, p)
+        if p[2] == 1.0 and not per_token:
+            segs[0][1][:] = 2  # (role_stream marks the sink chunk global; here really every chunk slides)
+        for oi, (x_len, roles) in enumerate(segs):
+            say("evict on a guessed capacity", (C, W, per_token), "run", ri, "op", oi, "x_len", x_len)
+            k = torch.randn(B, H, x_len, D, generator=g).to(dtype)
+            v = torch.randn(B, H, x_len, D, generator=g).to(dtype)
+            st.update(k, v, roles)
+            hip.update(k.cuda(), v.cuda(), one_hot_roles(roles, dtype=dtype).cuda())
+            st.post_update(x_len)
+            hip.post_update(x_len)
+            compare(hip, st, (ri, oi, x_len))
