@@ -123,14 +123,12 @@ int nats_prefill_tile_map(const uint8_t* roles, int64_t B, int64_t H_kv, int64_t
  */
 size_t nats_prefill_workspace_bytes(int64_t B, int64_t H_q, int64_t H_kv, int64_t L, int64_t D, int64_t C);
 
-/* Extra workspace bytes (behind the ones above; already included in nats_prefill_workspace_bytes) for two optional
- * forms of the bf16 launch.  Few query tiles over many key rows (a short segment over a long cache): several
+/* Extra workspace bytes (behind the ones above; already included in nats_prefill_workspace_bytes) for one optional
+ * form of the bf16 launch.  Few query tiles over many key rows (a short segment over a long cache): several
  * workgroups share the key tiles of one query tile and a second kernel merges their partial results, so that the
- * launch still fills the device (NATS_PREFILL_SPLIT=0 in the environment switches this off).  GQA groups of 4 q
- * heads or a multiple, on request (NATS_PREFILL_STREAM=1): the persistent kernel, one workgroup per CU walking a
- * precomputed list of (query tile, key tile) visits instead of one workgroup per query tile building its own.
+ * launch still fills the device (NATS_PREFILL_SPLIT=0 in the environment switches this off).
  * A call whose workspace is smaller runs one workgroup per query tile; results are the same to rounding.  0 for
- * shapes that use neither.  n_queries: new tokens of the call, n_rows: key rows (L for a prefill from an empty cache,
+ * shapes that do not use it.  n_queries: new tokens of the call, n_rows: key rows (L for a prefill from an empty cache,
  * n_ctx_data + x_len over a filled one).
  */
 size_t nats_prefill_sched_workspace_bytes(int64_t B, int64_t H_q, int64_t H_kv, int64_t n_queries, int64_t n_rows);

@@ -5,7 +5,6 @@
 //                              key tiles, or (kPacked) tiles assembled from the visible 16-row granules; with
 //                              n_split > 1 several workgroups share one tile list and leave partial results
 //   prefill_split_merge_kernel combines those partial results
-//   prefill_stream_kernel      persistent form of the first (one workgroup per CU, precomputed visit lists; opt in)
 //   prefill_simple_kernel      fp32 (or bf16) FMA kernel, one query row per lane; the fp32 parity path
 //
 // Mask semantics (components/masks/utils.py:89-94, components/cache/nats_chunk_layer_cache.py:462-511, 603-616):
@@ -43,9 +42,6 @@ struct PrefillArgs {
   int n_qg;      // query tile groups = ceil(n query tiles / qpw)
   int xcd_mode;  // 1: workgroups of one kv stream share an XCD (needs B*Hkv % 8 == 0)
   float scale;   // softmax scale
-  // persistent kernel only: the flat tile lists of the schedule
-  const int32_t* entries;
-  const int2* bounds;  // [workgroups] {first entry, end entry}
   // few query tiles over many key rows: n_split workgroups share the tile list of one (kv stream, head group,
   // query group) and leave partial results, which prefill_split_merge_kernel combines
   int n_split;      // 1: no split
@@ -894,621 +890,6 @@ __global__ __launch_bounds__(256) void prefill_split_merge_kernel(PrefillArgs a)
   }
 }
 
-// ---------------------------------------------------------------------------------------------------
-// Persistent variant for GQA groups of 4 and more (the kUniform case): one workgroup per CU walks a flat,
-// precomputed list of (item header, key tile, key tile, ..., item header, ...) entries, where an item is one
-// 64-row query tile of 4 q heads.  The K / V tile pipeline runs on across item boundaries (the first tiles of
-// the next item are in flight while the last ones of this item are computed), so the per-item cost that is
-// left is the output epilogue and the switch of the Q registers; the visit list, the pipeline fill and the
-// workgroup launch are paid once per workgroup instead of once per query tile.
-//
-// Schedule (three small kernels): count the visited key tiles of every (kv stream, query tile); prefix sums
-// over the items in processing order (XCD-major, so that the workgroups of XCD x = blockIdx % 8 work on the kv
-// streams x, x + 8, ...) and a split of every XCD's items into contiguous ranges of equal cost; the flat lists.
-// ---------------------------------------------------------------------------------------------------
-// List entries are 32-bit words.  Tile: key tile index | kEntNeedLim.  Item header (negative):
-// kEntHeader | kv stream << 20 | head group << 16 | query tile.
-constexpr int kEntHeader = int(0x80000000u);
-constexpr int kEntNeedLim = 0x40000000;  // some query of the item needs the element mask on this tile
-constexpr int kRing = 2048;              // list entries resident in LDS
-constexpr int kChunk = 256;              // entries per list transfer (64 lanes x 16 bytes)
-constexpr int kMaxStreamWgs = 1024;
-
-struct SchedArgs {
-  const int2* tile_lim;
-  int32_t* count;     // [n_streams * n_qt] visited key tiles of (kv stream, query tile)
-  int32_t* item_off;  // [n_streams * n_hg * n_qt] first list entry (the header) of every item
-  int2* bounds;       // [n_wg] {first entry, end entry} of every workgroup's list
-  int32_t* entries;
-  int n_streams, Hkv, n_hg, n_qt, n_wg, parts;
-  int Tk, base, r_begin, r_end, qt_first, qt_last;
-};
-
-// query tile qi of the region: first / last query token and last key tile
-__device__ __forceinline__ void sched_tile_range(const SchedArgs& a, int qi, int& r0, int& rlast, int& kt_end) {
-  const int qt = a.qt_first + qi;
-  r0 = max(qt * kTile, a.r_begin);
-  rlast = min(qt * kTile + kTile - 1, a.r_end - 1);
-  kt_end = (a.base + rlast) / kTile;
-}
-
-__global__ __launch_bounds__(256) void sched_count_kernel(SchedArgs a) {
-  const int idx = blockIdx.x * 4 + (threadIdx.x >> 6);
-  const int lane = threadIdx.x & 63;
-  if (idx >= a.n_streams * a.n_qt) return;
-  const int ks = idx / a.n_qt, qi = idx - ks * a.n_qt;
-  int r0, rlast, kt_end;
-  sched_tile_range(a, qi, r0, rlast, kt_end);
-  const int2* tl = a.tile_lim + (int64_t)ks * a.Tk;
-  int count = 0;
-  for (int t0 = 0; t0 <= kt_end; t0 += kWave) {
-    const int t = t0 + lane;
-    const bool v = t <= kt_end && tl[t].x >= r0;
-    count += __builtin_popcountll(__ballot(v));
-  }
-  if (lane == 0) a.count[idx] = count;
-}
-
-// Items of one part (the kv streams of one XCD, or all of them), heaviest query tiles first, are dealt to the
-// part's m workgroups in rounds, alternating the direction (0 .. m-1, m-1 .. 0, ...): the workgroups of a part
-// work on neighbouring query tiles of one kv stream at the same time, which keeps its K / V tiles in the XCD's
-// L2, and costs that grow or shrink along the order even out (costs that vary at random do not: at 5 / 15 / 80 %
-// global / local / sliding roles the busiest workgroup has 11 % more tiles than the average).  Thread w lists the
-// items of workgroup w.
-__global__ __launch_bounds__(kMaxStreamWgs) void sched_scan_kernel(SchedArgs a) {
-  __shared__ int wave_tot[kMaxStreamWgs / kWave];
-  const int w = threadIdx.x, lane = w & 63, wave = w >> 6;
-  const int m = a.n_wg / a.parts;
-  const int part_len = (a.n_streams / a.parts) * a.n_hg * a.n_qt;
-  const int part = w % a.parts, wl = w / a.parts;
-  auto item_of = [&](int k, int& item, int& cnt) {  // k-th item of this workgroup; false past the end
-    const int j = k * m + ((k & 1) ? m - 1 - wl : wl);
-    if (j >= part_len) return false;
-    const int sl = j / a.n_qt, qi = a.n_qt - 1 - (j - sl * a.n_qt);
-    const int ks = part + a.parts * (sl / a.n_hg), hg = sl % a.n_hg;
-    item = (ks * a.n_hg + hg) * a.n_qt + qi;
-    cnt = a.count[ks * a.n_qt + qi];
-    return true;
-  };
-  const int rounds = (part_len + m - 1) / m;
-  int total = 0;
-  if (w < a.n_wg) {
-    for (int k = 0; k < rounds; ++k) {
-      int item, cnt;
-      if (item_of(k, item, cnt)) total += cnt + 1;
-    }
-  }
-  int inc = total;
-#pragma unroll
-  for (int o = 1; o < kWave; o <<= 1) {
-    const int p = __shfl_up(inc, o);
-    if (lane >= o) inc += p;
-  }
-  if (lane == kWave - 1) wave_tot[wave] = inc;
-  __syncthreads();
-  int start = inc - total;
-  for (int i = 0; i < wave; ++i) start += wave_tot[i];
-  if (w < a.n_wg) {
-    a.bounds[w] = make_int2(start, start + total);
-    int off = start;
-    for (int k = 0; k < rounds; ++k) {
-      int item, cnt;
-      if (item_of(k, item, cnt)) {
-        a.item_off[item] = off;
-        off += cnt + 1;
-      }
-    }
-  }
-}
-
-__global__ __launch_bounds__(256) void sched_fill_kernel(SchedArgs a) {
-  const int i = blockIdx.x * 4 + (threadIdx.x >> 6);
-  const int lane = threadIdx.x & 63;
-  if (i >= a.n_streams * a.n_hg * a.n_qt) return;
-  const int qi = i % a.n_qt, sh = i / a.n_qt;
-  const int hg = sh % a.n_hg, ks = sh / a.n_hg;
-  int r0, rlast, kt_end;
-  sched_tile_range(a, qi, r0, rlast, kt_end);
-  const int2* tl = a.tile_lim + (int64_t)ks * a.Tk;
-  int32_t* out = a.entries + a.item_off[i];
-  if (lane == 0) out[0] = kEntHeader | (ks << 20) | (hg << 16) | (a.qt_first + qi);
-  int count = 1;
-  for (int t0 = 0; t0 <= kt_end; t0 += kWave) {
-    const int t = t0 + lane;
-    int2 lm = t <= kt_end ? tl[t] : make_int2(-1, -1);
-    const bool v = t <= kt_end && lm.x >= r0;
-    const uint64_t bits = __ballot(v);
-    if (v) {
-      // the element mask is needed on diagonal tiles and on tiles whose rows are not all visible to all queries
-      const bool need = t * kTile + kTile - 1 - a.base > r0 || lm.y < rlast;
-      out[count + __builtin_popcountll(bits & ((uint64_t(1) << lane) - 1))] = t | (need ? kEntNeedLim : 0);
-    }
-    count += __builtin_popcountll(bits);
-  }
-}
-
-template <int D>
-struct StreamSmem {
-  uint16_t k[4][kTile * D];  // tile g of the workgroup's tile sequence in k[g & 3]
-  uint16_t v[4][kTile * D];
-  int limk[8][kTile];        // row limits of tile g in limk[g & 7]
-  int32_t ring[kRing];       // list entries, entry r (relative to the first one of the workgroup) in ring[r % kRing]
-  unsigned char stage[kPrefillWaves][32 * 80];  // output staging: 32 rows x 32 head dims per wavefront
-};
-
-template <int D>
-__global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_stream_kernel(PrefillArgs a) {
-  constexpr int OCT = D / 8;
-  constexpr int DMA_PER_WAVE = OCT / kPrefillWaves;
-  constexpr int DSTEPS = D / 16;
-  constexpr int DT = D / 32;
-  constexpr int kHalf = kTile / 2;
-  static_assert(DMA_PER_WAVE >= 1, "tile rows are split over the wavefronts in 1 KiB transfers");
-
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  StreamSmem<D>& sm = *reinterpret_cast<StreamSmem<D>*>(smem_raw);
-
-  const int tid = threadIdx.x;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int sub = wave & 3;    // q head of the item's group of 4
-  const int half = wave >> 2;  // which 32 rows of the query tile
-  const int lane = tid & 63;
-  const int l32 = lane & 31;
-  const int hl = lane >> 5;
-
-  const int2 bnd = a.bounds[blockIdx.x];
-  const int e_base = __builtin_amdgcn_readfirstlane(bnd.x) & ~3;  // list transfers start at a multiple of 16 bytes
-  const int r_first = __builtin_amdgcn_readfirstlane(bnd.x) - e_base;
-  const int r_end = __builtin_amdgcn_readfirstlane(bnd.y) - e_base;
-  if (r_first >= r_end) return;
-  const int32_t* ent = a.entries + e_base;
-
-  // ---- list ring: chunk c (256 entries) lives in ring[(c & 7) * 256 ...]; wavefront c & 7 transfers it ----
-  auto load_chunk = [&](int c) {
-    if (wave == (c & 7)) {
-      __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint32_t*>(ent + (int64_t)c * kChunk) + lane * 4,
-                                       (uint32_t __attribute__((address_space(3)))*)(&sm.ring[(c & 7) * kChunk]), 16, 0, 0);
-    }
-  };
-  const int n_chunks = (r_end + kChunk - 1) / kChunk;
-#pragma unroll 1
-  for (int c = 0; c < min(n_chunks, 8); ++c) load_chunk(c);
-  int next_chunk = 8;  // next chunk to bring in; it replaces chunk next_chunk - 8 once the compute cursor has left that one
-  auto entry = [&](int r) { return __builtin_amdgcn_readfirstlane(sm.ring[r & (kRing - 1)]); };
-
-  const float c = a.scale * 1.4426950408889634f;
-
-  // ---- global -> LDS tile transfers (as in prefill_mfma_kernel) ---------------------------------------
-  int koff[DMA_PER_WAVE], voff[DMA_PER_WAVE];
-#pragma unroll
-  for (int j = 0; j < DMA_PER_WAVE; ++j) {
-    const int q = (wave * DMA_PER_WAVE + j) * kWave + lane;
-    const int row = q / OCT, pos = q % OCT;
-    koff[j] = int(row * a.ks_l + (pos ^ (row % OCT)) * 8);
-    voff[j] = int(row * a.vs_l + (pos ^ ((row & 3) << 1)) * 8);
-  }
-  auto issue_rows = [&](const uint16_t* base, int64_t stride, const int (&off)[DMA_PER_WAVE], uint16_t* dst, int kt,
-                        bool is_v) {
-    if (__builtin_expect(kt * kTile + kTile <= a.N, 1)) {
-      const uint16_t* tb = base + (int64_t)kt * kTile * stride;
-#pragma unroll
-      for (int j = 0; j < DMA_PER_WAVE; ++j) {
-        const int inst = wave * DMA_PER_WAVE + j;
-        __builtin_amdgcn_global_load_lds(tb + (int)off[j], (uint32_t __attribute__((address_space(3)))*)(dst + inst * kWave * 8), 16, 0, 0);
-      }
-    } else {
-#pragma unroll
-      for (int j = 0; j < DMA_PER_WAVE; ++j) {
-        const int inst = wave * DMA_PER_WAVE + j;
-        const int q = inst * kWave + lane;
-        const int row = q / OCT, pos = q % OCT;
-        const int n = min(kt * kTile + row, a.N - 1);
-        const int chunk = is_v ? pos ^ ((row & 3) << 1) : pos ^ (row % OCT);
-        __builtin_amdgcn_global_load_lds(base + (int64_t)n * stride + chunk * 8,
-                                         (uint32_t __attribute__((address_space(3)))*)(dst + inst * kWave * 8), 16, 0, 0);
-      }
-    }
-  };
-
-  // ---- list window: lane i holds entry cr0 + i (one LDS read per step); readers pick their entry with a lane read ----
-  int wv = kEntHeader, cr0 = r_first;
-  auto read_window = [&](int cr) {
-    cr0 = cr;
-    wv = sm.ring[(cr + lane) & (kRing - 1)];
-  };
-  // entry r, cr0 <= r < cr0 + 64; past the end of the list reads as a header
-  auto win = [&](int r) {
-    const int v = __builtin_amdgcn_readlane(wv, (r - cr0) & 63);
-    return r < r_end ? v : kEntHeader;
-  };
-
-  // ---- load cursors: the next K / V tile of the workgroup's tile sequence to put in flight -----------
-  struct Cursor {
-    int r;                 // next list entry
-    const uint16_t* base;  // K or V rows of the kv stream the cursor is in
-    const int32_t* lim;    // its row limits (K cursor)
-  };
-  Cursor kc{r_first, nullptr, nullptr}, vc{r_first, nullptr, nullptr};
-  auto stream_of = [&](int head, int& b, int& hkv) {
-    const int ks = (head >> 20) & 1023;
-    b = ks / a.Hkv;
-    hkv = ks - b * a.Hkv;
-  };
-  // A tile the cursor has reached, with what its transfer needs.
-  struct TileLoad {
-    int tile;  // list word of the tile, -1 at the end of the list
-    const uint16_t* base;
-    const int32_t* lim;
-  };
-  // (straight-line: between two tiles of the list there is at most one header, every item has a tile)
-  auto gather = [&](Cursor& cu, bool is_v) {
-    int w = win(cu.r);
-    if (__builtin_expect((w < 0) & (cu.r < r_end), 0)) {
-      int b, hkv;
-      stream_of(w, b, hkv);
-      if (is_v) {
-        cu.base = static_cast<const uint16_t*>(a.v) + b * a.vs_b + hkv * a.vs_h;
-      } else {
-        cu.base = static_cast<const uint16_t*>(a.k) + b * a.ks_b + hkv * a.ks_h;
-        cu.lim = a.tok_lim + (int64_t)(b * a.Hkv + hkv) * a.N;
-      }
-      ++cu.r;
-      w = win(cu.r);
-    }
-    cu.r += w >= 0;
-    return TileLoad{w, cu.base, cu.lim};  // a negative word: the list has ended
-  };
-  // tile index gi of the sequence goes to buffer gi & 3 (limits: slot gi & 7)
-  auto issue_k = [&](const TileLoad& t, int gi) {
-    if (t.tile >= 0) {
-      const int kt = t.tile & 0xffffff;
-      issue_rows(t.base, a.ks_l, koff, sm.k[gi & 3], kt, false);
-      // (asynchronous like the tile itself; rows beyond N are later than every query, which masks them whatever
-      // limit they get, so their address is clamped)
-      if ((t.tile & kEntNeedLim) && wave == 0)
-        __builtin_amdgcn_global_load_lds(t.lim + min(kt * kTile + lane, a.N - 1),
-                                         (uint32_t __attribute__((address_space(3)))*)(&sm.limk[gi & 7][0]), 4, 0, 0);
-    }
-  };
-  auto issue_v = [&](const TileLoad& t, int gi) {
-    if (t.tile >= 0) issue_rows(t.base, a.vs_l, voff, sm.v[gi & 3], t.tile & 0xffffff, true);
-  };
-
-  // ---- fragments and the tile arithmetic (as in prefill_mfma_kernel) -----------------------------------
-  auto k_frag = [&](const uint16_t* Kt, int kb, int s) {
-    const int row = kb * 32 + l32;
-    const int chunk = (s * 2 + hl) ^ (row % OCT);
-    return *reinterpret_cast<const bf16x8*>(Kt + row * D + chunk * 8);
-  };
-  const int r16 = lane & 15;
-  const int dsel = (lane >> 4) & 1;
-  auto v_frag = [&](const uint16_t* Vt, int t, int dt) {
-    const int chunk0 = dt * 4 + dsel * 2 + ((r16 & 3) >> 1);
-    const int half4 = (r16 & 1) * 4;
-    const int row_lo = t * 16 + hl * 4 + (r16 >> 2);
-    const int row_hi = row_lo + 8;
-    const uint16_t* pl = Vt + row_lo * D + ((chunk0 ^ ((row_lo & 3) << 1)) * 8) + half4;
-    const uint16_t* ph = Vt + row_hi * D + ((chunk0 ^ ((row_hi & 3) << 1)) * 8) + half4;
-    bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((bf16x4 __attribute__((address_space(3)))*)pl);
-    bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((bf16x4 __attribute__((address_space(3)))*)ph);
-    bf16x8 va = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-    return va;
-  };
-
-  bf16x8 qreg[DSTEPS];
-  f32x16 oacc[DT];
-  float m_run = -INFINITY;
-  float l_run = 0.f;
-  // Item context: first region token of this wavefront's rows and its output rows.  q0 / o_head belong to the item
-  // whose probabilities are being computed; *_nxt to the item after it and *_nx2 to the one after that (the Q
-  // fragments of an item are fetched while the last tile of the item two before it is still being finished, when
-  // the item in between has a single tile).
-  int q0 = 0, q0_nxt = 0, q0_nx2 = 0;
-  uint16_t* o_head = nullptr;
-  uint16_t* o_head_nxt = nullptr;
-  uint16_t* o_head_nx2 = nullptr;
-
-  auto qk_tile = [&](int buf, f32x16 (&sacc)[2]) {
-    const uint16_t* Kt = sm.k[buf];
-#pragma unroll
-    for (int s = 0; s < DSTEPS; ++s) {
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb) {
-        bf16x8 ka = k_frag(Kt, kb, s);
-        if (s == 0) {
-          const f32x16 z = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-          sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qreg[s], z, 0, 0, 0);
-        } else {
-          sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qreg[s], sacc[kb], 0, 0, 0);
-        }
-      }
-    }
-  };
-  auto mask_scores = [&](int kt, int slot, f32x16 (&sv)[2]) {
-    const int qtok = q0 + l32;
-#pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
-#pragma unroll
-      for (int g4 = 0; g4 < 4; ++g4) {
-        int kk = kb * 32 + g4 * 8 + hl * 4;
-        int4 lm = *reinterpret_cast<const int4*>(&sm.limk[slot][kk]);
-        const int lv[4] = {lm.x, lm.y, lm.z, lm.w};
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          int key = kt * kTile + kk + e - a.base;
-          bool vis = key <= qtok && qtok <= lv[e];
-          if (!vis) sv[kb][g4 * 4 + e] = -INFINITY;
-        }
-      }
-    }
-  };
-  auto row_max = [&](const f32x16 (&sv)[2]) {
-    float m = -INFINITY;
-#pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) m = fmaxf(m, sv[kb][i]);
-    return half_swap_max(m) * c;
-  };
-  auto rescale = [&](float mx) {
-    float m_new = fmaxf(m_run, mx);
-    float alpha = m_run == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_run - m_new);
-    l_run *= alpha;
-    m_run = m_new;
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) oacc[dt][i] *= alpha;
-  };
-  auto prob = [&](const f32x16 (&sv)[2], int n, float m_use, float& rs, bf16x8 (&pb)[4]) {
-    const int t = n >> 3, i = n & 7;
-    float p = __builtin_amdgcn_exp2f(fmaf(sv[t >> 1][(t & 1) * 8 + i], c, -m_use));
-    rs += p;
-    pb[t][i] = (__bf16)p;
-  };
-  auto finish_tile = [&](int vbuf, const f32x16 (&sv)[2]) {
-    const uint16_t* Vt = sm.v[vbuf];
-    const float m_use = m_run == -INFINITY ? 0.f : m_run;
-    float rs = 0.f;
-    bf16x8 pb[4];
-#pragma unroll
-    for (int n = 0; n < 32; ++n) prob(sv, n, m_use, rs, pb);
-    l_run += rs;
-#pragma unroll
-    for (int t = 0; t < 4; ++t)
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt) oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v_frag(Vt, t, dt), pb[t], oacc[dt], 0, 0, 0);
-  };
-  // q_next: not null when the scores this step computes are the last ones of their item; the Q fragments of the next
-  // item are then fetched as soon as the score MFMAs are issued and have landed when the step ends.
-  auto fused_step = [&](int kbuf_next, int vbuf, const f32x16 (&sv)[2], f32x16 (&sacc)[2], const uint4* q_next) {
-    const uint16_t* Kt = sm.k[kbuf_next];
-    const uint16_t* Vt = sm.v[vbuf];
-    constexpr int N_QK = 2 * DSTEPS;
-    constexpr int N_PV = 4 * DT;
-    constexpr int VA = 16 / N_QK > 0 ? 16 / N_QK : 1;
-    constexpr int VB = 16 / (N_PV / 2);
-    const float m_use = m_run == -INFINITY ? 0.f : m_run;
-    float rs = 0.f;
-    bf16x8 pb[4];
-    int n = 0;
-    __builtin_amdgcn_sched_barrier(0);
-    auto k_at = [&](int i) { return k_frag(Kt, i & 1, i >> 1); };
-    auto v_at = [&](int i) { return v_frag(Vt, i / DT, i % DT); };
-    bf16x8 kf[3], vf[3];
-    kf[0] = k_at(0);
-    kf[1] = k_at(1);
-#pragma unroll
-    for (int i = 0; i < N_QK; ++i) {
-      const int s = i >> 1, kb = i & 1;
-      if (i + 2 < N_QK) {
-        kf[(i + 2) % 3] = k_at(i + 2);
-      } else {
-        vf[(i + 2 - N_QK) % 3] = v_at(i + 2 - N_QK);
-      }
-      if (s == 0) {
-        const f32x16 z = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i % 3], qreg[s], z, 0, 0, 0);
-      } else {
-        sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i % 3], qreg[s], sacc[kb], 0, 0, 0);
-      }
-      if (n < 16) {
-#pragma unroll
-        for (int e = 0; e < VA; ++e) prob(sv, n++, m_use, rs, pb);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-    }
-#pragma unroll
-    for (; n < 16;) prob(sv, n++, m_use, rs, pb);
-    auto pv_phase = [&]() {
-      int m = n;
-#pragma unroll
-      for (int i = 0; i < N_PV; ++i) {
-        const int t = i / DT, dt = i % DT;
-        if (i + 2 < N_PV) vf[(i + 2) % 3] = v_at(i + 2);
-        oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[i % 3], pb[t], oacc[dt], 0, 0, 0);
-        if (t < 2) {
-#pragma unroll
-          for (int e = 0; e < VB; ++e) prob(sv, m++, m_use, rs, pb);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-      }
-    };
-    // (the phase is written out on both paths so that the wait for the Q fragments stays on the path that loads them)
-    if (__builtin_expect(q_next != nullptr, 0)) {
-#pragma unroll
-      for (int s = 0; s < DSTEPS; ++s) qreg[s] = __builtin_bit_cast(bf16x8, q_next[s * 2]);
-      __builtin_amdgcn_sched_barrier(0);
-      pv_phase();
-      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the new Q fragments are in their registers
-    } else {
-      __builtin_amdgcn_sched_barrier(0);
-      pv_phase();
-    }
-    l_run += rs;
-  };
-
-  // ---- item switch --------------------------------------------------------------------------------
-  // (The per-lane address arithmetic of the item switch starts from a lane id the compiler cannot see through:
-  // otherwise it is hoisted out of the tile loop and its registers are lost to the loop.)
-  auto fresh_lane = [&]() {
-    int x = lane;
-#if defined(__HIP_DEVICE_COMPILE__)
-    asm volatile("" : "+v"(x));
-#endif
-    return x;
-  };
-  // header word of an item: context of the item (into the second queue slot if `second`) and the address of this
-  // lane's Q fragments
-  auto q_source = [&](int headw, bool second) {
-    const int ln = fresh_lane();
-    const int l32 = ln & 31, hl = ln >> 5;
-    int b, hkv;
-    stream_of(headw, b, hkv);
-    const int hg = (headw >> 16) & 15, qt = headw & 0xffff;
-    const int hq = hkv * a.n_rep + hg * 4 + sub;
-    const int q0_new = qt * kTile + half * kHalf;
-    uint16_t* o_new = static_cast<uint16_t*>(a.o) + b * a.os_b + hq * a.os_h;
-    if (second) {
-      q0_nx2 = q0_new;
-      o_head_nx2 = o_new;
-    } else {
-      q0_nxt = q0_new;
-      o_head_nxt = o_new;
-    }
-    const uint16_t* qp = static_cast<const uint16_t*>(a.q) + b * a.qs_b + hq * a.qs_h;
-    const int row = min(max(q0_new + l32, a.r_begin), a.r_end - 1) - a.r_begin;
-    return reinterpret_cast<const uint4*>(qp + (int64_t)row * a.qs_l + hl * 8);
-  };
-  // O rows of the finished item leave through a wavefront-private LDS staging area, one block of 32 head dims at a
-  // time, so that every row is stored as 64 contiguous bytes; then the accumulators start over
-  auto item_epilogue = [&]() {
-    constexpr int kPitch = 80;
-    const int ln = fresh_lane();
-    const int l32 = ln & 31, hl = ln >> 5;
-    unsigned char* stage = sm.stage[wave];
-    const float inv = 1.f / half_swap_sum(l_run);
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-#pragma unroll
-      for (int g4 = 0; g4 < 4; ++g4) {
-        const int d = g4 * 8 + hl * 4;
-        // (the hardware conversion: round to nearest even, two values per instruction)
-        const bf16x4 ob = {(__bf16)(oacc[dt][g4 * 4 + 0] * inv), (__bf16)(oacc[dt][g4 * 4 + 1] * inv),
-                           (__bf16)(oacc[dt][g4 * 4 + 2] * inv), (__bf16)(oacc[dt][g4 * 4 + 3] * inv)};
-        const uint2 ou = __builtin_bit_cast(uint2, ob);
-        const uint32_t lo = ou.x, hi = ou.y;
-        *reinterpret_cast<uint2*>(stage + l32 * kPitch + d * 2) = make_uint2(lo, hi);
-      }
-      wave_lds_sync();
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        const int row = i * 16 + (ln >> 2), piece = ln & 3;
-        const int qtok = q0 + row;
-        const uint4 val = *reinterpret_cast<const uint4*>(stage + row * kPitch + piece * 16);
-        if (qtok >= a.r_begin && qtok < a.r_end)
-          *reinterpret_cast<uint4*>(o_head + (int64_t)(qtok - a.r_begin) * a.os_l + dt * 32 + piece * 8) = val;
-      }
-      wave_lds_sync();
-    }
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) oacc[dt][i] = 0.f;
-    m_run = -INFINITY;
-    l_run = 0.f;
-  };
-
-  // ---- prologue: the list is resident, the first item is set up, the first tiles are in flight ----------
-#pragma unroll
-  for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) oacc[dt][i] = 0.f;
-  __builtin_amdgcn_s_waitcnt(0);
-  __syncthreads();
-  int cr = r_first + 1;  // compute cursor: entry of the current tile (the list starts with a header)
-  read_window(r_first);
-  {
-    const int head0 = win(r_first);
-    const TileLoad k0 = gather(kc, false), k1 = gather(kc, false), k2 = gather(kc, false);
-    const TileLoad v0 = gather(vc, true), v1 = gather(vc, true);
-    const uint4* rp = q_source(head0, false);
-#pragma unroll
-    for (int s = 0; s < DSTEPS; ++s) qreg[s] = __builtin_bit_cast(bf16x8, rp[s * 2]);
-    q0 = q0_nxt;
-    o_head = o_head_nxt;
-    issue_k(k0, 0);
-    issue_v(v0, 0);
-    issue_k(k1, 1);
-    issue_v(v1, 1);
-    issue_k(k2, 2);
-  }
-  f32x16 sacc[2];
-  __builtin_amdgcn_s_waitcnt(0);
-  __syncthreads();
-  qk_tile(0, sacc);
-  // the Q fragments change as soon as the scores of an item's last tile are computed
-  if (win(cr + 1) < 0 && cr + 1 < r_end) {
-    const uint4* rp = q_source(win(cr + 1), false);
-#pragma unroll
-    for (int s = 0; s < DSTEPS; ++s) qreg[s] = __builtin_bit_cast(bf16x8, rp[s * 2]);
-  }
-  __builtin_amdgcn_s_waitcnt(0);
-  __syncthreads();  // k[0] is overwritten by the first step
-
-  // ---- tile loop -----------------------------------------------------------------------------------
-  // Two tiles of the workgroup's tile sequence share one step (transfers issued before the even tile, barrier after
-  // the odd one).  Every tile runs the same fused block: its probabilities and O += P V, woven with the scores of
-  // the next tile of the sequence, which may belong to the next item (whose Q fragments are in the registers by then).
-  int g = 0;  // index of the current tile in the sequence; its scores are in sacc
-  while (true) {
-    if ((g & 1) == 0) {
-      // every list entry the step needs is read, then the transfers are issued
-      read_window(cr);
-      const TileLoad k0 = gather(kc, false), k1 = gather(kc, false);
-      const TileLoad v0 = gather(vc, true), v1 = gather(vc, true);
-      if (next_chunk < n_chunks && cr / kChunk > next_chunk - 8) {  // the list chunk behind the compute cursor is replaced
-        load_chunk(next_chunk);
-        ++next_chunk;
-      }
-      issue_k(k0, g + 3);
-      issue_k(k1, g + 4);
-      issue_v(v0, g + 2);
-      issue_v(v1, g + 3);
-    }
-    const int cur = win(cr);
-    const bool last_of_item = win(cr + 1) < 0;
-    const int r_next = cr + 1 + last_of_item;  // next tile of the sequence (if r_next < r_end)
-    const bool is_end = last_of_item & (cr + 1 >= r_end);
-    // if the next tile is the last of its item, the Q fragments of the item after it come in during this step
-    const int after_next = win(r_next + 1);
-    const uint4* q_next = nullptr;
-    if (__builtin_expect((!is_end) & (after_next < 0) & (r_next + 1 < r_end), 0)) q_next = q_source(after_next, last_of_item);
-    {
-      f32x16 sv[2] = {sacc[0], sacc[1]};
-      if (cur & kEntNeedLim) mask_scores(cur & 0xffffff, g & 7, sv);
-      const float mx = row_max(sv);
-      if (__builtin_expect(__ballot(mx > m_run + kRescaleSlack) != 0, 0)) rescale(mx);
-      // (after the last tile of the list the block computes scores of a stale tile that nobody reads)
-      fused_step((g + 1) & 3, g & 3, sv, sacc, q_next);
-    }
-    if (__builtin_expect(last_of_item, 0)) {
-      item_epilogue();
-      q0 = q0_nxt;
-      o_head = o_head_nxt;
-      q0_nxt = q0_nx2;
-      o_head_nxt = o_head_nx2;
-    }
-    if (is_end) break;
-    cr = r_next;
-    if (g & 1) {
-      __builtin_amdgcn_s_waitcnt(0);  // the tiles in flight have landed in LDS
-      __syncthreads();                // ... for every wavefront, and the tiles of this step are no longer read
-    }
-    ++g;
-  }
-}
-
 template <int D, bool kUniform, bool kPacked = false>
 static int launch_prefill_mfma(const PrefillArgs& a, int64_t n_wg, hipStream_t st) {
   static bool configured[kMaxDevices] = {};  // per instantiation; the attribute is set once per device
@@ -1524,55 +905,6 @@ static int launch_prefill_mfma(const PrefillArgs& a, int64_t n_wg, hipStream_t s
   hipLaunchKernelGGL((prefill_mfma_kernel<D, kUniform, kPacked>), dim3((unsigned)n_wg), dim3(kPrefillWaves * kWave), smem, st, a);
   NATS_CHECK_LAUNCH("prefill_mfma_kernel");
   return NATS_OK;
-}
-
-// ---- schedule workspace and launch of the persistent kernel ---------------------------------------------
-struct StreamSched {
-  int32_t* count;
-  int32_t* item_off;
-  int2* bounds;
-  int32_t* entries;
-  int64_t max_entries;
-  size_t bytes;  // 0: the shape does not use the persistent kernel
-};
-
-// Upper bound of the list entries of one (kv stream, head group): the last of the n_qt query tiles sees at most
-// Tk key tiles, the j-th before it at most Tk - j + 1 (a partial last query tile may end in the same key tile as
-// its predecessor); one header per item.
-static int64_t sched_entries_per_stream(int64_t n_qt, int64_t Tk) {
-  int64_t n = 0;
-  for (int64_t j = 0; j < n_qt; ++j) {
-    int64_t t = Tk - j + 1;
-    t = t > Tk ? Tk : t;
-    n += (t > 1 ? t : 1) + 1;
-  }
-  return n;
-}
-
-// `ws` may be NULL (size query).  n_qt_max: upper bound of the 64-token query tiles of the call.
-static StreamSched carve_stream_sched(void* ws, int64_t B, int64_t H_q, int64_t H_kv, int64_t n_qt_max, int64_t Tk) {
-  StreamSched w{};
-  if (B <= 0 || H_kv <= 0 || H_q % H_kv != 0) return w;
-  const int64_t n_rep = H_q / H_kv;
-  if (n_rep < 4 || n_rep % 4 != 0 || B * H_kv > 1024 || n_rep / 4 > 16 || n_qt_max > 65535) return w;  // header word fields
-  const int64_t n_streams = B * H_kv, n_hg = n_rep / 4;
-  if (n_streams * n_hg * n_qt_max >= (int64_t(1) << 30)) return w;
-  const int64_t bound = n_streams * n_hg * sched_entries_per_stream(n_qt_max, Tk);
-  if (bound * (int64_t)sizeof(int32_t) > (int64_t(256) << 20)) return w;  // very long contexts keep the per-tile kernel
-  auto up = [](size_t x) { return (x + 255) & ~size_t(255); };
-  char* p = static_cast<char*>(ws);
-  size_t off = 0;
-  w.count = reinterpret_cast<int32_t*>(p + off);
-  off += up((size_t)(n_streams * n_qt_max) * sizeof(int32_t));
-  w.item_off = reinterpret_cast<int32_t*>(p + off);
-  off += up((size_t)(n_streams * n_hg * n_qt_max) * sizeof(int32_t));
-  w.bounds = reinterpret_cast<int2*>(p + off);
-  off += up((size_t)kMaxStreamWgs * sizeof(int2));
-  w.entries = reinterpret_cast<int32_t*>(p + off);
-  off += up((size_t)(bound + 2 * kChunk) * sizeof(int32_t));  // list transfers read whole chunks
-  w.max_entries = bound;
-  w.bytes = off;
-  return w;
 }
 
 static int device_cu_count() {
@@ -1603,44 +935,6 @@ static int choose_split(int64_t n_wg, int64_t Tk) {
 }
 static size_t split_partial_bytes(int64_t n_wg, int n_split, int64_t D) {
   return n_split <= 1 ? 0 : (size_t)n_wg * n_split * kPrefillWaves * (kTile / 2) * (D + 2) * sizeof(float);
-}
-
-template <int D>
-static int launch_prefill_stream(PrefillArgs a, const StreamSched& sw, hipStream_t st) {
-  int n_wg = device_cu_count();
-  if (n_wg <= 0) return fail(NATS_ERR_LAUNCH, "prefill: cannot read the number of compute units");
-  if (n_wg > kMaxStreamWgs) n_wg = kMaxStreamWgs;
-  SchedArgs sa{};
-  sa.tile_lim = a.tile_lim;
-  sa.count = sw.count; sa.item_off = sw.item_off; sa.bounds = sw.bounds; sa.entries = sw.entries;
-  sa.n_streams = a.B * a.Hkv; sa.Hkv = a.Hkv; sa.n_hg = a.n_hg;
-  sa.n_qt = a.qt_last - a.qt_first + 1;
-  const int n_items = sa.n_streams * sa.n_hg * sa.n_qt;
-  sa.parts = (sa.n_streams % 8 == 0 && n_wg % 8 == 0) ? 8 : 1;
-  sa.n_wg = n_wg;
-  sa.Tk = a.Tk; sa.base = a.base; sa.r_begin = a.r_begin; sa.r_end = a.r_end; sa.qt_first = a.qt_first; sa.qt_last = a.qt_last;
-  hipLaunchKernelGGL(sched_count_kernel, dim3((unsigned)((sa.n_streams * sa.n_qt + 3) / 4)), dim3(256), 0, st, sa);
-  NATS_CHECK_LAUNCH("sched_count_kernel");
-  hipLaunchKernelGGL(sched_scan_kernel, dim3(1), dim3((unsigned)((n_wg + kWave - 1) / kWave * kWave)), 0, st, sa);
-  NATS_CHECK_LAUNCH("sched_scan_kernel");
-  hipLaunchKernelGGL(sched_fill_kernel, dim3((unsigned)((n_items + 3) / 4)), dim3(256), 0, st, sa);
-  NATS_CHECK_LAUNCH("sched_fill_kernel");
-
-  a.entries = sw.entries;
-  a.bounds = sw.bounds;
-  static bool configured[kMaxDevices] = {};
-  const size_t smem = sizeof(StreamSmem<D>);
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail(NATS_ERR_LAUNCH, "prefill: no current device");
-  if (!configured[dev]) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_stream_kernel<D>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    if (e != hipSuccess) return fail(NATS_ERR_LAUNCH, "hipFuncSetAttribute(%zu bytes of LDS): %s", smem, hipGetErrorString(e));
-    configured[dev] = true;
-  }
-  hipLaunchKernelGGL((prefill_stream_kernel<D>), dim3((unsigned)n_wg), dim3(kPrefillWaves * kWave), smem, st, a);
-  NATS_CHECK_LAUNCH("prefill_stream_kernel");
-  return NATS_OK;
 }
 
 }  // namespace nats
@@ -1686,33 +980,16 @@ int check_common(const char* who, const SegmentShape& g, const int64_t* q_stride
   return NATS_OK;
 }
 
-// NATS_PREFILL_STREAM=1 in the environment selects the persistent kernel where the shape allows it
-bool use_stream_kernel() {
-  const char* e = getenv("NATS_PREFILL_STREAM");
-  return e && e[0] == '1';
-}
-
 bool use_packed_tiles() {
   const char* e = getenv("NATS_PREFILL_PACKED");
   return !(e && e[0] == '0');
 }
 
-// the schedule workspace behind the key-limit workspace, if the caller's buffer has room for it
-StreamSched sched_in_workspace(void* workspace, size_t workspace_bytes, size_t base_bytes, int64_t B, int64_t H_q,
-                               int64_t H_kv, int64_t n_qt, int64_t N, int dtype) {
-  StreamSched none{};
-  if (dtype != NATS_DTYPE_BF16) return none;
-  const int64_t Tk = (N + kTile - 1) / kTile;
-  StreamSched sw = carve_stream_sched(static_cast<char*>(workspace) + base_bytes, B, H_q, H_kv, n_qt, Tk);
-  if (sw.bytes == 0 || workspace_bytes < base_bytes + sw.bytes) return none;
-  return sw;
-}
-
 // key limits are in the workspace; launches the attention kernel of the segment
 int launch_segment(const char* who, const SegmentShape& g, const void* q, const void* k, const void* v, void* o,
                    const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
-                   const int64_t* o_strides, float sm_scale, int dtype, const PrefillWorkspace& w, const StreamSched& sw,
-                   void* extra, size_t extra_bytes, hipStream_t st) {
+                   const int64_t* o_strides, float sm_scale, int dtype, const PrefillWorkspace& w, void* extra,
+                   size_t extra_bytes, hipStream_t st) {
   PrefillArgs a{};
   a.q = q; a.k = k; a.v = v; a.o = o;
   a.tok_lim = w.tok_lim; a.tile_lim = w.tile_lim; a.gran_lim = w.gran_lim;
@@ -1755,9 +1032,8 @@ int launch_segment(const char* who, const SegmentShape& g, const void* q, const 
   // workgroup's four or two query tiles walk one list together, which costs the same as every wavefront skipping
   // on its own between shared barriers and lets small launches share their lists among workgroups.
   const bool packed = (g.C < kTile || hpw < 4) && use_packed_tiles();
-  const bool persistent = hpw == 4 && !packed && sw.bytes != 0 && use_stream_kernel();
   a.n_split = 1;
-  if ((hpw == 4 || packed) && !persistent) {  // the kernels in which every wavefront walks the whole tile list
+  if (hpw == 4 || packed) {  // the kernels in which every wavefront walks the whole tile list
     const int ns = choose_split(n_wg, a.Tk);
     if (ns > 1 && extra && extra_bytes >= split_partial_bytes(n_wg, ns, g.D)) {
       a.n_split = ns;
@@ -1788,8 +1064,6 @@ int launch_segment(const char* who, const SegmentShape& g, const void* q, const 
   // walks the whole list and the element mask sorts out what its own rows see)
   if (packed)
     return g.D == 64 ? launch_prefill_mfma<64, true, true>(a, n_wg, st) : launch_prefill_mfma<128, true, true>(a, n_wg, st);
-  if (hpw == 4 && sw.bytes != 0 && use_stream_kernel())
-    return g.D == 64 ? launch_prefill_stream<64>(a, sw, st) : launch_prefill_stream<128>(a, sw, st);
   if (hpw == 4) return g.D == 64 ? launch_prefill_mfma<64, true>(a, n_wg, st) : launch_prefill_mfma<128, true>(a, n_wg, st);
   return g.D == 64 ? launch_prefill_mfma<64, false>(a, n_wg, st) : launch_prefill_mfma<128, false>(a, n_wg, st);
 }
@@ -1807,16 +1081,13 @@ extern "C" size_t nats_prefill_sched_workspace_bytes(int64_t B, int64_t H_q, int
   // a segment over a filled cache starts anywhere inside a 64-token tile of its region
   const int64_t n_qt = n_rows == n_queries ? (n_queries + kTile - 1) / kTile : (n_queries + kTile - 2) / kTile + 1;
   const int64_t Tk = (n_rows + kTile - 1) / kTile;
-  const size_t sched = carve_stream_sched(nullptr, B, H_q, H_kv, n_qt, Tk).bytes;
-  // the partial results of a split launch use the same region (a launch is either split or persistent)
   const int64_t n_rep = H_q / H_kv;
   const int64_t hpw = n_rep % 4 == 0 ? 4 : n_rep % 2 == 0 ? 2 : 1;  // as in launch_segment
   // (a split launch never has more workgroups than the device has CUs, whatever the exact number of query tiles
   // turns out to be: room for that many partial results whenever a launch of this size may be split)
   const int64_t n_qg_min = (n_qt > 1 ? n_qt - 1 : 1) + 4 / hpw - 1;
   const int64_t n_wg_min = B * H_kv * (n_rep / hpw > 0 ? n_rep / hpw : 1) * (n_qg_min / (4 / hpw));
-  const size_t split = choose_split(n_wg_min, Tk) > 1 ? split_partial_bytes(device_cu_count(), 2, 128) / 2 : 0;
-  return sched > split ? sched : split;
+  return choose_split(n_wg_min, Tk) > 1 ? split_partial_bytes(device_cu_count(), 2, 128) / 2 : 0;
 }
 
 extern "C" size_t nats_prefill_past_workspace_bytes(int64_t B, int64_t H_kv, int64_t n_rows, int64_t S) {
@@ -1839,8 +1110,7 @@ extern "C" int nats_prefill_fwd(const void* q, const void* k, const void* v, con
   NATS_REQUIRE(workspace_bytes >= w.bytes, NATS_ERR_WORKSPACE, "%s: workspace %zu bytes < %zu", who, workspace_bytes, w.bytes);
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (int rc = prepare_key_limits(roles, B, H_kv, S, L, C, W, nullptr, w, st)) return rc;
-  const StreamSched sw = sched_in_workspace(workspace, workspace_bytes, w.bytes, B, H_q, H_kv, (L + kTile - 1) / kTile, L, dtype);
-  return launch_segment(who, g, q, k, v, o, q_strides, k_strides, v_strides, o_strides, sm_scale, dtype, w, sw,
+  return launch_segment(who, g, q, k, v, o, q_strides, k_strides, v_strides, o_strides, sm_scale, dtype, w,
                         static_cast<char*>(workspace) + w.bytes, workspace_bytes - w.bytes, st);
 }
 
@@ -1869,8 +1139,6 @@ extern "C" int nats_prefill_past_fwd(const void* q, const void* cache_k, const v
               state->gmin, state->tail, state->seen, state->fill_last, state->old_fill, state->update_chunk != 0};
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (int rc = prepare_key_limits(roles, B, H_kv, S, N, C, W, &pv, w, st)) return rc;
-  const int64_t n_qt = (state->old_fill + x_len - 1) / kTile - state->old_fill / kTile + 1;
-  const StreamSched sw = sched_in_workspace(workspace, workspace_bytes, w.bytes, B, H_q, H_kv, n_qt, N, dtype);
-  return launch_segment(who, g, q, cache_k, cache_v, o, q_strides, k_strides, v_strides, o_strides, sm_scale, dtype, w, sw,
+  return launch_segment(who, g, q, cache_k, cache_v, o, q_strides, k_strides, v_strides, o_strides, sm_scale, dtype, w,
                         static_cast<char*>(workspace) + w.bytes, workspace_bytes - w.bytes, st);
 }
