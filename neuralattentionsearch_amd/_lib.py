@@ -10,7 +10,8 @@ import functools
 import os
 
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_PKG_DIR, "libnats_hip.so")
+# (NATS_HIP_LIB names another build of the same library, e.g. to time two builds side by side)
+LIB_PATH = os.environ.get("NATS_HIP_LIB") or os.path.join(_PKG_DIR, "libnats_hip.so")
 
 c_i64 = ctypes.c_int64
 c_p = ctypes.c_void_p

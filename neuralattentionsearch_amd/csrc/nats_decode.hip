@@ -442,9 +442,18 @@ __global__ void decode_merge_balanced_kernel(const float* __restrict__ ws_acc, c
   o[(int64_t)head * D + d] = f32_to_bf16_bits(lsum > 0.f ? sum / lsum : 0.f);
 }
 
-template <int D>
+// T = float, or uint16_t for bf16 at the head dims the MFMA kernel does not take (16, 32, 256).
+template <typename T>
+__device__ __forceinline__ float dec_load(const T* p);
+template <>
+__device__ __forceinline__ float dec_load<float>(const float* p) { return *p; }
+template <>
+__device__ __forceinline__ float dec_load<uint16_t>(const uint16_t* p) { return bf16_bits_to_f32(*p); }
+
+template <typename T, int D>
 __global__ __launch_bounds__(256) void decode_split_f32_kernel(DecodeArgs a) {
-  constexpr int PER = D / 64;
+  constexpr int LANES = D < 64 ? D : 64;  // lanes that hold dimensions of a row
+  constexpr int PER = D / LANES;
   __shared__ float wacc[4][D];
   __shared__ float wm[4];
   __shared__ float wl[4];
@@ -452,14 +461,16 @@ __global__ __launch_bounds__(256) void decode_split_f32_kernel(DecodeArgs a) {
   const int split = blockIdx.x;
   const int head = blockIdx.y;  // b * Hq + hq
   const int b = head / a.Hq, hq = head % a.Hq, hkv = hq / a.n_rep;
-  const float* kp = static_cast<const float*>(a.k) + b * a.ks_b + hkv * a.ks_h;
-  const float* vp = static_cast<const float*>(a.v) + b * a.ks_b + hkv * a.ks_h;
+  const T* kp = static_cast<const T*>(a.k) + b * a.ks_b + hkv * a.ks_h;
+  const T* vp = static_cast<const T*>(a.v) + b * a.ks_b + hkv * a.ks_h;
   const uint8_t* valp = a.valid + b * a.vs_b + hkv * a.vs_h;
-  const float* qp = static_cast<const float*>(a.q) + (int64_t)head * D;
+  const T* qp = static_cast<const T*>(a.q) + (int64_t)head * D;
+  const bool live = lane < LANES;
+  const int d0 = live ? lane * PER : 0;
   float qv[PER], acc[PER];
 #pragma unroll
   for (int e = 0; e < PER; ++e) {
-    qv[e] = qp[lane * PER + e];
+    qv[e] = live ? dec_load<T>(qp + d0 + e) : 0.f;
     acc[e] = 0.f;
   }
   float m_run = -INFINITY, l_run = 0.f;
@@ -467,11 +478,11 @@ __global__ __launch_bounds__(256) void decode_split_f32_kernel(DecodeArgs a) {
   const int r_end = min(r_begin + a.rows_per_split, a.n_rows);
   for (int r = r_begin + wave; r < r_end; r += 4) {
     if (valp[r] == 0) continue;
-    const float* kr = kp + (int64_t)r * a.ks_r;
-    const float* vr = vp + (int64_t)r * a.ks_r;
+    const T* kr = kp + (int64_t)r * a.ks_r;
+    const T* vr = vp + (int64_t)r * a.ks_r;
     float dot = 0.f;
 #pragma unroll
-    for (int e = 0; e < PER; ++e) dot = fmaf(qv[e], kr[lane * PER + e], dot);
+    for (int e = 0; e < PER; ++e) dot = fmaf(qv[e], dec_load<T>(kr + d0 + e), dot);
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) dot += __shfl_xor(dot, off);
     float s = dot * a.scale;
@@ -480,11 +491,13 @@ __global__ __launch_bounds__(256) void decode_split_f32_kernel(DecodeArgs a) {
     float p = expf(s - m_new);
     l_run = l_run * alpha + p;
 #pragma unroll
-    for (int e = 0; e < PER; ++e) acc[e] = fmaf(p, vr[lane * PER + e], acc[e] * alpha);
+    for (int e = 0; e < PER; ++e) acc[e] = fmaf(p, dec_load<T>(vr + d0 + e), acc[e] * alpha);
     m_run = m_new;
   }
+  if (live) {
 #pragma unroll
-  for (int e = 0; e < PER; ++e) wacc[wave][lane * PER + e] = acc[e];
+    for (int e = 0; e < PER; ++e) wacc[wave][d0 + e] = acc[e];
+  }
   if (lane == 0) {
     wm[wave] = m_run;
     wl[wave] = l_run;
@@ -616,8 +629,9 @@ static int decode_fwd_impl(const void* q, const void* cache_k, const void* cache
                (long long)n_rows);
   NATS_REQUIRE(H_q % H_kv == 0, NATS_ERR_BAD_SHAPE, "nats_decode_fwd: H_q=%lld is not a multiple of H_kv=%lld",
                (long long)H_q, (long long)H_kv);
-  NATS_REQUIRE(D == 64 || D == 128, NATS_ERR_UNSUPPORTED, "nats_decode_fwd: head_dim %lld (supported: 64, 128)",
-               (long long)D);
+  NATS_REQUIRE(D == 16 || D == 32 || D == 64 || D == 128 || D == 256, NATS_ERR_UNSUPPORTED,
+               "nats_decode_fwd: head_dim %lld (supported: 16, 32, 64, 128, 256)", (long long)D);
+  const bool mfma = dtype == NATS_DTYPE_BF16 && (D == 64 || D == 128);  // other bf16 head dims take the plain kernel
   NATS_REQUIRE(dtype == NATS_DTYPE_BF16 || dtype == NATS_DTYPE_F32, NATS_ERR_BAD_DTYPE, "nats_decode_fwd: dtype %d", dtype);
   NATS_REQUIRE(n_rows < (int64_t(1) << 30) && B * H_q <= (int64_t(1) << 30), NATS_ERR_BAD_SHAPE,
                "nats_decode_fwd: problem too large");
@@ -631,7 +645,7 @@ static int decode_fwd_impl(const void* q, const void* cache_k, const void* cache
                need, max_bytes);
   NATS_REQUIRE(workspace_bytes >= need, NATS_ERR_WORKSPACE, "nats_decode_fwd: workspace %zu bytes < %zu", workspace_bytes,
                need);
-  if (dtype == NATS_DTYPE_BF16) {
+  if (mfma) {
     NATS_REQUIRE(kv_strides[0] % 8 == 0 && kv_strides[1] % 8 == 0 && kv_strides[2] % 8 == 0, NATS_ERR_BAD_SHAPE,
                  "nats_decode_fwd: bf16 cache strides must keep rows 16-byte aligned");
     NATS_REQUIRE((reinterpret_cast<uintptr_t>(cache_k) | reinterpret_cast<uintptr_t>(cache_v) |
@@ -641,7 +655,7 @@ static int decode_fwd_impl(const void* q, const void* cache_k, const void* cache
   hipStream_t st = static_cast<hipStream_t>(stream);
   DecodeArgs a;
   a.q = q; a.k = cache_k; a.v = cache_v; a.valid = valid; a.o = o;
-  a.row_end = dtype == NATS_DTYPE_BF16 ? row_end : nullptr;
+  a.row_end = mfma ? row_end : nullptr;
   a.tail_start = (int)tail_start;
   a.ks_b = kv_strides[0]; a.ks_h = kv_strides[1]; a.ks_r = kv_strides[2];
   a.vs_b = valid_strides[0]; a.vs_h = valid_strides[1];
@@ -654,16 +668,34 @@ static int decode_fwd_impl(const void* q, const void* cache_k, const void* cache
   a.ws_acc = static_cast<float*>(workspace);
   a.ws_ml = a.ws_acc + (size_t)B * H_q * a.nsplit * D;
 
-  if (dtype == NATS_DTYPE_F32) {
+  if (!mfma) {
     dim3 grid((unsigned)a.nsplit, (unsigned)(B * H_q));
-    if (D == 64) {
-      hipLaunchKernelGGL((decode_split_f32_kernel<64>), grid, dim3(256), 0, st, a);
-    } else {
-      hipLaunchKernelGGL((decode_split_f32_kernel<128>), grid, dim3(256), 0, st, a);
+    const bool f32 = dtype == NATS_DTYPE_F32;
+#define NATS_DECODE_PLAIN(DD)                                                                        \
+  case DD:                                                                                           \
+    if (f32) {                                                                                       \
+      hipLaunchKernelGGL((decode_split_f32_kernel<float, DD>), grid, dim3(256), 0, st, a);           \
+    } else {                                                                                         \
+      hipLaunchKernelGGL((decode_split_f32_kernel<uint16_t, DD>), grid, dim3(256), 0, st, a);        \
+    }                                                                                                \
+    break;
+    switch (D) {
+      NATS_DECODE_PLAIN(16)
+      NATS_DECODE_PLAIN(32)
+      NATS_DECODE_PLAIN(64)
+      NATS_DECODE_PLAIN(128)
+      default:
+      NATS_DECODE_PLAIN(256)
     }
+#undef NATS_DECODE_PLAIN
     NATS_CHECK_LAUNCH("decode_split_f32_kernel");
-    hipLaunchKernelGGL((decode_merge_kernel<false>), dim3((unsigned)(B * H_q)), dim3((unsigned)D), 0, st, a.ws_acc, a.ws_ml,
-                       o, a.nsplit, (int)D);
+    if (f32) {
+      hipLaunchKernelGGL((decode_merge_kernel<false>), dim3((unsigned)(B * H_q)), dim3((unsigned)D), 0, st, a.ws_acc, a.ws_ml,
+                         o, a.nsplit, (int)D);
+    } else {
+      hipLaunchKernelGGL((decode_merge_kernel<true>), dim3((unsigned)(B * H_q)), dim3((unsigned)D), 0, st, a.ws_acc, a.ws_ml,
+                         o, a.nsplit, (int)D);
+    }
     NATS_CHECK_LAUNCH("decode_merge_kernel");
     return NATS_OK;
   }

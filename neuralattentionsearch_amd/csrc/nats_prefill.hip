@@ -87,7 +87,7 @@ __device__ __forceinline__ void store_from_f32<uint16_t>(uint16_t* p, float x) {
 
 template <typename T, int D>
 __global__ __launch_bounds__(64) void prefill_simple_kernel(PrefillArgs a) {
-  constexpr int SUB = 32;
+  constexpr int SUB = D > 128 ? 16 : 32;  // (the staged K and V rows stay within the static LDS limit)
   __shared__ float Ks[SUB][D];
   __shared__ float Vs[SUB][D];
   __shared__ float Ss[SUB][kWave];
@@ -958,7 +958,8 @@ int check_common(const char* who, const SegmentShape& g, const int64_t* q_stride
                who, (long long)g.B, (long long)g.H_q, (long long)g.H_kv, (long long)g.x_len);
   NATS_REQUIRE(g.H_q % g.H_kv == 0, NATS_ERR_BAD_SHAPE, "%s: H_q=%lld is not a multiple of H_kv=%lld", who,
                (long long)g.H_q, (long long)g.H_kv);
-  NATS_REQUIRE(g.D == 64 || g.D == 128, NATS_ERR_UNSUPPORTED, "%s: head_dim %lld (supported: 64, 128)", who, (long long)g.D);
+  NATS_REQUIRE(g.D == 16 || g.D == 32 || g.D == 64 || g.D == 128 || g.D == 256, NATS_ERR_UNSUPPORTED,
+               "%s: head_dim %lld (supported: 16, 32, 64, 128, 256)", who, (long long)g.D);
   NATS_REQUIRE(is_pow2(g.C), NATS_ERR_UNSUPPORTED, "%s: chunk size %lld is not a power of two", who, (long long)g.C);
   NATS_REQUIRE(g.W >= 0 && g.W % g.C == 0, NATS_ERR_BAD_SHAPE, "%s: window %lld is not a multiple of chunk size %lld", who,
                (long long)g.W, (long long)g.C);
@@ -967,7 +968,7 @@ int check_common(const char* who, const SegmentShape& g, const int64_t* q_stride
   NATS_REQUIRE(k_strides[2] * kTile < (int64_t(1) << 30) && v_strides[2] * kTile < (int64_t(1) << 30) && k_strides[2] > 0 &&
                    v_strides[2] > 0,
                NATS_ERR_BAD_SHAPE, "%s: row strides %lld / %lld of k / v", who, (long long)k_strides[2], (long long)v_strides[2]);
-  if (dtype == NATS_DTYPE_BF16) {
+  if (dtype == NATS_DTYPE_BF16 && (g.D == 64 || g.D == 128)) {
     // 16-byte vector loads and stores of rows
     NATS_REQUIRE(q_strides[2] % 8 == 0 && k_strides[2] % 8 == 0 && v_strides[2] % 8 == 0 && o_strides[2] % 8 == 0 &&
                      q_strides[1] % 8 == 0 && k_strides[1] % 8 == 0 && v_strides[1] % 8 == 0 && o_strides[1] % 8 == 0 &&
@@ -1006,14 +1007,28 @@ int launch_segment(const char* who, const SegmentShape& g, const void* q, const 
   a.scale = sm_scale;
   a.hpw = 1; a.qpw = 1; a.n_hg = 1; a.n_qg = (int)n_qt; a.xcd_mode = 0;
 
-  if (dtype == NATS_DTYPE_F32) {
-    NATS_REQUIRE(g.B * g.H_q <= 65535, NATS_ERR_BAD_SHAPE, "%s: B*H_q too large for the fp32 kernel", who);
+  // fp32, and bf16 at the head dims the MFMA kernel does not take (16, 32, 256): the plain kernel
+  if (dtype == NATS_DTYPE_F32 || (g.D != 64 && g.D != 128)) {
+    NATS_REQUIRE(g.B * g.H_q <= 65535, NATS_ERR_BAD_SHAPE, "%s: B*H_q too large for the plain kernel", who);
     dim3 grid((unsigned)n_qt, (unsigned)(g.B * g.H_q));
-    if (g.D == 64) {
-      hipLaunchKernelGGL((prefill_simple_kernel<float, 64>), grid, dim3(64), 0, st, a);
-    } else {
-      hipLaunchKernelGGL((prefill_simple_kernel<float, 128>), grid, dim3(64), 0, st, a);
+    const bool f32 = dtype == NATS_DTYPE_F32;
+#define NATS_PREFILL_PLAIN(DD)                                                                     \
+  case DD:                                                                                         \
+    if (f32) {                                                                                     \
+      hipLaunchKernelGGL((prefill_simple_kernel<float, DD>), grid, dim3(64), 0, st, a);            \
+    } else {                                                                                       \
+      hipLaunchKernelGGL((prefill_simple_kernel<uint16_t, DD>), grid, dim3(64), 0, st, a);         \
+    }                                                                                              \
+    break;
+    switch (g.D) {
+      NATS_PREFILL_PLAIN(16)
+      NATS_PREFILL_PLAIN(32)
+      NATS_PREFILL_PLAIN(64)
+      NATS_PREFILL_PLAIN(128)
+      default:
+      NATS_PREFILL_PLAIN(256)
     }
+#undef NATS_PREFILL_PLAIN
     NATS_CHECK_LAUNCH("prefill_simple_kernel");
     return NATS_OK;
   }

@@ -38,12 +38,12 @@ def test_module_with_per_token_roles(lens, W):
     run_module(lens, 1, W)
 
 
-def run_module(lens, C, W, executor=None):
+def run_module(lens, C, W, executor=None, dim=512):
     from neuralattentionsearch_amd.attention import LlamaNAtSChunkAttentionLayer, apply_rotary_pos_emb
     from neuralattentionsearch_amd.cache import NAtSCache
     say("attention module", lens, C, W)
     torch.manual_seed(0)
-    B, dim, Hq, Hkv = 2, 512, 8, 2
+    B, Hq, Hkv = 2, 8, 2
     D = dim // Hq
     mod = LlamaNAtSChunkAttentionLayer(dim=dim, n_heads=Hq, n_kv_heads=Hkv, layer_id=0, local_seq_max_length=W,
                                        chunk_size=C).cuda().eval()
@@ -204,3 +204,9 @@ def test_module_with_an_executor_under_a_side_stream():
         run_module([300, 1, 1, 1, 120, 1, 1, 9, 200], 8, 16, executor=pool)
         run_module([200] + [1] * 20 + [90], 1, 16, executor=pool)
     side.synchronize()
+
+
+@pytest.mark.parametrize("dim", [128, 256, 2048])
+def test_module_with_other_head_dims(dim):
+    """Head dims 16, 32 and 256 (the reference's kernel accepts them too): prefill, segments and one-token steps."""
+    run_module([90, 1, 1, 40, 1, 1, 1, 17], 8, 16, dim=dim)

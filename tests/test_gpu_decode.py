@@ -104,6 +104,12 @@ def test_fp32(D):
     run_case(2, 4, 2, D, 128, 64, 12, torch.float32, seed=D, fill=3)
 
 
+@pytest.mark.parametrize("D", [16, 32, 256])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_other_head_dims(D, dtype):
+    run_case(2, 4, 2, D, 32, 8, 20, dtype, seed=D, fill=3)
+
+
 def test_strided_cache_views():
     """The cache handed over is a view of a larger capacity buffer, as the cache object does."""
     from neuralattentionsearch_amd import ops

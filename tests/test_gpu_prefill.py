@@ -53,6 +53,15 @@ def test_bf16_shapes(L, C, W, D):
     run_case(2, 8, 2, L, D, C, W, torch.bfloat16, seed=L + C)
 
 
+@pytest.mark.parametrize("D", [16, 32, 256])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_other_head_dims(D, dtype):
+    """The head dims the reference's kernel also accepts (models/transformer/triton/nats_flashattn_fwd.py:634) run
+    the plain kernel in both dtypes."""
+    run_case(2, 4, 2, 333, D, 8, 16, dtype, seed=D)
+    run_case(1, 2, 2, 200, D, 64, 128, dtype, seed=D + 1)
+
+
 def test_bf16_llama_head_shape_8_streams():
     # 32 q / 8 kv heads as in Llama-3-8B: exercises the XCD-aware workgroup mapping (B * H_kv % 8 == 0)
     run_case(1, 32, 8, 2048, 128, 64, 256, torch.bfloat16, seed=5, p=(0.05, 0.15, 0.8), scale_inputs=1 / math.sqrt(128) ** 0.5)
