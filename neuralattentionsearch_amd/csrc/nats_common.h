@@ -77,6 +77,7 @@ struct KeyLimArgs {
   int32_t* tok_lim;  // [streams, N] out, followed by one entry that holds -1 (the limit of a row nobody sees)
   int2* tile_lim;    // [streams, Tk] out {max, min}
   int2* gran_lim;    // [streams, Tk * 4] out {max, min} of every 16 rows
+  int32_t* ticket;   // out: one counter, set to zero (may be NULL)
   int Hkv, S, N, Tk, c_shift, C, W;
   int base, gmin, tail, seen, fill_last;
   int old_fill, token_mode;
@@ -88,6 +89,7 @@ struct PrefillWorkspace {
   int32_t* tok_lim;
   int2* tile_lim;
   int2* gran_lim;
+  int32_t* ticket;  // one counter, set to zero by the key-limit kernel (the attention kernel deals work from it)
   size_t bytes;
 };
 

@@ -41,6 +41,11 @@ struct PrefillArgs {
   int n_hg;      // head groups per kv head = n_rep / hpw
   int n_qg;      // query tile groups = ceil(n query tiles / qpw)
   int xcd_mode;  // 1: workgroups of one kv stream share an XCD (needs B*Hkv % 8 == 0)
+  // The query groups with the fewest visible keys (the last pool_ranks ranks of every stream) are not bound to a
+  // workgroup: the last workgroups of the grid draw one each from a counter (heaviest first), so that an XCD whose
+  // stream kept fewer keys visible, and which reaches its last workgroups earlier, takes the larger ones.
+  int pool_ranks;    // 0: every workgroup has its fixed query group
+  int32_t* ticket;   // the counter, zero at launch
   float scale;   // softmax scale
   // few query tiles over many key rows: n_split workgroups share the tile list of one (kv stream, head group,
   // query group) and leave partial results, which prefill_split_merge_kernel combines
@@ -213,6 +218,7 @@ struct PrefillSmem {
   int4 vlist[kWin];  // visited key tiles of the current window: {tile, max limit, min limit, -}
                      // packed tiles: the four 16-row granules of the tile ({id | mask flag, id, id, id}, -1 = none)
   int vcount;
+  int ticket;  // drawn pool item of this workgroup
 };
 constexpr int kGranPerTile = kTile / kGranule;
 constexpr int kPackedMaskFlag = 1 << 30;  // on the first granule id of a packed tile: some score of the tile is masked
@@ -224,8 +230,9 @@ constexpr int kPackedMaskFlag = 1 << 30;  // on the first granule id of a packed
 // the workgroup sees without a mask are packed among themselves and the rest (diagonal, partly visible, the remainder of the
 // first kind, padding) into tiles that go through the element mask.  The softmax does not care about the order
 // of the keys, so nothing else changes; without it a tile with one visible 16- or 32-row chunk costs a whole tile.
-template <int D, bool kUniform, bool kPacked = false>
-__global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(PrefillArgs a) {
+template <int D, bool kUniform, bool kPacked>
+__device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned char* smem_raw, int bid, int split, int ks,
+                                                  int hg, int rank) {
   static_assert(!kPacked || kUniform, "packed tiles are walked by every wavefront of the workgroup");
   constexpr int OCT = D / 8;                          // 16-byte chunks per row
   constexpr int DMA_PER_WAVE = OCT / kPrefillWaves;   // 1 KiB global->LDS transfers per wavefront and tensor
@@ -234,7 +241,6 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
   constexpr int kHalf = kTile / 2;
   static_assert(DMA_PER_WAVE >= 1, "tile rows are split over the wavefronts in 1 KiB transfers");
 
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   PrefillSmem<D>& sm = *reinterpret_cast<PrefillSmem<D>*>(smem_raw);
 
   const int tid = threadIdx.x;
@@ -245,15 +251,6 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
   const int l32 = lane & 31;
   const int hl = lane >> 5;
 
-  // ---- which (kv stream, head group, query group) -------------------------------------------------
-  int bid = blockIdx.x;
-  int split = 0;  // which share of the tile list (n_split > 1)
-  if (a.n_split > 1) {
-    split = bid % a.n_split;
-    bid /= a.n_split;
-  }
-  int ks, hg, rank;
-  map_workgroup(a, bid, ks, hg, rank);
   const int qg = a.n_qg - 1 - rank;  // heavy query groups first
   const int b = ks / a.Hkv, hkv = ks % a.Hkv;
   const int hq = hkv * a.n_rep + hg * a.hpw + (sub % a.hpw);
@@ -279,6 +276,16 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
   const int kt_end_group = (a.base + rlast_group) / kTile;
   const int my_kt_end = (a.base + tile_rlast) / kTile;
 
+  // ---- wavefront 0 asks for the tile summaries of the first kEarly * 64 key tiles before anything else is requested:
+  // memory operations complete in the order of their issue, so the wait for these (a trip to L2) does not include
+  // the Q rows (a trip to HBM), which stay in flight while the visit list is built and the first tiles are requested.
+  constexpr int kEarly = 8;
+  int2 tl_early[kEarly];
+  if (!kPacked && wave == 0) {
+#pragma unroll
+    for (int j = 0; j < kEarly; ++j) tl_early[j] = tl[min(j * kWave + lane, kt_end_group)];
+  }
+
   // ---- Q fragments: B operand, lane (query l32, k-group hl) --------------------------------------
   bf16x8 qreg[DSTEPS];
   {
@@ -299,6 +306,11 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
   float l_run = 0.f;
   const float c = a.scale * 1.4426950408889634f;
 
+  // V rows in LDS: the transposing read of a half wavefront covers 4 consecutive keys x 32 head dimensions (64 bytes
+  // of each row).  The 16-byte chunks of a row are permuted so that these four pieces fall into the four quarters of
+  // the 64 LDS banks: rows of 256 bytes (one row = all banks) move by a quarter per row, rows of 128 bytes (two rows
+  // = all banks) by a quarter per pair of rows.
+  auto v_swizzle = [](int row) { return OCT >= 16 ? (row & 3) << 2 : ((row >> 1) & 1) << 2; };
   // global -> LDS, one 64-key tile of K or of V; rows beyond N repeat row N-1 (their scores are masked,
   // so their probabilities are exactly 0 and a finite V row contributes nothing).  The lane's share of a
   // tile sits at fixed offsets from the tile's first row, computed once.
@@ -310,7 +322,7 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
     // (packed tiles: this wavefront's 8 rows of a tile lie in one granule; the offset counts from its first row)
     const int srow = kPacked ? row % kGranule : row;
     koff[j] = int(srow * a.ks_l + (pos ^ (row % OCT)) * 8);
-    voff[j] = int(srow * a.vs_l + (pos ^ ((row & 3) << 1)) * 8);
+    voff[j] = int(srow * a.vs_l + (pos ^ v_swizzle(row)) * 8);
   }
   auto issue_rows = [&](const uint16_t* base, int64_t stride, const int (&off)[DMA_PER_WAVE], uint16_t* dst, int kt,
                         bool is_v) {
@@ -328,7 +340,7 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
         const int q = inst * kWave + lane;
         const int row = q / OCT, pos = q % OCT;
         const int n = min(kt * kTile + row, a.N - 1);
-        const int chunk = is_v ? pos ^ ((row & 3) << 1) : pos ^ (row % OCT);
+        const int chunk = is_v ? pos ^ v_swizzle(row) : pos ^ (row % OCT);
         __builtin_amdgcn_global_load_lds(base + (int64_t)n * stride + chunk * 8,
                                          (uint32_t __attribute__((address_space(3)))*)(dst + inst * kWave * 8), 16, 0, 0);
       }
@@ -363,7 +375,7 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
         const int q = inst * kWave + lane;
         const int row = q / OCT, pos = q % OCT;
         const int n = min(gid * kGranule + row % kGranule, a.N - 1);
-        const int chunk = is_v ? pos ^ ((row & 3) << 1) : pos ^ (row % OCT);
+        const int chunk = is_v ? pos ^ v_swizzle(row) : pos ^ (row % OCT);
         __builtin_amdgcn_global_load_lds(base + (int64_t)n * stride + chunk * 8,
                                          (uint32_t __attribute__((address_space(3)))*)(dst + inst * kWave * 8), 16, 0, 0);
       }
@@ -407,8 +419,8 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
     const int half4 = (r16 & 1) * 4;
     const int row_lo = t * 16 + hl * 4 + (r16 >> 2);
     const int row_hi = row_lo + 8;
-    const uint16_t* pl = Vt + row_lo * D + ((chunk0 ^ ((row_lo & 3) << 1)) * 8) + half4;
-    const uint16_t* ph = Vt + row_hi * D + ((chunk0 ^ ((row_hi & 3) << 1)) * 8) + half4;
+    const uint16_t* pl = Vt + row_lo * D + ((chunk0 ^ v_swizzle(row_lo)) * 8) + half4;
+    const uint16_t* ph = Vt + row_hi * D + ((chunk0 ^ v_swizzle(row_hi)) * 8) + half4;
     bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((bf16x4 __attribute__((address_space(3)))*)pl);
     bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((bf16x4 __attribute__((address_space(3)))*)ph);
     bf16x8 va = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
@@ -430,6 +442,29 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
           sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qreg[s], sacc[kb], 0, 0, 0);
         }
       }
+    }
+  };
+  // The scores of the first tile of a list have nothing to run under: every K fragment is requested before the first
+  // matrix instruction, so that the LDS latency is paid once and not once per pair of instructions.
+  auto qk_tile_first = [&](int buf, f32x16 (&sacc)[2]) {
+    const uint16_t* Kt = sm.k[buf];
+    constexpr int N_QK = 2 * DSTEPS;
+    constexpr int AHEAD = N_QK < 8 ? N_QK : 8;  // fragments in flight
+    bf16x8 kf[AHEAD];
+#pragma unroll
+    for (int i = 0; i < AHEAD; ++i) kf[i] = k_frag(Kt, i & 1, i >> 1);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < N_QK; ++i) {
+      const int s = i >> 1, kb = i & 1;
+      if (s == 0) {
+        const f32x16 z = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i % AHEAD], qreg[s], z, 0, 0, 0);
+      } else {
+        sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i % AHEAD], qreg[s], sacc[kb], 0, 0, 0);
+      }
+      if (i + AHEAD < N_QK) kf[i % AHEAD] = k_frag(Kt, (i + AHEAD) & 1, (i + AHEAD) >> 1);
+      __builtin_amdgcn_sched_barrier(0);
     }
   };
   // ---- mask of a diagonal tile, or of a tile whose rows are not uniformly visible ---------------------
@@ -579,6 +614,48 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
 #pragma unroll
     for (int i = 0; i < 16; ++i) sacc[kb][i] = 0.f;
 
+  // Visit list of a window of whole tiles: wavefront 0 compacts the tiles some query of the group sees.  (The first
+  // window is built ahead of the window loop, from the summaries requested at the top of the kernel, so that those do
+  // not stay in registers through the tile loop.)
+  auto compact_round = [&](int t, int2 val, int& count) {
+    const bool v = t <= kt_end_group && val.x >= r0_group;
+    const uint64_t bits = __ballot(v);
+    if (v) sm.vlist[count + __builtin_popcountll(bits & ((uint64_t(1) << lane) - 1))] = make_int4(t, val.x, val.y, 0);
+    count += __builtin_popcountll(bits);
+  };
+  auto build_list = [&](int w0, bool first) {
+    // (rounds beyond the last tile the group may see are skipped: the tests on j are uniform)
+    int2 vals[kWin / kWave];
+#pragma unroll
+    for (int j = 0; j < kWin / kWave; ++j) {
+      if (w0 + j * kWave <= kt_end_group) {
+        if (first && j < kEarly) {
+          vals[j] = tl_early[j];
+        } else {
+          vals[j] = tl[min(w0 + j * kWave + lane, kt_end_group)];
+        }
+      }
+    }
+    int count = 0;
+#pragma unroll
+    for (int j = 0; j < kWin / kWave; ++j)
+      if (w0 + j * kWave <= kt_end_group) compact_round(w0 + j * kWave + lane, vals[j], count);
+    if (lane == 0) sm.vcount = count;
+  };
+  if (!kPacked && wave == 0) {
+    if (kt_end_group < kEarly * kWave) {
+      // every tile summary the list needs was requested at the top: nothing else is loaded here, and the wait for
+      // the summaries leaves the Q rows in flight
+      int count = 0;
+#pragma unroll
+      for (int j = 0; j < kEarly; ++j)
+        if (j * kWave <= kt_end_group) compact_round(j * kWave + lane, tl_early[j], count);
+      if (lane == 0) sm.vcount = count;
+    } else {
+      build_list(0, true);
+    }
+  }
+
   // (packed tiles: the window counts granules, and leaves room for the one tile the packing can add)
   const int g_end_group = (a.base + rlast_group) / kGranule;
   const int win_last = kPacked ? g_end_group : kt_end_group;
@@ -638,24 +715,7 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
       }
       if (lane == 0) sm.vcount = n_pt + n_mt;
     }
-    if (!kPacked && wave == 0) {
-      int2 vals[kWin / kWave];
-#pragma unroll
-      for (int j = 0; j < kWin / kWave; ++j) {
-        int t = w0 + j * kWave + lane;
-        vals[j] = t <= kt_end_group ? tl[t] : make_int2(-1, -1);
-      }
-      int count = 0;
-#pragma unroll
-      for (int j = 0; j < kWin / kWave; ++j) {
-        int t = w0 + j * kWave + lane;
-        bool v = t <= kt_end_group && vals[j].x >= r0_group;
-        uint64_t bits = __ballot(v);
-        if (v) sm.vlist[count + __builtin_popcountll(bits & ((uint64_t(1) << lane) - 1))] = make_int4(t, vals[j].x, vals[j].y, 0);
-        count += __builtin_popcountll(bits);
-      }
-      if (lane == 0) sm.vcount = count;
-    }
+    if (!kPacked && wave == 0 && w0 > 0) build_list(w0, false);
     __syncthreads();
     int n_vis = __builtin_amdgcn_readfirstlane(sm.vcount);
     int j0 = 0;  // first list entry of this workgroup's share
@@ -754,7 +814,7 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
       load_k(2, e2);
       __builtin_amdgcn_s_waitcnt(0);
       __syncthreads();
-      if (visits(e0.kt, e0.emax)) qk_tile(0, sacc);
+      if (visits(e0.kt, e0.emax)) qk_tile_first(0, sacc);
       __syncthreads();  // k[0] is overwritten by the first step
 
       for (int t = 0; t < n_vis; t += 2) {
@@ -829,6 +889,34 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
       }
     }
   }
+}
+
+// One (kv stream, head group, query group) per workgroup.  The workgroups at the end of the grid have no query group
+// of their own: each draws one of the pooled ones (the lightest of every stream, heaviest first) from a counter, so
+// that the XCDs whose streams kept fewer keys visible, and which get there earlier, take the larger ones.
+template <int D, bool kUniform, bool kPacked = false>
+__global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(PrefillArgs a) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  PrefillSmem<D>& sm = *reinterpret_cast<PrefillSmem<D>*>(smem_raw);
+  int bid = blockIdx.x;
+  int split = 0;  // which share of the tile list (n_split > 1)
+  if (a.n_split > 1) {
+    split = bid % a.n_split;
+    bid /= a.n_split;
+  }
+  const int ns = a.B * a.Hkv * a.n_hg;
+  int ks, hg, rank;
+  if (a.pool_ranks > 0 && bid >= (a.n_qg - a.pool_ranks) * ns) {
+    if (threadIdx.x == 0) sm.ticket = atomicAdd(a.ticket, 1);
+    __syncthreads();
+    const int t = __builtin_amdgcn_readfirstlane(sm.ticket);
+    rank = a.n_qg - a.pool_ranks + t / ns;
+    ks = (t % ns) / a.n_hg;
+    hg = (t % ns) % a.n_hg;
+  } else {
+    map_workgroup(a, bid, ks, hg, rank);
+  }
+  prefill_mfma_item<D, kUniform, kPacked>(a, smem_raw, bid, split, ks, hg, rank);
 }
 
 // Combines the partial results of the n_split workgroups that shared one tile list: grid = (the workgroups of the
@@ -1072,6 +1160,17 @@ int launch_segment(const char* who, const SegmentShape& g, const void* q, const 
     }
     NATS_CHECK_LAUNCH("prefill_split_merge_kernel");
     return NATS_OK;
+  }
+  // A launch of several rounds of workgroups per compute unit draws its lightest query groups from the counter
+  // (NATS_PREFILL_POOL = eighths of the query groups that are drawn, 0 = none).
+  {
+    const char* e = getenv("NATS_PREFILL_POOL");
+    const int eighths = e ? atoi(e) : 3;
+    const int n_cu = device_cu_count();
+    if (eighths > 0 && eighths <= 8 && w.ticket && n_cu > 0 && n_wg >= 4 * (int64_t)n_cu) {
+      a.pool_ranks = (int)((int64_t)a.n_qg * eighths / 8);
+      a.ticket = w.ticket;
+    }
   }
   // chunks shorter than a tile: tiles are packed from the 16-row granules that are visible (NATS_PREFILL_PACKED=0
   // in the environment keeps whole tiles, for comparison)

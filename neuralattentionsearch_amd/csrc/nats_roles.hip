@@ -128,6 +128,7 @@ __global__ __launch_bounds__(256) void key_lim_kernel(KeyLimArgs a) {
   const int stream = blockIdx.y;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int tile = blockIdx.x * 4 + wave;
+  if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0 && a.ticket) *a.ticket = 0;
   if (tile >= a.Tk) return;
   const int row = tile * kTile + lane;
   int32_t lim = -1;
@@ -272,6 +273,8 @@ PrefillWorkspace carve_prefill_workspace(void* ws, int64_t n_streams, int64_t S,
   off += up((size_t)(n_streams * Tk) * sizeof(int2));
   w.gran_lim = reinterpret_cast<int2*>(p + off);
   off += up((size_t)(n_streams * Tk * (kTile / kGranule)) * sizeof(int2));
+  w.ticket = reinterpret_cast<int32_t*>(p + off);
+  off += up(sizeof(int32_t));
   w.bytes = off;
   return w;
 }
@@ -287,6 +290,7 @@ int prepare_key_limits(const uint8_t* roles, int64_t B, int64_t H_kv, int64_t S,
   a.tok_lim = w.tok_lim;
   a.tile_lim = w.tile_lim;
   a.gran_lim = w.gran_lim;
+  a.ticket = w.ticket;
   a.Hkv = (int)H_kv; a.S = (int)S; a.N = (int)N; a.Tk = (int)((N + kTile - 1) / kTile);
   a.c_shift = ilog2(C); a.C = (int)C; a.W = (int)W;
   if (past) {
