@@ -884,8 +884,9 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
       const int row = id / OCT, piece = id % OCT;
       const int qtok = q0 + row;
       if (qtok >= a.r_begin && qtok < a.r_end) {
-        uint4 val = *reinterpret_cast<const uint4*>(stage + row * kRowPitch + piece * 16);
-        *reinterpret_cast<uint4*>(op + (int64_t)(qtok - a.r_begin) * a.os_l + piece * 8) = val;
+        // (streaming store: the output is written once and read by nobody here; it should not displace K / V tiles in L2)
+        const u32x4 val = *reinterpret_cast<const u32x4*>(stage + row * kRowPitch + piece * 16);
+        __builtin_nontemporal_store(val, reinterpret_cast<u32x4*>(op + (int64_t)(qtok - a.r_begin) * a.os_l + piece * 8));
       }
     }
   }
