@@ -30,13 +30,55 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-# HBM bytes per launch of the dominant kernels at the default workloads, from rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE scaled by a 1 GiB device copy (read factor 2.0, write factor 1.0); see profiles/.
-MEASURED_TRAFFIC = {  # bytes read + written per launch
-    "prefill": 225859 * 1024 * 2.0 + 262144 * 1024 * 1.0,
-    "decode": 889921 * 1024 * 2.0 + 1562 * 1024 * 1.0,
-    "evict": 272468 * 1024 * 2.0 + 554048 * 1024 * 1.0,
+# HBM bytes per launch of the dominant kernels at the default workloads come from profiler counter runs
+# (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, KiB per dispatch, scaled by what a 1 GiB device copy reads on the same
+# counters).  They are kept in bench_traffic.json together with a hash of the kernel sources they were measured on:
+# once a source has changed the figure is no longer reported (traffic: null) until the counters are read again and
+# recorded with `python bench.py --record-traffic prefill=<FETCH KiB>,<WRITE KiB> ...`.
+TRAFFIC_FILE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "bench_traffic.json")
+TRAFFIC_SOURCES = {
+    "prefill": ["nats_prefill.hip", "nats_roles.hip", "nats_common.h"],
+    "decode": ["nats_decode.hip", "nats_common.h"],
+    "evict": ["nats_evict.hip", "nats_common.h"],
 }
+
+
+def source_hash(names) -> str:
+    import hashlib
+    h = hashlib.sha256()
+    for n in names:
+        with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "neuralattentionsearch_amd", "csrc", n), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(key: str):
+    """(bytes read + written per launch, note) of a dominant kernel; bytes is None when there is no current figure."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            table = json.load(f)
+        e = table["kernels"][key]
+    except (OSError, KeyError, ValueError):
+        return None, "no counter figures recorded"
+    if e["source_hash"] != source_hash(TRAFFIC_SOURCES[key]):
+        return None, "kernel sources changed since the counters were read (" + e["profile"] + ")"
+    cal = table["calibration"]
+    return e["fetch_kib"] * 1024 * cal["fetch_factor"] + e["write_kib"] * 1024 * cal["write_factor"], e["profile"]
+
+
+def record_traffic(items):
+    """--record-traffic key=fetch_kib,write_kib ...: stores the figures with the hash of the present sources."""
+    with open(TRAFFIC_FILE) as f:
+        table = json.load(f)
+    for it in items:
+        key, vals = it.split("=")
+        fetch, write = (float(x) for x in vals.split(","))
+        table["kernels"][key].update(fetch_kib=fetch, write_kib=write, source_hash=source_hash(TRAFFIC_SOURCES[key]))
+    with open(TRAFFIC_FILE, "w") as f:
+        json.dump(table, f, indent=1)
+        f.write("\n")
+
+
 PEAK_HBM_GBS = 8000.0
 PEAK_BF16_TFLOPS = 2500.0
 METRIC = "NAtS prefill ms @32k (MFMA util); sparse-KV decode tok/s (HBM GB/s %peak)"
@@ -493,10 +535,15 @@ def main():
     ap.add_argument("--segments", type=int, default=4, help="segments of the `--only segments` leg")
     ap.add_argument("--segment-len", type=int, default=0, help="tokens per segment (default: prefill length / segments)")
     ap.add_argument("--only", choices=["prefill", "decode", "evict", "copy", "evict_stream", "segments", "role_step", "matvec", "llama"], default=None)
+    ap.add_argument("--record-traffic", nargs="+", metavar="KEY=FETCH_KIB,WRITE_KIB",
+                    help="store counter figures of prefill / decode / evict in bench_traffic.json and exit")
     ap.add_argument("--no-llama", action="store_true", help="skip the end-to-end Llama-3-8B-shape leg of the default run")
     ap.add_argument("--llama-prefill", type=int, default=16384)
     ap.add_argument("--llama-decode", type=int, default=512)
     args = ap.parse_args()
+    if args.record_traffic:
+        record_traffic(args.record_traffic)
+        return
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures the one-GPU hot path; it does not run on more than one GPU (--gpus 1 only)",
               file=sys.stderr)
@@ -546,18 +593,21 @@ def main():
     if pre:
         line["roofline"] = {"bound": "mfma", "achieved": pre["tflops_visited"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                             "frac": pre["tflops_visited"] / PEAK_BF16_TFLOPS,
-                            "traffic": MEASURED_TRAFFIC["prefill"] if args.prefill_len == 32768 and args.chunk_size == 64 else None,
                             "kernel": "prefill_mfma_kernel<128, true>"}
+        line["roofline"]["traffic"], line["roofline"]["traffic_source"] = (
+            measured_traffic("prefill") if args.prefill_len == 32768 and args.chunk_size == 64 else (None, "not the profiled workload"))
     if "decode" in res:
         d = res["decode"]
         line["roofline_decode"] = {"bound": "hbm", "achieved": d["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                                   "frac": d["frac_of_hbm_peak"], "traffic": MEASURED_TRAFFIC["decode"],
+                                   "frac": d["frac_of_hbm_peak"],
                                    "kernel": "decode_split_mfma_kernel<128,4> + decode_merge_balanced_kernel"}
+        line["roofline_decode"]["traffic"], line["roofline_decode"]["traffic_source"] = measured_traffic("decode")
     if "evict" in res:
         e = res["evict"]
         line["roofline_evict"] = {"bound": "hbm", "achieved": e["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                                  "frac": e["frac_of_hbm_peak"], "traffic": MEASURED_TRAFFIC["evict"],
+                                  "frac": e["frac_of_hbm_peak"],
                                   "kernel": "evict_plan_* + evict_apply_first_kernel (whole post_update)"}
+        line["roofline_evict"]["traffic"], line["roofline_evict"]["traffic_source"] = measured_traffic("evict")
     line["cpu_baseline"] = cpu
     if args.only in (None, "llama") and not args.no_llama:
         # the end-to-end workload: last, so that the kernel legs above are timed on a GPU that holds nothing else
