@@ -42,8 +42,8 @@ struct PrefillArgs {
   int n_qg;      // query tile groups = ceil(n query tiles / qpw)
   int xcd_mode;  // 1: workgroups of one kv stream share an XCD (needs B*Hkv % 8 == 0)
   // The query groups with the fewest visible keys (the last pool_ranks ranks of every stream) are not bound to a
-  // workgroup: the last workgroups of the grid draw one each from a counter (heaviest first), so that an XCD whose
-  // stream kept fewer keys visible, and which reaches its last workgroups earlier, takes the larger ones.
+  // workgroup: the last workgroups of the grid draw them from a counter (heaviest first) for as long as there are any,
+  // so that an XCD that reaches its last workgroups earlier takes more of them.
   int pool_ranks;    // 0: every workgroup has its fixed query group
   int32_t* ticket;   // the counter, zero at launch
   float scale;   // softmax scale
@@ -893,31 +893,49 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
 }
 
 // One (kv stream, head group, query group) per workgroup.  The workgroups at the end of the grid have no query group
-// of their own: each draws one of the pooled ones (the lightest of every stream, heaviest first) from a counter, so
-// that the XCDs whose streams kept fewer keys visible, and which get there earlier, take the larger ones.
+// of their own: they draw the pooled ones (the lightest of every stream, heaviest first) from a counter for as long
+// as there are any.  XCDs do not finish their fixed share at the same time (streams differ in how many keys their
+// roles keep visible, and the XCDs of one device differ in speed by a few percent): those that get to the pool
+// earlier take more of it.  The tile loop exists twice in the code, once for each kind of workgroup, so that the
+// loop around the pooled one costs the other nothing.
 template <int D, bool kUniform, bool kPacked = false>
-__global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(PrefillArgs a) {
+__global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(PrefillArgs args) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  PrefillSmem<D>& sm = *reinterpret_cast<PrefillSmem<D>*>(smem_raw);
   int bid = blockIdx.x;
   int split = 0;  // which share of the tile list (n_split > 1)
-  if (a.n_split > 1) {
-    split = bid % a.n_split;
-    bid /= a.n_split;
+  if (args.n_split > 1) {
+    split = bid % args.n_split;
+    bid /= args.n_split;
   }
-  const int ns = a.B * a.Hkv * a.n_hg;
-  int ks, hg, rank;
-  if (a.pool_ranks > 0 && bid >= (a.n_qg - a.pool_ranks) * ns) {
+  if (args.pool_ranks == 0 || bid < (args.n_qg - args.pool_ranks) * args.B * args.Hkv * args.n_hg) {
+    int ks, hg, rank;
+    map_workgroup(args, bid, ks, hg, rank);
+    prefill_mfma_item<D, kUniform, kPacked>(args, smem_raw, bid, split, ks, hg, rank);
+    return;
+  }
+  // The arguments are read afresh for every item (through a pointer the compiler cannot see through), so that none of
+  // them has to stay in a register from one item to the next.
+  PrefillSmem<D>& sm = *reinterpret_cast<PrefillSmem<D>*>(smem_raw);
+  static_assert(sizeof(PrefillArgs) % 4 == 0, "copied in 32-bit words");
+  struct ArgWords {
+    uint32_t w[sizeof(PrefillArgs) / 4];
+  };
+  auto argp = __builtin_amdgcn_kernarg_segment_ptr();
+  for (;;) {
+    asm volatile("" : "+s"(argp));
+    ArgWords aw;
+#pragma unroll
+    for (unsigned i = 0; i < sizeof(PrefillArgs) / 4; ++i) aw.w[i] = ((const __attribute__((opencl_constant)) uint32_t*)argp)[i];
+    const PrefillArgs a = __builtin_bit_cast(PrefillArgs, aw);
     if (threadIdx.x == 0) sm.ticket = atomicAdd(a.ticket, 1);
     __syncthreads();
     const int t = __builtin_amdgcn_readfirstlane(sm.ticket);
-    rank = a.n_qg - a.pool_ranks + t / ns;
-    ks = (t % ns) / a.n_hg;
-    hg = (t % ns) % a.n_hg;
-  } else {
-    map_workgroup(a, bid, ks, hg, rank);
+    const int ns = a.B * a.Hkv * a.n_hg;
+    if (t >= a.pool_ranks * ns) break;
+    prefill_mfma_item<D, kUniform, kPacked>(a, smem_raw, bid, split, (t % ns) / a.n_hg, (t % ns) % a.n_hg,
+                                            a.n_qg - a.pool_ranks + t / ns);
+    __syncthreads();  // the output staging of this item and the ticket are read before the next item writes LDS
   }
-  prefill_mfma_item<D, kUniform, kPacked>(a, smem_raw, bid, split, ks, hg, rank);
 }
 
 // Combines the partial results of the n_split workgroups that shared one tile list: grid = (the workgroups of the
@@ -1166,7 +1184,7 @@ int launch_segment(const char* who, const SegmentShape& g, const void* q, const 
   // (NATS_PREFILL_POOL = eighths of the query groups that are drawn, 0 = none).
   {
     const char* e = getenv("NATS_PREFILL_POOL");
-    const int eighths = e ? atoi(e) : 3;
+    const int eighths = e ? atoi(e) : 2;
     const int n_cu = device_cu_count();
     if (eighths > 0 && eighths <= 8 && w.ticket && n_cu > 0 && n_wg >= 4 * (int64_t)n_cu) {
       a.pool_ranks = (int)((int64_t)a.n_qg * eighths / 8);
