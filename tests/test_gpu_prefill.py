@@ -357,6 +357,42 @@ def test_rising_scores_in_split_lists_and_the_decode_kernel(split_lists):
         cache.post_update(n)
 
 
+@pytest.fixture
+def pooled_groups(monkeypatch):
+    def switch(eighths: int | None):
+        if eighths is None:
+            monkeypatch.delenv("NATS_PREFILL_POOL", raising=False)
+        else:
+            monkeypatch.setenv("NATS_PREFILL_POOL", str(eighths))
+    yield switch
+    monkeypatch.delenv("NATS_PREFILL_POOL", raising=False)
+
+
+@pytest.mark.parametrize("Hq,Hkv,L,C,W", [(32, 8, 32768, 64, 256),   # cfg2: eight streams, one per XCD
+                                          (24, 6, 12000, 64, 128),    # streams that do not fill the XCDs evenly
+                                          (8, 8, 20000, 32, 128),     # packed tiles, four query tiles per workgroup
+                                          (16, 8, 4096, 64, 256)])    # too few workgroups: nothing is pooled
+def test_pooled_query_groups_change_nothing(pooled_groups, Hq, Hkv, L, C, W):
+    """Large launches deal their lightest query groups from a counter.  Who computes a query group does not change
+    what is computed: the output is the same, bit for bit, with the pool switched off, at another pool size, and on a
+    second launch (the counter starts from zero every time)."""
+    from neuralattentionsearch_amd import ops
+    say("prefill pooled query groups", Hq, Hkv, L, C, W)
+    B, D = 1, 128
+    g = torch.Generator(device="cuda").manual_seed(3)
+    q = (torch.randn(B, Hq, L, D, generator=g, device="cuda") * 2.0).bfloat16()
+    k = (torch.randn(B, Hkv, L, D, generator=g, device="cuda") * 2.0).bfloat16()
+    v = torch.randn(B, Hkv, L, D, generator=g, device="cuda").bfloat16()
+    roles = to_dev(draw_roles(5, B, Hkv, -(-L // C), p=(0.05, 0.15, 0.8)))
+    outs = []
+    for eighths in (0, None, None, 5, 8):
+        pooled_groups(eighths)
+        outs.append(ops.prefill_attention(q, k, v, roles, C, W))
+    assert torch.isfinite(outs[0].float()).all()
+    for o in outs[1:]:
+        assert torch.equal(o, outs[0])
+
+
 def test_two_prefills_on_two_streams_equal_the_serial_results():
     """Scratch buffers are kept per stream: launches that run side by side on two streams do not share key limits."""
     from neuralattentionsearch_amd import ops
