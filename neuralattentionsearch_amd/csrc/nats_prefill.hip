@@ -42,10 +42,10 @@ struct PrefillArgs {
   int n_qg;      // query tile groups = ceil(n query tiles / qpw)
   int xcd_mode;  // 1: workgroups of one kv stream share an XCD (needs B*Hkv % 8 == 0)
   // The query groups with the fewest visible keys (the last pool_ranks ranks of every stream) are not bound to a
-  // workgroup: the last workgroups of the grid draw them from a counter (heaviest first) for as long as there are any,
-  // so that an XCD that reaches its last workgroups earlier takes more of them.
+  // workgroup: a few workgroups at the end of the grid draw them from counters, one queue per XCD (heaviest first),
+  // for as long as there are any, so that an XCD that reaches its last workgroups earlier takes more of them.
   int pool_ranks;    // 0: every workgroup has its fixed query group
-  int32_t* ticket;   // the counter, zero at launch
+  int32_t* ticket;   // one counter per XCD, kTicketStride entries apart, zero at launch
   float scale;   // softmax scale
   // few query tiles over many key rows: n_split workgroups share the tile list of one (kv stream, head group,
   // query group) and leave partial results, which prefill_split_merge_kernel combines
@@ -197,6 +197,7 @@ constexpr float kRescaleSlack = 8.0f;
 constexpr int kPrefillWaves = 8;
 constexpr int kMaxSplit = 32;  // workgroups that may share one tile list
 constexpr int kMaxDevices = 64;
+constexpr int kTicketStride = 32;  // int32 entries between the pool counters of two XCDs (128 bytes)
 
 // both halves of the wavefront get max / sum over lane and lane ^ 32 (one cross-half swap, no LDS round trip)
 __device__ __forceinline__ float half_swap_max(float v) {
@@ -218,7 +219,8 @@ struct PrefillSmem {
   int4 vlist[kWin];  // visited key tiles of the current window: {tile, max limit, min limit, -}
                      // packed tiles: the four 16-row granules of the tile ({id | mask flag, id, id, id}, -1 = none)
   int vcount;
-  int ticket;  // drawn pool item of this workgroup
+  int ticket;  // drawn pool item of this workgroup (-1: none left) and the queue it came from
+  int queue;
 };
 constexpr int kGranPerTile = kTile / kGranule;
 constexpr int kPackedMaskFlag = 1 << 30;  // on the first granule id of a packed tile: some score of the tile is masked
@@ -892,10 +894,10 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
   }
 }
 
-// One (kv stream, head group, query group) per workgroup.  The workgroups at the end of the grid have no query group
-// of their own: they draw the pooled ones (the lightest of every stream, heaviest first) from a counter for as long
-// as there are any.  XCDs do not finish their fixed share at the same time (streams differ in how many keys their
-// roles keep visible, and the XCDs of one device differ in speed by a few percent): those that get to the pool
+// One (kv stream, head group, query group) per workgroup.  The workgroups at the end of the grid (two per compute
+// unit) have no query group of their own: they draw the pooled ones (the lightest of every stream) from counters for
+// as long as there are any.  XCDs do not finish their fixed share at the same time (streams differ in how many keys
+// their roles keep visible, and the XCDs of one device differ in speed by a few percent): those that get to the pool
 // earlier take more of it.  The tile loop exists twice in the code, once for each kind of workgroup, so that the
 // loop around the pooled one costs the other nothing.
 template <int D, bool kUniform, bool kPacked = false>
@@ -913,6 +915,9 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
     prefill_mfma_item<D, kUniform, kPacked>(args, smem_raw, bid, split, ks, hg, rank);
     return;
   }
+  // Pooled query groups wait in one queue per XCD (that of their stream, heaviest first; every counter in a 128-byte
+  // line of its own).  A workgroup empties the queue of its own XCD, whose L2 holds the stream's tiles; then it looks
+  // at all counters, moves on to the fullest queue (twice at most), or ends.
   // The arguments are read afresh for every item (through a pointer the compiler cannot see through), so that none of
   // them has to stay in a register from one item to the next.
   PrefillSmem<D>& sm = *reinterpret_cast<PrefillSmem<D>*>(smem_raw);
@@ -921,19 +926,43 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
     uint32_t w[sizeof(PrefillArgs) / 4];
   };
   auto argp = __builtin_amdgcn_kernarg_segment_ptr();
+  int q = args.xcd_mode ? (bid & 7) : 0;
+  int moves = 0;  // queues of other XCDs this workgroup has moved on to (thread 0 keeps count)
   for (;;) {
     asm volatile("" : "+s"(argp));
     ArgWords aw;
 #pragma unroll
     for (unsigned i = 0; i < sizeof(PrefillArgs) / 4; ++i) aw.w[i] = ((const __attribute__((opencl_constant)) uint32_t*)argp)[i];
     const PrefillArgs a = __builtin_bit_cast(PrefillArgs, aw);
-    if (threadIdx.x == 0) sm.ticket = atomicAdd(a.ticket, 1);
+    const int nq = a.xcd_mode ? 8 : 1;
+    const int n_x = a.B * a.Hkv * a.n_hg / nq;  // items of one rank in one queue
+    const int qlen = a.pool_ranks * n_x;
+    if (threadIdx.x == 0) {
+      int t = atomicAdd(a.ticket + q * kTicketStride, 1);
+      if (t >= qlen && moves < 2 && nq > 1) {
+        int best = -1, best_left = 0;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const int left = qlen - __hip_atomic_load(a.ticket + i * kTicketStride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          if (left > best_left) best = i, best_left = left;
+        }
+        if (best >= 0) {
+          q = best;
+          ++moves;
+          t = atomicAdd(a.ticket + q * kTicketStride, 1);
+        }
+      }
+      sm.ticket = t < qlen ? t : -1;
+      sm.queue = q;
+    }
     __syncthreads();
     const int t = __builtin_amdgcn_readfirstlane(sm.ticket);
-    const int ns = a.B * a.Hkv * a.n_hg;
-    if (t >= a.pool_ranks * ns) break;
-    prefill_mfma_item<D, kUniform, kPacked>(a, smem_raw, bid, split, (t % ns) / a.n_hg, (t % ns) % a.n_hg,
-                                            a.n_qg - a.pool_ranks + t / ns);
+    const int q_now = __builtin_amdgcn_readfirstlane(sm.queue);
+    if (t < 0) break;
+    q = q_now;
+    const int sl = t % n_x;
+    const int ks = a.xcd_mode ? q + 8 * (sl / a.n_hg) : sl / a.n_hg;
+    prefill_mfma_item<D, kUniform, kPacked>(a, smem_raw, bid, split, ks, sl % a.n_hg, a.n_qg - a.pool_ranks + t / n_x);
     __syncthreads();  // the output staging of this item and the ticket are read before the next item writes LDS
   }
 }
@@ -1189,6 +1218,12 @@ int launch_segment(const char* who, const SegmentShape& g, const void* q, const 
     if (eighths > 0 && eighths <= 8 && w.ticket && n_cu > 0 && n_wg >= 4 * (int64_t)n_cu) {
       a.pool_ranks = (int)((int64_t)a.n_qg * eighths / 8);
       a.ticket = w.ticket;
+      // the drawing workgroups loop: two per compute unit are enough (the grid stays a multiple of 8, XCD by XCD)
+      const int64_t n_items = g.B * g.H_kv * a.n_hg;
+      const int64_t pooled = n_items * a.pool_ranks;
+      int64_t drawing = 2 * (int64_t)n_cu;
+      if (drawing > pooled) drawing = pooled;
+      n_wg = n_wg - pooled + (drawing + 7) / 8 * 8;
     }
   }
   // chunks shorter than a tile: tiles are packed from the 16-row granules that are visible (NATS_PREFILL_PACKED=0

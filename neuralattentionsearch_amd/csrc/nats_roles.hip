@@ -128,7 +128,7 @@ __global__ __launch_bounds__(256) void key_lim_kernel(KeyLimArgs a) {
   const int stream = blockIdx.y;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int tile = blockIdx.x * 4 + wave;
-  if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0 && a.ticket) *a.ticket = 0;
+  if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x < 8 && a.ticket) a.ticket[threadIdx.x * 32] = 0;
   if (tile >= a.Tk) return;
   const int row = tile * kTile + lane;
   int32_t lim = -1;
@@ -274,7 +274,7 @@ PrefillWorkspace carve_prefill_workspace(void* ws, int64_t n_streams, int64_t S,
   w.gran_lim = reinterpret_cast<int2*>(p + off);
   off += up((size_t)(n_streams * Tk * (kTile / kGranule)) * sizeof(int2));
   w.ticket = reinterpret_cast<int32_t*>(p + off);
-  off += up(sizeof(int32_t));
+  off += up(8 * 32 * sizeof(int32_t));  // eight counters, 128 bytes apart
   w.bytes = off;
   return w;
 }
