@@ -461,7 +461,7 @@ def cpu_baseline(args):
     """The oracle (a port of the reference's PyTorch path) on this host's cores, bounded samples."""
     from oracle import nats_oracle as orc
     cores = os.cpu_count() or 1
-    use = min(cores, 16)
+    use = min(cores, 16)  # (the CPU share of a one-GPU box, whatever its core count reads; reported as `cores`)
     torch.set_num_threads(use)
     D, C, W = 128, 64, 256
     samples = {}
