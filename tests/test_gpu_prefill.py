@@ -368,17 +368,20 @@ def pooled_groups(monkeypatch):
     monkeypatch.delenv("NATS_PREFILL_POOL", raising=False)
 
 
-@pytest.mark.parametrize("Hq,Hkv,L,C,W", [(32, 8, 32768, 64, 256),   # cfg2: eight streams, one per XCD
-                                          (24, 6, 12000, 64, 128),    # streams that do not fill the XCDs evenly
-                                          (8, 8, 20000, 32, 128),     # packed tiles, four query tiles per workgroup
-                                          (16, 8, 4096, 64, 256)])    # too few workgroups: nothing is pooled
-def test_pooled_query_groups_change_nothing(pooled_groups, Hq, Hkv, L, C, W):
+@pytest.mark.parametrize("B,Hq,Hkv,L,C,W", [(1, 32, 8, 32768, 64, 256),   # cfg2: eight streams, one per XCD
+                                            (1, 24, 6, 12000, 64, 128),    # streams that do not fill the XCDs evenly
+                                            (1, 8, 8, 20000, 32, 128),     # packed tiles, four query tiles per workgroup
+                                            (1, 64, 8, 6000, 64, 128),     # GQA groups of 8: two head groups per kv head
+                                            (2, 32, 8, 9000, 64, 256),     # sixteen streams: two per XCD queue
+                                            (3, 16, 8, 7000, 16, 64),      # 24 streams, packed tiles, groups of 2
+                                            (1, 16, 8, 4096, 64, 256)])    # too few workgroups: nothing is pooled
+def test_pooled_query_groups_change_nothing(pooled_groups, B, Hq, Hkv, L, C, W):
     """Large launches deal their lightest query groups from a counter.  Who computes a query group does not change
     what is computed: the output is the same, bit for bit, with the pool switched off, at another pool size, and on a
     second launch (the counter starts from zero every time)."""
     from neuralattentionsearch_amd import ops
-    say("prefill pooled query groups", Hq, Hkv, L, C, W)
-    B, D = 1, 128
+    say("prefill pooled query groups", B, Hq, Hkv, L, C, W)
+    D = 128
     g = torch.Generator(device="cuda").manual_seed(3)
     q = (torch.randn(B, Hq, L, D, generator=g, device="cuda") * 2.0).bfloat16()
     k = (torch.randn(B, Hkv, L, D, generator=g, device="cuda") * 2.0).bfloat16()
