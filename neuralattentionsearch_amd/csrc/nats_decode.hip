@@ -34,7 +34,8 @@ struct DecodeArgs {
   float scale;
   // balanced schedule of the bf16 kernel
   int2* head_table;  // [B*Hkv] {first partial slot, number of partials}
-  int n_wg;          // workgroups along x; every one takes the same number of 32-row tiles
+  int n_wg;          // workgroups along x
+  int share_first;   // 1/256ths of the tiles that go to the first half of the workgroups (128: equal shares)
 };
 
 __device__ __forceinline__ float exp2_guard(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -105,9 +106,10 @@ __device__ __forceinline__ void block_exclusive_scan(int* dst, int n, int* tmp) 
   __syncthreads();
 }
 
-// Balanced schedule: all 32-row tiles of all (b, kv head) streams form one list, cut into n_wg equal
-// ranges; a workgroup works through its range head by head and emits one partial (m, l, acc) per head it
-// touches.  No workgroup is empty and all finish together, whatever the per-head lengths are.
+// Balanced schedule: all 32-row tiles of all (b, kv head) streams form one list, cut into n_wg ranges (equal ones,
+// or larger ones for the first half of the workgroups, see decode_share_first); a workgroup works through its
+// range head by head and emits one partial (m, l, acc) per head it touches.  All finish together, whatever the
+// per-head lengths are.
 template <int D, int NREP>
 __global__ __launch_bounds__(256) void decode_split_mfma_kernel(DecodeArgs a) {
   constexpr int STEPS = D / 32;      // k-steps of the score MFMA
@@ -137,10 +139,16 @@ __global__ __launch_bounds__(256) void decode_split_mfma_kernel(DecodeArgs a) {
   __syncthreads();
   block_exclusive_scan(sm.tile_prefix, n_heads, sm.scan_tmp);
   const int total = sm.tile_prefix[n_heads];
-  const int tpw = (total + a.n_wg - 1) / a.n_wg;  // tiles per workgroup
+  // Tiles per workgroup: tpw_a for the first n_first workgroups (tiles [0, split)), tpw_b for the others.
+  const int n_first = a.share_first == 128 ? a.n_wg : a.n_wg / 2;
+  const int tpw_a = a.share_first == 128 ? (total + a.n_wg - 1) / a.n_wg
+                                         : max(1, (int)(((int64_t)total * a.share_first / 256 + n_first - 1) / n_first));
+  const int split = min(total, n_first * tpw_a);
+  const int tpw_b = max(1, (total - split + (a.n_wg - n_first) - 1) / max(1, a.n_wg - n_first));
+  auto wg_of = [&](int p) { return p < split ? p / tpw_a : n_first + (p - split) / tpw_b; };
   for (int h = tid; h < n_heads; h += 256) {
     int p0 = sm.tile_prefix[h], p1 = sm.tile_prefix[h + 1];
-    sm.slot_prefix[h] = p1 > p0 ? (p1 - 1) / tpw - p0 / tpw + 1 : 0;
+    sm.slot_prefix[h] = p1 > p0 ? wg_of(p1 - 1) - wg_of(p0) + 1 : 0;
   }
   __syncthreads();
   block_exclusive_scan(sm.slot_prefix, n_heads, sm.scan_tmp);
@@ -149,8 +157,8 @@ __global__ __launch_bounds__(256) void decode_split_mfma_kernel(DecodeArgs a) {
       a.head_table[h] = make_int2(sm.slot_prefix[h], sm.slot_prefix[h + 1] - sm.slot_prefix[h]);
     }
   }
-  int pos = wg * tpw;
-  const int pos_end = min(pos + tpw, total);
+  int pos = wg < n_first ? wg * tpw_a : split + (wg - n_first) * tpw_b;
+  const int pos_end = wg < n_first ? min(pos + tpw_a, split) : min(pos + tpw_b, total);
   if (pos >= pos_end) return;
   for (int h = tid; h < n_heads; h += 256) {
     if (sm.tile_prefix[h] <= pos && pos < sm.tile_prefix[h + 1]) sm.first_head = h;
@@ -222,7 +230,7 @@ __global__ __launch_bounds__(256) void decode_split_mfma_kernel(DecodeArgs a) {
     const int p0 = sm.tile_prefix[ks], p1 = sm.tile_prefix[ks + 1];
     const int seg_end = min(pos_end, p1);
     t_end = seg_end - p0;
-    slot = sm.slot_prefix[ks] + (wg - p0 / tpw);
+    slot = sm.slot_prefix[ks] + (wg - wg_of(p0));
     const int b = ks / a.Hkv, hkv = ks % a.Hkv;
     const int hq0 = hkv * a.n_rep + grp * NREP;
     kp = static_cast<const uint16_t*>(a.k) + b * a.ks_b + hkv * a.ks_h;
@@ -564,8 +572,7 @@ static void decode_split_geometry(int64_t B, int64_t H_kv, int64_t n_rows, int* 
   *nsplit = (int)((n_rows + 32 + r - 1) / r);
 }
 
-// workgroups of the balanced bf16 schedule: two per compute unit, fewer when there is little to do
-static int decode_balanced_workgroups(int64_t B, int64_t H_kv, int64_t n_rows) {
+static int compute_units_of_current_device() {
   static int n_cu_of[64] = {};  // compute units of every device, asked for once each
   int dev = 0, n_cu = 256;
   if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64) {
@@ -575,10 +582,30 @@ static int decode_balanced_workgroups(int64_t B, int64_t H_kv, int64_t n_rows) {
     }
     n_cu = n_cu_of[dev];
   }
+  return n_cu;
+}
+
+// workgroups of the balanced bf16 schedule: two per compute unit, fewer when there is little to do
+static int decode_balanced_workgroups(int64_t B, int64_t H_kv, int64_t n_rows) {
   int64_t upper = B * H_kv * ((n_rows + kDecTile - 1) / kDecTile + 1);  // tiles, at most
   int64_t want = (upper + 7) / 8;                                        // at least 8 tiles per workgroup
-  int64_t cap = 2 * (int64_t)n_cu;
+  int64_t cap = 2 * (int64_t)compute_units_of_current_device();
   return (int)(want < 1 ? 1 : (want > cap ? cap : want));
+}
+
+// Share of the tiles that the first half of the workgroups takes, in 1/256ths.  When the grid is exactly two
+// workgroups per compute unit, the first half of the grid is every unit's first resident workgroup, and that one
+// is served about twice as fast as the second while both are resident (measured with device timestamps: with equal
+// shares the first halves end after 210 us of a 285 us launch and the units then run half empty).  With 176/256 of
+// the tiles on the first half both halves end together.  NATS_DECODE_SHARE overrides the share (128: equal).
+static int decode_share_first(int n_wg, int groups) {
+  if (n_wg < 2 || n_wg % 2 != 0) return 128;
+  const char* e = getenv("NATS_DECODE_SHARE");
+  if (e) {
+    const int v = atoi(e);
+    return v > 0 && v < 256 ? v : 128;
+  }
+  return (groups == 1 && n_wg == 2 * compute_units_of_current_device()) ? 176 : 128;
 }
 
 static size_t align256(size_t x) { return (x + 255) & ~size_t(255); }
@@ -665,6 +692,7 @@ static int decode_fwd_impl(const void* q, const void* cache_k, const void* cache
   a.scale = sm_scale;
   a.head_table = nullptr;
   a.n_wg = 0;
+  a.share_first = 128;
   a.ws_acc = static_cast<float*>(workspace);
   a.ws_ml = a.ws_acc + (size_t)B * H_q * a.nsplit * D;
 
@@ -722,6 +750,7 @@ static int decode_fwd_impl(const void* q, const void* cache_k, const void* cache
     c.row_end = a.row_end ? a.row_end + b0 * H_kv : nullptr;
     c.o = static_cast<uint16_t*>(o) + b0 * H_q * D;
     c.n_wg = decode_balanced_workgroups(nb, H_kv, n_rows);
+    c.share_first = decode_share_first(c.n_wg, groups);
     c.head_table = static_cast<int2*>(workspace);
     c.ws_acc = reinterpret_cast<float*>(static_cast<char*>(workspace) + align256((size_t)(nb * H_kv) * sizeof(int2)));
     c.ws_ml = c.ws_acc + ((size_t)c.n_wg + (size_t)(nb * H_kv)) * (size_t)n_rep * D;
