@@ -81,6 +81,9 @@ class NAtSChunkLayerCache:
         self._await = None    # (sequence number, first) of an eviction whose scalars the host has not picked up yet
         self._redo = None     # what a first eviction launched on a guessed capacity needs if the guess was too small
         self._kept_share = None  # logical rows after the last first eviction / rows of the uncompacted cache
+        self._append_call = None  # ops.CacheAppendCall / ops.EvictInplaceCall prepared for the present buffers
+        self._inplace_call = None
+        self._inplace_params = None
         self.reset_cache()
 
     # -- state ----------------------------------------------------------------------------------
@@ -97,6 +100,7 @@ class NAtSChunkLayerCache:
         self._tokens_info = None
         self._roles = None
         self._buf_k = self._buf_v = self._buf_valid = self._buf_pos = None
+        self._append_call = self._inplace_call = None  # (they hold the buffers)
         self._n_rows = 0
         self._pending = None  # raw (K, V) of a first prefill not yet compacted
         self._last_result = None
@@ -318,9 +322,11 @@ class NAtSChunkLayerCache:
     def _write_rows(self, key_states, value_states, start: int, end: int):
         """Rows [start, end) of the cache, their valid bytes and stream positions: one kernel where the layouts
         allow 16-byte accesses, slice assignments otherwise."""
-        if ops.cache_append_ok(key_states, value_states, self._buf_k, self._buf_v):
-            ops.cache_append(key_states, value_states, self._buf_k, self._buf_v, self._buf_valid, self._buf_pos, start,
-                             self._seen_tokens)
+        call = self._append_call
+        if call is None or not call.matches(key_states, value_states, self._buf_k, self._buf_v, self._buf_valid, self._buf_pos):
+            call = self._append_call = ops.CacheAppendCall(key_states, value_states, self._buf_k, self._buf_v,
+                                                           self._buf_valid, self._buf_pos)
+        if call(key_states, value_states, start, self._seen_tokens):
             return
         self._buf_k[:, :, start:end] = key_states.to(self._buf_k.dtype)
         self._buf_v[:, :, start:end] = value_states.to(self._buf_v.dtype)
@@ -418,14 +424,30 @@ class NAtSChunkLayerCache:
         D = like.shape[3]
         if self._evict is None:
             self._evict = ops.EvictBuffers(self.device)
-        params = ops.evict_params(self.bsz, self.n_msks, D, C, W, S, x_len, fill, self.n_ctx_data, self._n_global_min,
-                                  self.sliding_queue_tail, first, max(self._rows, C))
-        ws, result = ops.evict_plan(roles, self.size_global_kv, self.size_local_kv, params, self._evict)
-        if src is None or not self._evict_first(src, roles, params, ws, result, first):
+        if src is None:
+            # a cache that holds rows: plan + in-place apply through the call prepared for these buffers
+            params = self._inplace_params
+            if params is None or params.D != D:
+                params = self._inplace_params = ops.evict_params(self.bsz, self.n_msks, D, C, W, S, 0, 0, 0, 0, 0, False, 0)
+            params.S, params.x_len, params.fill, params.first = S, x_len, fill, int(first)
+            params.n_ctx_data, params.gmin, params.tail = self.n_ctx_data, self._n_global_min, self.sliding_queue_tail
             params.n_alloc = self._rows
-            ops.evict_apply_inplace(self._buf_k, self._buf_v, self._buf_valid, self._buf_pos, roles, self.size_global_kv,
-                                    self.size_local_kv, params, ws, result)
+            call = self._inplace_call
+            if call is None or not call.matches(self._buf_k, self._buf_v, self._buf_valid, self._buf_pos, S):
+                call = self._inplace_call = ops.EvictInplaceCall(self._buf_k, self._buf_v, self._buf_valid, self._buf_pos,
+                                                                 self.size_global_kv, self.size_local_kv, self._evict,
+                                                                 self.bsz, self.n_msks, S)
+            call(roles, params)
             self._await = (params.seq, first)  # picked up when the host next needs n_ctx_data or the minimum global size
+        else:
+            params = ops.evict_params(self.bsz, self.n_msks, D, C, W, S, x_len, fill, self.n_ctx_data, self._n_global_min,
+                                      self.sliding_queue_tail, first, max(self._rows, C))
+            ws, result = ops.evict_plan(roles, self.size_global_kv, self.size_local_kv, params, self._evict)
+            if not self._evict_first(src, roles, params, ws, result, first):
+                params.n_alloc = self._rows
+                ops.evict_apply_inplace(self._buf_k, self._buf_v, self._buf_valid, self._buf_pos, roles,
+                                        self.size_global_kv, self.size_local_kv, params, ws, result)
+                self._await = (params.seq, first)
         # host-side bookkeeping (nats_chunk_layer_cache.py:400-413)
         n_ring = min(n_done, self.n_chunks_per_sw)
         start = 0 if first else self.sliding_queue_tail

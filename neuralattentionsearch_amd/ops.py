@@ -516,6 +516,78 @@ def cache_append(k: torch.Tensor, v: torch.Tensor, cache_k: torch.Tensor, cache_
                                         cache_k.element_size(), _stream(k)))
 
 
+class CacheAppendCall:
+    """`cache_append` for one pair of layouts (the new rows' and the cache's), with the checks made and the stride
+    arrays and buffer addresses prepared once: a caller that appends step after step into the same buffers pays one
+    library call per step.  `matches` says whether a prepared call still fits the tensors at hand."""
+
+    def __init__(self, k, v, cache_k, cache_v, valid, pos):
+        self.key = (k.shape, k.stride(), v.stride(), k.dtype, v.dtype, k.device)
+        self.bufs = (cache_k, cache_v, valid, pos)
+        self.ok = cache_append_ok(k, v, cache_k, cache_v)
+        if not self.ok:
+            return
+        e = 16 // cache_k.element_size()
+        fix = lambda t: tuple(st if n != 1 else e for st, n in zip(t.stride()[:3], t.shape[:3]))
+        B, H, x_len, D = k.shape
+        self.fn = _lib.load().nats_cache_append
+        self.head = (_ptr(cache_k), _ptr(cache_v), _ptr(valid), _ptr(pos), B, H, x_len, D)
+        self.n_rows = min(cache_k.shape[2], valid.shape[2])
+        self.tail = (i64_array(fix(k)), i64_array(fix(v)), i64_array(fix(cache_k)), i64_array(valid.stride()[:2]),
+                     cache_k.element_size())
+
+    def matches(self, k, v, cache_k, cache_v, valid, pos) -> bool:
+        b = self.bufs
+        return (b[0] is cache_k and b[1] is cache_v and b[2] is valid and b[3] is pos
+                and self.key == (k.shape, k.stride(), v.stride(), k.dtype, v.dtype, k.device))
+
+    def __call__(self, k, v, row0: int, pos0: int = 0) -> bool:
+        """Appends and returns True; False if these tensors cannot take the kernel (layout or alignment)."""
+        pk, pv = k.data_ptr(), v.data_ptr()
+        if not self.ok or (pk | pv) & 15:
+            return False
+        check(self.fn(pk, pv, *self.head, row0, self.n_rows, pos0, *self.tail, _stream(k)))
+        return True
+
+
+class EvictInplaceCall:
+    """Plan + in-place apply (`evict_plan`, `evict_apply_inplace`) for one set of cache buffers and role layout, checked
+    and prepared once; a call takes the roles of the step and the parameter struct."""
+
+    def __init__(self, cache_k, cache_v, valid, pos, size_global, size_local, buffers: "EvictBuffers", B, H_kv, S):
+        _require_cuda(cache_k, cache_v, valid, size_global, size_local)
+        if cache_k.shape != cache_v.shape or strides_differ(cache_k, cache_v) or cache_k.dtype != cache_v.dtype:
+            raise ValueError("cache_k and cache_v must share dtype and strides")
+        v8 = valid.view(torch.uint8) if valid.dtype == torch.bool else valid
+        if pos is not None and (pos.dtype != torch.int32 or pos.shape != v8.shape or strides_differ(pos, v8, 2)):
+            raise ValueError("pos must be int32 with the strides of valid")
+        lib = _lib.load()
+        self.bufs = (cache_k, cache_v, valid, pos)
+        self.S = S
+        self.buffers = buffers
+        ws = buffers.workspace(lib.nats_evict_workspace_bytes(B, H_kv, S))
+        self.ws = ws
+        self.plan, self.apply = lib.nats_evict_plan, lib.nats_evict_apply_inplace
+        self.sizes = (_ptr(size_global), _ptr(size_local))
+        self.plan_tail = (_ptr(ws), ws.numel(), _ptr(buffers.result), _ptr(buffers.mirror))
+        self.apply_head = (_ptr(cache_k), _ptr(cache_v), _ptr(v8), _ptr(pos))
+        self.apply_tail = (i64_array(cache_k.stride()[:3]), i64_array(v8.stride()[:2]), cache_k.element_size(), _ptr(ws),
+                           _ptr(buffers.result))
+
+    def matches(self, cache_k, cache_v, valid, pos, S) -> bool:
+        b = self.bufs
+        return (b[0] is cache_k and b[1] is cache_v and b[2] is valid and b[3] is pos and self.S == S
+                and self.ws is self.buffers.ws)
+
+    def __call__(self, roles: torch.Tensor, params: EvictParams):
+        if not roles.is_cuda or roles.dtype != torch.uint8 or not roles.is_contiguous():
+            raise ValueError("roles must be a contiguous uint8 GPU tensor")
+        params.seq = self.buffers.next_seq()
+        pr, ref, st = roles.data_ptr(), ctypes.byref(params), _stream(roles)
+        check(self.plan(pr, *self.sizes, ref, *self.plan_tail, st))
+        check(self.apply(*self.apply_head, pr, *self.sizes, ref, *self.apply_tail, st))
+
+
 def evict_apply_inplace(cache_k, cache_v, valid, pos, roles, size_global, size_local, params: EvictParams, ws, result):
     _require_cuda(cache_k, cache_v, valid, roles)
     lib = _lib.load()
