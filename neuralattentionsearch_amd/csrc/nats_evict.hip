@@ -376,6 +376,7 @@ struct TensorView {
   int upr;
 };
 
+constexpr int kFirstUnr = 4;  // 16-byte units a thread of the out-of-place kernel has in flight
 constexpr int kUnr = 4;  // moves per wavefront and batch
 constexpr int kNu = 2;   // units per lane and chunk slice (a slice holds at most 128 units)
 
@@ -581,14 +582,37 @@ __global__ __launch_bounds__(256) void evict_apply_first_kernel(ApplyArgs a) {
     const uint4* src =
         reinterpret_cast<const uint4*>(static_cast<const char*>(a.src[which]) + (b * a.ss_b + h * a.ss_h) * a.elem_bytes);
     const int64_t d_stride = a.ks_r * a.elem_bytes / 16, s_stride = a.ss_r * a.elem_bytes / 16;
-    for (int u = tid; u < C * upr; u += 256) {
-      int row = u / upr, col = u % upr;
-      int64_t drow = ci * C + row;
-      int64_t tok = src_chunk < 0 ? -1 : src_chunk * C + row;
-      // every row is read once and written once: both sides carry the streaming hint
-      u32x4 val = {0u, 0u, 0u, 0u};
-      if (tok >= 0 && tok < L && drow < res.n_ctx_data) val = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src + tok * s_stride + col));
-      __builtin_nontemporal_store(val, reinterpret_cast<u32x4*>(dst + drow * d_stride + col));
+    // Every row is read once and written once: both sides carry the streaming hint.  A thread has kFirstUnr loads
+    // in flight before its first store (a 64-row chunk of 256-byte rows is one trip).
+    const int n_units = C * upr;
+    const int row_step = 256 / upr, col_step = 256 % upr;
+    int row = tid / upr, col = tid % upr;
+    for (int u0 = tid; u0 < n_units; u0 += 256 * kFirstUnr) {
+      u32x4 val[kFirstUnr];
+      uint4* to[kFirstUnr];
+#pragma unroll
+      for (int k = 0; k < kFirstUnr; ++k) {
+        val[k] = u32x4{0u, 0u, 0u, 0u};
+        to[k] = nullptr;
+        if (u0 + k * 256 < n_units) {
+          const int64_t drow = ci * C + row;
+          const int64_t tok = src_chunk < 0 ? -1 : src_chunk * C + row;
+          to[k] = dst + drow * d_stride + col;
+          if (tok >= 0 && tok < L && drow < res.n_ctx_data) {
+            val[k] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src + tok * s_stride + col));
+          }
+        }
+        row += row_step;
+        col += col_step;
+        if (col >= upr) {
+          col -= upr;
+          ++row;
+        }
+      }
+#pragma unroll
+      for (int k = 0; k < kFirstUnr; ++k) {
+        if (to[k]) __builtin_nontemporal_store(val[k], reinterpret_cast<u32x4*>(to[k]));
+      }
     }
   } else {
     int32_t* dst = static_cast<int32_t*>(a.tensor[2]) + b * a.vs_b + h * a.vs_h;
