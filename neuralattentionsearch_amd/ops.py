@@ -494,13 +494,20 @@ def read_result(result: torch.Tensor) -> EvictResult:
     return EvictResult(*host)
 
 
-def cache_append_ok(k: torch.Tensor, v: torch.Tensor, cache_k: torch.Tensor, cache_v: torch.Tensor) -> bool:
-    """Whether `cache_append` takes these tensors: one dtype, 16-byte rows and strides everywhere."""
+def _append_layout_ok(k: torch.Tensor, v: torch.Tensor, cache_k: torch.Tensor, cache_v: torch.Tensor) -> bool:
+    """One dtype, 16-byte rows and strides everywhere, the cache itself at 16-byte addresses (the addresses of the
+    new rows are the caller's to check)."""
     e = 16 // cache_k.element_size()
     ts = (k, v, cache_k, cache_v)
-    return (all(t.is_cuda and t.dtype == cache_k.dtype and t.stride(-1) == 1 and t.data_ptr() % 16 == 0 for t in ts)
+    return (all(t.is_cuda and t.dtype == cache_k.dtype and t.stride(-1) == 1 for t in ts)
+            and (cache_k.data_ptr() | cache_v.data_ptr()) % 16 == 0
             and cache_k.shape[-1] % e == 0 and all(st % e == 0 for t in ts for st, n in zip(t.stride()[:3], t.shape[:3]) if n != 1)
             and not strides_differ(cache_k, cache_v))
+
+
+def cache_append_ok(k: torch.Tensor, v: torch.Tensor, cache_k: torch.Tensor, cache_v: torch.Tensor) -> bool:
+    """Whether `cache_append` takes these tensors: one dtype, 16-byte rows, strides and addresses everywhere."""
+    return _append_layout_ok(k, v, cache_k, cache_v) and (k.data_ptr() | v.data_ptr()) % 16 == 0
 
 
 def cache_append(k: torch.Tensor, v: torch.Tensor, cache_k: torch.Tensor, cache_v: torch.Tensor, valid: torch.Tensor,
@@ -524,7 +531,7 @@ class CacheAppendCall:
     def __init__(self, k, v, cache_k, cache_v, valid, pos):
         self.key = (k.shape, k.stride(), v.stride(), k.dtype, v.dtype, k.device)
         self.bufs = (cache_k, cache_v, valid, pos)
-        self.ok = cache_append_ok(k, v, cache_k, cache_v)
+        self.ok = _append_layout_ok(k, v, cache_k, cache_v)  # (the rows' addresses are checked per call)
         if not self.ok:
             return
         e = 16 // cache_k.element_size()

@@ -32,9 +32,10 @@ def compare(hip, st, where):
         assert np.array_equal(hip.token_positions.cpu().numpy().astype(np.int64), st.pos_k), (where, "index map")
 
 
-def drive(name, B, H, D, C, W, segs, dtype, seed, check_masks=True, attend_n_rep=0):
+def drive(name, B, H, D, C, W, segs, dtype, seed, check_masks=True, attend_n_rep=0, layout=None):
     """segs: list of (x_len, roles uint8 [B, H, S]).  With attend_n_rep > 0 every multi-token segment over a
-    non-empty cache also runs the segment attention kernel against masked attention on the oracle's cache."""
+    non-empty cache also runs the segment attention kernel against masked attention on the oracle's cache.
+    `layout(op index, k on the GPU, v on the GPU)` may return the same values in another memory layout."""
     from neuralattentionsearch_amd.cache import NAtSChunkLayerCache
     hip = NAtSChunkLayerCache(B, H, W, chunk_size=C, device="cuda", track_positions=True)
     st = ChunkCacheOracle(B=B, H=H, W=W, C=C)
@@ -46,7 +47,10 @@ def drive(name, B, H, D, C, W, segs, dtype, seed, check_masks=True, attend_n_rep
         v = torch.randn(B, H, x_len, D, generator=g).to(dtype)
         tsi = one_hot_roles(roles, dtype=dtype)
         ko, vo = st.update(k, v, roles)
-        kh, vh = hip.update(k.cuda(), v.cuda(), tsi.cuda())
+        kd, vd = k.cuda(), v.cuda()
+        if layout is not None:
+            kd, vd = layout(oi, kd, vd)
+        kh, vh = hip.update(kd, vd, tsi.cuda())
         assert torch.equal(kh.cpu().view(torch.int16 if dtype == torch.bfloat16 else torch.int32),
                            ko.contiguous().view(torch.int16 if dtype == torch.bfloat16 else torch.int32)), (name, oi, "update K")
         if check_masks:
@@ -123,6 +127,35 @@ def test_multi_segment_and_streaming_random(C, W):
     lens = [10 * C, 4 * C, C, C, 3 * C + 7, 2 * C - 7, 1, 1, 5 * C] + [C] * 6
     drive(f"multiseg_C{C}", 2, 3, 128, C, W, role_stream(rng, 2, 3, C, lens, (0.15, 0.25, 0.6)), torch.bfloat16, seed=C,
           check_masks=True, attend_n_rep=4)
+
+
+@pytest.mark.parametrize("C,W", [(64, 256), (8, 32)])
+def test_appended_rows_in_changing_layouts(C, W):
+    """The cache keeps calls prepared for the layout of the rows it was last handed and for its present buffers
+    (ops.CacheAppendCall, ops.EvictInplaceCall).  A stream whose segments arrive as contiguous tensors, as views of
+    a [B, L, H, D] projection output, inside wider rows at addresses that are and are not multiples of 16 bytes (same
+    strides; the latter take the slice-assignment path) and with elements that are not contiguous, long enough for
+    the capacity buffer to grow several times, leaves the oracle's bytes after every step."""
+    rng = np.random.default_rng(77 + C)
+    lens = [6 * C] + [C] * 5 + [2 * C + 3, C - 3] + [C] * 30 + [1] * (C + 2) + [C] * 4
+
+    def layout(oi, k, v):
+        B, H, L, D = k.shape
+        kind = (oi // 2) % 4  # (two steps in a row per kind, so that a prepared call is met again)
+        if kind == 1:  # [B, L, H, D] storage, as a projection leaves it
+            return (k.transpose(1, 2).contiguous().transpose(1, 2), v.transpose(1, 2).contiguous().transpose(1, 2))
+        if kind == 2:  # rows inside a wider buffer, every other time 8 bytes off a 16-byte address
+            off = 4 if oi % 2 else 0
+            z = lambda n, t: torch.zeros(B, H, L, n, dtype=t.dtype, device=t.device)
+            wide = lambda t: torch.cat([z(off, t), t, z(16 - off, t)], dim=-1)[..., off:off + D]
+            return wide(k), wide(v)
+        if kind == 3 and oi % 16 == 6:  # elements two apart
+            every_other = lambda t: torch.stack([t, t], dim=-1).reshape(B, H, L, 2 * D)[..., ::2]
+            return every_other(k), every_other(v)
+        return k, v
+
+    drive(f"layouts_C{C}", 2, 3, 128, C, W, role_stream(rng, 2, 3, C, lens, (0.15, 0.25, 0.6)), torch.bfloat16, seed=5 + C,
+          check_masks=False, layout=layout)
 
 
 @pytest.mark.parametrize("C,W,D,dtype,n_rep", [(64, 256, 128, torch.bfloat16, 4), (8, 32, 64, torch.bfloat16, 2),
