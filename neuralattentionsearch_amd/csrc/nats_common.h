@@ -68,7 +68,8 @@ struct PastView {
 };
 
 struct KeyLimArgs {
-  const int32_t* vis_lim;       // [streams, S] slot-level limits of the segment's roles
+  const uint8_t* roles;         // [streams, S]; if set, the kernel derives the slot-level limits itself (no past only)
+  const int32_t* vis_lim;       // [streams, S] slot-level limits of the segment's roles (used when roles is NULL)
   const int32_t* first_global;  // [streams] first global slot of the segment
   const uint8_t* valid;
   int64_t valid_s_b, valid_s_h;

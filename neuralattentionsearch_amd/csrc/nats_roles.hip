@@ -132,9 +132,37 @@ __global__ __launch_bounds__(256) void key_lim_kernel(KeyLimArgs a) {
   if (tile >= a.Tk) return;
   const int row = tile * kTile + lane;
   int32_t lim = -1;
+  // Slot-level limit of this lane's row from the roles themselves (as role_scan_kernel computes it: global ->
+  // INT32_MAX, sliding window -> slot + W / C, local -> the first global slot at or after it, the last slot counting
+  // as global): the wavefront's rows span at most 64 consecutive slots, so one ballot over the 64 slots from its first
+  // one answers most lanes, and the blocks that follow answer the rest with their first global slot.
+  int32_t v_inline = 0;
+  if (!kPast && a.roles) {
+    const uint8_t* r = a.roles + (int64_t)stream * a.S;
+    const bool in = row < a.N;
+    const int slot = in ? row >> a.c_shift : 0;
+    const int s0 = (tile * kTile) >> a.c_shift;  // slot of lane 0 (the tile starts inside N)
+    const uint8_t role = in ? r[slot] : uint8_t(NATS_ROLE_GLOBAL);
+    const bool want = in && role == NATS_ROLE_LOCAL;
+    int g = -1;
+    if (__ballot(want)) {
+      for (int blk = s0; blk < a.S; blk += kWave) {
+        const int n = blk + lane;
+        const bool is_g = n < a.S && (r[n] == NATS_ROLE_GLOBAL || n == a.S - 1);
+        const uint64_t bits = __ballot(is_g);
+        if (want && g < 0) {
+          const int rel = slot - blk;  // 0 .. 63 in the first block, negative afterwards
+          const uint64_t ahead = rel > 0 ? bits >> rel : bits;
+          if (ahead) g = (rel > 0 ? slot : blk) + __builtin_ctzll(ahead);
+        }
+        if (!__ballot(want && g < 0)) break;
+      }
+    }
+    v_inline = role == NATS_ROLE_GLOBAL ? kLimGlobal : role == NATS_ROLE_SW ? slot + (a.W >> a.c_shift) : g;
+  }
   if (row < a.N) {
     if (!kPast || row >= a.base) {
-      int32_t v = a.vis_lim[(int64_t)stream * a.S + ((row - a.base) >> a.c_shift)];
+      int32_t v = (!kPast && a.roles) ? v_inline : a.vis_lim[(int64_t)stream * a.S + ((row - a.base) >> a.c_shift)];
       int64_t t = (int64_t(v) + 1) * a.C - 1;
       lim = (v == kLimGlobal || t >= kLimGlobal) ? kLimGlobal : int32_t(t);
     } else {
@@ -283,8 +311,16 @@ PrefillWorkspace carve_prefill_workspace(void* ws, int64_t n_streams, int64_t S,
 int prepare_key_limits(const uint8_t* roles, int64_t B, int64_t H_kv, int64_t S, int64_t N, int64_t C, int64_t W,
                        const PastView* past, const PrefillWorkspace& w, hipStream_t st) {
   const int64_t n_streams = B * H_kv;
-  if (int rc = launch_role_scan(roles, n_streams, S, W, C, nullptr, w.vis_lim, w.first_global, st)) return rc;
   KeyLimArgs a{};
+  // A prefill from an empty cache needs the scan's result only inside the key-limit kernel, which then searches the
+  // roles itself (one launch less); streams so long that a run of local slots could make that search slow, and
+  // segments over a filled cache (which also need the first global slot), take the scan kernel.
+  const bool inline_scan = past == nullptr && S <= 8192;
+  if (inline_scan) {
+    a.roles = roles;
+  } else if (int rc = launch_role_scan(roles, n_streams, S, W, C, nullptr, w.vis_lim, w.first_global, st)) {
+    return rc;
+  }
   a.vis_lim = w.vis_lim;
   a.first_global = w.first_global;
   a.tok_lim = w.tok_lim;
