@@ -76,6 +76,23 @@ def test_prefill_mask_bit_exact(L, C, W):
     assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("L,C", [(2000, 1), (6000, 4), (6000, 8)])
+def test_prefill_mask_with_long_local_runs(L, C):
+    """Hundreds of local slots between two global ones: the search for the next global slot crosses several blocks
+    of 64 slots (the search inside the key-limit kernel that a prefill from an empty cache runs)."""
+    from neuralattentionsearch_amd import ops
+    say("prefill_mask long local runs", L, C)
+    rng = np.random.default_rng(L + C)
+    S = -(-L // C)
+    roles = rng.choice(3, size=(1, 2, S), p=(0.003, 0.9, 0.097)).astype(np.uint8)
+    roles[:, :, 0] = 0
+    roles[0, 1, S // 3:] = 1  # no global slot after the first third (the last slot counts as one)
+    W = 8 * C
+    want = orc.prefill_mask(roles, L, C, W)
+    got = ops.prefill_mask(to_dev(roles), L, C, W).cpu().numpy()
+    assert np.array_equal(got, want)
+
+
 def test_prefill_mask_worked_example():
     from neuralattentionsearch_amd import ops
     say("prefill_mask worked example")
