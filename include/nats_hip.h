@@ -310,7 +310,11 @@ int nats_evict_apply_inplace(void* cache_k, void* cache_v, uint8_t* valid, int32
  * ([B, H_kv, x_len, D], strides (b, h, row)) into a fresh cache of n_alloc rows, producing the same
  * bytes the in-place sequence would leave in rows [0, n_alloc) of [W zeros | K | pad].
  * Requires params->first == 1 and the cache to have been empty; n_alloc = ceil(result.n_ctx_data / C) * C
- * reproduces the reference's truncation (components/cache/nats_chunk_layer_cache.py:373-380).
+ * reproduces the reference's truncation (components/cache/nats_chunk_layer_cache.py:373-380).  A caller that does
+ * not know result.n_ctx_data yet may pass a larger n_alloc (a cache allocated on an estimate): rows from
+ * ceil(result.n_ctx_data / C) * C on are spare capacity and are not written at all, in none of the tensors; the
+ * caller zeroes them (valid 0, pos -1) when it extends the cache into them.  With a smaller n_alloc the call has
+ * to be made again into a large enough cache.
  */
 int nats_evict_apply_first(const void* src_k, const void* src_v, void* cache_k, void* cache_v, uint8_t* valid,
                            int32_t* pos, const uint8_t* roles, int64_t* size_global, int64_t* size_local,

@@ -101,6 +101,8 @@ class NAtSChunkLayerCache:
         self._roles = None
         self._buf_k = self._buf_v = self._buf_valid = self._buf_pos = None
         self._append_call = self._inplace_call = None  # (they hold the buffers)
+        self._uninit = False  # the buffers came from torch.empty and only the eviction kernel has written them
+        self._clean = None    # if set: buffer rows from this one on hold nothing yet, not even zeros
         self._n_rows = 0
         self._pending = None  # raw (K, V) of a first prefill not yet compacted
         self._last_result = None
@@ -184,6 +186,7 @@ class NAtSChunkLayerCache:
         self._gmin = int(res.gmin)
         if first:
             self._n_rows = math.ceil(self._n_ctx / self.chunk_size) * self.chunk_size
+            self._mark_spare()
 
     def _lazy(name):  # noqa: N805 -- a host scalar that a pending eviction result may still change
         def get(self):
@@ -238,6 +241,7 @@ class NAtSChunkLayerCache:
         """`zero=False` when the caller's kernel writes every row of every tensor itself."""
         B, H, D = like.shape[0], like.shape[1], like.shape[3]
         new = torch.zeros if zero else torch.empty
+        self._uninit, self._clean = not zero, None
         self._buf_k = new(B, H, rows, D, dtype=like.dtype, device=like.device)
         self._buf_v = new(B, H, rows, D, dtype=like.dtype, device=like.device)
         self._buf_valid = new(B, H, rows, dtype=torch.uint8, device=like.device)
@@ -249,8 +253,28 @@ class NAtSChunkLayerCache:
             self._buf_pos = torch.empty(B, H, rows, dtype=torch.int32, device=like.device)
         self._rows = rows
 
+    def _mark_spare(self):
+        """After a first eviction into buffers that came uninitialised: the out-of-place kernel writes the rows up to the
+        logical end of the cache only, the spare rows behind them hold nothing yet."""
+        if self._uninit and self._buf_k is not None and self._buf_k.shape[2] > self._n_rows:
+            self._clean = self._n_rows
+        self._uninit = False
+
+    def _init_rows(self, lo: int, hi: int):
+        """Buffer rows [lo, hi) as a fresh cache has them: zeros, not valid, no token."""
+        self._buf_k[:, :, lo:hi].zero_()
+        self._buf_v[:, :, lo:hi].zero_()
+        self._buf_valid[:, :, lo:hi].zero_()
+        if self._buf_pos is not None:
+            self._buf_pos[:, :, lo:hi].fill_(-1)
+
     def _grow(self, rows: int):
         cap = self._buf_k.shape[2]
+        if self._clean is not None and rows > self._clean:
+            # the cache extends into spare rows: the ones it takes now (all of them before the buffers are copied)
+            hi = cap if rows >= cap else rows
+            self._init_rows(self._clean, hi)
+            self._clean = hi if hi < cap else None
         if rows > cap:
             new_cap = max(rows, cap + max(cap // 2, 4 * self.chunk_size))
             new_cap = math.ceil(new_cap / self.chunk_size) * self.chunk_size
@@ -618,6 +642,7 @@ class NAtSLayerCache(NAtSChunkLayerCache):
         self._gmin = int(res.gmin)
         if first:
             self._n_rows = self._n_ctx
+            self._mark_spare()
 
     # -- evict + compact (nats_layer_cache.py:292-418) ---------------------------------------------
     def post_update(self, x_len: int):

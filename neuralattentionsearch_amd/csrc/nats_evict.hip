@@ -550,7 +550,9 @@ __global__ __launch_bounds__(256) void evict_apply_first_kernel(ApplyArgs a) {
   const int count = res.all_local ? 0 : hp.count;
   const bool tail_move = !res.all_local && partial && res.max_keep < S - 1;
 
-  const int64_t ci_end = min((int64_t)(blockIdx.x + 1) * a.chunks_per_wg, a.n_chunks);
+  // Destination chunks past the last one that holds live rows are spare capacity (a cache allocated on a guess of
+  // its size): they are left as they are; whoever extends the cache into them initialises them then.
+  const int64_t ci_end = min(min((int64_t)(blockIdx.x + 1) * a.chunks_per_wg, a.n_chunks), (res.n_ctx_data + C - 1) / C);
   for (int64_t ci = (int64_t)blockIdx.x * a.chunks_per_wg; ci < ci_end; ++ci) {
   // where the rows of this destination chunk come from: a source chunk of the raw prefill tensor
   // (-1 = zeros); the untouched part of [W zeros | K | pad] keeps its own rows
@@ -640,8 +642,6 @@ __global__ __launch_bounds__(256) void evict_apply_first_kernel(ApplyArgs a) {
             v = 1;
           }
         }
-        // rows of a cache that was allocated with room to spare, beyond what the reference's tensors hold
-        if (i >= (res.n_ctx_data + C - 1) / C * C) v = 0;
       }
       vrow[i] = v;
     }

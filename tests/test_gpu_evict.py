@@ -272,7 +272,7 @@ def test_cfg4_streamed_eviction_equals_bulk():
 
 
 @pytest.mark.parametrize("C,W,per_token", [(64, 256, False), (16, 32, False), (1, 32, True)])
-def test_a_reset_cache_evicts_its_next_prefill_on_a_guessed_capacity(C, W, per_token):
+def test_a_reset_cache_evicts_its_next_prefill_on_a_guessed_capacity(C, W, per_token, monkeypatch):
     """A cache object that is reset and fed a new prompt launches the first eviction into a cache sized from the share
     of rows it kept last time, before the plan kernel's numbers have reached the host.  The state must be the oracle's
     byte for byte whether the guess was right, too small (the eviction runs again at the right size), far too large
@@ -280,6 +280,17 @@ def test_a_reset_cache_evicts_its_next_prefill_on_a_guessed_capacity(C, W, per_t
     tokens appended afterwards must land in rows that look as the reference's zero padding does."""
     from neuralattentionsearch_amd.cache import NAtSChunkLayerCache, NAtSLayerCache
     from oracle.nats_oracle import TokenCacheOracle
+    # Uninitialised GPU memory holds 0x7f bytes for the length of this test (valid bytes that are not 0, positions
+    # that are not -1, values that are not 0), so that a spare row nobody initialised shows.
+    real_empty = torch.empty
+
+    def poisoned_empty(*args, **kwargs):
+        t = real_empty(*args, **kwargs)
+        if t.is_cuda and t.numel():
+            t.view(torch.uint8).fill_(0x7F)
+        return t
+
+    monkeypatch.setattr(torch, "empty", poisoned_empty)
     B, H, D, dtype = 2, 3, 64, torch.bfloat16
     hip = (NAtSLayerCache(B, H, W, device="cuda", track_positions=True) if per_token
            else NAtSChunkLayerCache(B, H, W, chunk_size=C, device="cuda", track_positions=True))
