@@ -74,6 +74,16 @@ def test_bf16_chunk_sizes_and_open_chunk(C, W, fill):
     run_case(3, 8, 2, 128, W, C, 30, torch.bfloat16, seed=C + fill, fill=fill)
 
 
+@pytest.mark.parametrize("share", [1, 37, 128, 176, 255])
+@pytest.mark.parametrize("B,Hkv,chunks", [(4, 8, 40), (1, 2, 3), (3, 1, 300)])
+def test_bf16_unequal_shares_of_the_two_halves_of_the_grid(share, B, Hkv, chunks, monkeypatch):
+    """The balanced schedule may give the first half of its workgroups another share of the tiles than the second
+    (NATS_DECODE_SHARE, in 1/256ths; large launches take 176 by themselves): any share, also the extreme ones that
+    leave one half with a single tile per workgroup or none, gives the oracle's result."""
+    monkeypatch.setenv("NATS_DECODE_SHARE", str(share))
+    run_case(B, 4 * Hkv, Hkv, 128, 256, 64, chunks, torch.bfloat16, seed=share + chunks, frac=(0.02, 1.0), fill=9)
+
+
 def test_bf16_single_sequence_long_cache():
     run_case(1, 32, 8, 128, 256, 64, 300, torch.bfloat16, seed=9, frac=(0.2, 1.0), fill=13)
 
