@@ -222,7 +222,7 @@ def decode_inputs(B, Hq, Hkv, D, C, W, ctx, seed, dev):
 
 
 def bench_decode(args, ops):
-    B, Hq, Hkv, D, C, W, ctx = 32, 32, 8, 128, 64, 256, 65536
+    B, Hq, Hkv, D, C, W, ctx = args.decode_batch, 32, 8, 128, 64, 256, args.decode_context
     q, k, v, valid, n_rows, (row_end, tail_start) = decode_inputs(B, Hq, Hkv, D, C, W, ctx, 0, "cuda")
     n_valid = int(valid[:, :, :n_rows].sum().item())
     bytes_alg = n_valid * D * 2 * 2 + 2 * q.numel() * 2
@@ -543,6 +543,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--prefill-len", type=int, default=32768)
     ap.add_argument("--chunk-size", type=int, default=64, help="chunk size of the prefill leg (the headline uses 64)")
+    ap.add_argument("--decode-batch", type=int, default=32, help="sequences of the decode leg (the headline uses 32)")
+    ap.add_argument("--decode-context", type=int, default=65536, help="context of the decode leg (the headline uses 65536)")
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--no-compare", action="store_true", help="skip the dense comparators of the prefill leg")
     ap.add_argument("--segments", type=int, default=4, help="segments of the `--only segments` leg")
@@ -614,7 +616,9 @@ def main():
         line["roofline_decode"] = {"bound": "hbm", "achieved": d["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
                                    "frac": d["frac_of_hbm_peak"],
                                    "kernel": "decode_split_mfma_kernel<128,4> + decode_merge_balanced_kernel"}
-        line["roofline_decode"]["traffic"], line["roofline_decode"]["traffic_source"] = measured_traffic("decode")
+        line["roofline_decode"]["traffic"], line["roofline_decode"]["traffic_source"] = (
+            measured_traffic("decode") if (args.decode_batch, args.decode_context) == (32, 65536)
+            else (None, "not the profiled workload"))
     if "evict" in res:
         e = res["evict"]
         line["roofline_evict"] = {"bound": "hbm", "achieved": e["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
