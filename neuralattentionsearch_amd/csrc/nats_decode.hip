@@ -393,34 +393,40 @@ __global__ __launch_bounds__(256) void decode_split_mfma_kernel(DecodeArgs a) {
   }
 }
 
-// merge the partials of one q head (balanced schedule): grid = B*Hq, block = D threads (one or two wavefronts).
-// The weights 2^(m_s - M) of the partials are computed side by side (thread s takes partial s) and kept in LDS;
-// the accumulators are then summed in partial order with four loads in flight.
+// merge the partials of one q head (balanced schedule): grid = B*Hq, block = G * D threads (G groups of D threads).
+// The weights 2^(m_s - M) of the partials are computed side by side (thread s takes partial s) and kept in LDS; group
+// g then sums the accumulators of the partials g, g + G, ... in that order with four loads in flight, and the groups'
+// sums are added in group order.  G = 1 for the few partials per head of a large batch; a single sequence, whose
+// heads are cut among many workgroups, takes up to eight groups (the kernel is one trip to memory per four partials
+// of a group, and nothing else).
+constexpr int kMergeRed = 16;  // wavefronts of the largest block (1024 threads)
 __global__ void decode_merge_balanced_kernel(const float* __restrict__ ws_acc, const float* __restrict__ ws_ml,
                                              const int2* __restrict__ head_table, uint16_t* __restrict__ o, int Hq, int Hkv,
                                              int D) {
-  extern __shared__ float merge_w[];  // [partials of the head] weights, then 2 x 4 floats for the block reductions
+  // [partials of the head] weights, 2 x kMergeRed floats for the block reductions, [G][D] sums of the groups
+  extern __shared__ float merge_w[];
   const int head = blockIdx.x;  // b * Hq + hq
-  const int d = threadIdx.x;
+  const int tid = threadIdx.x;
   const int n_rep = Hq / Hkv;
   const int b = head / Hq, hq = head % Hq;
   const int2 tab = head_table[b * Hkv + hq / n_rep];
   const int r = hq % n_rep;
   const int n = tab.y;
   float* red = merge_w + n;
+  float* part = red + 2 * kMergeRed;
   const int n_waves = (blockDim.x + kWave - 1) / kWave;
 
   float mloc = -INFINITY;
-  for (int s = d; s < n; s += blockDim.x) mloc = fmaxf(mloc, ws_ml[((int64_t)(tab.x + s) * n_rep + r) * 2]);
+  for (int s = tid; s < n; s += blockDim.x) mloc = fmaxf(mloc, ws_ml[((int64_t)(tab.x + s) * n_rep + r) * 2]);
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) mloc = fmaxf(mloc, __shfl_xor(mloc, off));
-  if ((d & 63) == 0) red[d >> 6] = mloc;
+  if ((tid & 63) == 0) red[tid >> 6] = mloc;
   __syncthreads();
   float M = red[0];
   for (int w = 1; w < n_waves; ++w) M = fmaxf(M, red[w]);
 
   float lloc = 0.f;
-  for (int s = d; s < n; s += blockDim.x) {
+  for (int s = tid; s < n; s += blockDim.x) {
     const int64_t prt = (int64_t)(tab.x + s) * n_rep + r;
     const float ms = ws_ml[prt * 2];
     const float f = (ms == -INFINITY) ? 0.f : exp2_guard(ms - M);
@@ -429,24 +435,36 @@ __global__ void decode_merge_balanced_kernel(const float* __restrict__ ws_acc, c
   }
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) lloc += __shfl_xor(lloc, off);
-  if ((d & 63) == 0) red[4 + (d >> 6)] = lloc;
+  if ((tid & 63) == 0) red[kMergeRed + (tid >> 6)] = lloc;
   __syncthreads();
-  float lsum = red[4];
-  for (int w = 1; w < n_waves; ++w) lsum += red[4 + w];
-  if (d >= D) return;
+  float lsum = red[kMergeRed];
+  for (int w = 1; w < n_waves; ++w) lsum += red[kMergeRed + w];
 
+  const int G = blockDim.x / D;
+  const int g = tid / D, d = tid % D;
   float sum = 0.f;
-  const float* acc = ws_acc + ((int64_t)tab.x * n_rep + r) * D + d;
-  const int64_t step = (int64_t)n_rep * D;
-  int s = 0;
-  for (; s + 4 <= n; s += 4) {
-    const float a0 = acc[(s + 0) * step], a1 = acc[(s + 1) * step], a2 = acc[(s + 2) * step], a3 = acc[(s + 3) * step];
-    sum = fmaf(a0, merge_w[s], sum);
-    sum = fmaf(a1, merge_w[s + 1], sum);
-    sum = fmaf(a2, merge_w[s + 2], sum);
-    sum = fmaf(a3, merge_w[s + 3], sum);
+  if (g < G) {
+    const float* acc = ws_acc + ((int64_t)tab.x * n_rep + r) * D + d;
+    const int64_t step = (int64_t)n_rep * D;
+    int s = g;
+    for (; s + 3 * G < n; s += 4 * G) {
+      const float a0 = acc[s * step], a1 = acc[(s + G) * step], a2 = acc[(s + 2 * G) * step], a3 = acc[(s + 3 * G) * step];
+      sum = fmaf(a0, merge_w[s], sum);
+      sum = fmaf(a1, merge_w[s + G], sum);
+      sum = fmaf(a2, merge_w[s + 2 * G], sum);
+      sum = fmaf(a3, merge_w[s + 3 * G], sum);
+    }
+    for (; s < n; s += G) sum = fmaf(acc[s * step], merge_w[s], sum);
   }
-  for (; s < n; ++s) sum = fmaf(acc[s * step], merge_w[s], sum);
+  if (G > 1) {
+    if (g < G) part[g * D + d] = sum;
+    __syncthreads();
+    if (g != 0) return;
+    sum = part[d];
+    for (int k = 1; k < G; ++k) sum += part[k * D + d];
+  } else if (g != 0) {
+    return;
+  }
   o[(int64_t)head * D + d] = f32_to_bf16_bits(lsum > 0.f ? sum / lsum : 0.f);
 }
 
@@ -773,8 +791,12 @@ static int decode_fwd_impl(const void* q, const void* cache_k, const void* cache
     if (rc) return rc;
     NATS_CHECK_LAUNCH("decode_split_mfma_kernel");
     // (a head has at most one partial per workgroup plus one)
-    const size_t merge_smem = ((size_t)c.n_wg + 2 + 8) * sizeof(float);
-    hipLaunchKernelGGL(decode_merge_balanced_kernel, dim3((unsigned)(nb * H_q)), dim3((unsigned)D), merge_smem, st, c.ws_acc,
+    // groups of the merge kernel's block: about four partials per group and head
+    const int64_t per_head = c.n_wg / (nb * H_kv) + 1;
+    int merge_groups = 1;
+    while (merge_groups < 8 && merge_groups * 4 < per_head && (merge_groups * 2) * D <= 1024) merge_groups *= 2;
+    const size_t merge_smem = ((size_t)c.n_wg + 2 + 2 * kMergeRed + (size_t)merge_groups * D) * sizeof(float);
+    hipLaunchKernelGGL(decode_merge_balanced_kernel, dim3((unsigned)(nb * H_q)), dim3((unsigned)(merge_groups * D)), merge_smem, st, c.ws_acc,
                        c.ws_ml, c.head_table, static_cast<uint16_t*>(c.o), (int)H_q, (int)H_kv, (int)D);
     NATS_CHECK_LAUNCH("decode_merge_balanced_kernel");
   }
