@@ -2,6 +2,8 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-cpu] [--no-llama] [--only prefill|decode|evict|evict_stream|segments|role_step|matvec|llama]
 
+    (other sizes of a single leg: --prefill-len L, --chunk-size C, --decode-batch B, --decode-context N)
+
 One step = one pass of a kernel family over one batch of synthetic input that is already resident in HBM:
 
 * prefill  role-masked chunked flash attention at the Llama-3-8B head shape, L = 32768 (the headline)
