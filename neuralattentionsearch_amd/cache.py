@@ -719,6 +719,33 @@ class NAtSCache(_CacheBase):
             return 0
         return self.cache_model[layer_idx]._seen_tokens
 
+    # What a transformers model asks of its cache while it prepares a forward pass (newer releases of that library
+    # build their causal mask from these; the NAtS attention layers ignore that mask and compute their own).  The base
+    # class answers them from a `layers` list its __init__ would have made, which does not exist here.
+    @property
+    def layers(self):
+        return self.cache_model
+
+    @property
+    def is_sliding(self):
+        return [False] * len(self.cache_model)
+
+    @property
+    def is_compileable(self) -> bool:
+        return False
+
+    @property
+    def is_initialized(self) -> bool:
+        return len(self.cache_model) > 0
+
+    def get_mask_sizes(self, query_length, layer_idx: int = 0):
+        """(kv_length, kv_offset) of the mask the caller is about to build: every token seen so far plus the new ones."""
+        n = query_length if isinstance(query_length, int) else int(query_length.shape[0])  # (older releases pass cache_position)
+        return self.get_seq_length(layer_idx) + n, 0
+
+    def get_max_length(self, layer_idx: int = 0):
+        return -1
+
     def generate_mask(self, layer_idx: int, x_len: int):
         return self.cache_model[layer_idx].generate_mask(x_len)
 

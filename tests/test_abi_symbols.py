@@ -152,3 +152,39 @@ def test_container_is_a_transformers_cache():
     assert cache.sliding_window_size == 256 and cache.chunk_size == 64
     cache.reset_cache()
     assert cache.cache_model == []
+
+
+def test_a_transformers_llama_model_takes_the_container_as_past_key_values():
+    """The reference's callers hand NAtSCache to a Hugging Face model (experiments/long_bench/hf_pred.py:173-184,
+    experiments/efficiency/eval_efficiency.py:297-340) whose attention layers they have patched
+    (models/transformer/hf/llama_nats_chunk.py).  Everything the unpatched parts of such a model ask of the cache
+    while they prepare a forward pass (sequence length, mask sizes, the sliding flags) must work on the container;
+    here the attention layers are stand-ins that return zeros, so no GPU is needed."""
+    pytest.importorskip("transformers")
+    import torch
+    from transformers import LlamaConfig, LlamaModel
+    from transformers.models.llama import modeling_llama
+    from neuralattentionsearch_amd.cache import NAtSCache
+
+    seen = []
+
+    def attention_stand_in(self, hidden_states, *args, **kwargs):
+        cache = kwargs.get("past_key_values", kwargs.get("past_key_value"))
+        seen.append(cache)
+        return torch.zeros_like(hidden_states), None
+
+    cfg = LlamaConfig(vocab_size=100, hidden_size=64, intermediate_size=128, num_hidden_layers=2, num_attention_heads=4,
+                      num_key_value_heads=2, max_position_embeddings=512)
+    model = LlamaModel(cfg).eval()
+    original = modeling_llama.LlamaAttention.forward
+    modeling_llama.LlamaAttention.forward = attention_stand_in
+    try:
+        cache = NAtSCache(16, 4)
+        with torch.no_grad():
+            out = model(input_ids=torch.randint(0, 100, (1, 12)), past_key_values=cache, use_cache=True)
+            out1 = model(input_ids=torch.randint(0, 100, (1, 1)), past_key_values=cache, use_cache=True)
+    finally:
+        modeling_llama.LlamaAttention.forward = original
+    assert out.last_hidden_state.shape == (1, 12, 64) and out1.last_hidden_state.shape == (1, 1, 64)
+    assert len(seen) == 4 and all(c is cache for c in seen)
+    assert cache.get_mask_sizes(5, 0) == (5, 0) and cache.is_sliding == [] and not cache.is_compileable

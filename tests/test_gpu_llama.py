@@ -173,6 +173,57 @@ def test_fused_role_step_gives_the_same_generation(method, prompt):
     assert kept[0] == kept[1]
 
 
+@pytest.mark.parametrize("C,W", [(8, 16), (1, 32)])
+def test_a_transformers_llama_with_patched_attention_layers(C, W):
+    """The way the reference is used (models/transformer/hf/llama_nats_chunk.py patches the attention layers of a
+    Hugging Face Llama, the callers pass a NAtSCache as past_key_values): a transformers LlamaForCausalLM whose
+    attention layers forward to this package's attention module, with the container as its cache, gives the logits
+    of the package's own model with the same weights, for a prompt, a later multi-token segment and one-token steps."""
+    pytest.importorskip("transformers")
+    from transformers import LlamaConfig, LlamaForCausalLM
+    from transformers.models.llama import modeling_llama
+    from neuralattentionsearch_amd.llama import NAtSLlamaConfig, NAtSLlamaForCausalLM
+    say("transformers llama with patched attention", C, W)
+    dims = dict(vocab_size=300, hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=4,
+                num_key_value_heads=2)
+    torch.manual_seed(3)
+    hf = LlamaForCausalLM(LlamaConfig(max_position_embeddings=2048, rms_norm_eps=1e-6, attention_bias=False,
+                                      mlp_bias=False, tie_word_embeddings=False, **dims)).cuda().float().eval()
+    cfg = NAtSLlamaConfig(rms_norm_eps=1e-6, rope_theta=10000.0, chunk_size=C, local_seq_max_length=W, **dims)
+    ours = NAtSLlamaForCausalLM(cfg).cuda().float().eval()
+    state = {k.removeprefix("model."): v for k, v in hf.state_dict().items()}
+    res = ours.load_state_dict(state, strict=False)
+    assert not res.unexpected_keys and all(k.endswith("proj_layer.weight") for k in res.missing_keys), res
+    with torch.no_grad():
+        for layer in ours.layers:  # the role projection has no counterpart in the plain model
+            layer.self_attn.proj_layer.weight.normal_(0.0, 0.5)
+
+    def nats_forward(self, hidden_states, position_embeddings=None, attention_mask=None, past_key_values=None, **kwargs):
+        start = past_key_values.get_seq_length(self.layer_idx)
+        return ours.layers[self.layer_idx].self_attn(hidden_states, position_embeddings, start, past_key_values), None
+
+    g = torch.Generator().manual_seed(11)
+    lens = [5 * max(C, 8) + 3, 2 * max(C, 8) + 1] + [1] * (2 * max(C, 16) + 2)
+    ids = [torch.randint(0, 300, (2, n), generator=g).cuda() for n in lens]
+    cache_hf, cache_own = ours.new_cache(), ours.new_cache()
+    original = modeling_llama.LlamaAttention.forward
+    modeling_llama.LlamaAttention.forward = nats_forward
+    try:
+        pos = 0
+        with torch.no_grad():
+            for i, x in enumerate(ids):
+                got = hf(input_ids=x, past_key_values=cache_hf, use_cache=True).logits
+                want = ours(x, pos, cache_own, all_logits=True).reshape(got.shape)
+                err = (got.float() - want.float()).abs().max().item()
+                assert err <= 2e-4, (i, x.shape, err)
+                pos += x.shape[1]
+    finally:
+        modeling_llama.LlamaAttention.forward = original
+    assert cache_hf.get_seq_length() == pos == cache_own.get_seq_length()
+    for a, b in zip(cache_hf.cache_model, cache_own.cache_model):
+        assert a.n_ctx_data == b.n_ctx_data and torch.equal(a.valid_tokens, b.valid_tokens)
+
+
 def test_full_size_llama3_8b_shape_prefill_16384_and_512_steps():
     """The end-to-end workload at its full size (32 layers, d_model 4096, 32 / 8 heads, FFN 14336, vocabulary 128256,
     bf16; 16384 prompt tokens, 512 greedy steps with eviction live), where no oracle run is affordable: properties
