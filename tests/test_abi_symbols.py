@@ -186,5 +186,6 @@ def test_a_transformers_llama_model_takes_the_container_as_past_key_values():
     finally:
         modeling_llama.LlamaAttention.forward = original
     assert out.last_hidden_state.shape == (1, 12, 64) and out1.last_hidden_state.shape == (1, 1, 64)
+    assert out.past_key_values is cache and out1.past_key_values is cache  # (the callers go on with output.past_key_values)
     assert len(seen) == 4 and all(c is cache for c in seen)
     assert cache.get_mask_sizes(5, 0) == (5, 0) and cache.is_sliding == [] and not cache.is_compileable
