@@ -135,6 +135,15 @@ class NAtSChunkLayerCache:
                     self._launch_first(src, roles, params, ws, result, rows)
         self._take_result(res, first)
 
+    def settle(self, wait: bool = True):
+        """A first eviction launched on a guessed capacity keeps the caller's K / V until the plan's numbers confirm the
+        guess (a guess that was too small is redone from those tensors).  `settle` ends that: with `wait` it takes
+        the numbers as soon as the plan kernel has written them, without it only if they are there already.  The
+        container calls it for a layer when the next layer has been queued, so that the tensors are held for about
+        one layer's work and the relaunch, if there is one, reads them before their owner's next forward pass."""
+        if self._redo is not None and (wait or self._evict.reported(self._await[0])):
+            self._resolve()
+
     def _logical_rows(self, n_ctx: int) -> int:
         """Rows the reference's cache tensors have after a first eviction that left n_ctx live rows (:373-380)."""
         return math.ceil(n_ctx / self.chunk_size) * self.chunk_size
@@ -166,6 +175,7 @@ class NAtSChunkLayerCache:
             self._launch_first(src, roles, params, ws, result, cap)
             self._redo = (src, roles, params, ws, result, full)
             self._await = (params.seq, first)
+            self.settle(wait=False)
             return True
         res = self._evict.wait(params.seq)
         if res.all_sw:  # the reference keeps the untruncated cache here (:283-288)
@@ -703,8 +713,15 @@ class NAtSCache(_CacheBase):
         self.chunk_size = chunk_size
         self.cached_x: list[torch.Tensor | None] = []
         self.track_positions = track_positions
+        self._spare_layers: list = []
 
     def reset_cache(self):
+        """dyn_cache.py:76-78: the container is empty afterwards.  The layer objects are kept aside and taken up again,
+        reset, by the next prompt's updates (same batch size, heads and device): they hold the eviction workspaces, the
+        pinned result mirror and the share of rows the last first eviction kept, from which the next first eviction
+        sizes its cache without waiting for its plan."""
+        old = self.cache_model + getattr(self, "_spare_layers", [])[len(self.cache_model):]
+        self._spare_layers = old
         self.cache_model = []
         self.cached_x = []
 
@@ -812,7 +829,10 @@ class NAtSCache(_CacheBase):
     def update(self, key_states, value_states, layer_idx: int, cache_kwargs: dict[str, Any] | None = None):
         if len(self.cache_model) <= layer_idx:
             bsz, n_kv_heads = key_states.shape[:2]
-            if self.chunk_size == 1:
+            new_cache = self._spare_layer(layer_idx, bsz, n_kv_heads, key_states.device)
+            if new_cache is not None:
+                new_cache.reset_cache()
+            elif self.chunk_size == 1:
                 new_cache = NAtSLayerCache(bsz, n_kv_heads, self.sliding_window_size, layer_id=layer_idx,
                                            device=key_states.device, track_positions=self.track_positions)
             else:
@@ -820,7 +840,23 @@ class NAtSCache(_CacheBase):
                                                 chunk_size=self.chunk_size, device=key_states.device,
                                                 track_positions=self.track_positions)
             self.cache_model.append(new_cache)
+        elif layer_idx == 0:
+            self.cache_model[-1].settle()  # (the last layer of the previous forward pass)
         return self.cache_model[layer_idx].update(key_states, value_states, **(cache_kwargs or {}))
+
+    def _spare_layer(self, layer_idx: int, bsz: int, n_kv_heads: int, device):
+        """The layer object a reset put aside for this index, if it fits the new prompt."""
+        spare = getattr(self, "_spare_layers", [])
+        if len(self.cache_model) != layer_idx or layer_idx >= len(spare) or spare[layer_idx] is None:
+            return None
+        c, spare[layer_idx] = spare[layer_idx], None
+        kind = NAtSLayerCache if self.chunk_size == 1 else NAtSChunkLayerCache
+        fits = (type(c) is kind and c.bsz == bsz and c.n_msks == n_kv_heads and c.device == torch.device(device)
+                and c.sliding_window_size == self.sliding_window_size and c.track_positions == self.track_positions
+                and (self.chunk_size == 1 or c.chunk_size == self.chunk_size))
+        return c if fits else None
 
     def post_update(self, layer_idx: int, x_len=1, **kwargs):
         self.cache_model[layer_idx].post_update(x_len=x_len)
+        if layer_idx > 0:
+            self.cache_model[layer_idx - 1].settle()

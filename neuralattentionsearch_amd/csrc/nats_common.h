@@ -36,6 +36,8 @@ constexpr int kWave = 64;
 constexpr int kTile = 64;  // prefill tile edge (queries and keys)
 constexpr int kGranule = 16;  // key rows whose limits are also summarised on their own (a quarter tile)
 constexpr int32_t kLimGlobal = 0x7fffffff;
+constexpr int kTicketQueues = 8;   // work counters of a prefill launch: one per XCD
+constexpr int kTicketStride = 32;  // int32 entries between two of them (128 bytes: a memory line each)
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));

@@ -197,7 +197,6 @@ constexpr float kRescaleSlack = 8.0f;
 constexpr int kPrefillWaves = 8;
 constexpr int kMaxSplit = 32;  // workgroups that may share one tile list
 constexpr int kMaxDevices = 64;
-constexpr int kTicketStride = 32;  // int32 entries between the pool counters of two XCDs (128 bytes)
 
 // both halves of the wavefront get max / sum over lane and lane ^ 32 (one cross-half swap, no LDS round trip)
 __device__ __forceinline__ float half_swap_max(float v) {

@@ -128,7 +128,7 @@ __global__ __launch_bounds__(256) void key_lim_kernel(KeyLimArgs a) {
   const int stream = blockIdx.y;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int tile = blockIdx.x * 4 + wave;
-  if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x < 8 && a.ticket) a.ticket[threadIdx.x * 32] = 0;
+  if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x < kTicketQueues && a.ticket) a.ticket[threadIdx.x * kTicketStride] = 0;
   if (tile >= a.Tk) return;
   const int row = tile * kTile + lane;
   int32_t lim = -1;

@@ -9,6 +9,7 @@ from __future__ import annotations
 import collections
 import ctypes
 import math
+import time
 import weakref
 
 import torch
@@ -21,7 +22,9 @@ EvictBrief = collections.namedtuple("EvictBrief", "n_ctx_data gmin all_sw all_lo
 ROLE_GLOBAL, ROLE_LOCAL, ROLE_SW = 0, 1, 2
 TILE = 64
 
-_workspaces: dict = {}
+# scratch buffers by (device, raw stream handle, purpose), least recently used first; at most _WORKSPACE_SLOTS of them
+_workspaces: "collections.OrderedDict" = collections.OrderedDict()
+_WORKSPACE_SLOTS = 32
 
 
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
@@ -63,7 +66,10 @@ def workspace(device, key: str, nbytes: int) -> torch.Tensor:
     """A scratch buffer per (device, current stream, purpose) that only ever grows.
 
     Calls of one purpose on one stream share the buffer, which the stream orders; calls on different streams (two
-    prefills side by side, a worker thread under the caller's stream) get buffers of their own."""
+    prefills side by side, a worker thread under the caller's stream) get buffers of their own.  The table keeps the
+    _WORKSPACE_SLOTS entries used last: a process that creates streams without end does not keep a buffer for every
+    stream it ever had (a dropped buffer goes back to torch's allocator, which orders its reuse after the work
+    queued on it)."""
     device = torch.device(device)
     idx = device.index if device.index is not None else torch.cuda.current_device()
     handle = _raw_stream(idx) if _raw_stream is not None else torch.cuda.current_stream(device).cuda_stream
@@ -72,6 +78,9 @@ def workspace(device, key: str, nbytes: int) -> torch.Tensor:
     if buf is None or buf.numel() < nbytes:
         buf = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
         _workspaces[k] = buf
+        while len(_workspaces) > _WORKSPACE_SLOTS:
+            _workspaces.popitem(last=False)
+    _workspaces.move_to_end(k)
     return buf
 
 
@@ -95,7 +104,7 @@ def roles_from_logits(logits: torch.Tensor, global_bias: float = 0.1, force_firs
                                      int(force_first_global), int(force_last_global), _ptr(roles), _ptr(one_hot),
                                      _stream(logits)))
     if one_hot is not None:
-        one_hot.nats_roles = roles  # whoever receives only the one-hot tensor finds the compact form on it
+        _attach_roles(one_hot, roles)  # whoever receives only the one-hot tensor finds the compact form on it
     return roles, one_hot
 
 
@@ -145,16 +154,24 @@ def role_step(x: torch.Tensor, weight: torch.Tensor, chunk_size: int, window: in
                              _ptr(roles), _ptr(one_hot), _ptr(logits), _ptr(carry), _ptr(end_idx), _ptr(vis_lim),
                              _stream(x)))
     if one_hot is not None:
-        one_hot.nats_roles = roles
+        _attach_roles(one_hot, roles)
     return {"roles": roles, "token_states_info": one_hot, "logits": logits, "carry": carry, "end_idx": end_idx,
             "vis_lim": vis_lim, "pad": pad}
 
 
+def _attach_roles(one_hot: torch.Tensor, roles: torch.Tensor) -> None:
+    """The compact roles travel with the one-hot tensor they were written with, together with the version counters of
+    both: an in-place edit of either afterwards (a slot forced global, a head masked) makes the pair stale."""
+    one_hot.nats_roles = roles
+    one_hot.nats_roles_version = (one_hot._version, roles._version)
+
+
 def roles_from_one_hot(token_states_info: torch.Tensor) -> torch.Tensor:
     """[B, H_kv, S, 3] one-hot float -> uint8 roles (index of the 1).  A tensor that `roles_from_logits` or
-    `role_step` produced carries its roles with it."""
+    `role_step` produced carries its roles with it; they are used while neither tensor has been written since."""
     roles = getattr(token_states_info, "nats_roles", None)
-    if roles is not None and roles.shape == token_states_info.shape[:-1] and roles.device == token_states_info.device:
+    if roles is not None and roles.shape == token_states_info.shape[:-1] and roles.device == token_states_info.device \
+            and getattr(token_states_info, "nats_roles_version", None) == (token_states_info._version, roles._version):
         return roles
     return token_states_info.argmax(-1).to(torch.uint8)
 
@@ -323,7 +340,7 @@ PER_TOKEN_UPDATE_CHUNK = 16  # update_chunk_size of the per-token cache as NAtSC
 def nats_prefill(q, k, v, end_seqs_idx, sliding_tokens, sm_scale, nats_chunk_size: int = 1, global_kv_size=None,
                  local_kv_size=None, valid_sw_tokens=None, n_ctx_data=None, sw_token_tails=None, n_rep: int = 1,
                  n_tokens_in_first_chunk: int = 0, local_seq_max_length: int = 4, return_masks: bool = False,
-                 block_n: int = 32):
+                 block_n: int = 32, seen_tokens: int | None = None, n_global_min: int | None = None):
     """Drop-in for nats_prefill of models/transformer/triton/nats_flashattn_fwd.py:617-725 (same argument
     names and meaning, returns (o, mask or None)).
 
@@ -337,9 +354,15 @@ def nats_prefill(q, k, v, end_seqs_idx, sliding_tokens, sm_scale, nats_chunk_siz
     n_ctx_data and sliding_queue_tail before the eviction of this segment; n_tokens_in_first_chunk the tokens of
     the open chunk cached before the segment.  The result is SDPA(q, k, v, cache.generate_mask(L_q)), the path
     this kernel form is checked against there, for a cache in the state those arguments describe: valid_tokens is
-    rebuilt from them (ring bits, a head's own rows, the open chunk), the window is taken as full
-    (_seen_tokens >= W; the arguments do not carry it), and nats_chunk_size == 1 means the per-token cache class
-    (`sliding_queue_tail` = the slot written last)."""
+    rebuilt from them (ring bits, a head's own rows, the open chunk), and nats_chunk_size == 1 means the per-token
+    cache class (`sliding_queue_tail` = the slot written last).
+
+    Two numbers of the cache are not among the reference's arguments; both may be passed here (the cache classes of
+    this package know them): `seen_tokens` = the cache's _seen_tokens before this segment, which decides whether the
+    ring has wrapped (:666-676 against :678-690) -- without it the window is taken as full, and a call whose other
+    arguments fit a ring that has not filled yet (fewer than W rows behind the ring and its last slot empty in
+    every head) is refused rather than answered for the wrong case; `n_global_min` = the cache's _n_global_min,
+    computed from global_kv_size (one device-to-host read) when it is not given."""
     if q.shape[1] // k.shape[1] != n_rep:
         raise ValueError(f"n_rep={n_rep} does not match {q.shape[1]} q heads / {k.shape[1]} kv heads")
     roles = _roles_from_kernel_arguments(end_seqs_idx, sliding_tokens)
@@ -360,11 +383,17 @@ def nats_prefill(q, k, v, end_seqs_idx, sliding_tokens, sm_scale, nats_chunk_siz
         raise ValueError(f"valid_sw_tokens must be [B, H_kv, W / C], got {tuple(valid_sw_tokens.shape)}")
     sg = global_kv_size.to(torch.int64).contiguous()
     sl = local_kv_size.to(torch.int64).contiguous()
+    if seen_tokens is None:
+        if n_ctx - W - old_fill < W and not bool(valid_sw_tokens[..., -1].any()):
+            raise ValueError("nats_prefill: these arguments fit a cache whose window has not filled yet as well as a "
+                             "full one; pass seen_tokens (the cache's _seen_tokens before this segment)")
+        seen_tokens = W
+    gmin = int(sg.min()) if n_global_min is None else int(n_global_min)
     rows = torch.arange(n_ctx, device=q.device)
     valid = rows < (sg + sl).unsqueeze(-1)                                       # a head's own global and local rows
     valid[:, :, :W] = valid_sw_tokens.bool().repeat_interleave(C, dim=-1)       # ring slots
     valid[:, :, n_ctx - old_fill:] = True                                        # the open chunk
-    state = past_state(n_ctx, old_fill, int(sg.min()), tail, W, old_fill,
+    state = past_state(n_ctx, old_fill, gmin, tail, int(seen_tokens), old_fill,
                        PER_TOKEN_UPDATE_CHUNK if C == 1 else 0)
     o = prefill_past_attention(q, k, v, valid, sg, sl, roles, C, W, state, sm_scale)
     mask = prefill_past_mask(valid, sg, sl, roles, x_len, C, W, state) if return_masks else None
@@ -426,19 +455,41 @@ def evict_params(B, H_kv, D, C, W, S, x_len, fill, n_ctx_data, gmin, tail, first
     return EvictParams(B, H_kv, D, C, W, S, x_len, fill, n_ctx_data, gmin, tail, int(first), n_alloc, 0, int(update_chunk))
 
 
+# Sequence numbers of eviction plans are drawn from one counter for the whole process, and the 16-byte pinned mirrors
+# the plan kernels report into are never handed back to the host allocator (a dropped EvictBuffers returns its mirror
+# to this pool): a plan kernel of a cache that has been dropped may still be queued, and whatever it writes late can
+# then neither land in memory that has a new owner outside this module nor carry a number a live cache waits for.
+_evict_seq = 0
+_mirror_pool: list = []
+
+
+def _next_evict_seq() -> int:
+    global _evict_seq
+    _evict_seq = _evict_seq % 0x7fffffff + 1
+    return _evict_seq
+
+
 class EvictBuffers:
     """What the eviction calls of one cache keep between calls: the plan workspace, the 64-byte result in device
     memory, which the apply kernels read, and 16 bytes of pinned host memory into which the plan kernel also writes
     the numbers the host needs (n_ctx_data, minimum global size, two flags) with the call's sequence number: the
     host polls for that number instead of synchronising with the stream."""
 
+    POLL_SECONDS = 0.1  # how long `wait` polls before it synchronises with the device instead
+
     def __init__(self, device):
         self.device = torch.device(device)
         self.ws = None
         self.result = torch.zeros(8, dtype=torch.int64, device=self.device)
-        self.mirror = torch.zeros(4, dtype=torch.int32).pin_memory()
+        self.mirror = _mirror_pool.pop() if _mirror_pool else torch.zeros(4, dtype=torch.int32).pin_memory()
         self.mirror_np = self.mirror.numpy()
         self.seq = 0
+
+    def __del__(self):
+        try:
+            _mirror_pool.append(self.mirror)
+        except Exception:  # (interpreter shutdown)
+            pass
 
     def workspace(self, nbytes: int) -> torch.Tensor:
         if self.ws is None or self.ws.numel() < nbytes:
@@ -447,19 +498,27 @@ class EvictBuffers:
         return self.ws
 
     def next_seq(self) -> int:
-        self.seq = self.seq % 0x7fffffff + 1
+        self.seq = _next_evict_seq()
         return self.seq
+
+    def reported(self, seq: int) -> bool:
+        """Whether the plan call numbered `seq` has written its result (one read, no waiting)."""
+        return int(self.mirror_np[0]) == seq
 
     def wait(self, seq: int) -> EvictBrief:
         """The short result of the plan call numbered `seq`, as soon as its kernel has written it."""
         m = self.mirror_np
-        for _ in range(200000):
-            if m[0] == seq:
-                break
-        else:  # (about a tenth of a second: something is slow; fall back to a synchronisation)
-            torch.cuda.synchronize(self.device)
-            if m[0] != seq:
-                raise RuntimeError(f"eviction plan {seq} never reported its result (mirror holds {int(m[0])})")
+        if m[0] != seq:
+            spins, deadline = 0, time.perf_counter() + self.POLL_SECONDS
+            while m[0] != seq:
+                spins += 1
+                if spins & 1023:
+                    continue
+                time.sleep(0)  # (lets other Python threads run)
+                if time.perf_counter() > deadline:  # something is slow: a synchronisation instead
+                    torch.cuda.synchronize(self.device)
+                    if m[0] != seq:
+                        raise RuntimeError(f"eviction plan {seq} never reported its result (mirror holds {int(m[0])})")
         flags = int(m[1])
         return EvictBrief(int(m[2]), int(m[3]), flags & 1, (flags >> 1) & 1)
 

@@ -23,7 +23,7 @@ def end_seq_idx_as_the_reference_computes_it(tsi):
     return S - 1 - torch.flip(torch.cummax(torch.flip(flags, (-1,)), -1)[1], (-1,))
 
 
-def run_smoke_pattern(B, H, n_rep, D, W, C, lens, dtype, seed):
+def run_smoke_pattern(B, H, n_rep, D, W, C, lens, dtype, seed, cache_scalars=False):
     from neuralattentionsearch_amd import ops
     from neuralattentionsearch_amd.cache import NAtSChunkLayerCache, NAtSLayerCache
     tol = 2e-2 if dtype == torch.bfloat16 else 1e-5
@@ -56,6 +56,8 @@ def run_smoke_pattern(B, H, n_rep, D, W, C, lens, dtype, seed):
             o, msk = ops.nats_prefill(q.cuda(), k2, v2, **common)
         else:
             want_mask = st.generate_mask(n)
+            if cache_scalars:  # the two numbers the reference's argument list does not carry
+                common.update(seen_tokens=cache._seen_tokens, n_global_min=cache._n_global_min)
             o, msk = ops.nats_prefill(
                 q.cuda(), k2, v2, **common,
                 n_tokens_in_first_chunk=cache.chunk_fill_size - n if C > 1 else 0,
@@ -92,6 +94,35 @@ def test_the_smoke_pattern_on_the_chunked_cache(C, W, lens):
 
 def test_per_token_cache_with_more_segments():
     run_smoke_pattern(2, 4, 4, 128, 64, 1, [300, 54, 160, 32], torch.bfloat16, seed=7)
+
+
+@pytest.mark.parametrize("C,W,lens", [(8, 32, [16, 8, 24, 40]), (4, 64, [20, 22, 30, 64])])
+def test_a_first_segment_shorter_than_the_window(C, W, lens):
+    """The ring has not wrapped when the later segments arrive: the limits of its slots follow the branch for
+    _seen_tokens < W (nats_chunk_layer_cache.py:666-676), which the call can only take when it is told the number of
+    tokens the cache has seen.  (Chunked cache only: a per-token cache that has seen fewer tokens than its window may
+    hold blocks of sliding-window tokens left in place behind a head's own rows, nats_layer_cache.py:316-327, which
+    the kernel's argument list cannot describe; `cache.segment_attention` covers that case.)"""
+    run_smoke_pattern(2, 2, 2, 64, W, C, lens, torch.float32, seed=50 + C, cache_scalars=True)
+    run_smoke_pattern(1, 2, 4, 128, W, C, lens, torch.bfloat16, seed=60 + C, cache_scalars=True)
+
+
+def test_an_unfilled_window_is_not_taken_for_a_full_one():
+    from neuralattentionsearch_amd import ops
+    say("nats_prefill seam: ambiguous ring")
+    W, C = 32, 8
+    q = torch.zeros(1, 2, 8, 64, device="cuda")
+    k = torch.zeros(1, 2, W + 16 + 8, 64, device="cuda")
+    idx = torch.zeros(1, 2, 1, dtype=torch.int64, device="cuda")
+    sizes = torch.full((1, 2), W + 8, dtype=torch.int64, device="cuda")
+    ring = torch.zeros(1, 2, W // C, dtype=torch.bool, device="cuda")
+    ring[..., 0] = True
+    kw = dict(nats_chunk_size=C, n_rep=1, local_seq_max_length=W, global_kv_size=sizes, local_kv_size=sizes - W,
+              valid_sw_tokens=ring, n_ctx_data=W + 16, sw_token_tails=16)
+    with pytest.raises(ValueError, match="seen_tokens"):
+        ops.nats_prefill(q, k, k, idx, idx.float(), 1.0, **kw)
+    o, _ = ops.nats_prefill(q, k, k, idx, idx.float(), 1.0, seen_tokens=16, **kw)
+    assert tuple(o.shape) == (1, 2, 8, 64)
 
 
 def test_arguments_are_checked():

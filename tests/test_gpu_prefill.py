@@ -424,3 +424,4 @@ def test_two_prefills_on_two_streams_equal_the_serial_results():
             st.synchronize()
         for o, want in zip(outs, serial):
             assert torch.equal(o, want), rep
+
