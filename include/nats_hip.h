@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define NATS_ABI_VERSION 7
+#define NATS_ABI_VERSION 8
 
 typedef enum {
   NATS_OK = 0,
@@ -332,6 +332,21 @@ int nats_cache_append(const void* k, const void* v, void* cache_k, void* cache_v
                       int64_t H_kv, int64_t x_len, int64_t D, int64_t row0, int64_t n_alloc, int64_t pos0,
                       const int64_t* k_strides, const int64_t* v_strides, const int64_t* cache_strides,
                       const int64_t* valid_strides, int elem_bytes, void* stream);
+
+/* nats_cache_append and, in the same launch, nats_evict_plan for the eviction that follows this update (the roles of
+ * the chunks the update completes are known when the rows arrive, NAtSChunkLayerCache.update / _post_update,
+ * components/cache/nats_chunk_layer_cache.py:171-256, 270-371): a stream that appends a chunk and evicts, step after
+ * step, then costs two launches per step, this one and nats_evict_apply_inplace.  `params` describe the coming
+ * post_update as they would for nats_evict_plan (n_alloc, n_ctx_data, gmin, tail as they stand before it; x_len = the
+ * rows appended here).  For params->S <= 32 and B * H_kv <= 4096; otherwise NATS_ERR_UNSUPPORTED (call the two
+ * entry points).
+ */
+int nats_cache_append_plan(const void* k, const void* v, void* cache_k, void* cache_v, uint8_t* valid, int32_t* pos,
+                           int64_t B, int64_t H_kv, int64_t x_len, int64_t D, int64_t row0, int64_t n_alloc, int64_t pos0,
+                           const int64_t* k_strides, const int64_t* v_strides, const int64_t* cache_strides,
+                           const int64_t* valid_strides, int elem_bytes, const uint8_t* roles, const int64_t* size_global,
+                           const int64_t* size_local, const nats_evict_params* params, void* workspace,
+                           size_t workspace_bytes, nats_evict_result* result, nats_evict_brief* result_mirror, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
  * Decode-step glue of the HF-shaped caller (models/transformer/hf/llama_nats_chunk.py:171-292 inside a Llama

@@ -20,7 +20,7 @@ c_i64p = ctypes.POINTER(ctypes.c_int64)
 NATS_DTYPE_BF16 = 0
 NATS_DTYPE_F32 = 1
 
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 
 class EvictParams(ctypes.Structure):
@@ -75,6 +75,9 @@ SIGNATURES = {
     "nats_evict_apply_first": (ctypes.c_int, [c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, ctypes.POINTER(EvictParams),
                                               c_i64p, c_i64p, c_i64p, ctypes.c_int, c_p, c_p, c_p]),
     "nats_cache_append": (ctypes.c_int, [c_p] * 6 + [c_i64] * 7 + [c_i64p] * 4 + [ctypes.c_int, c_p]),
+    "nats_cache_append_plan": (ctypes.c_int, [c_p] * 6 + [c_i64] * 7 + [c_i64p] * 4 + [ctypes.c_int, c_p, c_p, c_p,
+                                                                                        ctypes.POINTER(EvictParams), c_p,
+                                                                                        ctypes.c_size_t, c_p, c_p, c_p]),
     "nats_add_rms_norm": (ctypes.c_int, [c_p, c_p, c_p, c_p, c_p, c_i64, c_i64, ctypes.c_float, ctypes.c_int, c_i64,
                                          ctypes.c_int, c_p]),
     "nats_silu_mul": (ctypes.c_int, [c_p, c_p, c_i64, c_i64, ctypes.c_int, c_p]),

@@ -84,6 +84,7 @@ class NAtSChunkLayerCache:
         self._append_call = None  # ops.CacheAppendCall / ops.EvictInplaceCall prepared for the present buffers
         self._inplace_call = None
         self._inplace_params = None
+        self._planned = None  # (sequence number, roles, facts) of an eviction whose plan rode with the append of its rows
         self.reset_cache()
 
     # -- state ----------------------------------------------------------------------------------
@@ -101,6 +102,7 @@ class NAtSChunkLayerCache:
         self._roles = None
         self._buf_k = self._buf_v = self._buf_valid = self._buf_pos = None
         self._append_call = self._inplace_call = None  # (they hold the buffers)
+        self._planned = None
         self._uninit = False  # the buffers came from torch.empty and only the eviction kernel has written them
         self._clean = None    # if set: buffer rows from this one on hold nothing yet, not even zeros
         self._n_rows = 0
@@ -350,16 +352,47 @@ class NAtSChunkLayerCache:
         start = self.n_ctx_data
         end = start + x_len
         self._grow(math.ceil(end / self.chunk_size) * self.chunk_size)
-        self._write_rows(key_states, value_states, start, end)
+        self._write_rows(key_states, value_states, start, end, plan_ahead=True)
         return self._buf_k[:, :, :end], self._buf_v[:, :, :end]
 
-    def _write_rows(self, key_states, value_states, start: int, end: int):
+    def _inplace_prepare(self, x_len: int, seen_after: int):
+        """Parameter struct and prepared call of the in-place eviction that follows an update of x_len tokens, from the
+        state as it stands between that update and its post_update; also the facts the struct was filled from."""
+        C, W = self.chunk_size, self.sliding_window_size
+        roles, fill = self._roles, self.chunk_fill_size
+        S, D = roles.shape[-1], self._buf_k.shape[3]
+        params = self._inplace_params
+        if params is None or params.D != D:
+            params = self._inplace_params = ops.evict_params(self.bsz, self.n_msks, D, C, W, S, 0, 0, 0, 0, 0, False, 0)
+        facts = (S, x_len, fill, int(seen_after == x_len), self.n_ctx_data, self._n_global_min, self.sliding_queue_tail, self._rows)
+        (params.S, params.x_len, params.fill, params.first, params.n_ctx_data, params.gmin, params.tail, params.n_alloc) = facts
+        call = self._inplace_call
+        if call is None or not call.matches(self._buf_k, self._buf_v, self._buf_valid, self._buf_pos, S):
+            if self._evict is None:
+                self._evict = ops.EvictBuffers(self.device)
+            call = self._inplace_call = ops.EvictInplaceCall(self._buf_k, self._buf_v, self._buf_valid, self._buf_pos,
+                                                             self.size_global_kv, self.size_local_kv, self._evict,
+                                                             self.bsz, self.n_msks, S)
+        return params, call, facts
+
+    def _write_rows(self, key_states, value_states, start: int, end: int, plan_ahead: bool = False):
         """Rows [start, end) of the cache, their valid bytes and stream positions: one kernel where the layouts
-        allow 16-byte accesses, slice assignments otherwise."""
+        allow 16-byte accesses, slice assignments otherwise.  When the update completes a chunk and the roles are few,
+        the same launch plans the eviction its post_update will run (`plan_ahead`)."""
         call = self._append_call
         if call is None or not call.matches(key_states, value_states, self._buf_k, self._buf_v, self._buf_valid, self._buf_pos):
             call = self._append_call = ops.CacheAppendCall(key_states, value_states, self._buf_k, self._buf_v,
                                                            self._buf_valid, self._buf_pos)
+        self._planned = None
+        roles = self._roles
+        if (plan_ahead and roles is not None and self.chunk_fill_size >= self.chunk_size and call.ok
+                and roles.shape[-1] <= ops.EvictInplaceCall.PLAN_WITH_APPEND_SLOTS
+                and self.bsz * self.n_msks <= ops.EvictInplaceCall.PLAN_WITH_APPEND_HEADS):
+            x_len = end - start
+            params, plan, facts = self._inplace_prepare(x_len, self._seen_tokens + x_len)
+            if call(key_states, value_states, start, self._seen_tokens, plan=plan, roles=roles, params=params):
+                self._planned = (params.seq, roles, facts)
+                return
         if call(key_states, value_states, start, self._seen_tokens):
             return
         self._buf_k[:, :, start:end] = key_states.to(self._buf_k.dtype)
@@ -459,19 +492,15 @@ class NAtSChunkLayerCache:
         if self._evict is None:
             self._evict = ops.EvictBuffers(self.device)
         if src is None:
-            # a cache that holds rows: plan + in-place apply through the call prepared for these buffers
-            params = self._inplace_params
-            if params is None or params.D != D:
-                params = self._inplace_params = ops.evict_params(self.bsz, self.n_msks, D, C, W, S, 0, 0, 0, 0, 0, False, 0)
-            params.S, params.x_len, params.fill, params.first = S, x_len, fill, int(first)
-            params.n_ctx_data, params.gmin, params.tail = self.n_ctx_data, self._n_global_min, self.sliding_queue_tail
-            params.n_alloc = self._rows
-            call = self._inplace_call
-            if call is None or not call.matches(self._buf_k, self._buf_v, self._buf_valid, self._buf_pos, S):
-                call = self._inplace_call = ops.EvictInplaceCall(self._buf_k, self._buf_v, self._buf_valid, self._buf_pos,
-                                                                 self.size_global_kv, self.size_local_kv, self._evict,
-                                                                 self.bsz, self.n_msks, S)
-            call(roles, params)
+            # a cache that holds rows: plan + in-place apply through the call prepared for these buffers; the plan
+            # has run already if it rode with the append of these rows
+            params, call, facts = self._inplace_prepare(x_len, self._seen_tokens)
+            planned, self._planned = self._planned, None
+            if planned is not None and planned[1] is roles and planned[2] == facts:
+                params.seq = planned[0]
+                call.apply_planned(roles, params)
+            else:
+                call(roles, params)
             self._await = (params.seq, first)  # picked up when the host next needs n_ctx_data or the minimum global size
         else:
             params = ops.evict_params(self.bsz, self.n_msks, D, C, W, S, x_len, fill, self.n_ctx_data, self._n_global_min,
@@ -678,15 +707,32 @@ class NAtSLayerCache(NAtSChunkLayerCache):
         D = like.shape[3]
         if self._evict is None:
             self._evict = ops.EvictBuffers(self.device)
-        params = ops.evict_params(self.bsz, self.n_msks, D, 1, W, fill, x_len, fill, block_start, self._n_global_min,
-                                  self.sliding_queue_tail, first_ring, max(self._rows, 1), update_chunk=U)
-        ws, result = ops.evict_plan(roles, self.size_global_kv, self.size_local_kv, params, self._evict)
         self._row_end = None
-        if src is None or not self._evict_first(src, roles, params, ws, result, first_call):
+        if src is None:
+            # a cache that holds rows: plan + in-place apply through the call prepared for these buffers
+            params = self._inplace_params
+            if params is None or params.D != D:
+                params = self._inplace_params = ops.evict_params(self.bsz, self.n_msks, D, 1, W, fill, 0, 0, 0, 0, 0, False, 0,
+                                                                 update_chunk=U)
+            params.S, params.x_len, params.fill, params.first = fill, x_len, fill, int(first_ring)
+            params.n_ctx_data, params.gmin, params.tail = block_start, self._n_global_min, self.sliding_queue_tail
             params.n_alloc = self._rows
-            ops.evict_apply_inplace(self._buf_k, self._buf_v, self._buf_valid, self._buf_pos, roles, self.size_global_kv,
-                                    self.size_local_kv, params, ws, result)
+            call = self._inplace_call
+            if call is None or not call.matches(self._buf_k, self._buf_v, self._buf_valid, self._buf_pos, fill):
+                call = self._inplace_call = ops.EvictInplaceCall(self._buf_k, self._buf_v, self._buf_valid, self._buf_pos,
+                                                                 self.size_global_kv, self.size_local_kv, self._evict,
+                                                                 self.bsz, self.n_msks, fill)
+            call(roles, params)
             self._await = (params.seq, first_call)  # picked up when the host next needs n_ctx_data
+        else:
+            params = ops.evict_params(self.bsz, self.n_msks, D, 1, W, fill, x_len, fill, block_start, self._n_global_min,
+                                      self.sliding_queue_tail, first_ring, max(self._rows, 1), update_chunk=U)
+            ws, result = ops.evict_plan(roles, self.size_global_kv, self.size_local_kv, params, self._evict)
+            if not self._evict_first(src, roles, params, ws, result, first_call):
+                params.n_alloc = self._rows
+                ops.evict_apply_inplace(self._buf_k, self._buf_v, self._buf_valid, self._buf_pos, roles, self.size_global_kv,
+                                        self.size_local_kv, params, ws, result)
+                self._await = (params.seq, first_call)
         n_ring = min(fill, W)  # :437-445
         self.sliding_queue_tail = n_ring - 1 if first_ring else (self.sliding_queue_tail + n_ring) % W
         self.chunk_fill_size = 0

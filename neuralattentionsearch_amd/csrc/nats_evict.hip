@@ -683,6 +683,38 @@ __global__ __launch_bounds__(256) void cache_append_kernel(AppendArgs a) {
   }
 }
 
+// The append and the plan of the eviction that follows it in one launch: the last workgroup along x (of head 0,
+// tensor 0) has no rows to copy and runs the small plan kernel's work instead.  What the plan reads (roles, sizes,
+// the host's scalars) does not depend on the rows being appended.
+__global__ __launch_bounds__(256) void cache_append_plan_kernel(AppendArgs a, const uint8_t* __restrict__ roles,
+                                                                const int64_t* __restrict__ size_global,
+                                                                const int64_t* __restrict__ size_local, nats_evict_params p,
+                                                                char* __restrict__ ws, nats_evict_result* __restrict__ result,
+                                                                nats_evict_brief* __restrict__ result_mirror) {
+  if (blockIdx.x + 1 < gridDim.x) {
+    const int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int head = blockIdx.y, which = blockIdx.z;
+    const int b = head / a.H_kv, h = head % a.H_kv;
+    const int64_t l = u / a.upr;
+    const int col = (int)(u % a.upr);
+    if (l >= a.x_len) return;
+    const uint4* src = static_cast<const uint4*>(a.src[which]) + b * a.ss[which][0] + h * a.ss[which][1] + l * a.ss[which][2] + col;
+    uint4* dst = static_cast<uint4*>(a.dst[which]) + b * a.ds[0] + h * a.ds[1] + (a.row0 + l) * a.ds[2] + col;
+    *dst = *src;
+    if (which == 0 && col == 0) {
+      const int64_t at = b * a.vs_b + h * a.vs_h + a.row0 + l;
+      a.valid[at] = 1;
+      if (a.pos) a.pos[at] = (int32_t)(a.pos0 + l);
+    }
+    return;
+  }
+  if (blockIdx.y != 0 || blockIdx.z != 0) return;
+  const int n_heads = (int)(p.B * p.H_kv);
+  for (int head = threadIdx.x; head < n_heads; head += 256) plan_one_head_serial(roles, size_global, size_local, p, ws, head);
+  __syncthreads();  // (global writes of this workgroup are visible to it after the barrier)
+  plan_finalize(size_global, size_local, p, ws, result, result_mirror);
+}
+
 static int check_params(const char* who, const nats_evict_params* p) {
   NATS_REQUIRE(p, NATS_ERR_NULL_POINTER, "%s: params must not be NULL", who);
   NATS_REQUIRE(p->B > 0 && p->H_kv > 0 && p->D > 0 && p->S > 0, NATS_ERR_BAD_SHAPE, "%s: B=%lld H_kv=%lld D=%lld S=%lld", who,
@@ -826,11 +858,10 @@ extern "C" int nats_evict_apply_first(const void* src_k, const void* src_v, void
   return NATS_OK;
 }
 
-extern "C" int nats_cache_append(const void* k, const void* v, void* cache_k, void* cache_v, uint8_t* valid, int32_t* pos,
-                                 int64_t B, int64_t H_kv, int64_t x_len, int64_t D, int64_t row0, int64_t n_alloc, int64_t pos0,
-                                 const int64_t* k_strides, const int64_t* v_strides, const int64_t* cache_strides,
-                                 const int64_t* valid_strides, int elem_bytes, void* stream) {
-  const char* who = "nats_cache_append";
+static int fill_append_args(const char* who, AppendArgs& a, const void* k, const void* v, void* cache_k, void* cache_v,
+                            uint8_t* valid, int32_t* pos, int64_t B, int64_t H_kv, int64_t x_len, int64_t D, int64_t row0,
+                            int64_t n_alloc, int64_t pos0, const int64_t* k_strides, const int64_t* v_strides,
+                            const int64_t* cache_strides, const int64_t* valid_strides, int elem_bytes, dim3* grid) {
   NATS_REQUIRE(k && v && cache_k && cache_v && valid, NATS_ERR_NULL_POINTER, "%s: NULL pointer argument", who);
   NATS_REQUIRE(k_strides && v_strides && cache_strides && valid_strides, NATS_ERR_NULL_POINTER, "%s: NULL stride array", who);
   NATS_REQUIRE(B > 0 && H_kv > 0 && x_len > 0 && D > 0 && B * H_kv <= 65535, NATS_ERR_BAD_SHAPE,
@@ -839,7 +870,6 @@ extern "C" int nats_cache_append(const void* k, const void* v, void* cache_k, vo
                (long long)row0, (long long)(row0 + x_len), (long long)n_alloc);
   NATS_REQUIRE(elem_bytes == 2 || elem_bytes == 4, NATS_ERR_BAD_DTYPE, "%s: element size %d", who, elem_bytes);
   NATS_REQUIRE((D * elem_bytes) % 16 == 0, NATS_ERR_UNSUPPORTED, "%s: row of %lld bytes", who, (long long)(D * elem_bytes));
-  AppendArgs a;
   for (int i = 0; i < 3; ++i) {
     NATS_REQUIRE((k_strides[i] * elem_bytes) % 16 == 0 && (v_strides[i] * elem_bytes) % 16 == 0 &&
                      (cache_strides[i] * elem_bytes) % 16 == 0,
@@ -858,8 +888,51 @@ extern "C" int nats_cache_append(const void* k, const void* v, void* cache_k, vo
   a.x_len = (int)x_len; a.upr = (int)(D * elem_bytes / 16); a.H_kv = (int)H_kv;
   const int64_t units = x_len * a.upr;
   NATS_REQUIRE(units < (int64_t(1) << 38), NATS_ERR_BAD_SHAPE, "%s: too many rows", who);
-  dim3 grid((unsigned)((units + 255) / 256), (unsigned)(B * H_kv), 2u);
+  *grid = dim3((unsigned)((units + 255) / 256), (unsigned)(B * H_kv), 2u);
+  return NATS_OK;
+}
+
+extern "C" int nats_cache_append(const void* k, const void* v, void* cache_k, void* cache_v, uint8_t* valid, int32_t* pos,
+                                 int64_t B, int64_t H_kv, int64_t x_len, int64_t D, int64_t row0, int64_t n_alloc, int64_t pos0,
+                                 const int64_t* k_strides, const int64_t* v_strides, const int64_t* cache_strides,
+                                 const int64_t* valid_strides, int elem_bytes, void* stream) {
+  AppendArgs a;
+  dim3 grid;
+  if (int rc = fill_append_args("nats_cache_append", a, k, v, cache_k, cache_v, valid, pos, B, H_kv, x_len, D, row0, n_alloc,
+                                pos0, k_strides, v_strides, cache_strides, valid_strides, elem_bytes, &grid))
+    return rc;
   hipLaunchKernelGGL(cache_append_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream), a);
   NATS_CHECK_LAUNCH("cache_append_kernel");
+  return NATS_OK;
+}
+
+extern "C" int nats_cache_append_plan(const void* k, const void* v, void* cache_k, void* cache_v, uint8_t* valid, int32_t* pos,
+                                      int64_t B, int64_t H_kv, int64_t x_len, int64_t D, int64_t row0, int64_t n_alloc,
+                                      int64_t pos0, const int64_t* k_strides, const int64_t* v_strides,
+                                      const int64_t* cache_strides, const int64_t* valid_strides, int elem_bytes,
+                                      const uint8_t* roles, const int64_t* size_global, const int64_t* size_local,
+                                      const nats_evict_params* params, void* workspace, size_t workspace_bytes,
+                                      nats_evict_result* result, nats_evict_brief* result_mirror, void* stream) {
+  const char* who = "nats_cache_append_plan";
+  AppendArgs a;
+  dim3 grid;
+  if (int rc = fill_append_args(who, a, k, v, cache_k, cache_v, valid, pos, B, H_kv, x_len, D, row0, n_alloc, pos0, k_strides,
+                                v_strides, cache_strides, valid_strides, elem_bytes, &grid))
+    return rc;
+  NATS_REQUIRE(roles && size_global && size_local && workspace && result, NATS_ERR_NULL_POINTER, "%s: NULL pointer argument", who);
+  if (int rc = check_params(who, params)) return rc;
+  NATS_REQUIRE(params->B == B && params->H_kv == H_kv && params->x_len == x_len, NATS_ERR_BAD_SHAPE,
+               "%s: the eviction parameters describe another update (B=%lld H_kv=%lld x_len=%lld)", who, (long long)params->B,
+               (long long)params->H_kv, (long long)params->x_len);
+  NATS_REQUIRE(params->S <= 32 && B * H_kv <= 4096, NATS_ERR_UNSUPPORTED,
+               "%s: %lld role slots for %lld heads: the plan that rides with an append takes at most 32 for 4096 (use "
+               "nats_cache_append and nats_evict_plan)",
+               who, (long long)params->S, (long long)(B * H_kv));
+  size_t need = nats_evict_workspace_bytes(params->B, params->H_kv, params->S);
+  NATS_REQUIRE(workspace_bytes >= need, NATS_ERR_WORKSPACE, "%s: workspace %zu bytes < %zu", who, workspace_bytes, need);
+  grid.x += 1;  // the workgroup that plans
+  hipLaunchKernelGGL(cache_append_plan_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream), a, roles, size_global,
+                     size_local, *params, static_cast<char*>(workspace), result, result_mirror);
+  NATS_CHECK_LAUNCH("cache_append_plan_kernel");
   return NATS_OK;
 }

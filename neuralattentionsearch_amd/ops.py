@@ -597,6 +597,7 @@ class CacheAppendCall:
         fix = lambda t: tuple(st if n != 1 else e for st, n in zip(t.stride()[:3], t.shape[:3]))
         B, H, x_len, D = k.shape
         self.fn = _lib.load().nats_cache_append
+        self.fn_plan = _lib.load().nats_cache_append_plan
         self.head = (_ptr(cache_k), _ptr(cache_v), _ptr(valid), _ptr(pos), B, H, x_len, D)
         self.n_rows = min(cache_k.shape[2], valid.shape[2])
         self.tail = (i64_array(fix(k)), i64_array(fix(v)), i64_array(fix(cache_k)), i64_array(valid.stride()[:2]),
@@ -607,12 +608,19 @@ class CacheAppendCall:
         return (b[0] is cache_k and b[1] is cache_v and b[2] is valid and b[3] is pos
                 and self.key == (k.shape, k.stride(), v.stride(), k.dtype, v.dtype, k.device))
 
-    def __call__(self, k, v, row0: int, pos0: int = 0) -> bool:
-        """Appends and returns True; False if these tensors cannot take the kernel (layout or alignment)."""
+    def __call__(self, k, v, row0: int, pos0: int = 0, plan: "EvictInplaceCall | None" = None, roles=None, params=None) -> bool:
+        """Appends and returns True; False if these tensors cannot take the kernel (layout or alignment).  With `plan`
+        (and the roles and parameters of the eviction that will follow this update) the same launch also plans that
+        eviction, which `plan.apply_planned` then only has to apply."""
         pk, pv = k.data_ptr(), v.data_ptr()
         if not self.ok or (pk | pv) & 15:
             return False
-        check(self.fn(pk, pv, *self.head, row0, self.n_rows, pos0, *self.tail, _stream(k)))
+        if plan is None:
+            check(self.fn(pk, pv, *self.head, row0, self.n_rows, pos0, *self.tail, _stream(k)))
+        else:
+            params.seq = plan.buffers.next_seq()
+            check(self.fn_plan(pk, pv, *self.head, row0, self.n_rows, pos0, *self.tail, roles.data_ptr(), *plan.sizes,
+                               ctypes.byref(params), *plan.plan_tail, _stream(k)))
         return True
 
 
@@ -645,6 +653,8 @@ class EvictInplaceCall:
         return (b[0] is cache_k and b[1] is cache_v and b[2] is valid and b[3] is pos and self.S == S
                 and self.ws is self.buffers.ws)
 
+    PLAN_WITH_APPEND_SLOTS, PLAN_WITH_APPEND_HEADS = 32, 4096  # what nats_cache_append_plan takes
+
     def __call__(self, roles: torch.Tensor, params: EvictParams):
         if not roles.is_cuda or roles.dtype != torch.uint8 or not roles.is_contiguous():
             raise ValueError("roles must be a contiguous uint8 GPU tensor")
@@ -652,6 +662,11 @@ class EvictInplaceCall:
         pr, ref, st = roles.data_ptr(), ctypes.byref(params), _stream(roles)
         check(self.plan(pr, *self.sizes, ref, *self.plan_tail, st))
         check(self.apply(*self.apply_head, pr, *self.sizes, ref, *self.apply_tail, st))
+
+    def apply_planned(self, roles: torch.Tensor, params: EvictParams):
+        """The apply step alone, for an eviction whose plan rode with the append (`CacheAppendCall(..., plan=self)`):
+        `params` are the ones that launch was given, sequence number included."""
+        check(self.apply(*self.apply_head, roles.data_ptr(), *self.sizes, ctypes.byref(params), *self.apply_tail, _stream(roles)))
 
 
 def evict_apply_inplace(cache_k, cache_v, valid, pos, roles, size_global, size_local, params: EvictParams, ws, result):
