@@ -1,8 +1,8 @@
 """Benchmark of the NAtS sparse-attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-cpu] [--no-llama] [--only prefill|decode|evict|evict_stream|segments|role_step|matvec|llama]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-cpu] [--no-llama] [--no-extras] [--only prefill|decode|evict|evict_stream|segments|role_step|matvec|llama]
 
-    (other sizes of a single leg: --prefill-len L, --chunk-size C, --decode-batch B, --decode-context N)
+    (other sizes of a single leg: --prefill-len L, --chunk-size C, --decode-batch B, --decode-context N, --llama-chunk C)
 
 One step = one pass of a kernel family over one batch of synthetic input that is already resident in HBM:
 
@@ -10,7 +10,11 @@ One step = one pass of a kernel family over one batch of synthetic input that is
 * decode   one query token per sequence over the ragged, evicted KV cache (batch 32, context 65536)
 * evict    bulk eviction + compaction of a 16 x 8 x 65536 x 128 cache after its prefill
 * llama_e2e  the three together inside a random-weight Llama-3-8B-shape model: a 16384-token prefill, then 512 greedy
-           one-token steps with eviction live in all 32 layers (seconds for the prefill, ms per token)
+           one-token steps with eviction live in all 32 layers (seconds for the prefill, ms per token, peak memory);
+           llama_e2e_c1 the same with a role per token (the per-token cache class)
+* riding along under their own keys: prefill_c32 / prefill_c1 (the prefill at chunk sizes 32 and 1), decode_b1 (one
+           sequence), evict.cold (a layer cache that has never evicted), evict_stream (the eviction workload chunk by
+           chunk), segments (the prefill cut into four segments over one cache)
 
 Prints ONE JSON line.  `value` is the prefill time in ms; decode tokens/s, GB/s and the compaction GB/s
 ride along in the same line, each with its roofline fraction, next to a CPU baseline (the oracle, timed
@@ -87,32 +91,50 @@ METRIC = "NAtS prefill ms @32k (MFMA util); sparse-KV decode tok/s (HBM GB/s %pe
 
 
 def draw_roles(seed, B, H, S, p):
+    """Roles drawn directly (CPU legs, where no role kernel runs)."""
     rng = np.random.default_rng(seed)
     r = rng.choice(3, size=(B, H, S), p=p).astype(np.uint8)
     r[:, :, 0] = 0  # sink chunk
     return r
 
 
-def chunk_visibility_np(roles: np.ndarray, wc: int) -> np.ndarray:
-    """Vectorised chunk-level visibility with the causal cut: bool [B, H, S, S]."""
+# Role logits of the GPU legs: N(0, 1) per (chunk, head, option) plus these constants on (global, local, sliding window).
+# With the 0.1 the role kernel adds to the global logit (models/transformer/attention/nats_attention.py:96-109) the
+# first-maximum argmax then lands on the configured shares: P(option i) = int phi(z - b_i) prod_{j != i} Phi(z - b_j) dz
+# solved for b (sliding window fixed at 0).
+ROLE_LOGIT_BIAS = {
+    (0.05, 0.15, 0.80): (-2.17317727, -1.38648285, 0.0),   # prefill workload
+    (0.10, 0.15, 0.75): (-1.67833392, -1.31208150, 0.0),   # eviction workload
+}
+ROLE_GLOBAL_BIAS = 0.1
+
+
+def biased_role_logits(seed, B, S, H, shares, device="cuda"):
+    """fp32 [B, S, H, 3] logits whose argmax (through ops.roles_from_logits with the first chunk forced global) gives
+    roles in the shares (global, local, sliding window)."""
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(B, S, H, 3, generator=g) + torch.tensor(ROLE_LOGIT_BIAS[shares])
+    return x.to(device)
+
+
+def chunk_limits_np(roles: np.ndarray, wc: int) -> np.ndarray:
+    """Last query chunk that sees key chunk n, per (b, h, n): global -> S - 1, sliding window -> n + W / C, local ->
+    the next global chunk at or after n (the last chunk counts as one)."""
     B, H, S = roles.shape
     is_g = roles == 0
     flags = is_g.copy()
     flags[..., -1] = True
     idx = np.where(flags, np.arange(S), S)  # next global at or after n: reverse running minimum
     g = np.minimum.accumulate(idx[..., ::-1], axis=-1)[..., ::-1]
-    m = np.arange(S)[:, None]
-    n = np.arange(S)[None, :]
-    lim = np.where(is_g, np.iinfo(np.int32).max, np.where(roles == 2, np.arange(S) + wc, g))
-    return (n <= m)[None, None] & (m[None, None] <= lim[:, :, None, :])
+    lim = np.where(is_g, S - 1, np.where(roles == 2, np.arange(S) + wc, g))
+    return np.minimum(lim, S - 1)
 
 
 def prefill_flops(roles: np.ndarray, L: int, C: int, W: int, D: int, n_rep: int) -> tuple[float, float]:
     """Algorithmic FLOPs on the visited (query chunk, key chunk) pairs and the dense causal count."""
-    vis = chunk_visibility_np(roles, W // C)
     S = roles.shape[-1]
-    diag = np.eye(S, dtype=bool)[None, None]
-    off = (vis & ~diag).sum()
+    lim = chunk_limits_np(roles, W // C).astype(np.int64)
+    off = int((lim - np.arange(S)).sum())  # query chunks after n that see it
     n_streams = roles.shape[0] * roles.shape[1]
     pairs = off * C * C + n_streams * S * (C * (C + 1) // 2)
     dense = n_streams * (L * (L + 1) // 2)
@@ -150,18 +172,24 @@ def time_gpu(fn, steps: int, warmup: int):
 
 
 # --------------------------------------------------------------------------------------------------
-def bench_prefill(args, ops):
-    B, Hq, Hkv, L, D, C, W = 1, 32, 8, args.prefill_len, 128, args.chunk_size, 256
+def bench_prefill(args, ops, chunk_size=None, steps=None, warmup=None, compare=True, settle=True):
+    B, Hq, Hkv, L, D, C, W = 1, 32, 8, args.prefill_len, 128, chunk_size or args.chunk_size, 256
+    steps, warmup = steps or args.steps, args.warmup if warmup is None else warmup
     n_rep = Hq // Hkv
     dev = "cuda"
     g = torch.Generator(device=dev).manual_seed(0)
     q = (torch.randn(B, Hq, L, D, generator=g, device=dev) / math.sqrt(D)).bfloat16()
     k = (torch.randn(B, Hkv, L, D, generator=g, device=dev) / math.sqrt(D)).bfloat16()
     v = (torch.randn(B, Hkv, L, D, generator=g, device=dev) / math.sqrt(D)).bfloat16()
-    roles_np = draw_roles(0, B, Hkv, L // C, (0.05, 0.15, 0.80))
-    roles = torch.from_numpy(roles_np).to(dev)
+    logits = biased_role_logits(0, B, L // C, Hkv, (0.05, 0.15, 0.80), dev)
+    roles, _ = ops.roles_from_logits(logits, ROLE_GLOBAL_BIAS, True, False, with_one_hot=False)
+    roles_np = roles.cpu().numpy()
     out = torch.empty_like(q)
     flops, dense_flops = prefill_flops(roles_np, L, C, W, D, n_rep)
+
+    def sparse_step():  # the op as the attention module runs it: role logits -> roles -> masked attention
+        r, _ = ops.roles_from_logits(logits, ROLE_GLOBAL_BIAS, True, False, with_one_hot=False)
+        ops.prefill_attention(q, k, v, r, C, W, out=out)
 
     # Settling phase: the power management of the GPU takes some tens of milliseconds of matrix-heavy load to reach
     # its steady clock (the first launches after idle run up to 30 % slower than the settled ones), and a serving
@@ -169,31 +197,35 @@ def bench_prefill(args, ops):
     # kernel, so that a kernel trace of this run keeps the sparse workload's launches apart); the timed region itself
     # is W warm-up steps + K timed steps of the sparse workload, and the comparators are timed after it.
     roles_dense = torch.zeros_like(roles)
-    try:
-        for _ in range(3):
-            torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True)
-    except Exception:
-        for _ in range(6):
-            ops.prefill_attention(q, k, v, roles_dense, C, W, out=out)
+    if settle:
+        try:
+            for _ in range(3):
+                torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True)
+        except Exception:
+            for _ in range(6):
+                ops.prefill_attention(q, k, v, roles_dense, C, W, out=out)
 
-    wall, ev_mean, ev_min = time_gpu(lambda: ops.prefill_attention(q, k, v, roles, C, W, out=out), args.steps, args.warmup)
+    wall, ev_mean, ev_min = time_gpu(sparse_step, steps, warmup)
     res = {
         "ms": ev_mean, "ms_min": ev_min, "ms_wall": wall,
         "visited_fraction": flops / dense_flops, "algorithmic_tflop": flops / 1e12,
         "tflops_visited": flops / (ev_mean * 1e-3) / 1e12,
         "tokens_per_s": L / (ev_mean * 1e-3),
     }
-    res["shape"] = dict(B=B, Hq=Hq, Hkv=Hkv, L=L, D=D, C=C, W=W, roles="5% global / 15% local / 80% sliding")
-    if not args.no_compare:
+    shares = [float((roles_np == i).mean()) for i in range(3)]
+    res["shape"] = dict(B=B, Hq=Hq, Hkv=Hkv, L=L, D=D, C=C, W=W,
+                        roles="argmax of biased N(0,1) logits inside the timed op: %.1f%% global / %.1f%% local / %.1f%% sliding"
+                              % tuple(100 * x for x in shares))
+    if compare and not args.no_compare:
         # the same kernel on all-global roles = dense causal attention
-        _, dm, _ = time_gpu(lambda: ops.prefill_attention(q, k, v, roles_dense, C, W, out=out), max(2, args.steps // 4), 1)
+        _, dm, _ = time_gpu(lambda: ops.prefill_attention(q, k, v, roles_dense, C, W, out=out), max(2, steps // 4), 1)
         res["own_dense_causal_ms"] = dm
         res["own_dense_causal_tflops"] = dense_flops / (dm * 1e-3) / 1e12
         # a library dense causal flash attention of the same shape on the same GPU
         try:
             def sdpa():
                 return torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True)
-            _, sm, _ = time_gpu(sdpa, max(2, args.steps // 4), 1)
+            _, sm, _ = time_gpu(sdpa, max(2, steps // 4), 1)
             res["torch_sdpa_dense_causal_ms"] = sm
             res["torch_sdpa_dense_causal_tflops"] = dense_flops / (sm * 1e-3) / 1e12
             res["frac_of_dense_flash_throughput"] = res["tflops_visited"] / res["torch_sdpa_dense_causal_tflops"]
@@ -223,8 +255,8 @@ def decode_inputs(B, Hq, Hkv, D, C, W, ctx, seed, dev):
     return q, k, v, torch.from_numpy(valid).to(dev), n_rows, hint
 
 
-def bench_decode(args, ops):
-    B, Hq, Hkv, D, C, W, ctx = args.decode_batch, 32, 8, 128, 64, 256, args.decode_context
+def bench_decode(args, ops, batch=None, context=None):
+    B, Hq, Hkv, D, C, W, ctx = batch or args.decode_batch, 32, 8, 128, 64, 256, context or args.decode_context
     q, k, v, valid, n_rows, (row_end, tail_start) = decode_inputs(B, Hq, Hkv, D, C, W, ctx, 0, "cuda")
     n_valid = int(valid[:, :, :n_rows].sum().item())
     bytes_alg = n_valid * D * 2 * 2 + 2 * q.numel() * 2
@@ -242,28 +274,39 @@ def bench_decode(args, ops):
 
 
 def bench_evict(args, ops):
+    """Bulk eviction + compaction after a prefill.  `warm`: a layer cache that has been through a prompt before (what
+    NAtSCache.reset_cache leaves for the next prompt): the cache is allocated on the share of rows kept last time and the
+    apply kernel is launched without waiting for the plan.  `cold`: a layer cache that has never evicted (the first
+    prompt of a process): the host waits for the plan's row count before it allocates."""
     from neuralattentionsearch_amd.cache import NAtSChunkLayerCache
     B, Hkv, L, D, C, W = 16, 8, 65536, 128, 64, 512
     dev = "cuda"
     g = torch.Generator(device=dev).manual_seed(0)
     k = torch.randn(B, Hkv, L, D, generator=g, device=dev).bfloat16()
     v = torch.randn(B, Hkv, L, D, generator=g, device=dev).bfloat16()
-    roles_np = draw_roles(0, B, Hkv, L // C, (0.10, 0.15, 0.75))
-    tsi = torch.zeros(B, Hkv, L // C, 3, dtype=torch.bfloat16, device=dev)
-    tsi.scatter_(-1, torch.from_numpy(roles_np.astype(np.int64)).to(dev).unsqueeze(-1), 1.0)
-    roles = torch.from_numpy(roles_np).to(dev)
+    logits = biased_role_logits(0, B, L // C, Hkv, (0.10, 0.15, 0.75), dev)
+    roles0, _ = ops.roles_from_logits(logits, ROLE_GLOBAL_BIAS, True, False)
+    shares = [float((roles0 == i).float().mean().item()) for i in range(3)]
     cache = NAtSChunkLayerCache(B, Hkv, W, chunk_size=C, device=dev)
     moved = {}
 
-    def step():
+    def evict_into(c):
+        roles, tsi = ops.roles_from_logits(logits, ROLE_GLOBAL_BIAS, True, False)  # role logits -> roles + one-hot
+        c.update(k, v, tsi, roles=roles)
+        c.post_update(L)
+        moved["n_rows"] = c.cache_k.shape[2]  # (waits for the result of the plan kernel, as the next caller would)
+
+    def warm_step():
         cache.reset_cache()
-        cache.update(k, v, tsi, roles=roles)  # (one-hot and compact roles, as the role kernels hand them over)
-        cache.post_update(L)
-        moved["n_rows"] = cache.cache_k.shape[2]  # (waits for the result of the plan kernel, as the next caller would)
+        evict_into(cache)
+
+    def cold_step():
+        evict_into(NAtSChunkLayerCache(B, Hkv, W, chunk_size=C, device=dev))
 
     steps = max(3, args.steps // 2)
-    wall, ev_mean, ev_min = time_gpu(step, steps, 2)
+    wall, ev_mean, ev_min = time_gpu(warm_step, steps, 2)
     moved["rows"] = int(cache.last_evict_result.moved_rows)
+    c_wall, c_mean, c_min = time_gpu(cold_step, steps, 2)
     ring_rows = B * Hkv * W
     bytes_alg = (moved["rows"] + ring_rows) * D * 2 * 2 * 2  # rows x 256 B x (K, V) x (read + write)
     return {
@@ -271,8 +314,15 @@ def bench_evict(args, ops):
         "rows_moved": moved["rows"], "cache_rows_after": moved["n_rows"],
         "algorithmic_bytes": bytes_alg, "gbs": bytes_alg / (ev_mean * 1e-3) / 1e9,
         "frac_of_hbm_peak": bytes_alg / (ev_mean * 1e-3) / 1e9 / PEAK_HBM_GBS,
-        "note": "cache reset + update + whole post_update: plan kernel, its result through pinned memory, cache allocation, apply kernel",
-        "shape": dict(B=B, Hkv=Hkv, L=L, D=D, C=C, W=W, roles="10% global / 15% local / 75% sliding"),
+        "cold": {"ms": c_mean, "ms_min": c_min, "ms_wall": c_wall, "gbs": bytes_alg / (c_mean * 1e-3) / 1e9,
+                 "frac_of_hbm_peak": bytes_alg / (c_mean * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                 "note": "a fresh layer cache per step: role kernel, plan kernel, the host waits for its row count "
+                         "(pinned memory), allocation, apply kernel"},
+        "note": "role kernel + cache reset + update + whole post_update (plan kernel, apply kernel into a cache sized from "
+                "the previous prompt's kept share) + the wait for the plan's result",
+        "shape": dict(B=B, Hkv=Hkv, L=L, D=D, C=C, W=W,
+                      roles="argmax of biased N(0,1) logits inside the timed op: %.1f%% global / %.1f%% local / %.1f%% sliding"
+                            % tuple(100 * x for x in shares)),
     }
 
 
@@ -286,11 +336,10 @@ def bench_evict_stream(args, ops):
     g = torch.Generator(device=dev).manual_seed(0)
     k = torch.randn(B, Hkv, C, D, generator=g, device=dev).bfloat16()
     v = torch.randn(B, Hkv, C, D, generator=g, device=dev).bfloat16()
-    roles_np = draw_roles(0, B, Hkv, n_chunks, (0.10, 0.15, 0.75))
-    tsi_all = torch.zeros(B, Hkv, n_chunks, 3, dtype=torch.bfloat16, device=dev)
-    tsi_all.scatter_(-1, torch.from_numpy(roles_np.astype(np.int64)).to(dev).unsqueeze(-1), 1.0)
+    # (the roles of all 1024 steps come from one call of the role kernel ahead of the timed loop)
+    roles_all, tsi_all = ops.roles_from_logits(biased_role_logits(0, B, n_chunks, Hkv, (0.10, 0.15, 0.75), dev),
+                                               ROLE_GLOBAL_BIAS, True, False)
     tsis = [tsi_all[:, :, i:i + 1].contiguous() for i in range(n_chunks)]
-    roles_all = torch.from_numpy(roles_np).to(dev)
     roles = [roles_all[:, :, i:i + 1].contiguous() for i in range(n_chunks)]
     cache = NAtSChunkLayerCache(B, Hkv, W, chunk_size=C, device=dev)
 
@@ -308,7 +357,7 @@ def bench_evict_stream(args, ops):
     wall = time.perf_counter() - t0
     return {"total_s": wall, "us_per_chunk_step": wall / n_chunks * 1e6, "chunks": n_chunks,
             "cache_rows_after": int(cache.cache_k.shape[2]),
-            "note": "host-driven loop: update (one append kernel for 64 tokens) + post_update (plan kernel, in-place apply kernel; the plan's result reaches the host through pinned memory before the next append)",
+            "note": "host-driven loop: update (one kernel appends the 64 tokens and plans their eviction) + post_update (in-place apply kernel); the plan's result reaches the host through pinned memory before the next append",
             "shape": dict(B=B, Hkv=Hkv, L=L, D=D, C=C, W=W)}
 
 
@@ -326,10 +375,8 @@ def bench_segments(args, ops):
     q = (torch.randn(B, Hq, L, D, generator=g, device=dev) / math.sqrt(D)).bfloat16()
     k = (torch.randn(B, Hkv, L, D, generator=g, device=dev) / math.sqrt(D)).bfloat16()
     v = (torch.randn(B, Hkv, L, D, generator=g, device=dev) / math.sqrt(D)).bfloat16()
-    roles_np = draw_roles(0, B, Hkv, L // C, (0.05, 0.15, 0.80))
-    roles = torch.from_numpy(roles_np).to(dev)
-    tsi = torch.zeros(B, Hkv, L // C, 3, dtype=torch.bfloat16, device=dev)
-    tsi.scatter_(-1, roles.long().unsqueeze(-1), 1.0)
+    roles, tsi = ops.roles_from_logits(biased_role_logits(0, B, L // C, Hkv, (0.05, 0.15, 0.80), dev), ROLE_GLOBAL_BIAS,
+                                       True, False)
     sc = seg // C
     parts = [(q[:, :, i * seg:(i + 1) * seg], k[:, :, i * seg:(i + 1) * seg], v[:, :, i * seg:(i + 1) * seg],
               roles[:, :, i * sc:(i + 1) * sc].contiguous(), tsi[:, :, i * sc:(i + 1) * sc].contiguous()) for i in range(n_seg)]
@@ -420,42 +467,58 @@ def bench_matvec(args, ops):
     return out
 
 
-def bench_llama(args):
+def bench_llama(args, chunk_sizes=(64,)):
     """End to end at the Llama-3-8B shape with random weights: one prefill, then greedy decode steps with
-    eviction live in all 32 layers."""
+    eviction live in all 32 layers.  One set of weights serves every chunk size asked for (chunk size 1 = a role per
+    token and the per-token cache class); returns {chunk size: figures}."""
     from neuralattentionsearch_amd.llama import NAtSLlamaConfig, NAtSLlamaForCausalLM
     cfg = NAtSLlamaConfig.llama3_8b(fused_role_step=True)
     model = NAtSLlamaForCausalLM.random_init(cfg, seed=0)
     g = torch.Generator().manual_seed(0)
     ids = torch.randint(0, cfg.vocab_size, (1, args.llama_prefill), generator=g).cuda()
-    warm = model.new_cache()
-    logits = model(ids[:, :2048], 0, warm)  # loads every kernel and the GEMM heuristics once
-    for i in range(3):
-        logits = model(logits.argmax(-1, keepdim=True), 2048 + i, warm)
-    del warm
-    cache = model.new_cache()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    logits = model(ids, 0, cache)
-    torch.cuda.synchronize()
-    t_prefill = time.perf_counter() - t0
-    pos = args.llama_prefill
-    t0 = time.perf_counter()
-    for i in range(args.llama_decode):
-        logits = model(logits.argmax(-1, keepdim=True), pos, cache)
-        pos += 1
-    torch.cuda.synchronize()
-    t_decode = time.perf_counter() - t0
-    kept = [float(l.valid_tokens[:, :, :l.n_ctx_data].sum().item()) / (cfg.num_key_value_heads * pos) for l in cache.cache_model]
-    return {"prefill_s": t_prefill, "prefill_tokens_per_s": args.llama_prefill / t_prefill,
-            "decode_s": t_decode, "decode_tokens_per_s": args.llama_decode / t_decode,
-            "decode_ms_per_token": t_decode / args.llama_decode * 1e3,
-            "kept_fraction_mean": float(np.mean(kept)), "kept_fraction_min": float(np.min(kept)),
-            "kept_fraction_max": float(np.max(kept)),
-            "shape": dict(layers=cfg.num_hidden_layers, d_model=cfg.hidden_size, heads="32/8", head_dim=cfg.head_dim,
-                          ffn=cfg.intermediate_size, vocab=cfg.vocab_size, prefill=args.llama_prefill,
-                          decode_steps=args.llama_decode, chunk=cfg.chunk_size, window=cfg.local_seq_max_length),
-            "note": "random weights give near-uniform roles; prefill projections are library GEMMs; one-token steps use the matrix-vector, fused norm and rotary + append kernels"}
+    out = {}
+    for C in chunk_sizes:
+        cfg.chunk_size = C
+        for layer in model.layers:
+            layer.self_attn.chunk_size = C
+        warm = model.new_cache()
+        logits = model(ids[:, :2048], 0, warm)  # loads every kernel and the GEMM heuristics once
+        for i in range(3):
+            logits = model(logits.argmax(-1, keepdim=True), 2048 + i, warm)
+        del warm
+        torch.cuda.synchronize()
+        torch.cuda.reset_peak_memory_stats()
+        mem_before = torch.cuda.memory_allocated()
+        cache = model.new_cache()
+        t0 = time.perf_counter()
+        logits = model(ids, 0, cache)
+        torch.cuda.synchronize()
+        t_prefill = time.perf_counter() - t0
+        peak_prefill = torch.cuda.max_memory_allocated()
+        pos = args.llama_prefill
+        t0 = time.perf_counter()
+        for i in range(args.llama_decode):
+            logits = model(logits.argmax(-1, keepdim=True), pos, cache)
+            pos += 1
+        torch.cuda.synchronize()
+        t_decode = time.perf_counter() - t0
+        kept = [float(l.valid_tokens[:, :, :l.n_ctx_data].sum().item()) / (cfg.num_key_value_heads * pos) for l in cache.cache_model]
+        cache_bytes = sum(t.numel() * t.element_size() for l in cache.cache_model for t in (l._buf_k, l._buf_v, l._buf_valid) if t is not None)
+        out[C] = {"prefill_s": t_prefill, "prefill_tokens_per_s": args.llama_prefill / t_prefill,
+                  "decode_s": t_decode, "decode_tokens_per_s": args.llama_decode / t_decode,
+                  "decode_ms_per_token": t_decode / args.llama_decode * 1e3,
+                  "kept_fraction_mean": float(np.mean(kept)), "kept_fraction_min": float(np.min(kept)),
+                  "kept_fraction_max": float(np.max(kept)),
+                  # what the reference's harness prints beside its timings (experiments/efficiency/eval_efficiency.py:236-250)
+                  "max_memory_allocated_gb": torch.cuda.max_memory_allocated() / 1e9,
+                  "max_memory_allocated_prefill_gb": peak_prefill / 1e9,
+                  "weights_and_inputs_gb": mem_before / 1e9, "kv_cache_after_decode_gb": cache_bytes / 1e9,
+                  "shape": dict(layers=cfg.num_hidden_layers, d_model=cfg.hidden_size, heads="32/8", head_dim=cfg.head_dim,
+                                ffn=cfg.intermediate_size, vocab=cfg.vocab_size, prefill=args.llama_prefill,
+                                decode_steps=args.llama_decode, chunk=C, window=cfg.local_seq_max_length),
+                  "note": "random weights give near-uniform roles; prefill projections are library GEMMs; one-token steps use the matrix-vector, fused norm and rotary + append kernels"}
+        del cache, logits
+    return out
 
 
 # --------------------------------------------------------------------------------------------------
@@ -499,6 +562,18 @@ def cpu_baseline(args):
                    f"L=8192 {samples[8192]:.2f}s, L=16384 {samples[16384]:.2f}s; all 8 groups at L=16384 {t_all:.2f}s; "
                    f"value = that x (32768/16384)^2 (extrapolated, the [1,32,32768,32768] bool mask does not fit a host)"),
     }
+    # configs[0] whole, the one configuration the reference runs on a CPU: B=1, 8 heads, L=2048, D=64, fp32, chunk 64,
+    # window 128, roles = hard argmax of N(0, 1) logits; roles + mask + masked attention
+    g = torch.Generator().manual_seed(0)
+    q1, k1, v1 = (torch.randn(1, 8, 2048, 64, generator=g) for _ in range(3))
+    lg = torch.randn(1, 2048 // 64, 8, 3, generator=g)
+    reps, t0 = 0, time.perf_counter()
+    while reps < 3 or time.perf_counter() - t0 < 1.0:
+        r1 = orc.roles_from_logits(lg, 0.1, True, False)
+        orc.masked_attention(q1, k1, v1, orc.prefill_mask(r1, 2048, 64, 128))
+        reps += 1
+    out["cfg1_whole"] = {"value": (time.perf_counter() - t0) / reps * 1e3, "unit": "ms", "cores": use,
+                         "sample": f"configs[0] complete (B=1, H=8, L=2048, D=64, fp32, chunk 64, window 128), mean of {reps} runs"}
     # the same on one core, from the L = 8192 sample
     torch.set_num_threads(1)
     L = 8192
@@ -555,6 +630,9 @@ def main():
     ap.add_argument("--record-traffic", nargs="+", metavar="KEY=FETCH_KIB,WRITE_KIB",
                     help="store counter figures of prefill / decode / evict in bench_traffic.json and exit")
     ap.add_argument("--no-llama", action="store_true", help="skip the end-to-end Llama-3-8B-shape leg of the default run")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip the smaller legs of the default run (prefill at chunk 32 / 1, decode at batch 1, streamed eviction, segments, the per-token Llama leg)")
+    ap.add_argument("--llama-chunk", type=int, default=64, help="chunk size of `--only llama` (1 = a role per token)")
     ap.add_argument("--llama-prefill", type=int, default=16384)
     ap.add_argument("--llama-decode", type=int, default=512)
     args = ap.parse_args()
@@ -578,15 +656,24 @@ def main():
         print(json.dumps({"copy_bytes": 1 << 30}))
         return
     res = {}
+    extras = args.only is None and not args.no_extras  # the smaller legs that ride along in the default run
     if args.only in (None, "prefill"):
         res["prefill"] = bench_prefill(args, ops)
+    if extras:
+        # the chunk size of the reference's shipped Llama adapter (experiments/configs/finetune_distill.yaml:95) and a
+        # role per token, same shape, window and role shares
+        few = max(5, args.steps // 5)
+        res["prefill_c32"] = bench_prefill(args, ops, chunk_size=32, steps=few, warmup=3, compare=False, settle=False)
+        res["prefill_c1"] = bench_prefill(args, ops, chunk_size=1, steps=few, warmup=3, compare=False, settle=False)
     if args.only in (None, "decode"):
         res["decode"] = bench_decode(args, ops)
+    if extras:
+        res["decode_b1"] = bench_decode(args, ops, batch=1, context=65536)  # one sequence: the latency-bound end
     if args.only in (None, "evict"):
         res["evict"] = bench_evict(args, ops)
-    if args.only == "evict_stream":  # not part of the default run
+    if args.only == "evict_stream" or extras:
         res["evict_stream"] = bench_evict_stream(args, ops)
-    if args.only == "segments":  # not part of the default run
+    if args.only == "segments" or extras:
         res["segments"] = bench_segments(args, ops)
     if args.only == "role_step":  # not part of the default run
         res["role_step"] = bench_role_step(args, ops)
@@ -631,7 +718,14 @@ def main():
     if args.only in (None, "llama") and not args.no_llama:
         # the end-to-end workload: last, so that the kernel legs above are timed on a GPU that holds nothing else
         torch.cuda.empty_cache()
-        res["llama_e2e"] = bench_llama(args)
+        if args.only == "llama":
+            r = bench_llama(args, (args.llama_chunk,))
+            res["llama_e2e" if args.llama_chunk == 64 else f"llama_e2e_c{args.llama_chunk}"] = r[args.llama_chunk]
+        else:
+            r = bench_llama(args, (64,) if args.no_extras else (64, 1))
+            res["llama_e2e"] = r[64]
+            if 1 in r:
+                res["llama_e2e_c1"] = r[1]
     line.update(res)
     print(json.dumps(line))
 

@@ -284,7 +284,11 @@ size_t nats_evict_workspace_bytes(int64_t B, int64_t H_kv, int64_t S);
 
 /* Step 1, always: roles -> per-head plan in `workspace`, new sizes and the scalars in `result`.
  *   size_global / size_local [B, H_kv] int64, read here, rewritten by the apply step
- *   workspace: nats_evict_workspace_bytes(...) bytes (contents need not be kept between calls)
+ *   workspace: nats_evict_workspace_bytes(...) bytes.  Its first 256 bytes must be zero before the first call that
+ *              uses it and every call leaves them zero (a counter lives there); the rest need not be kept between
+ *              calls.  Calls that share a workspace must not overlap (calls on one stream do not).
+ *   With params->first the sizes are not read: a cache that has seen nothing holds the empty ring (size_global = W,
+ *   size_local = 0) whatever the tensors contain; the apply step writes them.
  *   result_mirror: NULL, or 16 bytes (16-byte aligned) that receive the short form of the result in one store, meant
  *              for pinned host memory: a host that sees its own params->seq there has n_ctx_data, gmin and the two
  *              flags without synchronising with the stream

@@ -75,7 +75,7 @@ class NAtSChunkLayerCache:
         self._sizes = torch.empty(2, bsz, n_msks, device=device, dtype=torch.long)
         self._sizes_init = torch.zeros(2, bsz, n_msks, device=device, dtype=torch.long)
         self._sizes_init[0] = sliding_window_size
-        self.size_global_kv, self.size_local_kv = self._sizes[0], self._sizes[1]
+        self._sizes_stale = True  # the tensors do not hold the empty cache's sizes yet (written when someone needs them)
         self._row_end = None  # size_global_kv + size_local_kv, kept between evictions
         self._evict = None    # ops.EvictBuffers, made by the first eviction
         self._await = None    # (sequence number, first) of an eviction whose scalars the host has not picked up yet
@@ -88,9 +88,27 @@ class NAtSChunkLayerCache:
         self.reset_cache()
 
     # -- state ----------------------------------------------------------------------------------
+    # size_global_kv / size_local_kv [B, H] int64 (nats_chunk_layer_cache.py:60-66).  A reset does not write them: the
+    # eviction of a first prefill knows what an empty cache holds and writes the new sizes itself; whoever else wants
+    # them first (a read of the attributes, an eviction that is not the first) has them written then.
+    def _fresh_sizes(self):
+        self._resolve()  # (a first eviction still on its way may turn out to have left the sizes alone)
+        if self._sizes_stale:
+            self._sizes_stale = False
+            torch.add(self._sizes_init, 0, out=self._sizes)  # (a kernel; a tensor copy would go through the runtime's copy path)
+        return self._sizes
+
+    @property
+    def size_global_kv(self):
+        return self._fresh_sizes()[0]
+
+    @property
+    def size_local_kv(self):
+        return self._fresh_sizes()[1]
+
     def reset_cache(self):
         self._await = self._redo = None  # (a result still on its way belongs to the state that is dropped here)
-        torch.add(self._sizes_init, 0, out=self._sizes)  # (a kernel; a tensor copy would go through the runtime's copy path)
+        self._sizes_stale = True
         self._row_end = None
         self.sliding_queue_tail = 0
         self.chunk_fill_size = 0
@@ -135,6 +153,7 @@ class NAtSChunkLayerCache:
                 self._kept_share = rows / full
                 if rows > self._buf_k.shape[2]:  # the guess was too small: once more, at the right size
                     self._launch_first(src, roles, params, ws, result, rows)
+                self._sizes_stale = False  # the out-of-place kernel has written them
         self._take_result(res, first)
 
     def settle(self, wait: bool = True):
@@ -163,7 +182,7 @@ class NAtSChunkLayerCache:
         if k_raw.stride(-1) != 1 or ops.strides_differ(k_raw, v_raw):
             k_raw, v_raw = k_raw.contiguous(), v_raw.contiguous()
         ops.evict_apply_first(k_raw, v_raw, self._buf_k, self._buf_v, self._buf_valid, self._buf_pos, roles,
-                              self.size_global_kv, self.size_local_kv, params, ws, result)
+                              self._sizes[0], self._sizes[1], params, ws, result)  # (writes the sizes unless every chunk slides)
 
     def _evict_first(self, src, roles, params, ws, result, first: bool):
         """The eviction of a first prefill that is still raw K / V.  The size of the compacted cache is a result of
@@ -186,6 +205,7 @@ class NAtSChunkLayerCache:
         rows = self._logical_rows(int(res.n_ctx_data))
         self._kept_share = rows / full
         self._launch_first(src, roles, params, ws, result, rows)
+        self._sizes_stale = False  # the out-of-place kernel has written them
         self._take_result(res, first)
         return True
 
@@ -505,7 +525,8 @@ class NAtSChunkLayerCache:
         else:
             params = ops.evict_params(self.bsz, self.n_msks, D, C, W, S, x_len, fill, self.n_ctx_data, self._n_global_min,
                                       self.sliding_queue_tail, first, max(self._rows, C))
-            ws, result = ops.evict_plan(roles, self.size_global_kv, self.size_local_kv, params, self._evict)
+            # (the first tokens of the cache: the plan does not read the size tensors, which may not have been reset)
+            ws, result = ops.evict_plan(roles, self._sizes[0], self._sizes[1], params, self._evict)
             if not self._evict_first(src, roles, params, ws, result, first):
                 params.n_alloc = self._rows
                 ops.evict_apply_inplace(self._buf_k, self._buf_v, self._buf_valid, self._buf_pos, roles,
@@ -727,7 +748,8 @@ class NAtSLayerCache(NAtSChunkLayerCache):
         else:
             params = ops.evict_params(self.bsz, self.n_msks, D, 1, W, fill, x_len, fill, block_start, self._n_global_min,
                                       self.sliding_queue_tail, first_ring, max(self._rows, 1), update_chunk=U)
-            ws, result = ops.evict_plan(roles, self.size_global_kv, self.size_local_kv, params, self._evict)
+            # (the first tokens of the cache: the plan does not read the size tensors, which may not have been reset)
+            ws, result = ops.evict_plan(roles, self._sizes[0], self._sizes[1], params, self._evict)
             if not self._evict_first(src, roles, params, ws, result, first_call):
                 params.n_alloc = self._rows
                 ops.evict_apply_inplace(self._buf_k, self._buf_v, self._buf_valid, self._buf_pos, roles, self.size_global_kv,

@@ -35,7 +35,16 @@ struct HeadPlan {
   int32_t all_local; // every slot of this head is local
 };
 
-constexpr size_t kPlanHeaderBytes = 256;
+constexpr size_t kPlanHeaderBytes = 256;  // (its first word: the ticket counter of evict_plan_heads_kernel, zero between launches)
+
+// The sizes a head brings into an eviction.  A cache that has seen nothing before these tokens (p.first) holds the
+// empty ring and no local rows whatever its size tensors contain: they need not have been reset.
+__device__ __forceinline__ long long old_size_global(const nats_evict_params& p, const int64_t* __restrict__ size_global, int h) {
+  return p.first ? (long long)p.W : (long long)size_global[h];
+}
+__device__ __forceinline__ long long old_size_local(const nats_evict_params& p, const int64_t* __restrict__ size_local, int h) {
+  return p.first ? 0LL : (long long)size_local[h];
+}
 
 __host__ __device__ inline size_t plan_lists_offset(int64_t n_heads) {
   return (kPlanHeaderBytes + (size_t)n_heads * sizeof(HeadPlan) + 255) & ~size_t(255);
@@ -77,6 +86,7 @@ __device__ __forceinline__ void load_roles(const uint8_t* __restrict__ r, int S,
   }
 }
 
+template <bool kCoherent = false>
 __device__ __forceinline__ void plan_one_head(const uint8_t* __restrict__ roles, const int64_t* __restrict__ size_global,
                                               const int64_t* __restrict__ size_local, const nats_evict_params& p,
                                               char* __restrict__ ws, int head, int lane) {
@@ -89,7 +99,7 @@ __device__ __forceinline__ void plan_one_head(const uint8_t* __restrict__ roles,
   HeadPlan* plans = reinterpret_cast<HeadPlan*>(ws + kPlanHeaderBytes);
   int32_t* keep = reinterpret_cast<int32_t*>(ws + plan_lists_offset(n_heads)) + (int64_t)head * S;
   const uint8_t* r = roles + (int64_t)head * S;
-  const long long sg = size_global[head], sl = size_local[head];
+  const long long sg = old_size_global(p, size_global, head), sl = old_size_local(p, size_local, head);
   HeadPlan hp;
   if (p.x_len == 1 && !p.update_chunk) {
     // one completed chunk is scattered for every head (:289-330)
@@ -156,7 +166,17 @@ __device__ __forceinline__ void plan_one_head(const uint8_t* __restrict__ roles,
     hp.all_sw = n_sw == S;
     hp.all_local = n_loc == S;
   }
-  if (lane == 0) plans[head] = hp;
+  if (lane == 0) {
+    if (kCoherent) {
+      // (read by another workgroup of the same launch: written through to where every compute unit reads it)
+      const uint64_t* w = reinterpret_cast<const uint64_t*>(&hp);
+      uint64_t* dst = reinterpret_cast<uint64_t*>(plans + head);
+#pragma unroll
+      for (int i = 0; i < (int)(sizeof(HeadPlan) / 8); ++i) __hip_atomic_store(dst + i, w[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    } else {
+      plans[head] = hp;
+    }
+  }
 }
 
 // The same plan for a head with few role slots, computed by one lane on its own (no wave-wide steps), so that a
@@ -173,7 +193,7 @@ __device__ __forceinline__ void plan_one_head_serial(const uint8_t* __restrict__
   HeadPlan* plans = reinterpret_cast<HeadPlan*>(ws + kPlanHeaderBytes);
   int32_t* keep = reinterpret_cast<int32_t*>(ws + plan_lists_offset(n_heads)) + (int64_t)head * S;
   const uint8_t* r = roles + (int64_t)head * S;
-  const long long sg = size_global[head], sl = size_local[head];
+  const long long sg = old_size_global(p, size_global, head), sl = old_size_local(p, size_local, head);
   HeadPlan hp;
   if (p.x_len == 1 && !p.update_chunk) {
     int r0 = r[0], rl = r[S - 1];
@@ -236,6 +256,9 @@ __device__ __forceinline__ void fold(PlanAgg& a, const PlanAgg& b) {
   a.sum_keep += b.sum_keep;
 }
 
+static_assert(sizeof(HeadPlan) == 32, "a head plan travels as four 64-bit words");
+
+template <bool kCoherent = false>
 __device__ __forceinline__ void plan_finalize(const int64_t* __restrict__ size_global, const int64_t* __restrict__ size_local,
                                               const nats_evict_params& p, char* __restrict__ ws,
                                               nats_evict_result* __restrict__ result,
@@ -254,8 +277,17 @@ __device__ __forceinline__ void plan_finalize(const int64_t* __restrict__ size_g
   w.max_tot_new = 0; w.max_tot_old = 0; w.max_tot_alllocal = 0;
   w.min_sg_new = 0x7fffffffffffffffLL; w.min_sg_old = 0x7fffffffffffffffLL; w.sum_keep = 0;
   for (int h = tid; h < n_heads; h += 256) {
-    const HeadPlan hp = plans[h];
-    const long long sg = size_global[h], sl = size_local[h];
+    HeadPlan hp;
+    if (kCoherent) {  // plans written by other workgroups of this launch
+      uint64_t w[sizeof(HeadPlan) / 8];
+      const uint64_t* src = reinterpret_cast<const uint64_t*>(plans + h);
+#pragma unroll
+      for (int i = 0; i < (int)(sizeof(HeadPlan) / 8); ++i) w[i] = __hip_atomic_load(src + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      hp = *reinterpret_cast<const HeadPlan*>(w);
+    } else {
+      hp = plans[h];
+    }
+    const long long sg = old_size_global(p, size_global, h), sl = old_size_local(p, size_local, h);
     PlanAgg x;
     x.all_sw = hp.all_sw; x.all_local = hp.all_local;
     x.max_keep = hp.count; x.max_end = hp.count + hp.dst_base;
@@ -309,8 +341,8 @@ __device__ __forceinline__ void plan_finalize(const int64_t* __restrict__ size_g
   if (all_local_flag) {
     // every slot local: nothing moves and only the local size grows (:747-749, :356)
     for (int h = tid; h < n_heads; h += 256) {
-      plans[h].sg_new = size_global[h];
-      plans[h].sl_new = size_local[h] + (long long)n_done * C;
+      plans[h].sg_new = old_size_global(p, size_global, h);
+      plans[h].sl_new = old_size_local(p, size_local, h) + (long long)n_done * C;
     }
   }
 }
@@ -328,21 +360,28 @@ __global__ __launch_bounds__(256) void evict_plan_small_kernel(const uint8_t* __
   plan_finalize(size_global, size_local, p, ws, result, result_mirror);
 }
 
-// Many role bytes (a prefill): a wavefront per head over the whole device, then one workgroup folds the heads.
+// Many role bytes (a prefill): a wavefront per head over the whole device; the workgroup that draws the launch's last
+// ticket (a counter at the start of the workspace, zero between launches) folds the heads.  The per-head plans cross
+// from the other workgroups to that one inside the launch, so they are written and read past the caches.
 __global__ __launch_bounds__(256) void evict_plan_heads_kernel(const uint8_t* __restrict__ roles,
                                                                const int64_t* __restrict__ size_global,
                                                                const int64_t* __restrict__ size_local, nats_evict_params p,
-                                                               char* __restrict__ ws) {
+                                                               char* __restrict__ ws, nats_evict_result* __restrict__ result,
+                                                               nats_evict_brief* __restrict__ result_mirror) {
+  __shared__ int last;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int head = blockIdx.x * 4 + wave;
-  if (head < (int)(p.B * p.H_kv)) plan_one_head(roles, size_global, size_local, p, ws, head, lane);
-}
-
-__global__ __launch_bounds__(256) void evict_plan_finalize_kernel(const int64_t* __restrict__ size_global,
-                                                                  const int64_t* __restrict__ size_local, nats_evict_params p,
-                                                                  char* __restrict__ ws, nats_evict_result* __restrict__ result,
-                                                                  nats_evict_brief* __restrict__ result_mirror) {
-  plan_finalize(size_global, size_local, p, ws, result, result_mirror);
+  if (head < (int)(p.B * p.H_kv)) plan_one_head<true>(roles, size_global, size_local, p, ws, head, lane);
+  __builtin_amdgcn_s_waitcnt(0);  // this workgroup's plans have arrived before it is counted
+  __syncthreads();
+  if (tid == 0) {
+    int32_t* ticket = reinterpret_cast<int32_t*>(ws);
+    const int t = atomicAdd(ticket, 1);
+    last = t == (int)gridDim.x - 1;
+    if (last) atomicExch(ticket, 0);
+  }
+  __syncthreads();
+  if (last) plan_finalize<true>(size_global, size_local, p, ws, result, result_mirror);
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -763,11 +802,8 @@ extern "C" int nats_evict_plan(const uint8_t* roles, const int64_t* size_global,
     return NATS_OK;
   }
   hipLaunchKernelGGL(evict_plan_heads_kernel, dim3(n_wg), dim3(256), 0, st, roles, size_global, size_local, *params,
-                     static_cast<char*>(workspace));
-  NATS_CHECK_LAUNCH("evict_plan_heads_kernel");
-  hipLaunchKernelGGL(evict_plan_finalize_kernel, dim3(1), dim3(256), 0, st, size_global, size_local, *params,
                      static_cast<char*>(workspace), result, result_mirror);
-  NATS_CHECK_LAUNCH("evict_plan_finalize_kernel");
+  NATS_CHECK_LAUNCH("evict_plan_heads_kernel");
   return NATS_OK;
 }
 

@@ -494,7 +494,8 @@ class EvictBuffers:
     def workspace(self, nbytes: int) -> torch.Tensor:
         if self.ws is None or self.ws.numel() < nbytes:
             have = 0 if self.ws is None else self.ws.numel()
-            self.ws = torch.empty(max(int(nbytes), 2 * have, 4096), dtype=torch.uint8, device=self.device)
+            # (zeros: the plan kernel's ticket counter at the start of the workspace is zero between launches)
+            self.ws = torch.zeros(max(int(nbytes), 2 * have, 4096), dtype=torch.uint8, device=self.device)
         return self.ws
 
     def next_seq(self) -> int:
@@ -536,7 +537,7 @@ def evict_plan(roles: torch.Tensor, size_global: torch.Tensor, size_local: torch
     lib = _lib.load()
     nbytes = lib.nats_evict_workspace_bytes(params.B, params.H_kv, params.S)
     if buffers is None:
-        ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=roles.device)
+        ws = torch.zeros(max(nbytes, 256), dtype=torch.uint8, device=roles.device)  # (its first 256 bytes must be zero)
         result = torch.empty(8, dtype=torch.int64, device=roles.device)
         mirror = None
     else:
