@@ -70,7 +70,9 @@ int nats_roles_from_logits(const void* logits, int dtype, int64_t B, int64_t S, 
  * With total = pre_fill + L:  total < C  -> no chunk completes, only carry_out = statistic so far is written;
  * otherwise S = ceil(total / C) role slots are produced, the open last one (total % C != 0) forced global and
  * its statistic written to carry_out.
- *   roles     [B, H_kv, S] uint8 out
+ *   roles     [B, H_kv, S] uint8 out; roles_head_stride = 0: contiguous, else the entries between the roles of two
+ *             consecutive (b, kv head) streams (>= S): the roles land in a slice of a wider [B, H_kv, U] buffer, as
+ *             the per-token cache keeps the roles of its pending tokens (nats_layer_cache.py:196-200); no index scan then
  *   one_hot   [B, H_kv, S, 3] out, dtype of x, may be NULL
  *   logits    [B, S, H_kv, 3] out (before the bias), dtype of x, may be NULL
  *   end_idx / vis_lim  [B, H_kv, S] as nats_role_scan, may be NULL
@@ -79,8 +81,8 @@ int nats_roles_from_logits(const void* logits, int dtype, int64_t B, int64_t S, 
  */
 int nats_role_step(const void* x, const void* carry_in, const void* weight, int dtype, int64_t B, int64_t L, int64_t dim,
                    int64_t H_kv, int64_t C, int64_t W, int64_t pre_fill, int merge_max, float global_bias,
-                   int force_first_global, const int64_t* x_strides, uint8_t* roles, void* one_hot, void* logits,
-                   void* carry_out, int64_t* end_idx, int32_t* vis_lim, void* stream);
+                   int force_first_global, const int64_t* x_strides, uint8_t* roles, int64_t roles_head_stride,
+                   void* one_hot, void* logits, void* carry_out, int64_t* end_idx, int32_t* vis_lim, void* stream);
 
 /* next-global index and the per-slot visibility limit derived from it.
  * Replaces the first half of generate_hard_seq_masks (components/masks/utils.py:85-87).
@@ -401,15 +403,19 @@ int nats_rope_qk(const void* q, const void* k, const void* cos, const void* sin,
  *   q_out[b, h, l]            = rope(q[b, h, l])            [B, H_q, x_len, D] contiguous
  *   cache_k[b, h, row0 + l]   = rope(k[b, h, l]),  cache_v[b, h, row0 + l] = v[b, h, l]
  *   valid[b, h, row0 + l] = 1, pos[b, h, row0 + l] = pos0 + l (pos may be NULL)
+ *   clear_row >= 0: also valid[b, h, clear_row] = 0 for every (b, h), a row below row0: the ring slot that the
+ *   per-token cache switches off after a step whose eviction is deferred (NAtSLayerCache._post_update,
+ *   components/cache/nats_layer_cache.py:300-310), written with the next step's rows.  -1: none.
  *   q [B, H_q, x_len, D], k / v [B, H_kv, x_len, D]: strides (b, h, l), last dimension contiguous
  *   cos / sin [B, x_len, D]: strides (b, l);  cache_k / cache_v [B, H_kv, n_alloc, D]: strides (b, h, row)
  *   valid / pos [B, H_kv, n_alloc]: strides (b, h)
  */
 int nats_rope_append(const void* q, const void* k, const void* v, const void* cos, const void* sin, void* q_out,
                      void* cache_k, void* cache_v, uint8_t* valid, int32_t* pos, int64_t B, int64_t H_q, int64_t H_kv,
-                     int64_t x_len, int64_t D, int64_t row0, int64_t n_alloc, int64_t pos0, const int64_t* q_strides,
-                     const int64_t* k_strides, const int64_t* v_strides, const int64_t* cos_strides,
-                     const int64_t* cache_strides, const int64_t* valid_strides, int dtype, void* stream);
+                     int64_t x_len, int64_t D, int64_t row0, int64_t n_alloc, int64_t pos0, int64_t clear_row,
+                     const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                     const int64_t* cos_strides, const int64_t* cache_strides, const int64_t* valid_strides, int dtype,
+                     void* stream);
 
 #ifdef __cplusplus
 }

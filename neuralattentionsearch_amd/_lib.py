@@ -48,7 +48,8 @@ SIGNATURES = {
     "nats_roles_from_logits": (ctypes.c_int, [c_p, ctypes.c_int, c_i64, c_i64, c_i64, ctypes.c_float, ctypes.c_int,
                                               ctypes.c_int, c_p, c_p, c_p]),
     "nats_role_step": (ctypes.c_int, [c_p, c_p, c_p, ctypes.c_int, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64,
-                                      ctypes.c_int, ctypes.c_float, ctypes.c_int, c_i64p, c_p, c_p, c_p, c_p, c_p, c_p, c_p]),
+                                      ctypes.c_int, ctypes.c_float, ctypes.c_int, c_i64p, c_p, c_i64, c_p, c_p, c_p, c_p,
+                                      c_p, c_p]),
     "nats_role_scan": (ctypes.c_int, [c_p, c_i64, c_i64, c_i64, c_i64, c_i64, c_p, c_p, c_p]),
     "nats_prefill_mask": (ctypes.c_int, [c_p, c_i64, c_i64, c_i64, c_i64, c_i64, c_p, c_p, ctypes.c_size_t, c_p]),
     "nats_prefill_tile_map": (ctypes.c_int, [c_p, c_i64, c_i64, c_i64, c_i64, c_i64, c_p, c_p, ctypes.c_size_t, c_p]),
@@ -83,7 +84,7 @@ SIGNATURES = {
     "nats_silu_mul": (ctypes.c_int, [c_p, c_p, c_i64, c_i64, ctypes.c_int, c_p]),
     "nats_matvec": (ctypes.c_int, [c_p, c_p, c_p] + [c_i64] * 6 + [ctypes.c_int, ctypes.c_int, c_p]),
     "nats_rope_qk": (ctypes.c_int, [c_p] * 6 + [c_i64] * 5 + [c_i64p] * 3 + [ctypes.c_int, c_p]),
-    "nats_rope_append": (ctypes.c_int, [c_p] * 10 + [c_i64] * 8 + [c_i64p] * 6 + [ctypes.c_int, c_p]),
+    "nats_rope_append": (ctypes.c_int, [c_p] * 10 + [c_i64] * 9 + [c_i64p] * 6 + [ctypes.c_int, c_p]),
 }
 
 _lib = None

@@ -569,10 +569,26 @@ class NAtSLayerCache(NAtSChunkLayerCache):
 
     def reset_cache(self):
         super().reset_cache()
+        self._clear_slot = None  # ring slot whose valid byte is to be switched off (see post_update) and has not been yet
         self._in_chunk = None   # uint8 [B, H, U]: roles of the pending tokens (:196-200, :218)
         self._block = None      # roles of the whole pending block as of the last update (_tokens_info, :209-219)
+        self._block_fill = 0
         self._mask_roles = None  # the block as of the last multi-token update (:229-231)
         self._live_end = self.sliding_window_size  # n_ctx_data after the last eviction that moved rows
+
+    # A step whose eviction is deferred switches off one ring slot (:300-310).  Nothing reads the valid bytes between
+    # that step's attention and the next step's, so the byte is written with the next step's rows (one kernel less per
+    # token) -- or at once for whoever looks at the valid bytes before.
+    def _flush_clear(self):
+        slot, self._clear_slot = self._clear_slot, None
+        if slot is not None and self._buf_valid is not None:
+            self._buf_valid[:, :, slot] = 0
+
+    @property
+    def valid_tokens(self):
+        self._materialize_pending()
+        self._flush_clear()
+        return None if self._buf_valid is None else self._buf_valid[:, :, :self._rows].view(torch.bool)
 
     # -- append (nats_layer_cache.py:167-286) ------------------------------------------------------
     def _pad_rows(self, n: int) -> int:
@@ -602,6 +618,23 @@ class NAtSLayerCache(NAtSChunkLayerCache):
     def _full_rows(self, x_len: int) -> int:
         return self.sliding_window_size + self._pad_rows(x_len)
 
+    def role_destination(self, x_len: int = 1):
+        """Where the roles of the next x_len tokens belong among the pending ones: a uint8 [B, H, x_len] view into which
+        a role kernel may write them directly (`ops.role_step(..., roles_out=...)`); handed to `update` /
+        `append_rotated` as `roles` it costs no copy.  None when the tokens do not fit the pending buffer."""
+        U = self.update_chunk_size
+        if self._in_chunk is None:
+            self._in_chunk = torch.zeros(self.bsz, self.n_msks, U, dtype=torch.uint8, device=self.device)
+        at = self.chunk_fill_size
+        return self._in_chunk[:, :, at:at + x_len] if at + x_len <= U else None
+
+    def _pending_block(self):
+        """uint8 [B, H, fill] contiguous: the roles of the whole pending block (made from the buffer when asked for;
+        a full buffer is the block itself)."""
+        if self._block is None:
+            self._block = self._in_chunk[:, :, :self._block_fill].contiguous()
+        return self._block
+
     def _note_roles(self, token_states_info, roles):
         """Roles of the new tokens join the pending block."""
         U = self.update_chunk_size
@@ -615,11 +648,15 @@ class NAtSLayerCache(NAtSChunkLayerCache):
         if fill > U:
             self._block = torch.cat([self._in_chunk[:, :, :last], roles], dim=2).contiguous()
         else:
-            self._in_chunk[:, :, last:fill] = roles
-            self._block = self._in_chunk[:, :, :fill].contiguous()
-        self._roles = self._block
+            in_place = (roles.data_ptr() == self._in_chunk.data_ptr() + last and roles.stride(1) == U
+                        and (self.bsz == 1 or roles.stride(0) == self.n_msks * U) and (x_len == 1 or roles.stride(2) == 1))
+            if not in_place:  # (a role kernel that was given `role_destination` has written them already)
+                self._in_chunk[:, :, last:fill] = roles
+            self._block = None
+        self._block_fill = fill
+        self._roles = None
         if x_len > 1:
-            self._mask_roles = self._block
+            self._mask_roles = self._pending_block()
 
     def update(self, key_states: torch.Tensor, value_states: torch.Tensor, token_states_info: torch.Tensor | None,
                roles: torch.Tensor | None = None):
@@ -639,6 +676,7 @@ class NAtSLayerCache(NAtSChunkLayerCache):
                 self._materialize_pending()  # nothing will be evicted by the coming post_update
             return key_states, value_states
         self._materialize_pending()
+        self._flush_clear()
         start = self.n_ctx_data
         end = start + x_len
         self._grow(end)
@@ -658,8 +696,9 @@ class NAtSLayerCache(NAtSChunkLayerCache):
         start = self.n_ctx_data
         end = start + x_len
         self._grow(end)
+        clear, self._clear_slot = self._clear_slot, None
         q_rot = ops.rope_append(q, key_states, value_states, cos, sin, self._buf_k, self._buf_v, self._buf_valid,
-                                self._buf_pos, start, self._seen_tokens)
+                                self._buf_pos, start, self._seen_tokens, -1 if clear is None else clear)
         return q_rot, self._buf_k[:, :, :end], self._buf_v[:, :, :end]
 
     # -- masks (nats_layer_cache.py:155-162, 469-554) ------------------------------------------------
@@ -674,6 +713,7 @@ class NAtSLayerCache(NAtSChunkLayerCache):
         if self._seen_tokens == 0:
             return ops.prefill_mask(self._mask_roles, x_len, 1, self.sliding_window_size)
         self._materialize_pending()
+        self._flush_clear()
         return ops.prefill_past_mask(self._buf_valid, self.size_global_kv, self.size_local_kv, self._mask_roles, x_len, 1,
                                      self.sliding_window_size, self.past_state(x_len))
 
@@ -717,12 +757,14 @@ class NAtSLayerCache(NAtSChunkLayerCache):
             # the eviction is deferred; the ring slot the next token would take is switched off (:300-310)
             slot = fill if self._seen_tokens < U else (fill + self.sliding_queue_tail + 1) % W
             self._materialize_pending()
-            self._buf_valid[:, :, slot] = 0
+            self._flush_clear()
+            self._clear_slot = slot  # (written with the next step's rows, or by whoever reads the valid bytes first)
             self.chunk_fill_size_last = fill
             return
+        self._flush_clear()
         first_ring = fill == self._seen_tokens   # the block holds every token seen so far (:439)
         first_call = self._seen_tokens == x_len  # (:404)
-        roles = self._block
+        roles = self._pending_block()
         src = self._pending
         like = src[0] if src is not None else self._buf_k
         D = like.shape[3]

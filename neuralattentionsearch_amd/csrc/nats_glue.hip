@@ -304,6 +304,7 @@ struct RopeAppendArgs {
   int Hq, Hkv, x_len, D;
   int64_t row0;
   int pos0;
+  int64_t clear_row;  // >= 0: valid[b, h, clear_row] is set to 0 for every (b, h) (a row below row0)
 };
 
 // grid (x_len, Hq + 2 * Hkv, B); one thread per element of the head vector (D <= 256)
@@ -333,6 +334,7 @@ __global__ void rope_append_kernel(RopeAppendArgs a) {
       if (d == 0) {
         a.valid[b * a.valid_s[0] + h * a.valid_s[1] + a.row0 + l] = 1;
         if (a.pos) a.pos[b * a.valid_s[0] + h * a.valid_s[1] + a.row0 + l] = a.pos0 + l;
+        if (l == 0 && a.clear_row >= 0) a.valid[b * a.valid_s[0] + h * a.valid_s[1] + a.clear_row] = 0;
       }
     }
   } else {
@@ -531,11 +533,13 @@ extern "C" int nats_matvec(const void* w, const void* x, void* y, int64_t x_rows
 extern "C" int nats_rope_append(const void* q, const void* k, const void* v, const void* cos, const void* sin, void* q_out,
                                 void* cache_k, void* cache_v, uint8_t* valid, int32_t* pos, int64_t B, int64_t H_q,
                                 int64_t H_kv, int64_t x_len, int64_t D, int64_t row0, int64_t n_alloc, int64_t pos0,
-                                const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
-                                const int64_t* cos_strides, const int64_t* cache_strides, const int64_t* valid_strides,
-                                int dtype, void* stream) {
+                                int64_t clear_row, const int64_t* q_strides, const int64_t* k_strides,
+                                const int64_t* v_strides, const int64_t* cos_strides, const int64_t* cache_strides,
+                                const int64_t* valid_strides, int dtype, void* stream) {
   NATS_REQUIRE(q && k && v && cos && sin && q_out && cache_k && cache_v && valid, NATS_ERR_NULL_POINTER,
                "nats_rope_append: NULL pointer");
+  NATS_REQUIRE(clear_row < row0, NATS_ERR_BAD_SHAPE, "nats_rope_append: clear_row=%lld is not below row0=%lld",
+               (long long)clear_row, (long long)row0);
   NATS_REQUIRE(q_strides && k_strides && v_strides && cos_strides && cache_strides && valid_strides, NATS_ERR_NULL_POINTER,
                "nats_rope_append: NULL stride array");
   NATS_REQUIRE(B > 0 && H_q > 0 && H_kv > 0 && x_len > 0 && B <= 65535 && H_q + 2 * H_kv <= 65535, NATS_ERR_BAD_SHAPE,
@@ -556,6 +560,7 @@ extern "C" int nats_rope_append(const void* q, const void* k, const void* v, con
   }
   a.Hq = (int)H_q; a.Hkv = (int)H_kv; a.x_len = (int)x_len; a.D = (int)D;
   a.row0 = row0; a.pos0 = (int)pos0;
+  a.clear_row = clear_row;
   hipStream_t st = static_cast<hipStream_t>(stream);
   dim3 grid((unsigned)x_len, (unsigned)(H_q + 2 * H_kv), (unsigned)B);
   const unsigned threads = (unsigned)((D + 63) / 64 * 64);

@@ -183,11 +183,19 @@ class NAtSLlamaAttention(nn.Module):
         if pre_fill + 1 < C:
             if not statistic_done:
                 past_key_value.update_nats_cached_x_in_chunk(hidden_states, idx, self.chunk_merge_method)
+        elif self.fused_role_step and C == 1 and (dest := past_key_value.cache_model[idx].role_destination(1)) is not None:
+            # a per-token cache takes the role straight into its buffer of pending roles; nothing else needs it
+            ops.role_step_token(hidden_states, self.proj_layer.weight, self.local_seq_max_length, dest,
+                                merge_max=self.chunk_merge_method == ChunkMergeType.MAX, global_bias=0.0,
+                                force_first_global=start_pos < C)
+            past_key_value._update_cache_x(None, idx)
+            roles = dest
         elif self.fused_role_step:
+            dest = None
             step = ops.role_step(hidden_states, self.proj_layer.weight, C, self.local_seq_max_length, pre_fill=pre_fill,
                                  carry_in=past_key_value.get_nats_cached_x_in_chunk(idx) if pre_fill else None,
                                  merge_max=self.chunk_merge_method == ChunkMergeType.MAX, global_bias=0.0,
-                                 force_first_global=start_pos < C)
+                                 force_first_global=start_pos < C, with_one_hot=dest is None, roles_out=dest)
             past_key_value._update_cache_x(step["carry"], idx)
             roles, tsi = step["roles"], step["token_states_info"]
         else:

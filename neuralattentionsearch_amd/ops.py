@@ -111,14 +111,16 @@ def roles_from_logits(logits: torch.Tensor, global_bias: float = 0.1, force_firs
 def role_step(x: torch.Tensor, weight: torch.Tensor, chunk_size: int, window: int, pre_fill: int = 0,
               carry_in: torch.Tensor | None = None, merge_max: bool = False, global_bias: float = 0.1,
               force_first_global: bool = False, with_one_hot: bool = True, with_logits: bool = False,
-              with_scan: bool = False) -> dict:
+              with_scan: bool = False, roles_out: torch.Tensor | None = None) -> dict:
     """Chunk pooling of hidden states + role projection + argmax (+ next-global scan) in one call.
 
     x [B, L, dim] hidden states of the new tokens, weight [H_kv * 3, dim] (proj_layer.weight), carry_in
     [B, 1, dim] or [B, dim] the running statistic of the open chunk (required when pre_fill > 0).
     Returns a dict with `roles` uint8 [B, H_kv, S] (None while no chunk completes), `token_states_info`,
     `logits` [B, S, H_kv, 3], `carry` [B, 1, dim] (statistic of the open chunk, None if every chunk is
-    complete), `end_idx`, `vis_lim`, and `pad`.
+    complete), `end_idx`, `vis_lim`, and `pad`.  `roles_out`: a uint8 [B, H_kv, S] view into which the roles are
+    written instead of a new tensor (its last dimension contiguous, its first two laid out as those of a contiguous
+    [B, H_kv, U] tensor: a slice of the per-token cache's pending roles); not together with `with_scan`.
     components/cache/dyn_cache.py:117-171, models/transformer/attention/nats_chunk_attention.py:64-95."""
     _require_cuda(x, weight, carry_in)
     lib = _lib.load()
@@ -143,7 +145,15 @@ def role_step(x: torch.Tensor, weight: torch.Tensor, chunk_size: int, window: in
     S = 0 if total < C else math.ceil(total / C)
     pad = 0 if S == 0 else S * C - total
     dev, dt = x.device, x.dtype
-    roles = torch.empty(B, H, S, dtype=torch.uint8, device=dev) if S else None
+    roles_hs = 0
+    if roles_out is not None and S:
+        hs = roles_out.stride(1)
+        if (tuple(roles_out.shape) != (B, H, S) or roles_out.dtype != torch.uint8 or not roles_out.is_cuda or with_scan
+                or (S > 1 and roles_out.stride(2) != 1) or hs < S or (B > 1 and roles_out.stride(0) != H * hs)):
+            raise ValueError("roles_out must be a uint8 [B, H_kv, S] slice of a contiguous [B, H_kv, U] tensor")
+        roles, roles_hs = roles_out, hs
+    else:
+        roles = torch.empty(B, H, S, dtype=torch.uint8, device=dev) if S else None
     one_hot = torch.empty(B, H, S, 3, dtype=dt, device=dev) if S and with_one_hot else None
     logits = torch.empty(B, S, H, 3, dtype=dt, device=dev) if S and with_logits else None
     carry = torch.empty(B, 1, dim, dtype=dt, device=dev) if (S == 0 or pad) else None
@@ -151,7 +161,7 @@ def role_step(x: torch.Tensor, weight: torch.Tensor, chunk_size: int, window: in
     vis_lim = torch.empty(B, H, S, dtype=torch.int32, device=dev) if S and with_scan else None
     check(lib.nats_role_step(_ptr(x), _ptr(carry_in), _ptr(weight), _dtype_code(x), B, L, dim, H, C, window, pre_fill,
                              int(merge_max), float(global_bias), int(force_first_global), i64_array(x.stride()[:2]),
-                             _ptr(roles), _ptr(one_hot), _ptr(logits), _ptr(carry), _ptr(end_idx), _ptr(vis_lim),
+                             _ptr(roles), roles_hs, _ptr(one_hot), _ptr(logits), _ptr(carry), _ptr(end_idx), _ptr(vis_lim),
                              _stream(x)))
     if one_hot is not None:
         _attach_roles(one_hot, roles)
@@ -164,6 +174,23 @@ def _attach_roles(one_hot: torch.Tensor, roles: torch.Tensor) -> None:
     both: an in-place edit of either afterwards (a slot forced global, a head masked) makes the pair stale."""
     one_hot.nats_roles = roles
     one_hot.nats_roles_version = (one_hot._version, roles._version)
+
+
+def role_step_token(x: torch.Tensor, weight: torch.Tensor, window: int, roles_out: torch.Tensor, merge_max: bool = False,
+                    global_bias: float = 0.1, force_first_global: bool = False) -> None:
+    """`role_step` for one token per sequence with a role per token (chunk size 1): x [B, 1, dim] -> the roles, written
+    into `roles_out` (uint8 [B, H_kv, 1], a slice of the per-token cache's pending roles, `role_destination`).  Nothing
+    is allocated and nothing returned: the call a decoding loop makes once per layer and token."""
+    B, L, dim = x.shape
+    H = weight.shape[0] // 3
+    hs = roles_out.stride(1)
+    if (L != 1 or not x.is_cuda or weight.dtype != x.dtype or weight.shape[1] != dim or x.stride(-1) != 1
+            or not weight.is_contiguous() or tuple(roles_out.shape) != (B, H, 1) or roles_out.dtype != torch.uint8
+            or (B > 1 and roles_out.stride(0) != H * hs)):
+        raise ValueError("role_step_token takes x [B, 1, dim], weight [H_kv * 3, dim] and roles_out uint8 [B, H_kv, 1]")
+    check(_lib.load().nats_role_step(x.data_ptr(), None, weight.data_ptr(), _dtype_code(x), B, 1, dim, H, 1, window, 0,
+                                     int(merge_max), float(global_bias), int(force_first_global), i64_array(x.stride()[:2]),
+                                     roles_out.data_ptr(), hs, None, None, None, None, None, _stream(x)))
 
 
 def roles_from_one_hot(token_states_info: torch.Tensor) -> torch.Tensor:
@@ -833,10 +860,11 @@ def rope_qk(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, sin: torch.Tens
 
 def rope_append(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
                 cache_k: torch.Tensor, cache_v: torch.Tensor, valid: torch.Tensor, pos: torch.Tensor | None, row0: int,
-                pos0: int = 0) -> torch.Tensor:
+                pos0: int = 0, clear_row: int = -1) -> torch.Tensor:
     """Rotary embedding of q and k, and k / v written to rows [row0, row0 + x_len) of the cache with their valid
     bytes (and stream positions).  q [B, H_q, x_len, D], k / v [B, H_kv, x_len, D] (any strides, last dimension
-    contiguous), cos / sin [B, x_len, D].  Returns the rotated q, contiguous."""
+    contiguous), cos / sin [B, x_len, D].  `clear_row` >= 0: the valid byte of that row (below row0) is set to 0 in
+    every head.  Returns the rotated q, contiguous."""
     _require_cuda(q, k, v, cos, sin, cache_k, cache_v, valid, pos)
     B, Hq, x_len, D = q.shape
     Hkv = k.shape[1]
@@ -857,7 +885,7 @@ def rope_append(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cos: torch.Te
     n_alloc = min(cache_k.shape[2], valid.shape[2])
     check(_lib.load().nats_rope_append(
         _ptr(q), _ptr(k), _ptr(v), _ptr(cos), _ptr(sin), _ptr(q_out), _ptr(cache_k), _ptr(cache_v), _ptr(valid), _ptr(pos),
-        B, Hq, Hkv, x_len, D, int(row0), n_alloc, int(pos0), i64_array(q.stride()[:3]), i64_array(k.stride()[:3]),
+        B, Hq, Hkv, x_len, D, int(row0), n_alloc, int(pos0), int(clear_row), i64_array(q.stride()[:3]), i64_array(k.stride()[:3]),
         i64_array(v.stride()[:3]), i64_array(cos.stride()[:2]), i64_array(cache_k.stride()[:3]),
         i64_array(valid.stride()[:2]), _dtype_code(q), _stream(q)))
     return q_out
