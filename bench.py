@@ -141,13 +141,18 @@ def prefill_flops(roles: np.ndarray, L: int, C: int, W: int, D: int, n_rep: int)
     return 4.0 * D * n_rep * pairs, 4.0 * D * n_rep * dense
 
 
-def time_gpu(fn, steps: int, warmup: int):
-    """Time of `fn` on the current stream: W untimed calls, then exactly K calls between one pair of HIP events
+def time_gpu(fn, steps: int, warmup: int, settle_ms: float = 0.0):
+    """Time of `fn` on the current stream: W untimed calls (for a leg of a few microseconds per call `settle_ms` keeps
+    the untimed calls going for that long: after host-side set-up the GPU has dropped to its idle clock, and a few
+    hundred microseconds of warm-up do not bring it back), then exactly K calls between one pair of HIP events
     (and one pair of synchronisations), so that the launches follow each other as they do in use.  Returns
     (host wall time per step, GPU time per step, best single step); the best step comes from a short extra loop
     with an event pair around every call, which costs each call about ten microseconds of markers and is
     therefore not what the mean is taken from."""
     for _ in range(warmup):
+        fn()
+    t_settle = time.perf_counter() + settle_ms * 1e-3
+    while time.perf_counter() < t_settle:
         fn()
     torch.cuda.synchronize()
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -262,7 +267,7 @@ def bench_decode(args, ops, batch=None, context=None):
     bytes_alg = n_valid * D * 2 * 2 + 2 * q.numel() * 2
     wall, ev_mean, ev_min = time_gpu(
         lambda: ops.decode_attention(q, k, v, valid, n_rows, row_end=row_end, tail_start=tail_start),
-        args.steps * 5, args.warmup)
+        args.steps * 5, args.warmup, settle_ms=60.0 if B < 8 else 0.0)
     return {
         "ms": ev_mean, "ms_min": ev_min, "ms_wall": wall,
         "tokens_per_s_per_layer": B / (ev_mean * 1e-3),
