@@ -93,6 +93,14 @@ struct PrefillWorkspace {
   int2* tile_lim;
   int2* gran_lim;
   int32_t* ticket;  // one counter, set to zero by the key-limit kernel (the attention kernel deals work from it)
+  // long-lived rows (see long_rows_kernel): per stream the ascending list of their row ids, their limits, the number
+  // of list entries before every 16-row granule, and the least limit of every 64 list entries
+  int32_t* long_rows;    // [streams, long_cap]
+  int32_t* long_lim;     // [streams, long_cap]
+  int32_t* long_before;  // [streams, n_gran + 1]
+  int32_t* long_tmin;    // [streams, long_cap / 64]
+  int64_t long_cap;      // list entries per stream: N rounded up to whole tiles, plus one tile of padding
+  int64_t n_gran;        // 16-row granules per stream
   size_t bytes;
 };
 
@@ -100,6 +108,8 @@ PrefillWorkspace carve_prefill_workspace(void* ws, int64_t n_streams, int64_t S,
 int prepare_key_limits(const uint8_t* roles, int64_t B, int64_t H_kv, int64_t S, int64_t N, int64_t C, int64_t W,
                        const PastView* past, const PrefillWorkspace& w, hipStream_t st);
 int check_past_state(const char* who, const nats_past_state* ps, int64_t x_len, int64_t C, int64_t W);
+// Fills the long-lived-row lists of the workspace from its key limits (after prepare_key_limits on the same stream).
+int launch_long_rows(const PrefillWorkspace& w, int64_t n_streams, int64_t N, int64_t base, int64_t t_long, hipStream_t st);
 
 // Orders LDS traffic between the lanes of one wavefront (no workgroup barrier needed for wave-private LDS).
 __device__ __forceinline__ void wave_lds_sync() {

@@ -52,6 +52,13 @@ struct PrefillArgs {
   int n_split;      // 1: no split
   float* part_acc;  // [workgroup, split, wavefront, 32 rows, D]
   float* part_ml;   // [workgroup, split, wavefront, 32 rows, 2] running maximum (base-2 exponent) and row sum
+  // packed tiles of chunks shorter than a granule: rows more than t_long tokens behind a query group come from the
+  // lists of long-lived rows (long_rows_kernel), gathered row by row; NULL = every row is walked granule by granule
+  const int32_t* long_rows;
+  const int32_t* long_lim;
+  const int32_t* long_before;
+  const int32_t* long_tmin;
+  int long_cap, n_gran, t_long;
 };
 
 // workgroup index -> (kv stream, head group, rank of the query group; heavy query groups come first)
@@ -214,7 +221,8 @@ struct PrefillSmem {
   uint16_t k[4][kTile * D];  // tile j of the visit list in k[j & 3]
   uint16_t v[4][kTile * D];
   int limk[8][kTile];        // row limits of tile j in limk[j & 7]
-  int posk[8][kTile];        // packed tiles: region token of every key row (a row is visible up to limk and from posk on)
+  int posk[8][kTile];        // packed tiles: region token of every key row (a row is visible up to limk and from posk on);
+                             // tiles gathered from the long-lived rows: the cache row of every key row
   int4 vlist[kWin];  // visited key tiles of the current window: {tile, max limit, min limit, -}
                      // packed tiles: the four 16-row granules of the tile ({id | mask flag, id, id, id}, -1 = none)
   int vcount;
@@ -223,6 +231,7 @@ struct PrefillSmem {
 };
 constexpr int kGranPerTile = kTile / kGranule;
 constexpr int kPackedMaskFlag = 1 << 30;  // on the first granule id of a packed tile: some score of the tile is masked
+constexpr int kFarTileFlag = 1 << 29;     // ... the entry is tile (id & 0xffffff) of the stream's list of long-lived rows
 
 // kUniform: the wavefronts are the q heads of ONE query tile (GQA groups of 4 and more), so every tile of
 // the visit list is visited by every wavefront and the tile loop has no per-wavefront branches.
@@ -276,6 +285,23 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
   const int my_rlast = min(q0 + kHalf - 1, a.r_end - 1);
   const int kt_end_group = (a.base + rlast_group) / kTile;
   const int my_kt_end = (a.base + tile_rlast) / kTile;
+
+  // Rows more than t_long tokens behind the group's first query: only the stream's long-lived rows can be visible
+  // there (long_rows_kernel); the first n_far entries of their list lie below near_row0, the row from which the
+  // group walks granule by granule.
+  const bool far_mode = kPacked && a.long_rows != nullptr;
+  int near_row0 = 0, n_far = 0;
+  const int32_t* lrows = nullptr;
+  const int32_t* llim = nullptr;
+  const int32_t* ltmin = nullptr;
+  if (far_mode) {
+    near_row0 = max(0, a.base + r0_group - a.t_long) & ~(kGranule - 1);
+    n_far = __builtin_amdgcn_readfirstlane(a.long_before[(int64_t)ks * (a.n_gran + 1) + near_row0 / kGranule]);
+    lrows = a.long_rows + (int64_t)ks * a.long_cap;
+    llim = a.long_lim + (int64_t)ks * a.long_cap;
+    ltmin = a.long_tmin + (int64_t)ks * (a.long_cap / kTile);
+  }
+  const int n_far_tiles = (n_far + kTile - 1) / kTile;
 
   // ---- wavefront 0 asks for the tile summaries of the first kEarly * 64 key tiles before anything else is requested:
   // memory operations complete in the order of their issue, so the wait for these (a trip to L2) does not include
@@ -382,10 +408,35 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
       }
     }
   };
+  // a tile of the list of long-lived rows: the cache row of every tile row is in posk[slot] (requested a step ahead)
+  auto issue_rows_far = [&](const uint16_t* base, int64_t stride, uint16_t* dst, int slot, bool is_v) {
+#pragma unroll
+    for (int j = 0; j < DMA_PER_WAVE; ++j) {
+      const int inst = wave * DMA_PER_WAVE + j;  // uniform
+      const int q = inst * kWave + lane;
+      const int row = q / OCT, pos = q % OCT;
+      const int n = max(0, min(sm.posk[slot][row], a.N - 1));  // (padding entries hold INT_MAX and the limit -1)
+      const int chunk = is_v ? pos ^ v_swizzle(row) : pos ^ (row % OCT);
+      __builtin_amdgcn_global_load_lds(base + (int64_t)n * stride + chunk * 8,
+                                       (uint32_t __attribute__((address_space(3)))*)(dst + inst * kWave * 8), 16, 0, 0);
+    }
+  };
   auto granule_of = [&](int id0, int id1, int id2, int id3, int which) {
     return which == 0 ? (id0 & ~kPackedMaskFlag) : which == 1 ? id1 : which == 2 ? id2 : id3;
   };
   auto issue_k_p = [&](int id0, int id1, int id2, int id3, int buf, int slot) {
+    if (id0 & kFarTileFlag) {
+      issue_rows_far(kp, a.ks_l, sm.k[buf], slot, false);
+      if ((id0 & kPackedMaskFlag) && wave == 0) {
+        int ln = lane;
+#if defined(__HIP_DEVICE_COMPILE__)
+        asm volatile("" : "+v"(ln));
+#endif
+        __builtin_amdgcn_global_load_lds(llim + (int64_t)(id0 & 0xffffff) * kTile + ln,
+                                         (uint32_t __attribute__((address_space(3)))*)(&sm.limk[slot][0]), 4, 0, 0);
+      }
+      return;
+    }
     issue_rows_p(kp, a.ks_l, koff, sm.k[buf], granule_of(id0, id1, id2, id3, wave >> 1), false);
     if ((id0 & kPackedMaskFlag) && wave == 0) {
       // limits and region tokens of the 64 rows, for the element mask (asynchronous like the tile itself).
@@ -402,7 +453,11 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
       sm.posk[slot][ln] = real ? row - a.base : 0x7fffffff;
     }
   };
-  auto issue_v_p = [&](int id0, int id1, int id2, int id3, int buf) {
+  auto issue_v_p = [&](int id0, int id1, int id2, int id3, int buf, int slot) {
+    if (id0 & kFarTileFlag) {
+      issue_rows_far(vp, a.vs_l, sm.v[buf], slot, true);
+      return;
+    }
     issue_rows_p(vp, a.vs_l, voff, sm.v[buf], granule_of(id0, id1, id2, id3, wave >> 1), true);
   };
 
@@ -488,8 +543,10 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
     }
   };
   // packed tile: every key row carries its own region token
-  auto mask_scores_p = [&](int slot, f32x16 (&sv)[2]) {
+  // (a tile of long-lived rows: posk holds cache rows, and the rows from near_row0 on belong to the granule walk)
+  auto mask_scores_p = [&](int slot, f32x16 (&sv)[2], bool far_tile) {
     const int qtok = q0 + l32;
+    const int bound = far_tile ? near_row0 - 1 : qtok;
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
@@ -501,7 +558,7 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
         const int pv[4] = {ps.x, ps.y, ps.z, ps.w};
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          const bool vis = pv[e] <= qtok && qtok <= lv[e];
+          const bool vis = pv[e] <= bound && qtok <= lv[e];
           if (!vis) sv[kb][g4 * 4 + e] = -INFINITY;
         }
       }
@@ -661,9 +718,22 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
   const int g_end_group = (a.base + rlast_group) / kGranule;
   const int win_last = kPacked ? g_end_group : kt_end_group;
   constexpr int kWinStep = kPacked ? (kWin - 1) * kGranPerTile : kWin;
-  for (int w0 = 0; w0 <= win_last; w0 += kWinStep) {
+  int f0 = 0;                                // first tile of the long-lived rows in this window
+  bool far_win = far_mode && n_far_tiles > 0;  // windows of gathered tiles come first, then the granule walk
+  for (int w0 = far_mode ? near_row0 / kGranule : 0; w0 <= win_last;) {
     // ---- visit list of this window: wavefront 0 compacts the tiles some query tile of the group sees ----
-    if (kPacked && wave == 0) {
+    if (kPacked && far_win && wave == 0) {
+      // tiles [f0, f0 + count) of the list; a tile needs no mask when all its rows lie below near_row0 and every
+      // query of the group sees every one of them
+      const int cnt = min(kWin - 1, n_far_tiles - f0);
+      for (int i = lane; i < cnt; i += kWave) {
+        const int t = f0 + i;
+        const bool plain = (t + 1) * kTile <= n_far && ltmin[t] >= rlast_group;
+        sm.vlist[i] = make_int4(kFarTileFlag | (plain ? 0 : kPackedMaskFlag) | t, 0, 0, 0);
+      }
+      if (lane == 0) sm.vcount = cnt;
+    }
+    if (kPacked && !far_win && wave == 0) {
       // granules seen without a mask and granules that need one, each kind in its own list (staged in the tile
       // buffers, which are idle here), then four ids per tile
       int* plain_ids = reinterpret_cast<int*>(&sm.k[0][0]);
@@ -769,7 +839,7 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
       auto load_v = [&](int j, const Entry& e) {
         if (j < n_vis) {
           if (kPacked) {
-            issue_v_p(e.kt, e.emax, e.emin, e.e3, j & 3);
+            issue_v_p(e.kt, e.emax, e.emin, e.e3, j & 3, j & 7);
           } else {
             issue_v(e.kt, j & 3);
           }
@@ -788,7 +858,7 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
                                     : (ec.kt * kTile + kTile - 1 - a.base <= my_r0 && ec.emin >= my_rlast);
           if (!full) {
             if (kPacked) {
-              mask_scores_p(t & 7, sv);
+              mask_scores_p(t & 7, sv, (ec.kt & kFarTileFlag) != 0);
             } else {
               mask_scores(ec.kt, t & 7, sv);
             }
@@ -807,6 +877,24 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
         }
       };
 
+      // gathered tiles: the cache rows of tile j of the window go to posk[j & 7] a step before its K rows are
+      // requested (asynchronous; the step's wait and barrier make them visible to every wavefront)
+      auto load_ids = [&](int j) {
+        if (kPacked && far_win && j < n_vis && wave == 0) {
+          int ln = lane;
+#if defined(__HIP_DEVICE_COMPILE__)
+          asm volatile("" : "+v"(ln));
+#endif
+          __builtin_amdgcn_global_load_lds(lrows + (int64_t)(f0 + j0 + j) * kTile + ln,
+                                           (uint32_t __attribute__((address_space(3)))*)(&sm.posk[j & 7][0]), 4, 0, 0);
+        }
+      };
+      if (kPacked && far_win) {
+#pragma unroll
+        for (int j = 0; j < 5; ++j) load_ids(j);
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+      }
       Entry e0 = read_entry(0), e1 = read_entry(1), e2 = read_entry(2);
       load_k(0, e0);
       load_v(0, e0);
@@ -824,14 +912,22 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
         load_k(t + 4, e4);
         load_v(t + 2, e2);
         load_v(t + 3, e3);
+        load_ids(t + 5);
+        load_ids(t + 6);
         process_tile(t, e0, e1);
         if (t + 1 < n_vis) process_tile(t + 1, e1, e2);
         e0 = e2; e1 = e3; e2 = e4;
         __builtin_amdgcn_s_waitcnt(0);  // the tiles in flight have landed in LDS
         __syncthreads();                // ... for every wavefront, and the tiles of this step are no longer read
       }
-    } else if (w0 + kWinStep <= win_last) {
+    } else if (far_win || w0 + kWinStep <= win_last) {
       __syncthreads();  // (nobody may still be reading this window's count when wavefront 0 starts the next list)
+    }
+    if (far_win) {
+      f0 += kWin - 1;
+      far_win = f0 < n_far_tiles;
+    } else {
+      w0 += kWinStep;
     }
   }
 
@@ -1121,6 +1217,11 @@ bool use_packed_tiles() {
   return !(e && e[0] == '0');
 }
 
+bool use_far_rows() {
+  const char* e = getenv("NATS_PREFILL_FAR");
+  return !(e && e[0] == '0');
+}
+
 // key limits are in the workspace; launches the attention kernel of the segment
 int launch_segment(const char* who, const SegmentShape& g, const void* q, const void* k, const void* v, void* o,
                    const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
@@ -1182,6 +1283,15 @@ int launch_segment(const char* who, const SegmentShape& g, const void* q, const 
   // workgroup's four or two query tiles walk one list together, which costs the same as every wavefront skipping
   // on its own between shared barriers and lets small launches share their lists among workgroups.
   const bool packed = (g.C < kTile || hpw < 4) && use_packed_tiles();
+  // Chunks shorter than a granule: a granule far behind a query mostly holds a visible row or two among invisible
+  // ones, so the rows more than a window (and a granule) behind a query group are taken from the lists of
+  // long-lived rows instead, row by row (NATS_PREFILL_FAR=0 in the environment walks every granule, for comparison).
+  if (packed && g.C < kGranule && use_far_rows()) {
+    a.t_long = (int)(g.W + kGranule);
+    if (int rc = launch_long_rows(w, g.B * g.H_kv, g.N, g.base, a.t_long, st)) return rc;
+    a.long_rows = w.long_rows; a.long_lim = w.long_lim; a.long_before = w.long_before; a.long_tmin = w.long_tmin;
+    a.long_cap = (int)w.long_cap; a.n_gran = (int)w.n_gran;
+  }
   a.n_split = 1;
   if (hpw == 4 || packed) {  // the kernels in which every wavefront walks the whole tile list
     const int ns = choose_split(n_wg, a.Tk);

@@ -303,8 +303,114 @@ PrefillWorkspace carve_prefill_workspace(void* ws, int64_t n_streams, int64_t S,
   off += up((size_t)(n_streams * Tk * (kTile / kGranule)) * sizeof(int2));
   w.ticket = reinterpret_cast<int32_t*>(p + off);
   off += up(8 * 32 * sizeof(int32_t));  // eight counters, 128 bytes apart
+  w.long_cap = (Tk + 1) * kTile;
+  w.n_gran = Tk * (kTile / kGranule);
+  w.long_rows = reinterpret_cast<int32_t*>(p + off);
+  off += up((size_t)(n_streams * w.long_cap) * sizeof(int32_t));
+  w.long_lim = reinterpret_cast<int32_t*>(p + off);
+  off += up((size_t)(n_streams * w.long_cap) * sizeof(int32_t));
+  w.long_before = reinterpret_cast<int32_t*>(p + off);
+  off += up((size_t)(n_streams * (w.n_gran + 1)) * sizeof(int32_t));
+  w.long_tmin = reinterpret_cast<int32_t*>(p + off);
+  off += up((size_t)(n_streams * (Tk + 1)) * sizeof(int32_t));
   w.bytes = off;
   return w;
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Long-lived rows.  With chunks shorter than a 16-row granule most granules far behind a query hold a row or two
+// that it still sees (a global token among sliding-window tokens), and walking them granule by granule loads and
+// multiplies mostly invisible rows.  A row is long-lived when some query more than t_long tokens after it may see it:
+// tok_lim[n] >= (n - base) + t_long.  Per stream the kernel lists these rows in ascending order with their limits,
+// counts the list entries before every granule, and notes the least limit of every 64 entries.  A query group whose
+// first token is r0 then takes, of the rows below base + r0 - t_long, exactly the listed ones (any other row there has
+// tok_lim < r0 and is seen by nobody in the group), gathered 64 to a tile, and walks only the rows from there on
+// granule by granule.  One workgroup per stream; a thread owns one granule per round.
+// ---------------------------------------------------------------------------------------------------
+constexpr int kLongThreads = 1024;
+
+__global__ __launch_bounds__(kLongThreads) void long_rows_kernel(const int32_t* __restrict__ tok_lim, int N, int base,
+                                                                 int t_long, int n_gran, int long_cap,
+                                                                 int32_t* __restrict__ long_rows,
+                                                                 int32_t* __restrict__ long_lim,
+                                                                 int32_t* __restrict__ long_before,
+                                                                 int32_t* __restrict__ long_tmin) {
+  __shared__ int wave_tot[kLongThreads / kWave];
+  __shared__ int carry;
+  const int ks = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int32_t* lim = tok_lim + (int64_t)ks * N;
+  int32_t* rows_o = long_rows + (int64_t)ks * long_cap;
+  int32_t* lim_o = long_lim + (int64_t)ks * long_cap;
+  int32_t* before_o = long_before + (int64_t)ks * (n_gran + 1);
+  if (tid == 0) carry = 0;
+  __syncthreads();
+  for (int g0 = 0; g0 < n_gran; g0 += kLongThreads) {
+    const int g = g0 + tid;
+    int lv[kGranule];
+    unsigned bits = 0;
+#pragma unroll
+    for (int i = 0; i < kGranule; ++i) {
+      const int n = g * kGranule + i;
+      lv[i] = (g < n_gran && n < N) ? lim[n] : -1;
+      if (lv[i] >= 0 && lv[i] >= n - base + t_long) bits |= 1u << i;
+    }
+    const int cnt = __builtin_popcount(bits);
+    int incl = cnt;
+#pragma unroll
+    for (int o = 1; o < kWave; o <<= 1) {
+      const int y = __shfl_up(incl, o);
+      if (lane >= o) incl += y;
+    }
+    if (lane == kWave - 1) wave_tot[wave] = incl;
+    __syncthreads();
+    int off = carry + incl - cnt;
+    int total = 0;
+#pragma unroll
+    for (int w = 0; w < kLongThreads / kWave; ++w) {
+      const int t = wave_tot[w];
+      if (w < wave) off += t;
+      total += t;
+    }
+    if (g < n_gran) before_o[g] = off;
+#pragma unroll
+    for (int i = 0; i < kGranule; ++i) {
+      if (bits & (1u << i)) {
+        rows_o[off] = g * kGranule + i;
+        lim_o[off] = lv[i];
+        ++off;
+      }
+    }
+    __syncthreads();
+    if (tid == 0) carry += total;
+    __syncthreads();
+  }
+  const int total = carry;
+  if (tid == 0) before_o[n_gran] = total;
+  const int n_tiles = (total + kTile - 1) / kTile + 1;  // (one tile of padding: a reader may run one tile ahead)
+  for (int i = total + tid; i < n_tiles * kTile; i += kLongThreads) {
+    rows_o[i] = 0x7fffffff;
+    lim_o[i] = -1;
+  }
+  // least limit of every 64 entries (the entries were written by other threads of this workgroup: they are read
+  // past the first-level cache, after a fence and a barrier)
+  __threadfence();
+  __syncthreads();
+  int32_t* tmin_o = long_tmin + (int64_t)ks * (long_cap / kTile);
+  for (int t = wave; t < n_tiles; t += kLongThreads / kWave) {
+    int m = __hip_atomic_load(lim_o + t * kTile + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) m = min(m, __shfl_xor(m, o));
+    if (lane == 0) tmin_o[t] = m;
+  }
+}
+
+int launch_long_rows(const PrefillWorkspace& w, int64_t n_streams, int64_t N, int64_t base, int64_t t_long, hipStream_t st) {
+  NATS_REQUIRE(n_streams <= 0x7fffffff, NATS_ERR_BAD_SHAPE, "long_rows_kernel: %lld streams", (long long)n_streams);
+  hipLaunchKernelGGL(long_rows_kernel, dim3((unsigned)n_streams), dim3(kLongThreads), 0, st, w.tok_lim, (int)N, (int)base,
+                     (int)t_long, (int)w.n_gran, (int)w.long_cap, w.long_rows, w.long_lim, w.long_before, w.long_tmin);
+  NATS_CHECK_LAUNCH("long_rows_kernel");
+  return NATS_OK;
 }
 
 // roles -> vis_lim, first_global -> tok_lim, tile_lim.  `past` may be NULL (prefill from an empty cache).

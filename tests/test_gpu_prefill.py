@@ -280,6 +280,68 @@ def test_packed_tiles_on_segments_over_a_filled_cache(packed_tiles):
         assert (x - y).abs().max().item() <= 2e-2
 
 
+# ---- chunks shorter than a granule: rows far behind a query come from the lists of long-lived rows ----------------
+@pytest.fixture
+def far_rows(monkeypatch):
+    def switch(on: bool):
+        monkeypatch.setenv("NATS_PREFILL_FAR", "1" if on else "0")
+    yield switch
+    monkeypatch.delenv("NATS_PREFILL_FAR", raising=False)
+
+
+@pytest.mark.parametrize("Hq,Hkv,L,C,W,p", [
+    (32, 8, 32768, 1, 256, (0.05, 0.15, 0.8)),     # the headline shape with a role per token
+    (4, 1, 70016, 1, 64, (0.97, 0.02, 0.01)),      # 1060 tiles of long-lived rows: two windows of gathered tiles
+    (8, 2, 40000, 4, 32, (0.004, 0.5, 0.496)),     # long runs of local tokens: long-lived rows with finite limits
+    (4, 4, 20000, 2, 16, (0.05, 0.15, 0.8)),       # one q head per kv head: four query tiles share the gathered tiles
+])
+def test_long_lived_rows_full_size_sampled_rows(Hq, Hkv, L, C, W, p):
+    say("prefill gathered rows, sampled rows", Hq, Hkv, L, C, W, p)
+    check_sampled_rows(1, Hq, Hkv, L, 128, C, W, n_samples=64, p=p)
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,L,D,C,W,p", [
+    (2, 8, 2, 1500, 128, 1, 4, (0.1, 0.3, 0.6)),
+    (1, 8, 2, 1100, 64, 2, 8, (0.05, 0.5, 0.45)),
+    (1, 4, 2, 900, 128, 8, 16, (0.2, 0.3, 0.5)),    # groups of 2
+    (1, 2, 2, 700, 128, 4, 8, (0.3, 0.3, 0.4)),     # groups of 1
+    (1, 8, 2, 1300, 128, 1, 16, (0.0, 0.0, 1.0)),   # no long-lived row but the first
+    (1, 8, 2, 1300, 128, 1, 16, (1.0, 0.0, 0.0)),   # every row is long-lived
+])
+def test_long_lived_rows_against_the_oracle(B, Hq, Hkv, L, D, C, W, p):
+    """Small windows, so that most of every query's keys come through the gathered tiles."""
+    run_case(B, Hq, Hkv, L, D, C, W, torch.bfloat16, seed=L, p=p)
+
+
+def test_gathered_rows_agree_with_the_granule_walk(far_rows):
+    """The same keys reach the softmax in another order, on a first prefill and on segments over a per-token cache
+    (cache rows below the open chunk: ring, kept rows, pending tokens)."""
+    from neuralattentionsearch_amd import ops
+    from neuralattentionsearch_amd.cache import NAtSLayerCache
+    say("prefill gathered rows vs granule walk")
+    B, Hq, Hkv, D, W = 1, 8, 2, 128, 32
+    outs = []
+    for on in (False, True):
+        far_rows(on)
+        gg = torch.Generator().manual_seed(5)
+        cache = NAtSLayerCache(B, Hkv, W, device="cuda")
+        res = []
+        for n, seed in ((3000, 1), (700, 2), (45, 3), (1200, 4)):
+            q = torch.randn(B, Hq, n, D, generator=gg).bfloat16().cuda()
+            k = torch.randn(B, Hkv, n, D, generator=gg).bfloat16().cuda()
+            v = torch.randn(B, Hkv, n, D, generator=gg).bfloat16().cuda()
+            first = cache.get_seq_length() == 0
+            roles = draw_roles(seed, B, Hkv, n, p=(0.1, 0.2, 0.7), first_global=first)
+            tsi = orc.one_hot_roles(roles).bfloat16().cuda()
+            kk, vv = cache.update(k, v, tsi)
+            res.append((ops.prefill_attention(q, kk, vv, to_dev(roles), 1, W) if first else cache.segment_attention(q)).float())
+            cache.post_update(n)
+        outs.append(res)
+    for x, y in zip(*outs):
+        assert torch.isfinite(y).all()
+        assert (x - y).abs().max().item() <= 2e-2
+
+
 # ---- running maxima that keep rising: the rescaling branch of every variant ------------------------------------
 def rising_inputs(B, Hq, Hkv, L, D, step_rows, step_nats, seed):
     """q, k, v whose scores grow by `step_nats` every `step_rows` keys (a common direction u: q carries sqrt(D) u,
