@@ -81,6 +81,9 @@ struct KeyLimArgs {
   int2* tile_lim;    // [streams, Tk] out {max, min}
   int2* gran_lim;    // [streams, Tk * 4] out {max, min} of every 16 rows
   int32_t* ticket;   // out: one counter, set to zero (may be NULL)
+  int4* tile_long;   // [streams, Tk] out (may be NULL): per 64-row tile the long-lived rows every later query sees, those
+                     // with a last query, and the greatest limit among the latter (see long_rows_kernel)
+  int t_long;
   int Hkv, S, N, Tk, c_shift, C, W;
   int base, gmin, tail, seen, fill_last;
   int old_fill, token_mode;
@@ -93,14 +96,17 @@ struct PrefillWorkspace {
   int2* tile_lim;
   int2* gran_lim;
   int32_t* ticket;  // one counter, set to zero by the key-limit kernel (the attention kernel deals work from it)
-  // long-lived rows (see long_rows_kernel): per stream the ascending list of their row ids, their limits, the number
-  // of list entries before every 16-row granule, and the least limit of every 64 list entries
-  int32_t* long_rows;    // [streams, long_cap]
-  int32_t* long_lim;     // [streams, long_cap]
-  int32_t* long_before;  // [streams, n_gran + 1]
-  int32_t* long_tmin;    // [streams, long_cap / 64]
-  int64_t long_cap;      // list entries per stream: N rounded up to whole tiles, plus one tile of padding
+  // long-lived rows (see long_rows_kernel): per stream two ascending lists of row ids with their limits (A: rows every
+  // later query sees, B: rows with a last query), the number of entries
+  // of each list before every 16-row granule, and for every 64-token region tile the first entry of B that matters
+  int32_t* long_rows;    // [streams, 2, long_cap]
+  int32_t* long_lim;     // [streams, 2, long_cap]
+  int4* tile_long;       // [streams, Tk] counts of both kinds per 64-row tile, from the key-limit kernel
+  int32_t* long_before;  // [streams, 2, n_gran + 1]
+  int32_t* long_alive;   // [streams, n_rtile]
+  int64_t long_cap;      // entries per list: N rounded up to whole tiles, plus one tile of padding
   int64_t n_gran;        // 16-row granules per stream
+  int64_t n_rtile;       // entries of long_alive per stream
   size_t bytes;
 };
 
@@ -109,7 +115,9 @@ int prepare_key_limits(const uint8_t* roles, int64_t B, int64_t H_kv, int64_t S,
                        const PastView* past, const PrefillWorkspace& w, hipStream_t st);
 int check_past_state(const char* who, const nats_past_state* ps, int64_t x_len, int64_t C, int64_t W);
 // Fills the long-lived-row lists of the workspace from its key limits (after prepare_key_limits on the same stream).
-int launch_long_rows(const PrefillWorkspace& w, int64_t n_streams, int64_t N, int64_t base, int64_t t_long, hipStream_t st);
+int launch_long_rows(const PrefillWorkspace& w, int64_t n_streams, int64_t N, int64_t base, int64_t W, hipStream_t st);
+// rows that a query more than this many tokens behind them may still see are long-lived
+inline int64_t long_row_threshold(int64_t W) { return W + kGranule; }
 
 // Orders LDS traffic between the lanes of one wavefront (no workgroup barrier needed for wave-private LDS).
 __device__ __forceinline__ void wave_lds_sync() {

@@ -54,11 +54,11 @@ struct PrefillArgs {
   float* part_ml;   // [workgroup, split, wavefront, 32 rows, 2] running maximum (base-2 exponent) and row sum
   // packed tiles of chunks shorter than a granule: rows more than t_long tokens behind a query group come from the
   // lists of long-lived rows (long_rows_kernel), gathered row by row; NULL = every row is walked granule by granule
-  const int32_t* long_rows;
-  const int32_t* long_lim;
-  const int32_t* long_before;
-  const int32_t* long_tmin;
-  int long_cap, n_gran, t_long;
+  const int32_t* long_rows;    // [streams, 2, long_cap]: list A (rows every later query sees), list B (rows with a last query)
+  const int32_t* long_lim;     // [streams, 2, long_cap]
+  const int32_t* long_before;  // [streams, 2, n_gran + 1] entries of A / of B before every granule
+  const int32_t* long_alive;   // [streams, n_rtile] first entry of B that a query of the 64-token region tile may see
+  int long_cap, n_gran, n_rtile, t_long;
 };
 
 // workgroup index -> (kv stream, head group, rank of the query group; heavy query groups come first)
@@ -231,7 +231,7 @@ struct PrefillSmem {
 };
 constexpr int kGranPerTile = kTile / kGranule;
 constexpr int kPackedMaskFlag = 1 << 30;  // on the first granule id of a packed tile: some score of the tile is masked
-constexpr int kFarTileFlag = 1 << 29;     // ... the entry is tile (id & 0xffffff) of the stream's list of long-lived rows
+constexpr int kFarTileFlag = 1 << 29;     // ... the entry is a tile of long-lived rows: 64 list entries from the second field on
 
 // kUniform: the wavefronts are the q heads of ONE query tile (GQA groups of 4 and more), so every tile of
 // the visit list is visited by every wavefront and the tile loop has no per-wavefront branches.
@@ -287,21 +287,24 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
   const int my_kt_end = (a.base + tile_rlast) / kTile;
 
   // Rows more than t_long tokens behind the group's first query: only the stream's long-lived rows can be visible
-  // there (long_rows_kernel); the first n_far entries of their list lie below near_row0, the row from which the
-  // group walks granule by granule.
+  // there (long_rows_kernel).  Below near_row0, the row from which the group walks granule by granule, lie the first
+  // n_far_a entries of list A and the first b_hi of list B, of which those before b_lo are seen by nobody here.
   const bool far_mode = kPacked && a.long_rows != nullptr;
-  int near_row0 = 0, n_far = 0;
+  int near_row0 = 0, n_far_a = 0, b_lo = 0, b_hi = 0;
   const int32_t* lrows = nullptr;
   const int32_t* llim = nullptr;
-  const int32_t* ltmin = nullptr;
   if (far_mode) {
     near_row0 = max(0, a.base + r0_group - a.t_long) & ~(kGranule - 1);
-    n_far = __builtin_amdgcn_readfirstlane(a.long_before[(int64_t)ks * (a.n_gran + 1) + near_row0 / kGranule]);
-    lrows = a.long_rows + (int64_t)ks * a.long_cap;
-    llim = a.long_lim + (int64_t)ks * a.long_cap;
-    ltmin = a.long_tmin + (int64_t)ks * (a.long_cap / kTile);
+    const int32_t* bef = a.long_before + (int64_t)ks * 2 * (a.n_gran + 1) + near_row0 / kGranule;
+    n_far_a = __builtin_amdgcn_readfirstlane(bef[0]);
+    b_hi = __builtin_amdgcn_readfirstlane(bef[a.n_gran + 1]);
+    b_lo = __builtin_amdgcn_readfirstlane(a.long_alive[(int64_t)ks * a.n_rtile + r0_group / kTile]);
+    b_lo = min(b_lo, b_hi);
+    lrows = a.long_rows + (int64_t)ks * 2 * a.long_cap;
+    llim = a.long_lim + (int64_t)ks * 2 * a.long_cap;
   }
-  const int n_far_tiles = (n_far + kTile - 1) / kTile;
+  const int n_far_ta = (n_far_a + kTile - 1) / kTile;  // gathered tiles of list A, then of list B
+  const int n_far_tiles = n_far_ta + (b_hi - b_lo + kTile - 1) / kTile;
 
   // ---- wavefront 0 asks for the tile summaries of the first kEarly * 64 key tiles before anything else is requested:
   // memory operations complete in the order of their issue, so the wait for these (a trip to L2) does not include
@@ -432,7 +435,7 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
 #if defined(__HIP_DEVICE_COMPILE__)
         asm volatile("" : "+v"(ln));
 #endif
-        __builtin_amdgcn_global_load_lds(llim + (int64_t)(id0 & 0xffffff) * kTile + ln,
+        __builtin_amdgcn_global_load_lds(llim + id1 + ln,
                                          (uint32_t __attribute__((address_space(3)))*)(&sm.limk[slot][0]), 4, 0, 0);
       }
       return;
@@ -723,13 +726,18 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
   for (int w0 = far_mode ? near_row0 / kGranule : 0; w0 <= win_last;) {
     // ---- visit list of this window: wavefront 0 compacts the tiles some query tile of the group sees ----
     if (kPacked && far_win && wave == 0) {
-      // tiles [f0, f0 + count) of the list; a tile needs no mask when all its rows lie below near_row0 and every
-      // query of the group sees every one of them
+      // gathered tiles [f0, f0 + count): whole tiles of list A need no mask (every query sees their rows, and they
+      // lie below near_row0); the last one of A and the tiles of B go through it
       const int cnt = min(kWin - 1, n_far_tiles - f0);
       for (int i = lane; i < cnt; i += kWave) {
         const int t = f0 + i;
-        const bool plain = (t + 1) * kTile <= n_far && ltmin[t] >= rlast_group;
-        sm.vlist[i] = make_int4(kFarTileFlag | (plain ? 0 : kPackedMaskFlag) | t, 0, 0, 0);
+        int4 d;
+        if (t < n_far_ta) {
+          d = make_int4(kFarTileFlag | ((t + 1) * kTile <= n_far_a ? 0 : kPackedMaskFlag), t * kTile, 0, 0);
+        } else {
+          d = make_int4(kFarTileFlag | kPackedMaskFlag, a.long_cap + b_lo + (t - n_far_ta) * kTile, 0, 0);
+        }
+        sm.vlist[i] = d;
       }
       if (lane == 0) sm.vcount = cnt;
     }
@@ -885,7 +893,8 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
 #if defined(__HIP_DEVICE_COMPILE__)
           asm volatile("" : "+v"(ln));
 #endif
-          __builtin_amdgcn_global_load_lds(lrows + (int64_t)(f0 + j0 + j) * kTile + ln,
+          const int start = __builtin_amdgcn_readfirstlane(sm.vlist[j0 + j].y);
+          __builtin_amdgcn_global_load_lds(lrows + start + ln,
                                            (uint32_t __attribute__((address_space(3)))*)(&sm.posk[j & 7][0]), 4, 0, 0);
         }
       };
@@ -1287,10 +1296,10 @@ int launch_segment(const char* who, const SegmentShape& g, const void* q, const 
   // ones, so the rows more than a window (and a granule) behind a query group are taken from the lists of
   // long-lived rows instead, row by row (NATS_PREFILL_FAR=0 in the environment walks every granule, for comparison).
   if (packed && g.C < kGranule && use_far_rows()) {
-    a.t_long = (int)(g.W + kGranule);
-    if (int rc = launch_long_rows(w, g.B * g.H_kv, g.N, g.base, a.t_long, st)) return rc;
-    a.long_rows = w.long_rows; a.long_lim = w.long_lim; a.long_before = w.long_before; a.long_tmin = w.long_tmin;
-    a.long_cap = (int)w.long_cap; a.n_gran = (int)w.n_gran;
+    a.t_long = (int)long_row_threshold(g.W);
+    if (int rc = launch_long_rows(w, g.B * g.H_kv, g.N, g.base, g.W, st)) return rc;
+    a.long_rows = w.long_rows; a.long_lim = w.long_lim; a.long_before = w.long_before; a.long_alive = w.long_alive;
+    a.long_cap = (int)w.long_cap; a.n_gran = (int)w.n_gran; a.n_rtile = (int)w.n_rtile;
   }
   a.n_split = 1;
   if (hpw == 4 || packed) {  // the kernels in which every wavefront walks the whole tile list

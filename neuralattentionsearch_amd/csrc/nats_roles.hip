@@ -70,44 +70,76 @@ __global__ void roles_kernel(const void* __restrict__ logits, int64_t B, int64_t
 }
 
 // ---------------------------------------------------------------------------------------------------
-// One wavefront per (b, h): reverse scan in blocks of 64 slots with a ballot per block.
+// Reverse scan per (b, h) in blocks of 64 slots with a ballot per block.
 // end_idx[n] = first global slot >= n, the last slot counting as global (components/masks/utils.py:85-87).
 // vis_lim[n] = last query slot that sees key slot n:
 //   global -> INT32_MAX, sliding window -> n + W / C, local -> end_idx[n]
 // (components/masks/utils.py:92 and components/cache/nats_chunk_layer_cache.py:603-611).
 // ---------------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(64) void role_scan_kernel(const uint8_t* __restrict__ roles, int64_t S, int32_t wc,
-                                                      int64_t* __restrict__ end_idx, int32_t* __restrict__ vis_lim,
-                                                      int32_t* __restrict__ first_global) {
+// A workgroup takes kScanWaves * kScanSpan consecutive slots of one stream, a wavefront kScanSpan of them: it first
+// looks for the first global slot of its span (and the last wavefront for the first one behind the workgroup's slots,
+// which is usually a block or two away), then walks its span from the end with what follows it as the carry.
+constexpr int kScanWaves = 16;
+constexpr int kScanSpan = 256;
+
+__global__ __launch_bounds__(kScanWaves * kWave) void role_scan_kernel(const uint8_t* __restrict__ roles, int64_t S,
+                                                                       int32_t wc, int64_t* __restrict__ end_idx,
+                                                                       int32_t* __restrict__ vis_lim,
+                                                                       int32_t* __restrict__ first_global) {
+  __shared__ int64_t first_g[kScanWaves + 1];
   const int64_t stream = blockIdx.x;
   const uint8_t* r = roles + stream * S;
   const int lane = lane_id();
-  int64_t carry = S - 1;
-  for (int64_t base = ((S - 1) / kWave) * kWave; base >= 0; base -= kWave) {
-    int64_t n = base + lane;
-    bool in = n < S;
-    uint8_t role = in ? r[n] : uint8_t(NATS_ROLE_LOCAL);
-    bool is_g = in && (role == NATS_ROLE_GLOBAL || n == S - 1);
-    uint64_t bits = __ballot(is_g);
-    uint64_t ahead = bits >> lane;  // bit 0 = this slot
-    int64_t g = ahead ? n + __builtin_ctzll(ahead) : carry;
-    if (in) {
-      if (end_idx) end_idx[stream * S + n] = g;
-      if (vis_lim) {
-        int32_t lim;
-        if (role == NATS_ROLE_GLOBAL) {
-          lim = kLimGlobal;
-        } else if (role == NATS_ROLE_SW) {
-          lim = int32_t(n) + wc;
-        } else {
-          lim = int32_t(g);
-        }
-        vis_lim[stream * S + n] = lim;
-      }
+  const int wave = threadIdx.x >> 6;
+  const int64_t seg0 = int64_t(blockIdx.y) * (kScanWaves * kScanSpan);
+  const int64_t span0 = seg0 + wave * kScanSpan;
+  const int64_t span1 = min(span0 + kScanSpan, S);
+  auto first_global_in = [&](int64_t lo, int64_t hi) {  // first global slot in [lo, hi), or S
+    for (int64_t b = lo; b < hi; b += kWave) {
+      const int64_t n = b + lane;
+      const bool is_g = n < hi && (r[n] == NATS_ROLE_GLOBAL || n == S - 1);
+      const uint64_t bits = __ballot(is_g);
+      if (bits) return b + __builtin_ctzll(bits);
     }
-    if (bits) carry = base + __builtin_ctzll(bits);
+    return S;
+  };
+  const int64_t mine = first_global_in(span0, span1);
+  if (lane == 0) first_g[wave] = mine;
+  if (wave == kScanWaves - 1) {
+    const int64_t behind = first_global_in(min(seg0 + kScanWaves * kScanSpan, S), S);
+    if (lane == 0) first_g[kScanWaves] = behind < S ? behind : S - 1;
   }
-  if (first_global && lane == 0) first_global[stream] = int32_t(carry);  // end_idx[0]
+  __syncthreads();
+  int64_t carry = first_g[kScanWaves];
+  for (int w = kScanWaves - 1; w > wave; --w)
+    if (first_g[w] < S) carry = first_g[w];
+  if (span0 < S) {
+    for (int64_t base = span0 + ((span1 - 1 - span0) / kWave) * kWave; base >= span0; base -= kWave) {
+      int64_t n = base + lane;
+      bool in = n < span1;
+      uint8_t role = in ? r[n] : uint8_t(NATS_ROLE_LOCAL);
+      bool is_g = in && (role == NATS_ROLE_GLOBAL || n == S - 1);
+      uint64_t bits = __ballot(is_g);
+      uint64_t ahead = bits >> lane;  // bit 0 = this slot
+      int64_t g = ahead ? n + __builtin_ctzll(ahead) : carry;
+      if (in) {
+        if (end_idx) end_idx[stream * S + n] = g;
+        if (vis_lim) {
+          int32_t lim;
+          if (role == NATS_ROLE_GLOBAL) {
+            lim = kLimGlobal;
+          } else if (role == NATS_ROLE_SW) {
+            lim = int32_t(n) + wc;
+          } else {
+            lim = int32_t(g);
+          }
+          vis_lim[stream * S + n] = lim;
+        }
+      }
+      if (bits) carry = base + __builtin_ctzll(bits);
+    }
+  }
+  if (first_global && blockIdx.y == 0 && wave == 0 && lane == 0) first_global[stream] = int32_t(carry);  // end_idx[0]
 }
 
 // Per key row the last query token (counted from the start of the open-chunk region) that sees it, and
@@ -241,6 +273,16 @@ __global__ __launch_bounds__(256) void key_lim_kernel(KeyLimArgs a) {
     mn = min(mn, __shfl_xor(mn, off));
   }
   if (lane == 0) a.tile_lim[(int64_t)stream * a.Tk + tile] = make_int2(mx, mn);
+  if (a.tile_long) {
+    const bool is_long = row < a.N && lim >= 0 && lim >= row - a.base + a.t_long;
+    const bool kind_a = is_long && lim == kLimGlobal;
+    const bool kind_b = is_long && !kind_a;
+    int mb = kind_b ? lim : -1;
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) mb = max(mb, __shfl_xor(mb, off));
+    const int na = __builtin_popcountll(__ballot(kind_a)), nb = __builtin_popcountll(__ballot(kind_b));
+    if (lane == 0) a.tile_long[(int64_t)stream * a.Tk + tile] = make_int4(na, nb, mb, 0);
+  }
   if (stream == 0 && tile == 0 && lane == 0) a.tok_lim[(int64_t)gridDim.y * a.N] = -1;
 }
 
@@ -267,8 +309,10 @@ __global__ void tile_map_kernel(const int2* __restrict__ tile_lim, int64_t T, ui
 
 int launch_role_scan(const uint8_t* roles, int64_t n_streams, int64_t S, int64_t W, int64_t C, int64_t* end_idx,
                      int32_t* vis_lim, int32_t* first_global, hipStream_t st) {
-  hipLaunchKernelGGL(role_scan_kernel, dim3((unsigned)n_streams), dim3(kWave), 0, st, roles, S, int32_t(W / C), end_idx,
-                     vis_lim, first_global);
+  const int64_t n_seg = (S + kScanWaves * kScanSpan - 1) / (kScanWaves * kScanSpan);
+  NATS_REQUIRE(n_seg <= 65535, NATS_ERR_BAD_SHAPE, "role_scan_kernel: %lld role slots per stream", (long long)S);
+  hipLaunchKernelGGL(role_scan_kernel, dim3((unsigned)n_streams, (unsigned)n_seg), dim3(kScanWaves * kWave), 0, st, roles, S,
+                     int32_t(W / C), end_idx, vis_lim, first_global);
   NATS_CHECK_LAUNCH("role_scan_kernel");
   return NATS_OK;
 }
@@ -305,14 +349,17 @@ PrefillWorkspace carve_prefill_workspace(void* ws, int64_t n_streams, int64_t S,
   off += up(8 * 32 * sizeof(int32_t));  // eight counters, 128 bytes apart
   w.long_cap = (Tk + 1) * kTile;
   w.n_gran = Tk * (kTile / kGranule);
+  w.n_rtile = Tk + 2;
   w.long_rows = reinterpret_cast<int32_t*>(p + off);
-  off += up((size_t)(n_streams * w.long_cap) * sizeof(int32_t));
+  off += up((size_t)(n_streams * 2 * w.long_cap) * sizeof(int32_t));
   w.long_lim = reinterpret_cast<int32_t*>(p + off);
-  off += up((size_t)(n_streams * w.long_cap) * sizeof(int32_t));
+  off += up((size_t)(n_streams * 2 * w.long_cap) * sizeof(int32_t));
+  w.tile_long = reinterpret_cast<int4*>(p + off);
+  off += up((size_t)(n_streams * Tk) * sizeof(int4));
   w.long_before = reinterpret_cast<int32_t*>(p + off);
-  off += up((size_t)(n_streams * (w.n_gran + 1)) * sizeof(int32_t));
-  w.long_tmin = reinterpret_cast<int32_t*>(p + off);
-  off += up((size_t)(n_streams * (Tk + 1)) * sizeof(int32_t));
+  off += up((size_t)(n_streams * 2 * (w.n_gran + 1)) * sizeof(int32_t));
+  w.long_alive = reinterpret_cast<int32_t*>(p + off);
+  off += up((size_t)(n_streams * w.n_rtile) * sizeof(int32_t));
   w.bytes = off;
   return w;
 }
@@ -321,94 +368,145 @@ PrefillWorkspace carve_prefill_workspace(void* ws, int64_t n_streams, int64_t S,
 // Long-lived rows.  With chunks shorter than a 16-row granule most granules far behind a query hold a row or two
 // that it still sees (a global token among sliding-window tokens), and walking them granule by granule loads and
 // multiplies mostly invisible rows.  A row is long-lived when some query more than t_long tokens after it may see it:
-// tok_lim[n] >= (n - base) + t_long.  Per stream the kernel lists these rows in ascending order with their limits,
-// counts the list entries before every granule, and notes the least limit of every 64 entries.  A query group whose
-// first token is r0 then takes, of the rows below base + r0 - t_long, exactly the listed ones (any other row there has
-// tok_lim < r0 and is seen by nobody in the group), gathered 64 to a tile, and walks only the rows from there on
-// granule by granule.  One workgroup per stream; a thread owns one granule per round.
+// tok_lim[n] >= (n - base) + t_long.  A query group whose first token is r0 finds, among the rows below
+// base + r0 - t_long, its visible rows among the long-lived ones only (any other row there has tok_lim < r0).
+// Per stream the kernel writes two lists of row ids with their limits, each in ascending row order:
+//   A  long-lived rows that every later query sees (global tokens, kept cache rows);
+//   B  long-lived rows with a last query that sees them (local tokens far from their next global token, ring rows):
+//      the entries before the first one at which the running maximum of the limits along the list reaches r0 are
+//      invisible from r0 on, and `alive` holds that first entry for every 64-token region tile;
+// and for each list the number of entries before every granule.  The attention kernel gathers the entries of A
+// below its first granule-walked row, and those of B from `alive` on, 64 to a tile.
+// A wavefront per 64-row tile; what lies before a tile comes from the per-tile counts the key-limit kernel left.
 // ---------------------------------------------------------------------------------------------------
-constexpr int kLongThreads = 1024;
+constexpr int kLongWaves = 16;  // 64-row tiles per workgroup
 
-__global__ __launch_bounds__(kLongThreads) void long_rows_kernel(const int32_t* __restrict__ tok_lim, int N, int base,
-                                                                 int t_long, int n_gran, int long_cap,
-                                                                 int32_t* __restrict__ long_rows,
-                                                                 int32_t* __restrict__ long_lim,
-                                                                 int32_t* __restrict__ long_before,
-                                                                 int32_t* __restrict__ long_tmin) {
-  __shared__ int wave_tot[kLongThreads / kWave];
-  __shared__ int carry;
-  const int ks = blockIdx.x;
+__global__ __launch_bounds__(kLongWaves * kWave) void long_rows_kernel(const int32_t* __restrict__ tok_lim,
+                                                                       const int4* __restrict__ tile_long, int N, int Tk,
+                                                                       int base, int t_long, int n_gran, int long_cap,
+                                                                       int n_rtile, int32_t* __restrict__ long_rows,
+                                                                       int32_t* __restrict__ long_lim,
+                                                                       int32_t* __restrict__ long_before,
+                                                                       int32_t* __restrict__ long_alive) {
+  __shared__ int red_a[kLongWaves], red_b[kLongWaves], red_m[kLongWaves];
+  const int ks = blockIdx.y;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int32_t* lim = tok_lim + (int64_t)ks * N;
-  int32_t* rows_o = long_rows + (int64_t)ks * long_cap;
-  int32_t* lim_o = long_lim + (int64_t)ks * long_cap;
-  int32_t* before_o = long_before + (int64_t)ks * (n_gran + 1);
-  if (tid == 0) carry = 0;
-  __syncthreads();
-  for (int g0 = 0; g0 < n_gran; g0 += kLongThreads) {
-    const int g = g0 + tid;
-    int lv[kGranule];
-    unsigned bits = 0;
+  const int t0 = blockIdx.x * kLongWaves;  // first tile of this workgroup
+  const int tile = t0 + wave;
+  const int4* tl = tile_long + (int64_t)ks * Tk;
+  // entries of both lists, and the greatest limit in B, in the tiles before this workgroup's
+  int sa = 0, sb = 0, sm = -1;
+  for (int t = tid; t < t0; t += kLongWaves * kWave) {
+    const int4 c = tl[t];
+    sa += c.x;
+    sb += c.y;
+    sm = max(sm, c.z);
+  }
 #pragma unroll
-    for (int i = 0; i < kGranule; ++i) {
-      const int n = g * kGranule + i;
-      lv[i] = (g < n_gran && n < N) ? lim[n] : -1;
-      if (lv[i] >= 0 && lv[i] >= n - base + t_long) bits |= 1u << i;
+  for (int o = 32; o >= 1; o >>= 1) {
+    sa += __shfl_xor(sa, o);
+    sb += __shfl_xor(sb, o);
+    sm = max(sm, __shfl_xor(sm, o));
+  }
+  if (lane == 0) {
+    red_a[wave] = sa;
+    red_b[wave] = sb;
+    red_m[wave] = sm;
+  }
+  __syncthreads();
+  int base_a = 0, base_b = 0, run_max = -1;
+#pragma unroll
+  for (int w = 0; w < kLongWaves; ++w) {
+    base_a += red_a[w];
+    base_b += red_b[w];
+    run_max = max(run_max, red_m[w]);
+  }
+  // ... and in the tiles of this workgroup before this wavefront's
+  {
+    int4 c = make_int4(0, 0, -1, 0);
+    if (lane < wave && t0 + lane < Tk) c = tl[t0 + lane];
+    int ca = c.x, cb = c.y, cm = c.z;
+#pragma unroll
+    for (int o = 8; o >= 1; o >>= 1) {
+      ca += __shfl_xor(ca, o);
+      cb += __shfl_xor(cb, o);
+      cm = max(cm, __shfl_xor(cm, o));
     }
-    const int cnt = __builtin_popcount(bits);
-    int incl = cnt;
+    base_a += __shfl(ca, 0);
+    base_b += __shfl(cb, 0);
+    run_max = max(run_max, __shfl(cm, 0));
+  }
+  int32_t* rows_a = long_rows + (int64_t)ks * 2 * long_cap;
+  int32_t* lims_a = long_lim + (int64_t)ks * 2 * long_cap;
+  int32_t* rows_b = rows_a + long_cap;
+  int32_t* lims_b = lims_a + long_cap;
+  int32_t* before_a = long_before + (int64_t)ks * 2 * (n_gran + 1);
+  int32_t* before_b = before_a + (n_gran + 1);
+  int32_t* alive = long_alive + (int64_t)ks * n_rtile;
+  if (tile < Tk) {
+    const int row = tile * kTile + lane;
+    const int lim = row < N ? tok_lim[(int64_t)ks * N + row] : -1;
+    const bool is_long = lim >= 0 && lim >= row - base + t_long;
+    const bool kind_a = is_long && lim == kLimGlobal;
+    const bool kind_b = is_long && !kind_a;
+    const uint64_t bits_a = __ballot(kind_a), bits_b = __ballot(kind_b);
+    const uint64_t below = (uint64_t(1) << lane) - 1;
+    const int off_a = base_a + __builtin_popcountll(bits_a & below);
+    const int off_b = base_b + __builtin_popcountll(bits_b & below);
+    if ((lane & (kGranule - 1)) == 0) {
+      before_a[row / kGranule] = off_a;
+      before_b[row / kGranule] = off_b;
+    }
+    if (kind_a) {
+      rows_a[off_a] = row;
+      lims_a[off_a] = lim;
+    }
+    // running maximum of the limits of B up to and without this lane's row
+    int incl = kind_b ? lim : -1;
 #pragma unroll
     for (int o = 1; o < kWave; o <<= 1) {
       const int y = __shfl_up(incl, o);
-      if (lane >= o) incl += y;
+      if (lane >= o) incl = max(incl, y);
     }
-    if (lane == kWave - 1) wave_tot[wave] = incl;
-    __syncthreads();
-    int off = carry + incl - cnt;
-    int total = 0;
-#pragma unroll
-    for (int w = 0; w < kLongThreads / kWave; ++w) {
-      const int t = wave_tot[w];
-      if (w < wave) off += t;
-      total += t;
+    int prev = __shfl_up(incl, 1);
+    if (lane == 0) prev = -1;
+    prev = max(prev, run_max);
+    if (kind_b) {
+      rows_b[off_b] = row;
+      lims_b[off_b] = lim;
+      // this entry is the first that matters to the region tiles whose first token lies in (prev, max(prev, lim)]
+      const int t_lo = prev < 0 ? 0 : prev / kTile + 1;
+      const int t_hi = min(max(prev, lim) / kTile, n_rtile - 1);
+      for (int t = t_lo; t <= t_hi; ++t) alive[t] = off_b;
     }
-    if (g < n_gran) before_o[g] = off;
-#pragma unroll
-    for (int i = 0; i < kGranule; ++i) {
-      if (bits & (1u << i)) {
-        rows_o[off] = g * kGranule + i;
-        lim_o[off] = lv[i];
-        ++off;
+    if (tile == Tk - 1) {
+      // the ends of the lists: totals, padding (A is read in whole tiles, a tile of B may start at any entry), and
+      // the region tiles that begin behind every limit in B
+      const int n_a = base_a + __builtin_popcountll(bits_a), n_b = base_b + __builtin_popcountll(bits_b);
+      const int all_max = max(run_max, __shfl(incl, kWave - 1));
+      if (lane == 0) {
+        before_a[n_gran] = n_a;
+        before_b[n_gran] = n_b;
       }
+      for (int i = n_a + lane; i < (n_a + kTile - 1) / kTile * kTile; i += kWave) {
+        rows_a[i] = 0x7fffffff;
+        lims_a[i] = -1;
+      }
+      rows_b[n_b + lane] = 0x7fffffff;
+      lims_b[n_b + lane] = -1;
+      for (int t = (all_max < 0 ? 0 : all_max / kTile + 1) + lane; t < n_rtile; t += kWave) alive[t] = n_b;
     }
-    __syncthreads();
-    if (tid == 0) carry += total;
-    __syncthreads();
-  }
-  const int total = carry;
-  if (tid == 0) before_o[n_gran] = total;
-  const int n_tiles = (total + kTile - 1) / kTile + 1;  // (one tile of padding: a reader may run one tile ahead)
-  for (int i = total + tid; i < n_tiles * kTile; i += kLongThreads) {
-    rows_o[i] = 0x7fffffff;
-    lim_o[i] = -1;
-  }
-  // least limit of every 64 entries (the entries were written by other threads of this workgroup: they are read
-  // past the first-level cache, after a fence and a barrier)
-  __threadfence();
-  __syncthreads();
-  int32_t* tmin_o = long_tmin + (int64_t)ks * (long_cap / kTile);
-  for (int t = wave; t < n_tiles; t += kLongThreads / kWave) {
-    int m = __hip_atomic_load(lim_o + t * kTile + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-#pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) m = min(m, __shfl_xor(m, o));
-    if (lane == 0) tmin_o[t] = m;
   }
 }
 
-int launch_long_rows(const PrefillWorkspace& w, int64_t n_streams, int64_t N, int64_t base, int64_t t_long, hipStream_t st) {
-  NATS_REQUIRE(n_streams <= 0x7fffffff, NATS_ERR_BAD_SHAPE, "long_rows_kernel: %lld streams", (long long)n_streams);
-  hipLaunchKernelGGL(long_rows_kernel, dim3((unsigned)n_streams), dim3(kLongThreads), 0, st, w.tok_lim, (int)N, (int)base,
-                     (int)t_long, (int)w.n_gran, (int)w.long_cap, w.long_rows, w.long_lim, w.long_before, w.long_tmin);
+int launch_long_rows(const PrefillWorkspace& w, int64_t n_streams, int64_t N, int64_t base, int64_t W, hipStream_t st) {
+  NATS_REQUIRE(n_streams <= 65535, NATS_ERR_BAD_SHAPE, "long_rows_kernel: %lld streams", (long long)n_streams);
+  const int64_t Tk = (N + kTile - 1) / kTile;
+  dim3 grid((unsigned)((Tk + kLongWaves - 1) / kLongWaves), (unsigned)n_streams);
+  // (the threshold is the one the key-limit kernel counted the tiles' rows with)
+  hipLaunchKernelGGL(long_rows_kernel, grid, dim3(kLongWaves * kWave), 0, st, w.tok_lim, w.tile_long, (int)N, (int)Tk,
+                     (int)base, (int)long_row_threshold(W), (int)w.n_gran, (int)w.long_cap, (int)w.n_rtile, w.long_rows, w.long_lim,
+                     w.long_before, w.long_alive);
   NATS_CHECK_LAUNCH("long_rows_kernel");
   return NATS_OK;
 }
@@ -433,6 +531,8 @@ int prepare_key_limits(const uint8_t* roles, int64_t B, int64_t H_kv, int64_t S,
   a.tile_lim = w.tile_lim;
   a.gran_lim = w.gran_lim;
   a.ticket = w.ticket;
+  a.tile_long = w.tile_long;
+  a.t_long = (int)long_row_threshold(W);
   a.Hkv = (int)H_kv; a.S = (int)S; a.N = (int)N; a.Tk = (int)((N + kTile - 1) / kTile);
   a.c_shift = ilog2(C); a.C = (int)C; a.W = (int)W;
   if (past) {
