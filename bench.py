@@ -391,7 +391,7 @@ def bench_segments(args, ops):
     def run(count: bool = False):
         cache.reset_cache()
         for i, (qs, ks, vs, rs, ts) in enumerate(parts):
-            kc, vc = cache.update(ks, vs, ts)
+            kc, vc = cache.update(ks, vs, ts, roles=rs)  # (roles and one-hot as the role kernel hands them over together)
             if i == 0:
                 ops.prefill_attention(qs, kc, vc, rs, C, W)
             else:

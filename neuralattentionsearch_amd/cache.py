@@ -314,8 +314,9 @@ class NAtSChunkLayerCache:
             def widen(t, fill):
                 shape = list(t.shape)
                 shape[2] = new_cap
-                n = torch.full(shape, fill, dtype=t.dtype, device=t.device)
+                n = torch.empty(shape, dtype=t.dtype, device=t.device)
                 n[:, :, :cap] = t
+                n[:, :, cap:].fill_(fill)
                 return n
 
             self._buf_k = widen(self._buf_k, 0)
