@@ -121,7 +121,9 @@ int nats_prefill_tile_map(const uint8_t* roles, int64_t B, int64_t H_kv, int64_t
  *   roles [B, H_kv, S] uint8, S = ceil(L / C)
  *   workspace: nats_prefill_workspace_bytes(...) bytes of device memory (contents need not be kept).  It belongs to
  *   the call until its kernels have run: besides the per-key limits it holds the counter from which a large launch
- *   deals its lightest query groups, so two calls that may overlap on the device need a workspace each.
+ *   deals its lightest query groups and, for chunks shorter than 16 tokens, the lists of the rows that stay visible
+ *   for more than a window (those rows are gathered row by row instead of walked in 16-row granules), so two calls
+ *   that may overlap on the device need a workspace each.
  * D in {16, 32, 64, 128, 256} (the head dims of nats_flashattn_fwd.py:634); C a power of two; W % C == 0;
  * H_q % H_kv == 0.
  * dtype bf16 with D 64 or 128 runs QK^T and PV on bf16 MFMA with fp32 softmax state; dtype f32, and bf16 at the
