@@ -424,10 +424,9 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
                                        (uint32_t __attribute__((address_space(3)))*)(dst + inst * kWave * 8), 16, 0, 0);
     }
   };
-  auto granule_of = [&](int id0, int id1, int id2, int id3, int which) {
-    return which == 0 ? (id0 & ~kPackedMaskFlag) : which == 1 ? id1 : which == 2 ? id2 : id3;
-  };
-  auto issue_k_p = [&](int id0, int id1, int id2, int id3, int buf, int slot) {
+  // (id0: the first field of the list entry, with its flags; mine: this wavefront's granule of the tile, or the first
+  // list entry of a gathered tile; idx: the entry's place in the list)
+  auto issue_k_p = [&](int id0, int mine, int idx, int buf, int slot) {
     if (id0 & kFarTileFlag) {
       issue_rows_far(kp, a.ks_l, sm.k[buf], slot, false);
       if ((id0 & kPackedMaskFlag) && wave == 0) {
@@ -435,12 +434,12 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
 #if defined(__HIP_DEVICE_COMPILE__)
         asm volatile("" : "+v"(ln));
 #endif
-        __builtin_amdgcn_global_load_lds(llim + id1 + ln,
+        __builtin_amdgcn_global_load_lds(llim + mine + ln,
                                          (uint32_t __attribute__((address_space(3)))*)(&sm.limk[slot][0]), 4, 0, 0);
       }
       return;
     }
-    issue_rows_p(kp, a.ks_l, koff, sm.k[buf], granule_of(id0, id1, id2, id3, wave >> 1), false);
+    issue_rows_p(kp, a.ks_l, koff, sm.k[buf], mine, false);
     if ((id0 & kPackedMaskFlag) && wave == 0) {
       // limits and region tokens of the 64 rows, for the element mask (asynchronous like the tile itself).
       // (The lane id is taken afresh so that nothing derived from it has to live across the tile loop.)
@@ -448,7 +447,8 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
 #if defined(__HIP_DEVICE_COMPILE__)
       asm volatile("" : "+v"(ln));
 #endif
-      const int gid = granule_of(id0, id1, id2, id3, ln >> 4);
+      int gid = reinterpret_cast<const int*>(&sm.vlist[idx])[ln >> 4];
+      if ((ln >> 4) == 0) gid &= ~kPackedMaskFlag;
       const int row = gid * kGranule + (ln & (kGranule - 1));
       const bool real = gid >= 0 && row < a.N;
       const int32_t* src = real ? lim + row : a.tok_lim + (int64_t)a.B * a.Hkv * a.N;  // (the entry that holds -1)
@@ -456,12 +456,12 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
       sm.posk[slot][ln] = real ? row - a.base : 0x7fffffff;
     }
   };
-  auto issue_v_p = [&](int id0, int id1, int id2, int id3, int buf, int slot) {
+  auto issue_v_p = [&](int id0, int mine, int buf, int slot) {
     if (id0 & kFarTileFlag) {
       issue_rows_far(vp, a.vs_l, sm.v[buf], slot, true);
       return;
     }
-    issue_rows_p(vp, a.vs_l, voff, sm.v[buf], granule_of(id0, id1, id2, id3, wave >> 1), true);
+    issue_rows_p(vp, a.vs_l, voff, sm.v[buf], mine, true);
   };
 
   auto k_frag = [&](const uint16_t* Kt, int kb, int s) {
@@ -821,24 +821,33 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
       // One step handles two tiles of the list (2s, 2s + 1) between two workgroup barriers.  At its start the
       // K tiles 2s + 1, 2s + 2 and the V tiles 2s, 2s + 1 are in LDS and the scores of tile 2s in registers; the
       // step puts K tiles 2s + 3, 2s + 4 and V tiles 2s + 2, 2s + 3 in flight.
-      // (packed tiles: kt, emax, emin, e3 are the four granule ids, kt with the mask flag)
+      // (packed tiles: kt is the entry's first field with its flags, emax this wavefront's granule of the tile -- or
+      // the first list entry of a gathered tile -- and emin the entry's place in the list)
       struct Entry {
-        int kt, emax, emin, e3;
+        int kt, emax, emin;
       };
       auto read_entry = [&](int j) {
-        Entry r = {0, 0, 0, 0};
+        Entry r = {0, 0, 0};
         if (j < n_vis) {
-          int kt, emax, emin;
-          entry(j, kt, emax, emin);
-          r.kt = kt; r.emax = emax; r.emin = emin;
-          if (kPacked) r.e3 = __builtin_amdgcn_readfirstlane(sm.vlist[j0 + j].w);
+          if (kPacked) {
+            const int* ep = reinterpret_cast<const int*>(&sm.vlist[j0 + j]);
+            r.kt = __builtin_amdgcn_readfirstlane(ep[0]);
+            const int sel = (r.kt & kFarTileFlag) ? 1 : wave >> 1;
+            const int mine = __builtin_amdgcn_readfirstlane(ep[sel]);
+            r.emax = sel == 0 ? mine & ~kPackedMaskFlag : mine;
+            r.emin = j0 + j;
+          } else {
+            int kt, emax, emin;
+            entry(j, kt, emax, emin);
+            r.kt = kt; r.emax = emax; r.emin = emin;
+          }
         }
         return r;
       };
       auto load_k = [&](int j, const Entry& e) {
         if (j < n_vis) {
           if (kPacked) {
-            issue_k_p(e.kt, e.emax, e.emin, e.e3, j & 3, j & 7);
+            issue_k_p(e.kt, e.emax, e.emin, j & 3, j & 7);
           } else {
             issue_k(e.kt, j & 3, j & 7, group_needs_lim(e.kt, e.emin));
           }
@@ -847,7 +856,7 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
       auto load_v = [&](int j, const Entry& e) {
         if (j < n_vis) {
           if (kPacked) {
-            issue_v_p(e.kt, e.emax, e.emin, e.e3, j & 3, j & 7);
+            issue_v_p(e.kt, e.emax, j & 3, j & 7);
           } else {
             issue_v(e.kt, j & 3);
           }
