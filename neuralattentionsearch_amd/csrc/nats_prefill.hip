@@ -749,17 +749,35 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
       const int2* gl = a.gran_lim + (int64_t)ks * a.Tk * kGranPerTile;
       const int g_hi = min(w0 + kWinStep - 1, g_end_group);
       int n_plain = 0, n_mask = 0;
-      for (int gb = w0; gb <= g_hi; gb += 16 * kWave) {
-        int2 vals[16];
+      // first the 64-row tiles that somebody in the group sees (one summary per tile), then only their granules
+      int* cand = reinterpret_cast<int*>(&sm.k[1][0]);
+      const int t_lo = w0 / kGranPerTile, t_hi = g_hi / kGranPerTile;
+      int n_c = 0;
+      for (int tb = t_lo; tb <= t_hi; tb += 8 * kWave) {
+        int mx[8];
 #pragma unroll
-        for (int u = 0; u < 16; ++u) {
-          const int g = gb + u * kWave + lane;
-          vals[u] = g <= g_hi ? gl[g] : make_int2(-1, -1);
+        for (int u = 0; u < 8; ++u) {
+          const int t = tb + u * kWave + lane;
+          mx[u] = t <= t_hi ? tl[t].x : -1;
         }
 #pragma unroll
-        for (int u = 0; u < 16; ++u) {
-          const int g = gb + u * kWave + lane;
-          const bool vis = g <= g_hi && vals[u].x >= r0_group;
+        for (int u = 0; u < 8; ++u) {
+          const bool vis = mx[u] >= r0_group && tb + u * kWave + lane <= t_hi;
+          const uint64_t bv = __ballot(vis);
+          if (vis) cand[n_c + __builtin_popcountll(bv & ((uint64_t(1) << lane) - 1))] = tb + u * kWave + lane;
+          n_c += __builtin_popcountll(bv);
+        }
+      }
+      wave_lds_sync();
+      for (int cb = 0; cb < n_c; cb += kWave) {
+        const int t = cb + lane < n_c ? cand[cb + lane] : -1;
+        int2 vals[kGranPerTile];
+#pragma unroll
+        for (int u = 0; u < kGranPerTile; ++u) vals[u] = t >= 0 ? gl[t * kGranPerTile + u] : make_int2(-1, -1);
+#pragma unroll
+        for (int u = 0; u < kGranPerTile; ++u) {
+          const int g = t * kGranPerTile + u;
+          const bool vis = t >= 0 && g >= w0 && g <= g_hi && vals[u].x >= r0_group;
           const int last_pos = g * kGranule + kGranule - 1 - a.base;
           const bool plain = vis && vals[u].y >= rlast_group && last_pos <= r0_group && (g + 1) * kGranule <= a.N;
           const bool masked = vis && !plain;
