@@ -240,9 +240,13 @@ constexpr int kFarTileFlag = 1 << 29;     // ... the entry is a tile of long-liv
 // the workgroup sees without a mask are packed among themselves and the rest (diagonal, partly visible, the remainder of the
 // first kind, padding) into tiles that go through the element mask.  The softmax does not care about the order
 // of the keys, so nothing else changes; without it a tile with one visible 16- or 32-row chunk costs a whole tile.
-template <int D, bool kUniform, bool kPacked>
+// (kMode: 0 whole tiles, 1 packed tiles, 2 packed tiles with the rows far behind a query gathered from the lists of
+// long-lived rows)
+template <int D, bool kUniform, int kMode>
 __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned char* smem_raw, int bid, int split, int ks,
                                                   int hg, int rank) {
+  constexpr bool kPacked = kMode != 0;
+  constexpr bool kFar = kMode == 2;
   static_assert(!kPacked || kUniform, "packed tiles are walked by every wavefront of the workgroup");
   constexpr int OCT = D / 8;                          // 16-byte chunks per row
   constexpr int DMA_PER_WAVE = OCT / kPrefillWaves;   // 1 KiB global->LDS transfers per wavefront and tensor
@@ -289,7 +293,7 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
   // Rows more than t_long tokens behind the group's first query: only the stream's long-lived rows can be visible
   // there (long_rows_kernel).  Below near_row0, the row from which the group walks granule by granule, lie the first
   // n_far_a entries of list A and the first b_hi of list B, of which those before b_lo are seen by nobody here.
-  const bool far_mode = kPacked && a.long_rows != nullptr;
+  const bool far_mode = kFar;
   int near_row0 = 0, n_far_a = 0, b_lo = 0, b_hi = 0;
   const int32_t* lrows = nullptr;
   const int32_t* llim = nullptr;
@@ -427,7 +431,7 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
   // (id0: the first field of the list entry, with its flags; mine: this wavefront's granule of the tile, or the first
   // list entry of a gathered tile; idx: the entry's place in the list)
   auto issue_k_p = [&](int id0, int mine, int idx, int buf, int slot) {
-    if (id0 & kFarTileFlag) {
+    if (kFar && (id0 & kFarTileFlag)) {
       issue_rows_far(kp, a.ks_l, sm.k[buf], slot, false);
       if ((id0 & kPackedMaskFlag) && wave == 0) {
         int ln = lane;
@@ -457,7 +461,7 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
     }
   };
   auto issue_v_p = [&](int id0, int mine, int buf, int slot) {
-    if (id0 & kFarTileFlag) {
+    if (kFar && (id0 & kFarTileFlag)) {
       issue_rows_far(vp, a.vs_l, sm.v[buf], slot, true);
       return;
     }
@@ -725,7 +729,7 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
   bool far_win = far_mode && n_far_tiles > 0;  // windows of gathered tiles come first, then the granule walk
   for (int w0 = far_mode ? near_row0 / kGranule : 0; w0 <= win_last;) {
     // ---- visit list of this window: wavefront 0 compacts the tiles some query tile of the group sees ----
-    if (kPacked && far_win && wave == 0) {
+    if (kFar && far_win && wave == 0) {
       // gathered tiles [f0, f0 + count): whole tiles of list A need no mask (every query sees their rows, and they
       // lie below near_row0); the last one of A and the tiles of B go through it
       const int cnt = min(kWin - 1, n_far_tiles - f0);
@@ -850,7 +854,7 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
           if (kPacked) {
             const int* ep = reinterpret_cast<const int*>(&sm.vlist[j0 + j]);
             r.kt = __builtin_amdgcn_readfirstlane(ep[0]);
-            const int sel = (r.kt & kFarTileFlag) ? 1 : wave >> 1;
+            const int sel = (kFar && (r.kt & kFarTileFlag)) ? 1 : wave >> 1;
             const int mine = __builtin_amdgcn_readfirstlane(ep[sel]);
             r.emax = sel == 0 ? mine & ~kPackedMaskFlag : mine;
             r.emin = j0 + j;
@@ -893,7 +897,7 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
                                     : (ec.kt * kTile + kTile - 1 - a.base <= my_r0 && ec.emin >= my_rlast);
           if (!full) {
             if (kPacked) {
-              mask_scores_p(t & 7, sv, (ec.kt & kFarTileFlag) != 0);
+              mask_scores_p(t & 7, sv, kFar && (ec.kt & kFarTileFlag) != 0);
             } else {
               mask_scores(ec.kt, t & 7, sv);
             }
@@ -915,7 +919,7 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
       // gathered tiles: the cache rows of tile j of the window go to posk[j & 7] a step before its K rows are
       // requested (asynchronous; the step's wait and barrier make them visible to every wavefront)
       auto load_ids = [&](int j) {
-        if (kPacked && far_win && j < n_vis && wave == 0) {
+        if (kFar && far_win && j < n_vis && wave == 0) {
           int ln = lane;
 #if defined(__HIP_DEVICE_COMPILE__)
           asm volatile("" : "+v"(ln));
@@ -925,7 +929,7 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
                                            (uint32_t __attribute__((address_space(3)))*)(&sm.posk[j & 7][0]), 4, 0, 0);
         }
       };
-      if (kPacked && far_win) {
+      if (kFar && far_win) {
 #pragma unroll
         for (int j = 0; j < 5; ++j) load_ids(j);
         __builtin_amdgcn_s_waitcnt(0);
@@ -1031,7 +1035,7 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
 // their roles keep visible, and the XCDs of one device differ in speed by a few percent): those that get to the pool
 // earlier take more of it.  The tile loop exists twice in the code, once for each kind of workgroup, so that the
 // loop around the pooled one costs the other nothing.
-template <int D, bool kUniform, bool kPacked = false>
+template <int D, bool kUniform, int kMode = 0>
 __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(PrefillArgs args) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   int bid = blockIdx.x;
@@ -1043,7 +1047,7 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
   if (args.pool_ranks == 0 || bid < (args.n_qg - args.pool_ranks) * args.B * args.Hkv * args.n_hg) {
     int ks, hg, rank;
     map_workgroup(args, bid, ks, hg, rank);
-    prefill_mfma_item<D, kUniform, kPacked>(args, smem_raw, bid, split, ks, hg, rank);
+    prefill_mfma_item<D, kUniform, kMode>(args, smem_raw, bid, split, ks, hg, rank);
     return;
   }
   // Pooled query groups wait in one queue per XCD (that of their stream, heaviest first; every counter in a 128-byte
@@ -1093,7 +1097,7 @@ __global__ __launch_bounds__(kPrefillWaves * kWave) void prefill_mfma_kernel(Pre
     q = q_now;
     const int sl = t % n_x;
     const int ks = a.xcd_mode ? q + 8 * (sl / a.n_hg) : sl / a.n_hg;
-    prefill_mfma_item<D, kUniform, kPacked>(a, smem_raw, bid, split, ks, sl % a.n_hg, a.n_qg - a.pool_ranks + t / n_x);
+    prefill_mfma_item<D, kUniform, kMode>(a, smem_raw, bid, split, ks, sl % a.n_hg, a.n_qg - a.pool_ranks + t / n_x);
     __syncthreads();  // the output staging of this item and the ticket are read before the next item writes LDS
   }
 }
@@ -1157,19 +1161,19 @@ __global__ __launch_bounds__(256) void prefill_split_merge_kernel(PrefillArgs a)
   }
 }
 
-template <int D, bool kUniform, bool kPacked = false>
+template <int D, bool kUniform, int kMode = 0>
 static int launch_prefill_mfma(const PrefillArgs& a, int64_t n_wg, hipStream_t st) {
   static bool configured[kMaxDevices] = {};  // per instantiation; the attribute is set once per device
   const size_t smem = sizeof(PrefillSmem<D>);
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail(NATS_ERR_LAUNCH, "prefill: no current device");
   if (!configured[dev]) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_mfma_kernel<D, kUniform, kPacked>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_mfma_kernel<D, kUniform, kMode>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return fail(NATS_ERR_LAUNCH, "hipFuncSetAttribute(%zu bytes of LDS): %s", smem, hipGetErrorString(e));
     configured[dev] = true;
   }
-  hipLaunchKernelGGL((prefill_mfma_kernel<D, kUniform, kPacked>), dim3((unsigned)n_wg), dim3(kPrefillWaves * kWave), smem, st, a);
+  hipLaunchKernelGGL((prefill_mfma_kernel<D, kUniform, kMode>), dim3((unsigned)n_wg), dim3(kPrefillWaves * kWave), smem, st, a);
   NATS_CHECK_LAUNCH("prefill_mfma_kernel");
   return NATS_OK;
 }
@@ -1330,6 +1334,11 @@ int launch_segment(const char* who, const SegmentShape& g, const void* q, const 
     a.long_rows = w.long_rows; a.long_lim = w.long_lim; a.long_before = w.long_before; a.long_alive = w.long_alive;
     a.long_cap = (int)w.long_cap; a.n_gran = (int)w.n_gran; a.n_rtile = (int)w.n_rtile;
   }
+  auto launch_packed = [&](const PrefillArgs& pa, int64_t n) {
+    if (pa.long_rows)
+      return g.D == 64 ? launch_prefill_mfma<64, true, 2>(pa, n, st) : launch_prefill_mfma<128, true, 2>(pa, n, st);
+    return g.D == 64 ? launch_prefill_mfma<64, true, 1>(pa, n, st) : launch_prefill_mfma<128, true, 1>(pa, n, st);
+  };
   a.n_split = 1;
   if (hpw == 4 || packed) {  // the kernels in which every wavefront walks the whole tile list
     const int ns = choose_split(n_wg, a.Tk);
@@ -1343,7 +1352,7 @@ int launch_segment(const char* who, const SegmentShape& g, const void* q, const 
     const int64_t n_launch = n_wg * a.n_split;
     int rc;
     if (packed) {
-      rc = g.D == 64 ? launch_prefill_mfma<64, true, true>(a, n_launch, st) : launch_prefill_mfma<128, true, true>(a, n_launch, st);
+      rc = launch_packed(a, n_launch);
     } else {
       rc = g.D == 64 ? launch_prefill_mfma<64, true>(a, n_launch, st) : launch_prefill_mfma<128, true>(a, n_launch, st);
     }
@@ -1378,7 +1387,7 @@ int launch_segment(const char* who, const SegmentShape& g, const void* q, const 
   // (GQA groups of 1 and 2: the workgroup's 2 or 4 query tiles form one group for the packing, every wavefront
   // walks the whole list and the element mask sorts out what its own rows see)
   if (packed)
-    return g.D == 64 ? launch_prefill_mfma<64, true, true>(a, n_wg, st) : launch_prefill_mfma<128, true, true>(a, n_wg, st);
+    return launch_packed(a, n_wg);
   if (hpw == 4) return g.D == 64 ? launch_prefill_mfma<64, true>(a, n_wg, st) : launch_prefill_mfma<128, true>(a, n_wg, st);
   return g.D == 64 ? launch_prefill_mfma<64, false>(a, n_wg, st) : launch_prefill_mfma<128, false>(a, n_wg, st);
 }
