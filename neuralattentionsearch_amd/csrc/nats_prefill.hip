@@ -729,10 +729,20 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
   bool far_win = far_mode && n_far_tiles > 0;  // windows of gathered tiles come first, then the granule walk
   for (int w0 = far_mode ? near_row0 / kGranule : 0; w0 <= win_last;) {
     // ---- visit list of this window: wavefront 0 compacts the tiles some query tile of the group sees ----
+    // far_cnt gathered tiles at the head of the list; the granule walk joins the window that holds the last of them
+    // when its tiles fit behind (the usual case: one pass of the tile pipeline per workgroup)
+    int far_cnt = 0;
+    bool with_near = !far_win;
+    if (kFar && far_win) {
+      far_cnt = min(kWin - 1, n_far_tiles - f0);
+      const int n_near = g_end_group - w0 + 1;  // granules of the walk
+      with_near = f0 + far_cnt == n_far_tiles && n_near <= kWinStep &&
+                  far_cnt + (n_near + kGranPerTile - 1) / kGranPerTile + 1 <= kWin - 1;
+    }
     if (kFar && far_win && wave == 0) {
       // gathered tiles [f0, f0 + count): whole tiles of list A need no mask (every query sees their rows, and they
       // lie below near_row0); the last one of A and the tiles of B go through it
-      const int cnt = min(kWin - 1, n_far_tiles - f0);
+      const int cnt = far_cnt;
       for (int i = lane; i < cnt; i += kWave) {
         const int t = f0 + i;
         int4 d;
@@ -743,9 +753,9 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
         }
         sm.vlist[i] = d;
       }
-      if (lane == 0) sm.vcount = cnt;
+      if (lane == 0 && !with_near) sm.vcount = cnt;
     }
-    if (kPacked && !far_win && wave == 0) {
+    if (kPacked && with_near && wave == 0) {
       // granules seen without a mask and granules that need one, each kind in its own list (staged in the tile
       // buffers, which are idle here), then four ids per tile
       int* plain_ids = reinterpret_cast<int*>(&sm.k[0][0]);
@@ -812,9 +822,9 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
           d.z = o + 2 < n_mask ? mask_ids[o + 2] : -1;
           d.w = o + 3 < n_mask ? mask_ids[o + 3] : -1;
         }
-        sm.vlist[i] = d;
+        sm.vlist[far_cnt + i] = d;
       }
-      if (lane == 0) sm.vcount = n_pt + n_mt;
+      if (lane == 0) sm.vcount = far_cnt + n_pt + n_mt;
     }
     if (!kPacked && wave == 0 && w0 > 0) build_list(w0, false);
     __syncthreads();
@@ -919,7 +929,7 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
       // gathered tiles: the cache rows of tile j of the window go to posk[j & 7] a step before its K rows are
       // requested (asynchronous; the step's wait and barrier make them visible to every wavefront)
       auto load_ids = [&](int j) {
-        if (kFar && far_win && j < n_vis && wave == 0) {
+        if (kFar && j < n_vis && j0 + j < far_cnt && wave == 0) {
           int ln = lane;
 #if defined(__HIP_DEVICE_COMPILE__)
           asm volatile("" : "+v"(ln));
@@ -929,7 +939,7 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
                                            (uint32_t __attribute__((address_space(3)))*)(&sm.posk[j & 7][0]), 4, 0, 0);
         }
       };
-      if (kFar && far_win) {
+      if (kFar && j0 < far_cnt) {
 #pragma unroll
         for (int j = 0; j < 5; ++j) load_ids(j);
         __builtin_amdgcn_s_waitcnt(0);
@@ -960,15 +970,14 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
         __builtin_amdgcn_s_waitcnt(0);  // the tiles in flight have landed in LDS
         __syncthreads();                // ... for every wavefront, and the tiles of this step are no longer read
       }
-    } else if (far_win || w0 + kWinStep <= win_last) {
+    } else if (!with_near || w0 + kWinStep <= win_last) {
       __syncthreads();  // (nobody may still be reading this window's count when wavefront 0 starts the next list)
     }
     if (far_win) {
-      f0 += kWin - 1;
+      f0 += far_cnt;
       far_win = f0 < n_far_tiles;
-    } else {
-      w0 += kWinStep;
     }
+    if (with_near) w0 += kWinStep;
   }
 
   // ---- a share of the tile list: the unnormalised sums, the running maximum and the row sum leave as they are ----
