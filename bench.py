@@ -667,9 +667,10 @@ def main():
     if extras:
         # the chunk size of the reference's shipped Llama adapter (experiments/configs/finetune_distill.yaml:95) and a
         # role per token, same shape, window and role shares
-        few = max(5, args.steps // 5)
-        res["prefill_c32"] = bench_prefill(args, ops, chunk_size=32, steps=few, warmup=3, compare=False, settle=False)
-        res["prefill_c1"] = bench_prefill(args, ops, chunk_size=1, steps=few, warmup=3, compare=False, settle=False)
+        # (the clock is settled again before each: the set-up of a leg's inputs leaves the GPU idle for a while)
+        few = max(10, args.steps // 2)
+        res["prefill_c32"] = bench_prefill(args, ops, chunk_size=32, steps=few, warmup=10, compare=False)
+        res["prefill_c1"] = bench_prefill(args, ops, chunk_size=1, steps=few, warmup=10, compare=False)
     if args.only in (None, "decode"):
         res["decode"] = bench_decode(args, ops)
     if extras:
