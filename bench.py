@@ -142,9 +142,9 @@ def prefill_flops(roles: np.ndarray, L: int, C: int, W: int, D: int, n_rep: int)
 
 
 def time_gpu(fn, steps: int, warmup: int, settle_ms: float = 0.0):
-    """Time of `fn` on the current stream: W untimed calls (for a leg of a few microseconds per call `settle_ms` keeps
-    the untimed calls going for that long: after host-side set-up the GPU has dropped to its idle clock, and a few
-    hundred microseconds of warm-up do not bring it back), then exactly K calls between one pair of HIP events
+    """Time of `fn` on the current stream: W untimed calls (`settle_ms` keeps the untimed calls going for that long:
+    after the host-side set-up of a leg's inputs the GPU has dropped to its idle clock, and a few milliseconds of
+    warm-up do not always bring it back), then exactly K calls between one pair of HIP events
     (and one pair of synchronisations), so that the launches follow each other as they do in use.  Returns
     (host wall time per step, GPU time per step, best single step); the best step comes from a short extra loop
     with an event pair around every call, which costs each call about ten microseconds of markers and is
@@ -267,7 +267,7 @@ def bench_decode(args, ops, batch=None, context=None):
     bytes_alg = n_valid * D * 2 * 2 + 2 * q.numel() * 2
     wall, ev_mean, ev_min = time_gpu(
         lambda: ops.decode_attention(q, k, v, valid, n_rows, row_end=row_end, tail_start=tail_start),
-        args.steps * 5, args.warmup, settle_ms=60.0 if B < 8 else 0.0)
+        args.steps * 5, args.warmup, settle_ms=60.0)
     return {
         "ms": ev_mean, "ms_min": ev_min, "ms_wall": wall,
         "tokens_per_s_per_layer": B / (ev_mean * 1e-3),
@@ -309,7 +309,7 @@ def bench_evict(args, ops):
         evict_into(NAtSChunkLayerCache(B, Hkv, W, chunk_size=C, device=dev))
 
     steps = max(3, args.steps // 2)
-    wall, ev_mean, ev_min = time_gpu(warm_step, steps, 2)
+    wall, ev_mean, ev_min = time_gpu(warm_step, steps, 2, settle_ms=30.0)
     moved["rows"] = int(cache.last_evict_result.moved_rows)
     c_wall, c_mean, c_min = time_gpu(cold_step, steps, 2)
     ring_rows = B * Hkv * W
