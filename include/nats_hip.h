@@ -78,6 +78,8 @@ int nats_roles_from_logits(const void* logits, int dtype, int64_t B, int64_t S, 
  *   end_idx / vis_lim  [B, H_kv, S] as nats_role_scan, may be NULL
  * The pooled statistic and the logits are rounded to the dtype of x where the torch ops round them; logits
  * are accumulated in fp32 in an order of their own, so they agree with a library GEMM to rounding only.
+ * C must be a power of two here (NATS_ERR_UNSUPPORTED otherwise): the chunk mean is sum * (1 / C), which is torch's
+ * mean bit for bit only then.  The other entry points take any chunk size that divides the window.
  */
 int nats_role_step(const void* x, const void* carry_in, const void* weight, int dtype, int64_t B, int64_t L, int64_t dim,
                    int64_t H_kv, int64_t C, int64_t W, int64_t pre_fill, int merge_max, float global_bias,
@@ -124,7 +126,7 @@ int nats_prefill_tile_map(const uint8_t* roles, int64_t B, int64_t H_kv, int64_t
  *   deals its lightest query groups and, for chunks shorter than 16 tokens, the lists of the rows that stay visible
  *   for more than a window (those rows are gathered row by row instead of walked in 16-row granules), so two calls
  *   that may overlap on the device need a workspace each.
- * D in {16, 32, 64, 128, 256} (the head dims of nats_flashattn_fwd.py:634); C a power of two; W % C == 0;
+ * D in {16, 32, 64, 128, 256} (the head dims of nats_flashattn_fwd.py:634); C > 0; W % C == 0;
  * H_q % H_kv == 0.
  * dtype bf16 with D 64 or 128 runs QK^T and PV on bf16 MFMA with fp32 softmax state; dtype f32, and bf16 at the
  * other head dims, run an fp32 FMA kernel.

@@ -1240,7 +1240,7 @@ int check_common(const char* who, const SegmentShape& g, const int64_t* q_stride
                (long long)g.H_q, (long long)g.H_kv);
   NATS_REQUIRE(g.D == 16 || g.D == 32 || g.D == 64 || g.D == 128 || g.D == 256, NATS_ERR_UNSUPPORTED,
                "%s: head_dim %lld (supported: 16, 32, 64, 128, 256)", who, (long long)g.D);
-  NATS_REQUIRE(is_pow2(g.C), NATS_ERR_UNSUPPORTED, "%s: chunk size %lld is not a power of two", who, (long long)g.C);
+  NATS_REQUIRE(g.C > 0 && g.C < (int64_t(1) << 30), NATS_ERR_BAD_SHAPE, "%s: chunk size %lld", who, (long long)g.C);
   NATS_REQUIRE(g.W >= 0 && g.W % g.C == 0, NATS_ERR_BAD_SHAPE, "%s: window %lld is not a multiple of chunk size %lld", who,
                (long long)g.W, (long long)g.C);
   NATS_REQUIRE(dtype == NATS_DTYPE_BF16 || dtype == NATS_DTYPE_F32, NATS_ERR_BAD_DTYPE, "%s: dtype %d", who, dtype);
@@ -1458,7 +1458,7 @@ extern "C" int nats_prefill_past_fwd(const void* q, const void* cache_k, const v
                NATS_ERR_NULL_POINTER, "%s: NULL pointer argument", who);
   NATS_REQUIRE(q_strides && k_strides && v_strides && valid_strides && o_strides, NATS_ERR_NULL_POINTER,
                "%s: NULL stride array", who);
-  NATS_REQUIRE(is_pow2(C) && W >= 0 && W % C == 0, NATS_ERR_BAD_SHAPE, "%s: chunk size %lld, window %lld", who,
+  NATS_REQUIRE(C > 0 && W >= 0 && W % C == 0, NATS_ERR_BAD_SHAPE, "%s: chunk size %lld, window %lld", who,
                (long long)C, (long long)W);
   if (int rc = check_past_state(who, state, x_len, C, W)) return rc;
   const int64_t base = state->n_ctx_data - state->old_fill;

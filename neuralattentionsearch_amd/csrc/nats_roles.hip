@@ -169,11 +169,13 @@ __global__ __launch_bounds__(256) void key_lim_kernel(KeyLimArgs a) {
   // as global): the wavefront's rows span at most 64 consecutive slots, so one ballot over the 64 slots from its first
   // one answers most lanes, and the blocks that follow answer the rest with their first global slot.
   int32_t v_inline = 0;
+  // (x / C for x >= 0; a shift when the chunk size is a power of two)
+  auto slot_of = [&](int x) { return a.c_shift >= 0 ? x >> a.c_shift : x / a.C; };
   if (!kPast && a.roles) {
     const uint8_t* r = a.roles + (int64_t)stream * a.S;
     const bool in = row < a.N;
-    const int slot = in ? row >> a.c_shift : 0;
-    const int s0 = (tile * kTile) >> a.c_shift;  // slot of lane 0 (the tile starts inside N)
+    const int slot = in ? slot_of(row) : 0;
+    const int s0 = slot_of(tile * kTile);  // slot of lane 0 (the tile starts inside N)
     const uint8_t role = in ? r[slot] : uint8_t(NATS_ROLE_GLOBAL);
     const bool want = in && role == NATS_ROLE_LOCAL;
     int g = -1;
@@ -190,11 +192,11 @@ __global__ __launch_bounds__(256) void key_lim_kernel(KeyLimArgs a) {
         if (!__ballot(want && g < 0)) break;
       }
     }
-    v_inline = role == NATS_ROLE_GLOBAL ? kLimGlobal : role == NATS_ROLE_SW ? slot + (a.W >> a.c_shift) : g;
+    v_inline = role == NATS_ROLE_GLOBAL ? kLimGlobal : role == NATS_ROLE_SW ? slot + slot_of(a.W) : g;
   }
   if (row < a.N) {
     if (!kPast || row >= a.base) {
-      int32_t v = (!kPast && a.roles) ? v_inline : a.vis_lim[(int64_t)stream * a.S + ((row - a.base) >> a.c_shift)];
+      int32_t v = (!kPast && a.roles) ? v_inline : a.vis_lim[(int64_t)stream * a.S + slot_of(row - a.base)];
       int64_t t = (int64_t(v) + 1) * a.C - 1;
       lim = (v == kLimGlobal || t >= kLimGlobal) ? kLimGlobal : int32_t(t);
     } else {
@@ -228,7 +230,7 @@ __global__ __launch_bounds__(256) void key_lim_kernel(KeyLimArgs a) {
           }
         }
       } else if (row < a.W) {
-        const int s = row >> a.c_shift;
+        const int s = slot_of(row);
         if (!val) {
           lim = -1;
         } else if (a.seen >= a.W) {
@@ -534,7 +536,7 @@ int prepare_key_limits(const uint8_t* roles, int64_t B, int64_t H_kv, int64_t S,
   a.tile_long = w.tile_long;
   a.t_long = (int)long_row_threshold(W);
   a.Hkv = (int)H_kv; a.S = (int)S; a.N = (int)N; a.Tk = (int)((N + kTile - 1) / kTile);
-  a.c_shift = ilog2(C); a.C = (int)C; a.W = (int)W;
+  a.c_shift = is_pow2(C) ? ilog2(C) : -1; a.C = (int)C; a.W = (int)W;
   if (past) {
     a.valid = past->valid; a.valid_s_b = past->valid_s_b; a.valid_s_h = past->valid_s_h;
     a.size_global = past->size_global; a.size_local = past->size_local;
@@ -575,7 +577,7 @@ extern "C" int nats_roles_from_logits(const void* logits, int dtype, int64_t B, 
 }
 
 static int check_cw(const char* who, int64_t C, int64_t W) {
-  NATS_REQUIRE(is_pow2(C), NATS_ERR_UNSUPPORTED, "%s: chunk size %lld is not a power of two", who, (long long)C);
+  NATS_REQUIRE(C > 0 && C < (int64_t(1) << 30), NATS_ERR_BAD_SHAPE, "%s: chunk size %lld", who, (long long)C);
   NATS_REQUIRE(W >= 0 && W % C == 0, NATS_ERR_BAD_SHAPE, "%s: window %lld is not a multiple of chunk size %lld", who,
                (long long)W, (long long)C);
   return NATS_OK;

@@ -150,7 +150,8 @@ class NAtSLlamaAttention(nn.Module):
         self.v_proj = nn.Linear(cfg.hidden_size, self.num_key_value_heads * self.head_dim, bias=False)
         self.o_proj = nn.Linear(self.num_heads * self.head_dim, cfg.hidden_size, bias=False)
         self.proj_layer = nn.Linear(cfg.hidden_size, self.num_key_value_heads * 3, bias=False)  # :315-318
-        self.fused_role_step = cfg.fused_role_step
+        # (the fused role step takes chunk sizes that are a power of two; others go through the torch ops)
+        self.fused_role_step = cfg.fused_role_step and cfg.chunk_size & (cfg.chunk_size - 1) == 0
         self.qkv_weight = None
 
     def fuse(self):

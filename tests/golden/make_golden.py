@@ -99,6 +99,13 @@ def scenarios():
                     segs=[(24, "rand"), (9, "rand"), (1, "rand"), (1, "rand"), (13, "rand"), (3, "rand")]))
     out.append(dict(name="chunk1_first_lt_w", B=1, H=2, D=2, C=1, W=8, p=(0.15, 0.25, 0.6),
                     segs=[(3, "rand"), (4, "rand")] + [(1, "rand")] * 12 + [(10, "rand")]))
+    # chunk sizes that are no power of two (the class only asks for W % C == 0, :47)
+    out.append(dict(name="chunk3_prefill_decode_w6", B=2, H=2, D=2, C=3, W=6, p=mix, segs=[(20, "rand")] + [(1, "rand")] * 15))
+    out.append(dict(name="chunk6_multiseg_w12", B=2, H=3, D=2, C=6, W=12, p=mix,
+                    segs=[(40, "rand"), (13, "rand"), (1, "rand"), (1, "rand"), (22, "rand"), (6, "rand")]))
+    out.append(dict(name="chunk12_stream_w24", B=1, H=2, D=2, C=12, W=24, p=(0.15, 0.25, 0.6),
+                    segs=[(12, "rand")] * 8 + [(5, "rand"), (30, "rand")]))
+    out.append(dict(name="chunk3_first_lt_w12", B=1, H=2, D=2, C=3, W=12, p=mix, segs=[(4, "rand"), (5, "rand"), (20, "rand")]))
     return out
 
 

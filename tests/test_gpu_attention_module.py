@@ -20,12 +20,14 @@ def rope_tables(B, start, n, D, device):
     return emb.cos()[None].expand(B, -1, -1), emb.sin()[None].expand(B, -1, -1)
 
 
-@pytest.mark.parametrize("L,C,W,steps", [(100, 16, 32, 40), (64, 16, 32, 20), (5, 8, 16, 30), (1, 8, 16, 30)])
+@pytest.mark.parametrize("L,C,W,steps", [(100, 16, 32, 40), (64, 16, 32, 20), (5, 8, 16, 30), (1, 8, 16, 30),
+                                         (100, 12, 36, 40), (50, 3, 12, 20)])  # (chunk sizes that are no power of two)
 def test_module_prefill_and_decode(L, C, W, steps):
     run_module([L] + [1] * steps, C, W)
 
 
-@pytest.mark.parametrize("lens,C,W", [([70, 45, 1, 1, 33, 16, 1, 90], 16, 32), ([3, 9, 40, 1, 1, 1, 25], 8, 16)])
+@pytest.mark.parametrize("lens,C,W", [([70, 45, 1, 1, 33, 16, 1, 90], 16, 32), ([3, 9, 40, 1, 1, 1, 25], 8, 16),
+                                      ([70, 45, 1, 1, 33, 16, 1, 90], 6, 24)])
 def test_module_segments_over_a_filled_cache(lens, C, W):
     """Multi-token segments after the first one run the segment kernel over the evicted cache."""
     run_module(lens, C, W)

@@ -53,6 +53,16 @@ def test_bf16_shapes(L, C, W, D):
     run_case(2, 8, 2, L, D, C, W, torch.bfloat16, seed=L + C)
 
 
+@pytest.mark.parametrize("L,C,W,D,dtype", [(700, 3, 12, 128, torch.bfloat16), (900, 6, 24, 64, torch.bfloat16),
+                                           (1000, 12, 36, 128, torch.bfloat16), (1300, 24, 48, 128, torch.bfloat16),
+                                           (1500, 48, 96, 128, torch.bfloat16), (2000, 96, 192, 128, torch.bfloat16),
+                                           (500, 6, 12, 64, torch.float32), (700, 96, 96, 128, torch.float32)])
+def test_chunk_sizes_that_are_no_power_of_two(L, C, W, D, dtype):
+    """The reference's cache only asks for W % C == 0 (nats_chunk_layer_cache.py:47): chunks that straddle 16-row
+    granules and 64-row tiles.  The golden scenarios with chunk sizes 3, 6 and 12 cover the cache side."""
+    run_case(2, 8, 2, L, D, C, W, dtype, seed=L + C)
+
+
 @pytest.mark.parametrize("D", [16, 32, 256])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_other_head_dims(D, dtype):
