@@ -116,6 +116,9 @@ __global__ __launch_bounds__(256) void decode_split_mfma_kernel(DecodeArgs a) {
   constexpr int OCT = D / 8;         // 16-byte chunks per row
   constexpr int NDMA = kDecTile * OCT / kWave;  // 1 KiB transfers per V tile
   constexpr int DB = D / 16;         // 16-dim blocks of O^T
+  // V rows in LDS have their 16-byte chunks permuted so that the transposing reads of a half wavefront (four rows,
+  // 32 bytes of each) spread over the banks; rows of 64 bytes only have four chunks to permute
+  auto v_swz = [](int row) { return OCT >= 8 ? (row & 3) << 1 : (row >> 2) & 3; };
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   DecodeSmem<D, NREP>& sm = *reinterpret_cast<DecodeSmem<D, NREP>*>(smem_raw);
@@ -216,7 +219,7 @@ __global__ __launch_bounds__(256) void decode_split_mfma_kernel(DecodeArgs a) {
       const int q = j * kWave + lane;  // chunk slot in the LDS tile
       const int row = q / OCT, cpos = q % OCT;
       const int src_row = ((m >> row) & 1) ? row : fv;
-      const int chunk = cpos ^ ((row & 3) << 1);
+      const int chunk = cpos ^ v_swz(row);
       __builtin_amdgcn_global_load_lds(vp + (int64_t)(r0 + src_row) * a.ks_r + chunk * 8,
                                        (uint32_t __attribute__((address_space(3)))*)(&sm.v[wave][buf][j * kWave * 8]), 16, 0,
                                        kAuxStream);
@@ -330,8 +333,8 @@ __global__ __launch_bounds__(256) void decode_split_mfma_kernel(DecodeArgs a) {
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
           const int chunk0 = db * 2 + ((l16 & 3) >> 1);
-          const uint16_t* plo = Vt + row_lo * D + ((chunk0 ^ ((row_lo & 3) << 1)) * 8) + half * 4;
-          const uint16_t* phi = Vt + row_hi * D + ((chunk0 ^ ((row_hi & 3) << 1)) * 8) + half * 4;
+          const uint16_t* plo = Vt + row_lo * D + ((chunk0 ^ v_swz(row_lo)) * 8) + half * 4;
+          const uint16_t* phi = Vt + row_hi * D + ((chunk0 ^ v_swz(row_hi)) * 8) + half * 4;
           bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((bf16x4 __attribute__((address_space(3)))*)plo);
           bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((bf16x4 __attribute__((address_space(3)))*)phi);
           bf16x8 va = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
@@ -676,7 +679,7 @@ static int decode_fwd_impl(const void* q, const void* cache_k, const void* cache
                (long long)H_q, (long long)H_kv);
   NATS_REQUIRE(D == 16 || D == 32 || D == 64 || D == 128 || D == 256, NATS_ERR_UNSUPPORTED,
                "nats_decode_fwd: head_dim %lld (supported: 16, 32, 64, 128, 256)", (long long)D);
-  const bool mfma = dtype == NATS_DTYPE_BF16 && (D == 64 || D == 128);  // other bf16 head dims take the plain kernel
+  const bool mfma = dtype == NATS_DTYPE_BF16 && (D == 32 || D == 64 || D == 128);  // other bf16 head dims take the plain kernel
   NATS_REQUIRE(dtype == NATS_DTYPE_BF16 || dtype == NATS_DTYPE_F32, NATS_ERR_BAD_DTYPE, "nats_decode_fwd: dtype %d", dtype);
   NATS_REQUIRE(n_rows < (int64_t(1) << 30) && B * H_q <= (int64_t(1) << 30), NATS_ERR_BAD_SHAPE,
                "nats_decode_fwd: problem too large");
@@ -779,6 +782,13 @@ static int decode_fwd_impl(const void* q, const void* cache_k, const void* cache
         case 4: rc = launch_mfma<128, 4>(c, groups, st); break;
         case 2: rc = launch_mfma<128, 2>(c, groups, st); break;
         default: rc = launch_mfma<128, 1>(c, groups, st); break;
+      }
+    } else if (D == 32) {
+      switch (nrep_k) {
+        case 8: rc = launch_mfma<32, 8>(c, groups, st); break;
+        case 4: rc = launch_mfma<32, 4>(c, groups, st); break;
+        case 2: rc = launch_mfma<32, 2>(c, groups, st); break;
+        default: rc = launch_mfma<32, 1>(c, groups, st); break;
       }
     } else {
       switch (nrep_k) {

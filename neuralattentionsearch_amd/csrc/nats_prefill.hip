@@ -249,11 +249,15 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
   constexpr bool kFar = kMode == 2;
   static_assert(!kPacked || kUniform, "packed tiles are walked by every wavefront of the workgroup");
   constexpr int OCT = D / 8;                          // 16-byte chunks per row
-  constexpr int DMA_PER_WAVE = OCT / kPrefillWaves;   // 1 KiB global->LDS transfers per wavefront and tensor
+  constexpr int N_INST = kTile * OCT / kWave;         // 1 KiB global->LDS transfers per tile
+  constexpr int DMA_PER_WAVE = (N_INST + kPrefillWaves - 1) / kPrefillWaves;  // ... per wavefront and tensor (with rows
+                                                      // of 64 bytes a tile is four transfers: wavefronts 0-3 issue one each)
   constexpr int DSTEPS = D / 16;
   constexpr int DT = D / 32;
   constexpr int kHalf = kTile / 2;
-  static_assert(DMA_PER_WAVE >= 1, "tile rows are split over the wavefronts in 1 KiB transfers");
+  static_assert(DMA_PER_WAVE >= 1 && N_INST % DMA_PER_WAVE == 0, "tile rows are split over the wavefronts in 1 KiB transfers");
+  // first tile row of this wavefront's transfers -> its granule of a packed tile
+  constexpr int kRowsPerInst = kWave / OCT;
 
   PrefillSmem<D>& sm = *reinterpret_cast<PrefillSmem<D>*>(smem_raw);
 
@@ -344,7 +348,8 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
   // of each row).  The 16-byte chunks of a row are permuted so that these four pieces fall into the four quarters of
   // the 64 LDS banks: rows of 256 bytes (one row = all banks) move by a quarter per row, rows of 128 bytes (two rows
   // = all banks) by a quarter per pair of rows.
-  auto v_swizzle = [](int row) { return OCT >= 16 ? (row & 3) << 2 : ((row >> 1) & 1) << 2; };
+  // (rows of 64 bytes: four rows = all banks and the four pieces of a read are one contiguous 256 bytes)
+  auto v_swizzle = [](int row) { return OCT >= 16 ? (row & 3) << 2 : OCT >= 8 ? ((row >> 1) & 1) << 2 : 0; };
   // global -> LDS, one 64-key tile of K or of V; rows beyond N repeat row N-1 (their scores are masked,
   // so their probabilities are exactly 0 and a finite V row contributes nothing).  The lane's share of a
   // tile sits at fixed offsets from the tile's first row, computed once.
@@ -365,7 +370,8 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
 #pragma unroll
       for (int j = 0; j < DMA_PER_WAVE; ++j) {
         const int inst = wave * DMA_PER_WAVE + j;
-        __builtin_amdgcn_global_load_lds(tb + (int)off[j], (uint32_t __attribute__((address_space(3)))*)(dst + inst * kWave * 8), 16, 0, 0);
+        if (inst < N_INST)
+          __builtin_amdgcn_global_load_lds(tb + (int)off[j], (uint32_t __attribute__((address_space(3)))*)(dst + inst * kWave * 8), 16, 0, 0);
       }
     } else {
 #pragma unroll
@@ -375,8 +381,9 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
         const int row = q / OCT, pos = q % OCT;
         const int n = min(kt * kTile + row, a.N - 1);
         const int chunk = is_v ? pos ^ v_swizzle(row) : pos ^ (row % OCT);
-        __builtin_amdgcn_global_load_lds(base + (int64_t)n * stride + chunk * 8,
-                                         (uint32_t __attribute__((address_space(3)))*)(dst + inst * kWave * 8), 16, 0, 0);
+        if (inst < N_INST)
+          __builtin_amdgcn_global_load_lds(base + (int64_t)n * stride + chunk * 8,
+                                           (uint32_t __attribute__((address_space(3)))*)(dst + inst * kWave * 8), 16, 0, 0);
       }
     }
   };
@@ -400,7 +407,8 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
 #pragma unroll
       for (int j = 0; j < DMA_PER_WAVE; ++j) {
         const int inst = wave * DMA_PER_WAVE + j;
-        __builtin_amdgcn_global_load_lds(tb + (int)off[j], (uint32_t __attribute__((address_space(3)))*)(dst + inst * kWave * 8), 16, 0, 0);
+        if (inst < N_INST)
+          __builtin_amdgcn_global_load_lds(tb + (int)off[j], (uint32_t __attribute__((address_space(3)))*)(dst + inst * kWave * 8), 16, 0, 0);
       }
     } else {
 #pragma unroll
@@ -410,8 +418,9 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
         const int row = q / OCT, pos = q % OCT;
         const int n = min(gid * kGranule + row % kGranule, a.N - 1);
         const int chunk = is_v ? pos ^ v_swizzle(row) : pos ^ (row % OCT);
-        __builtin_amdgcn_global_load_lds(base + (int64_t)n * stride + chunk * 8,
-                                         (uint32_t __attribute__((address_space(3)))*)(dst + inst * kWave * 8), 16, 0, 0);
+        if (inst < N_INST)
+          __builtin_amdgcn_global_load_lds(base + (int64_t)n * stride + chunk * 8,
+                                           (uint32_t __attribute__((address_space(3)))*)(dst + inst * kWave * 8), 16, 0, 0);
       }
     }
   };
@@ -422,10 +431,11 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
       const int inst = wave * DMA_PER_WAVE + j;  // uniform
       const int q = inst * kWave + lane;
       const int row = q / OCT, pos = q % OCT;
-      const int n = max(0, min(sm.posk[slot][row], a.N - 1));  // (padding entries hold INT_MAX and the limit -1)
+      const int n = max(0, min(sm.posk[slot][row & (kTile - 1)], a.N - 1));  // (padding entries hold INT_MAX and the limit -1)
       const int chunk = is_v ? pos ^ v_swizzle(row) : pos ^ (row % OCT);
-      __builtin_amdgcn_global_load_lds(base + (int64_t)n * stride + chunk * 8,
-                                       (uint32_t __attribute__((address_space(3)))*)(dst + inst * kWave * 8), 16, 0, 0);
+      if (inst < N_INST)
+        __builtin_amdgcn_global_load_lds(base + (int64_t)n * stride + chunk * 8,
+                                         (uint32_t __attribute__((address_space(3)))*)(dst + inst * kWave * 8), 16, 0, 0);
     }
   };
   // (id0: the first field of the list entry, with its flags; mine: this wavefront's granule of the tile, or the first
@@ -864,7 +874,10 @@ __device__ __forceinline__ void prefill_mfma_item(const PrefillArgs& a, unsigned
           if (kPacked) {
             const int* ep = reinterpret_cast<const int*>(&sm.vlist[j0 + j]);
             r.kt = __builtin_amdgcn_readfirstlane(ep[0]);
-            const int sel = (kFar && (r.kt & kFarTileFlag)) ? 1 : wave >> 1;
+            // (this wavefront's granule: the one its first transferred row lies in; a wavefront without transfers
+            // reads the last one and does not use it)
+            const int my_gran = min(wave * DMA_PER_WAVE * kRowsPerInst / kGranule, kGranPerTile - 1);
+            const int sel = (kFar && (r.kt & kFarTileFlag)) ? 1 : my_gran;
             const int mine = __builtin_amdgcn_readfirstlane(ep[sel]);
             r.emax = sel == 0 ? mine & ~kPackedMaskFlag : mine;
             r.emin = j0 + j;
@@ -1248,7 +1261,7 @@ int check_common(const char* who, const SegmentShape& g, const int64_t* q_stride
   NATS_REQUIRE(k_strides[2] * kTile < (int64_t(1) << 30) && v_strides[2] * kTile < (int64_t(1) << 30) && k_strides[2] > 0 &&
                    v_strides[2] > 0,
                NATS_ERR_BAD_SHAPE, "%s: row strides %lld / %lld of k / v", who, (long long)k_strides[2], (long long)v_strides[2]);
-  if (dtype == NATS_DTYPE_BF16 && (g.D == 64 || g.D == 128)) {
+  if (dtype == NATS_DTYPE_BF16 && (g.D == 32 || g.D == 64 || g.D == 128)) {
     // 16-byte vector loads and stores of rows
     NATS_REQUIRE(q_strides[2] % 8 == 0 && k_strides[2] % 8 == 0 && v_strides[2] % 8 == 0 && o_strides[2] % 8 == 0 &&
                      q_strides[1] % 8 == 0 && k_strides[1] % 8 == 0 && v_strides[1] % 8 == 0 && o_strides[1] % 8 == 0 &&
@@ -1293,7 +1306,7 @@ int launch_segment(const char* who, const SegmentShape& g, const void* q, const 
   a.hpw = 1; a.qpw = 1; a.n_hg = 1; a.n_qg = (int)n_qt; a.xcd_mode = 0;
 
   // fp32, and bf16 at the head dims the MFMA kernel does not take (16, 32, 256): the plain kernel
-  if (dtype == NATS_DTYPE_F32 || (g.D != 64 && g.D != 128)) {
+  if (dtype == NATS_DTYPE_F32 || (g.D != 32 && g.D != 64 && g.D != 128)) {
     NATS_REQUIRE(g.B * g.H_q <= 65535, NATS_ERR_BAD_SHAPE, "%s: B*H_q too large for the plain kernel", who);
     dim3 grid((unsigned)n_qt, (unsigned)(g.B * g.H_q));
     const bool f32 = dtype == NATS_DTYPE_F32;
@@ -1343,10 +1356,13 @@ int launch_segment(const char* who, const SegmentShape& g, const void* q, const 
     a.long_rows = w.long_rows; a.long_lim = w.long_lim; a.long_before = w.long_before; a.long_alive = w.long_alive;
     a.long_cap = (int)w.long_cap; a.n_gran = (int)w.n_gran; a.n_rtile = (int)w.n_rtile;
   }
+  // (head dim -> instantiation)
+#define NATS_PREFILL_BY_D(UNI, MODE, PA, NWG)                                                  \
+  (g.D == 32 ? launch_prefill_mfma<32, UNI, MODE>(PA, NWG, st)                                 \
+             : g.D == 64 ? launch_prefill_mfma<64, UNI, MODE>(PA, NWG, st) : launch_prefill_mfma<128, UNI, MODE>(PA, NWG, st))
   auto launch_packed = [&](const PrefillArgs& pa, int64_t n) {
-    if (pa.long_rows)
-      return g.D == 64 ? launch_prefill_mfma<64, true, 2>(pa, n, st) : launch_prefill_mfma<128, true, 2>(pa, n, st);
-    return g.D == 64 ? launch_prefill_mfma<64, true, 1>(pa, n, st) : launch_prefill_mfma<128, true, 1>(pa, n, st);
+    if (pa.long_rows) return NATS_PREFILL_BY_D(true, 2, pa, n);
+    return NATS_PREFILL_BY_D(true, 1, pa, n);
   };
   a.n_split = 1;
   if (hpw == 4 || packed) {  // the kernels in which every wavefront walks the whole tile list
@@ -1363,10 +1379,12 @@ int launch_segment(const char* who, const SegmentShape& g, const void* q, const 
     if (packed) {
       rc = launch_packed(a, n_launch);
     } else {
-      rc = g.D == 64 ? launch_prefill_mfma<64, true>(a, n_launch, st) : launch_prefill_mfma<128, true>(a, n_launch, st);
+      rc = NATS_PREFILL_BY_D(true, 0, a, n_launch);
     }
     if (rc) return rc;
-    if (g.D == 64) {
+    if (g.D == 32) {
+      hipLaunchKernelGGL((prefill_split_merge_kernel<32>), dim3((unsigned)n_wg, kPrefillWaves * (kTile / 2) * 8 / 256), dim3(256), 0, st, a);
+    } else if (g.D == 64) {
       hipLaunchKernelGGL((prefill_split_merge_kernel<64>), dim3((unsigned)n_wg, kPrefillWaves * (kTile / 2) * 16 / 256), dim3(256), 0, st, a);
     } else {
       hipLaunchKernelGGL((prefill_split_merge_kernel<128>), dim3((unsigned)n_wg, kPrefillWaves * (kTile / 2) * 32 / 256), dim3(256), 0, st, a);
@@ -1397,8 +1415,9 @@ int launch_segment(const char* who, const SegmentShape& g, const void* q, const 
   // walks the whole list and the element mask sorts out what its own rows see)
   if (packed)
     return launch_packed(a, n_wg);
-  if (hpw == 4) return g.D == 64 ? launch_prefill_mfma<64, true>(a, n_wg, st) : launch_prefill_mfma<128, true>(a, n_wg, st);
-  return g.D == 64 ? launch_prefill_mfma<64, false>(a, n_wg, st) : launch_prefill_mfma<128, false>(a, n_wg, st);
+  if (hpw == 4) return NATS_PREFILL_BY_D(true, 0, a, n_wg);
+  return NATS_PREFILL_BY_D(false, 0, a, n_wg);
+#undef NATS_PREFILL_BY_D
 }
 
 }  // namespace

@@ -64,7 +64,7 @@ def run_case(B, Hq, Hkv, D, W, C, n_max_chunks, dtype, seed=0, frac=(0.1, 1.0), 
 
 
 @pytest.mark.parametrize("n_rep", [1, 2, 3, 4, 5, 6, 7, 8, 12, 16])
-@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("D", [32, 64, 128])
 def test_bf16_group_sizes(n_rep, D):
     run_case(2, 2 * n_rep, 2, D, 128, 64, 20, torch.bfloat16, seed=n_rep + D)
 

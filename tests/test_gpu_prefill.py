@@ -63,6 +63,13 @@ def test_chunk_sizes_that_are_no_power_of_two(L, C, W, D, dtype):
     run_case(2, 8, 2, L, D, C, W, dtype, seed=L + C)
 
 
+@pytest.mark.parametrize("Hq,Hkv,L,C,W", [(8, 2, 1000, 64, 128), (8, 2, 777, 32, 64), (4, 4, 900, 16, 32), (4, 2, 650, 1, 16),
+                                          (8, 2, 2100, 128, 256)])
+def test_head_dim_32_on_the_matrix_kernels(Hq, Hkv, L, C, W):
+    """Rows of 64 bytes: a tile is four transfers (wavefronts 0-3 issue one each), one score MFMA step per 16 dims."""
+    run_case(2, Hq, Hkv, L, 32, C, W, torch.bfloat16, seed=L + 32)
+
+
 @pytest.mark.parametrize("D", [16, 32, 256])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_other_head_dims(D, dtype):
