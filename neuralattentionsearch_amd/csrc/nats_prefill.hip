@@ -2,8 +2,10 @@
 //
 // Kernels (they share the per-row limits and the tile / granule summaries of the key-limit stage):
 //   prefill_mfma_kernel        bf16, QK^T and PV on v_mfma_f32_32x32x16_bf16, fp32 online softmax; walks whole 64-row
-//                              key tiles, or (kPacked) tiles assembled from the visible 16-row granules; with
-//                              n_split > 1 several workgroups share one tile list and leave partial results
+//                              key tiles (kMode 0), tiles assembled from the visible 16-row granules (kMode 1), or, for
+//                              chunks shorter than a granule, tiles gathered row by row from the lists of long-lived
+//                              rows far behind a query plus granules near it (kMode 2); with n_split > 1 several
+//                              workgroups share one tile list and leave partial results
 //   prefill_split_merge_kernel combines those partial results
 //   prefill_simple_kernel      fp32 (or bf16) FMA kernel, one query row per lane; the fp32 parity path
 //
@@ -235,7 +237,7 @@ constexpr int kFarTileFlag = 1 << 29;     // ... the entry is a tile of long-liv
 
 // kUniform: the wavefronts are the q heads of ONE query tile (GQA groups of 4 and more), so every tile of
 // the visit list is visited by every wavefront and the tile loop has no per-wavefront branches.
-// kPacked (with kUniform, for chunks shorter than a tile): a tile is assembled from four 16-row granules taken
+// kPacked (kMode 1 and 2, with kUniform, for chunks shorter than a tile): a tile is assembled from four 16-row granules taken
 // from anywhere in the key rows.  Granules no query of the workgroup sees are left out, granules every query of
 // the workgroup sees without a mask are packed among themselves and the rest (diagonal, partly visible, the remainder of the
 // first kind, padding) into tiles that go through the element mask.  The softmax does not care about the order
