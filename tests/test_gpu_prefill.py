@@ -330,6 +330,13 @@ def test_long_lived_rows_against_the_oracle(B, Hq, Hkv, L, D, C, W, p):
     run_case(B, Hq, Hkv, L, D, C, W, torch.bfloat16, seed=L, p=p)
 
 
+@pytest.mark.parametrize("L", [1, 2, 15, 16, 17, 31, 63, 64, 65, 129])
+@pytest.mark.parametrize("C,W", [(1, 1), (1, 4), (2, 4), (8, 8), (3, 6)])
+def test_short_sequences_with_short_chunks(L, C, W):
+    """Fewer rows than a granule, a tile, and a few more: the lists of long-lived rows of one or two tiles."""
+    run_case(1, 4, 1, L, 64, C, W, torch.bfloat16, seed=L * 7 + C, p=(0.3, 0.3, 0.4))
+
+
 def test_gathered_rows_agree_with_the_granule_walk(far_rows):
     """The same keys reach the softmax in another order, on a first prefill and on segments over a per-token cache
     (cache rows below the open chunk: ring, kept rows, pending tokens)."""
