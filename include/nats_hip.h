@@ -263,7 +263,10 @@ typedef struct {
                            first row of that block, tail = the ring slot written last, first = 1 if the block holds
                            every token seen so far.  Ring rows are copied whatever the role (valid only if
                            sliding-window), rows at and beyond the new n_ctx_data keep their contents, and a block of
-                           sliding-window tokens only leaves n_ctx_data where it is. */
+                           sliding-window tokens only leaves n_ctx_data where it is.  U = 1 (nothing is deferred, W >= 2):
+                           a one-token step is the class's one-step branch (:328-367): the token's row goes to row
+                           size_global (a global token) or size_global + size_local (any other) of every head and to ring
+                           slot tail + 2 (slot 1 for the first token ever), unless it is sliding-window on every head. */
 } nats_evict_params;
 
 typedef struct {

@@ -555,15 +555,18 @@ class NAtSLayerCache(NAtSChunkLayerCache):
         [P, n_ctx_data)               the pending block
 
     Storage (capacity buffer, deferred first prefill) and the kernels are those of the chunked class with one-token
-    chunks; the state machine is this class's own."""
+    chunks; the state machine is this class's own.  With `update_chunk_size == 1` nothing is deferred and a one-token
+    step is the reference's one-step branch (:328-367), which the kernels take from `update_chunk == 1, x_len == 1`."""
 
     def __init__(self, bsz: int, n_msks: int, sliding_window_size: int, layer_id: int = 0, update_chunk_size: int = 16,
                  device: torch.device | str = "cuda", track_positions: bool = False):
         if sliding_window_size < update_chunk_size:  # nats_layer_cache.py:77-78
             raise NotImplementedError("The sliding window size must be greater or equal to the update chunk size!")
-        if update_chunk_size < 2:
-            raise NotImplementedError("update_chunk_size == 1 (the one-step branch, nats_layer_cache.py:328-367) is not "
-                                      "built; the container always uses 16")
+        if update_chunk_size < 1:
+            raise ValueError("update_chunk_size must be positive")
+        if update_chunk_size == 1 and sliding_window_size < 2:
+            # nats_layer_cache.py:344 writes ring slot 1 at the first one-token call, which a window of one does not have
+            raise NotImplementedError("update_chunk_size == 1 needs a sliding window of at least two tokens")
         self.update_chunk_size = update_chunk_size
         super().__init__(bsz, n_msks, sliding_window_size, layer_id=layer_id, chunk_size=1, device=device,
                          track_positions=track_positions)
@@ -766,6 +769,9 @@ class NAtSLayerCache(NAtSChunkLayerCache):
         first_ring = fill == self._seen_tokens   # the block holds every token seen so far (:439)
         first_call = self._seen_tokens == x_len  # (:404)
         roles = self._pending_block()
+        if x_len == 1 and self._pending is not None:
+            # (update_chunk_size == 1: the first token ever is evicted at once, by the one-step branch :328-367, in place)
+            self._materialize_pending()
         src = self._pending
         like = src[0] if src is not None else self._buf_k
         D = like.shape[3]

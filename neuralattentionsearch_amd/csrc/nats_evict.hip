@@ -46,6 +46,11 @@ __device__ __forceinline__ long long old_size_local(const nats_evict_params& p, 
   return p.first ? 0LL : (long long)size_local[h];
 }
 
+// A one-token step that completes a chunk scatters that chunk for every head (nats_chunk_layer_cache.py:289-330); the
+// per-token cache does the same with its one token when nothing is deferred (update_chunk_size == 1,
+// nats_layer_cache.py:328-367), with the same arithmetic for the sizes.
+__host__ __device__ inline bool one_step_scatter(const nats_evict_params& p) { return p.x_len == 1 && p.update_chunk <= 1; }
+
 __host__ __device__ inline size_t plan_lists_offset(int64_t n_heads) {
   return (kPlanHeaderBytes + (size_t)n_heads * sizeof(HeadPlan) + 255) & ~size_t(255);
 }
@@ -101,7 +106,7 @@ __device__ __forceinline__ void plan_one_head(const uint8_t* __restrict__ roles,
   const uint8_t* r = roles + (int64_t)head * S;
   const long long sg = old_size_global(p, size_global, head), sl = old_size_local(p, size_local, head);
   HeadPlan hp;
-  if (p.x_len == 1 && !p.update_chunk) {
+  if (one_step_scatter(p)) {
     // one completed chunk is scattered for every head (:289-330)
     int r0 = r[0], rl = r[S - 1];
     bool is_g = r0 == NATS_ROLE_GLOBAL;
@@ -195,7 +200,7 @@ __device__ __forceinline__ void plan_one_head_serial(const uint8_t* __restrict__
   const uint8_t* r = roles + (int64_t)head * S;
   const long long sg = old_size_global(p, size_global, head), sl = old_size_local(p, size_local, head);
   HeadPlan hp;
-  if (p.x_len == 1 && !p.update_chunk) {
+  if (one_step_scatter(p)) {
     int r0 = r[0], rl = r[S - 1];
     bool is_g = r0 == NATS_ROLE_GLOBAL;
     long long dst = is_g ? sg : sg + sl;
@@ -306,7 +311,7 @@ __device__ __forceinline__ void plan_finalize(const int64_t* __restrict__ size_g
     const PlanAgg t = agg[0];
     nats_evict_result res;
     res.all_sw = t.all_sw;
-    res.all_local = (p.x_len != 1 || p.update_chunk) && t.all_local && !t.all_sw;
+    res.all_local = !one_step_scatter(p) && t.all_local && !t.all_sw;
     res.max_keep = t.max_keep;
     res.max_end = t.max_end;
     res.seq = p.seq;
@@ -321,7 +326,7 @@ __device__ __forceinline__ void plan_finalize(const int64_t* __restrict__ size_g
     } else {
       res.n_ctx_data = t.max_tot_new + partial;
       res.gmin = t.min_sg_new;
-      bool tail_move = (p.x_len != 1 || p.update_chunk) && partial && t.max_keep < S - 1;  // :840
+      bool tail_move = !one_step_scatter(p) && partial && t.max_keep < S - 1;  // :840
       res.moved_rows = (t.sum_keep + (tail_move ? n_heads : 0)) * (long long)C;
     }
     *result = res;
@@ -450,8 +455,11 @@ __device__ void apply_inplace_body(const ApplyArgs& a, TensorView<U> t, int head
   // 1. ring insert (:391-437)
   const bool token = p.update_chunk != 0;
   const int n_ring = n_done < wc ? n_done : wc;
-  // the chunked cache's tail is the next slot to write, the per-token cache's the slot written last
-  const int start_chunk = p.first ? 0 : token ? (int)((p.tail + 1) % p.W) : (int)(p.tail / p.C);
+  // the chunked cache's tail is the next slot to write, the per-token cache's the slot written last; its one-step
+  // branch writes one slot further on (nats_layer_cache.py:340-345: slot 1 for the first token ever, else tail + 2,
+  // while the tail itself advances by one), unless every head's token is sliding-window (:316-317)
+  const int skip = token && one_step_scatter(p) && !res.all_sw ? 1 : 0;
+  const int start_chunk = p.first ? skip : token ? (int)((p.tail + 1 + skip) % p.W) : (int)(p.tail / p.C);
   for (int j = wave; j < n_ring; j += 4) {
     int slot = n_done - n_ring + j;
     bool is_sw = r[slot] == NATS_ROLE_SW;
@@ -470,7 +478,7 @@ __device__ void apply_inplace_body(const ApplyArgs& a, TensorView<U> t, int head
   // 2. ordered chunk moves, each batch read completely before it is written
   int n_moves;
   bool tail_move = false;
-  if (p.x_len == 1 && !token) {
+  if (one_step_scatter(p)) {
     n_moves = 1;
   } else if (res.all_local) {
     n_moves = 0;
@@ -768,7 +776,8 @@ static int check_params(const char* who, const nats_evict_params* p) {
   NATS_REQUIRE(p->update_chunk >= 0 && (p->update_chunk == 0 || (p->C == 1 && p->fill >= p->update_chunk && p->update_chunk <= p->W)),
                NATS_ERR_BAD_SHAPE, "%s: update_chunk=%lld needs chunk size 1, a window and a pending block of at least that many tokens",
                who, (long long)p->update_chunk);
-  NATS_REQUIRE(p->x_len != 1 || p->S == 1 || p->update_chunk, NATS_ERR_BAD_SHAPE, "%s: a one-token step completes exactly one chunk", who);
+  NATS_REQUIRE(p->x_len != 1 || p->S == 1 || p->update_chunk > 1, NATS_ERR_BAD_SHAPE, "%s: a one-token step completes exactly one chunk", who);
+  NATS_REQUIRE(p->update_chunk != 1 || p->W >= 2, NATS_ERR_UNSUPPORTED, "%s: update_chunk=1 needs a window of at least two tokens", who);
   NATS_REQUIRE(p->n_ctx_data >= p->W && p->gmin >= p->W && p->tail >= 0 && p->tail < p->W && p->tail % p->C == 0,
                NATS_ERR_BAD_SHAPE, "%s: n_ctx_data=%lld gmin=%lld tail=%lld", who, (long long)p->n_ctx_data,
                (long long)p->gmin, (long long)p->tail);

@@ -19,7 +19,7 @@ How each function is pinned (see tests/test_oracle_*.py):
 * masked_attention ............. torch SDPA with a bool mask is the library routine itself
 * ChunkCacheOracle.update / generate_mask / post_update
                                  golden vectors written by the reference's NAtSChunkLayerCache on CPU
-                                 (tests/golden/make_golden.py), 24 scenarios / 270 calls (chunk sizes 1 to 4), compared on
+                                 (tests/golden/make_golden.py), 28 scenarios / 305 calls (chunk sizes 1 to 12), compared on
                                  every byte of cache_k, cache_v, valid_tokens, sizes and scalars
 * decode_attention ............. equals masked_attention restricted to the valid rows (gather, then dense
                                  softmax); checked against torch SDPA
@@ -29,15 +29,15 @@ How each function is pinned (see tests/test_oracle_*.py):
 
 * TokenCacheOracle.update / generate_mask / post_update (the per-token class, chunk_size == 1)
                                  golden vectors written by the reference's NAtSLayerCache on CPU
-                                 (tests/golden/make_golden_token.py), 25 scenarios / 893 calls: every mask and,
+                                 (tests/golden/make_golden_token.py), 30 scenarios / 1030 calls: every mask and,
                                  after every post_update, every byte of cache_k, cache_v, valid_tokens, the sizes
                                  and the scalars (deferred 16-token eviction, ring insert, all-sliding and
                                  all-local blocks, multi-token segments over pending tokens, first segments
-                                 shorter than the window and than the update chunk, update chunks of 4 and 8)
+                                 shorter than the window and than the update chunk, update chunks of 4 and 8, and the
+                                 one-step branch of update chunk 1, :328-367, in five scenarios)
 
-Functions with parity unpinned: none of the above.  Not restated: the branch of the per-token class for
-update_chunk_size == 1 (cache/nats_layer_cache.py:328-367), which the container never constructs
-(dyn_cache.py:183-185 leaves the default of 16); TokenCacheOracle refuses U == 1.
+Functions with parity unpinned: none of the above.  Not restated: update_chunk_size == 1 with a window of one token
+(cache/nats_layer_cache.py:344 then writes ring slot 1 of a ring that has only slot 0); TokenCacheOracle refuses it.
 """
 from __future__ import annotations
 
@@ -574,8 +574,10 @@ class TokenCacheOracle:
     def __post_init__(self):
         if self.W < self.U:  # :77-78
             raise NotImplementedError("The sliding window size must be greater or equal to the update chunk size!")
-        if self.U == 1:
-            raise NotImplementedError("the one-step branch of update_chunk_size == 1 (:328-367) is not restated")
+        if self.U == 1 and self.W < 2:
+            # :344 writes ring slot 1 at the first one-token call without reducing it modulo W: with W == 1 that is the
+            # token's own row, outside the ring
+            raise NotImplementedError("update_chunk_size == 1 is restated for windows of at least two tokens")
         self.size_global = np.full((self.B, self.H), self.W, dtype=np.int64)
         self.size_local = np.zeros((self.B, self.H), dtype=np.int64)
         self.n_ctx_data = self.W
@@ -718,7 +720,55 @@ class TokenCacheOracle:
             self._ring_insert()
             self.fill = self.fill_last = 0
             return
-        self._ring_insert()
+        if x_len == 1 and U == 1:  # :328-367: the one-step branch, every head scatters its one token
+            self._one_step(block[:, :, 0])
+        else:
+            self._ring_insert()
+            self._merge_block(block, fill)
+        self.size_local += fill  # :393
+        assert not (self.size_local < 0).any()
+        self.n_ctx_data = int((self.size_global + self.size_local).max())  # :394
+        old_gmin = self.gmin  # :565 uses the minimum from before this call
+        if self.n_ctx_data != old_gmin:
+            idx = np.arange(old_gmin, self.n_ctx_data)
+            end = (self.size_global + self.size_local)[:, :, None]
+            self.valid[:, :, old_gmin:self.n_ctx_data] = idx[None, None, :] < end
+        self.gmin = int(self.size_global.min())
+        if self.seen == x_len:  # :404-408
+            n = self.n_ctx_data
+            self.cache_k, self.cache_v = self.cache_k[:, :, :n], self.cache_v[:, :, :n]
+            self.valid, self.pos_k = self.valid[:, :, :n], self.pos_k[:, :, :n]
+        self.fill = self.fill_last = 0
+
+    def _one_step(self, role: np.ndarray):
+        """:328-367 (update_chunk_size == 1, one new token, not sliding-window on every head).  The token's row
+        (n_ctx_data - 1, where update() put it) is written to ring slot tail + 2 (slot 1 for the first token ever;
+        `tail` itself advances by one, :340-345) and to row size_global (a global token, which thereby drops the
+        head's local rows) or size_global + size_local (local and sliding-window tokens alike); the slot is valid iff
+        the token is sliding-window.  The sizes are left so that the common `size_local += 1` (:393) completes them."""
+        W, src = self.W, self.n_ctx_data - 1
+        if self.seen == 1:
+            slot, self.tail = 1, 0
+        else:
+            slot = (1 + self.tail + 1) % W
+            self.tail = (self.tail + 1) % W
+        is_g = role == ROLE_GLOBAL
+        is_sw = role == ROLE_SW
+        dst = np.where(is_g, self.size_global, self.size_global + self.size_local)  # :335-337
+        self.valid[:, :, slot] = is_sw  # :347
+        new_k, new_v, new_p = self.cache_k[:, :, src].clone(), self.cache_v[:, :, src].clone(), self.pos_k[:, :, src].copy()
+        for b in range(self.B):
+            for h in range(self.H):
+                for row in (int(dst[b, h]), slot):  # :351-355
+                    self.cache_k[b, h, row] = new_k[b, h]
+                    self.cache_v[b, h, row] = new_v[b, h]
+                    self.pos_k[b, h, row] = new_p[b, h]
+        dec_local = np.where(is_g, self.size_local + 1, 0) + is_sw  # :357-361
+        self.size_global = self.size_global + is_g  # :365
+        self.size_local = self.size_local - dec_local  # :366
+
+    def _merge_block(self, block: np.ndarray, fill: int):
+        B, H = self.B, self.H
         if not (block == ROLE_LOCAL).all():  # :651-770 + cache_update.py:25-76 (chunk_size 1)
             P = self.n_ctx_data - fill  # :759
             moves = []
@@ -745,20 +795,6 @@ class TokenCacheOracle:
             for (b, h), (sg, sl) in new_sizes.items():
                 self.size_global[b, h] = sg
                 self.size_local[b, h] = sl
-        self.size_local += fill  # :393
-        assert not (self.size_local < 0).any()
-        self.n_ctx_data = int((self.size_global + self.size_local).max())  # :394
-        old_gmin = self.gmin  # :565 uses the minimum from before this call
-        if self.n_ctx_data != old_gmin:
-            idx = np.arange(old_gmin, self.n_ctx_data)
-            end = (self.size_global + self.size_local)[:, :, None]
-            self.valid[:, :, old_gmin:self.n_ctx_data] = idx[None, None, :] < end
-        self.gmin = int(self.size_global.min())
-        if self.seen == x_len:  # :404-408
-            n = self.n_ctx_data
-            self.cache_k, self.cache_v = self.cache_k[:, :, :n], self.cache_v[:, :, :n]
-            self.valid, self.pos_k = self.valid[:, :, :n], self.pos_k[:, :, :n]
-        self.fill = self.fill_last = 0
 
 
 def kept_token_fraction(cache: ChunkCacheOracle) -> float:

@@ -97,10 +97,19 @@ def scenarios():
                     segs=[(32, "rand"), (16, "all_s"), (12, "rand"), (20, "rand")] + one(8)))
     # streaming in blocks of exactly one update chunk
     out.append(dict(name="stream_blocks_w16", B=2, H=2, W=16, p=(0.15, 0.25, 0.6), segs=[(16, "rand")] * 12))
-    # other update chunk sizes the class accepts (W >= U); 1 would take the one-step branch (:328-367), which
-    # NAtSCache never constructs and which is not recorded
+    # other update chunk sizes the class accepts (W >= U)
     out.append(dict(name="update_chunk4_w8", B=2, H=2, W=8, U=4, p=mix, segs=[(11, "rand")] + one(13) + [(6, "rand"), (9, "rand")] + one(6)))
     out.append(dict(name="update_chunk8_w8", B=1, H=3, W=8, U=8, p=mix, segs=[(20, "rand")] + one(20) + [(10, "rand")] + one(9)))
+    # update chunk 1: nothing is deferred; a one-token step that is not sliding-window on every head takes the one-step
+    # branch (:328-367), which NAtSCache never constructs (dyn_cache.py:183-185 leaves the default of 16)
+    out.append(dict(name="update_chunk1_w8", B=2, H=3, W=8, U=1, p=mix, segs=[(11, "rand")] + one(30)))
+    out.append(dict(name="update_chunk1_decode_from_empty_w4", B=2, H=2, W=4, U=1, p=mix, segs=one(30)))
+    out.append(dict(name="update_chunk1_w2_swheavy", B=1, H=3, W=2, U=1, p=sw_heavy, segs=one(24)))
+    out.append(dict(name="update_chunk1_special_roles_w8", B=1, H=2, W=8, U=1, p=mix,
+                    segs=[(9, "rand")] + one(4, "all_s") + one(6) + one(3, "all_l") + one(3, "all_g") + one(5, "all_s")
+                    + one(8)))
+    out.append(dict(name="update_chunk1_multiseg_w8", B=2, H=2, W=8, U=1, p=mix,
+                    segs=one(3) + [(5, "rand")] + one(4) + [(12, "rand"), (2, "rand")] + one(6) + [(3, "all_s")] + one(5)))
     for sc in out:
         sc.setdefault("D", 2)
         sc.setdefault("U", 16)

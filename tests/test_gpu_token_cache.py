@@ -122,3 +122,17 @@ def test_container_builds_the_per_token_class_for_chunk_size_one():
     assert c1.get_nats_chunk_fill_size(0) == 0  # as the reference's container answers for chunk_size == 1
     with pytest.raises(NotImplementedError):
         NAtSCache(8, 1).update(k, k, 0, {"token_states_info": tsi})  # window below the update chunk size
+
+
+@pytest.mark.parametrize("W,D,dtype,n_rep,p", [(16, 64, torch.float32, 2, (0.3, 0.3, 0.4)),
+                                               (64, 128, torch.bfloat16, 4, (0.1, 0.2, 0.7)),
+                                               (2, 128, torch.bfloat16, 1, (0.2, 0.2, 0.6))])
+def test_random_streams_without_deferral(W, D, dtype, n_rep, p):
+    """update_chunk_size == 1: every call evicts; one-token steps take the reference's one-step branch
+    (nats_layer_cache.py:328-367) unless the token is sliding-window on every head."""
+    rng = np.random.default_rng(7 * W + D)
+    lens = [1] * 5 + [3 * W + 5] + [1] * 50 + [W // 2 + 3, 1, 1, 2 * W + 5, 2] + [1] * 30 + [300]
+    segs = role_stream(rng, 2, 4, lens, p)
+    for i in (8, 9, 30):  # some steps whose token is sliding-window on every head (:316-327 instead of :328-367)
+        segs[i] = (1, np.full((2, 4, 1), 2, np.uint8))
+    drive(f"random_U1_W{W}", 2, 4, D, W, 1, segs, dtype, seed=W, n_rep=n_rep)
