@@ -703,7 +703,7 @@ def main():
     if pre:
         line["roofline"] = {"bound": "mfma", "achieved": pre["tflops_visited"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                             "frac": pre["tflops_visited"] / PEAK_BF16_TFLOPS,
-                            "kernel": "prefill_mfma_kernel<128, true>"}
+                            "kernel": "prefill_mfma_kernel<128, true, 0>"}
         line["roofline"]["traffic"], line["roofline"]["traffic_source"] = (
             measured_traffic("prefill") if args.prefill_len == 32768 and args.chunk_size == 64 else (None, "not the profiled workload"))
     if "decode" in res:
