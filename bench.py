@@ -178,7 +178,7 @@ def time_gpu(fn, steps: int, warmup: int, settle_ms: float = 0.0):
 
 # --------------------------------------------------------------------------------------------------
 def bench_prefill(args, ops, chunk_size=None, steps=None, warmup=None, compare=True, settle=True):
-    B, Hq, Hkv, L, D, C, W = 1, 32, 8, args.prefill_len, 128, chunk_size or args.chunk_size, 256
+    B, Hq, Hkv, L, D, C, W = 1, 32, 8, args.prefill_len, args.head_dim, chunk_size or args.chunk_size, 256
     steps, warmup = steps or args.steps, args.warmup if warmup is None else warmup
     n_rep = Hq // Hkv
     dev = "cuda"
@@ -261,7 +261,7 @@ def decode_inputs(B, Hq, Hkv, D, C, W, ctx, seed, dev):
 
 
 def bench_decode(args, ops, batch=None, context=None):
-    B, Hq, Hkv, D, C, W, ctx = batch or args.decode_batch, 32, 8, 128, 64, 256, context or args.decode_context
+    B, Hq, Hkv, D, C, W, ctx = batch or args.decode_batch, 32, 8, args.head_dim, 64, 256, context or args.decode_context
     q, k, v, valid, n_rows, (row_end, tail_start) = decode_inputs(B, Hq, Hkv, D, C, W, ctx, 0, "cuda")
     n_valid = int(valid[:, :, :n_rows].sum().item())
     bytes_alg = n_valid * D * 2 * 2 + 2 * q.numel() * 2
@@ -627,6 +627,8 @@ def main():
     ap.add_argument("--chunk-size", type=int, default=64, help="chunk size of the prefill leg (the headline uses 64)")
     ap.add_argument("--decode-batch", type=int, default=32, help="sequences of the decode leg (the headline uses 32)")
     ap.add_argument("--decode-context", type=int, default=65536, help="context of the decode leg (the headline uses 65536)")
+    ap.add_argument("--head-dim", type=int, default=128, choices=[32, 64, 128, 256],
+                    help="head dim of `--only prefill` / `--only decode` (the headline uses 128)")
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--no-compare", action="store_true", help="skip the dense comparators of the prefill leg")
     ap.add_argument("--segments", type=int, default=4, help="segments of the `--only segments` leg")
@@ -697,22 +699,24 @@ def main():
         "ms_per_step": pre["ms"] if pre else None,
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": f"prefill B=1 Hq=32 Hkv=8 D=128 L={args.prefill_len} chunk {args.chunk_size} window 256, roles 5/15/80 "
+        "config": {"workload": f"prefill B=1 Hq=32 Hkv=8 D={args.head_dim} L={args.prefill_len} chunk {args.chunk_size} window 256, roles 5/15/80 "
                                "(global/local/sliding); decode and compaction ride along under their own keys"},
     }
     if pre:
         line["roofline"] = {"bound": "mfma", "achieved": pre["tflops_visited"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                             "frac": pre["tflops_visited"] / PEAK_BF16_TFLOPS,
-                            "kernel": "prefill_mfma_kernel<128, true, 0>"}
+                            "kernel": "prefill_mfma_wide_kernel" if args.head_dim == 256
+                                      else f"prefill_mfma_kernel<{args.head_dim}, true, {0 if args.chunk_size >= 64 else 1 if args.chunk_size >= 16 else 2}>"}
         line["roofline"]["traffic"], line["roofline"]["traffic_source"] = (
-            measured_traffic("prefill") if args.prefill_len == 32768 and args.chunk_size == 64 else (None, "not the profiled workload"))
+            measured_traffic("prefill") if (args.prefill_len, args.chunk_size, args.head_dim) == (32768, 64, 128)
+            else (None, "not the profiled workload"))
     if "decode" in res:
         d = res["decode"]
         line["roofline_decode"] = {"bound": "hbm", "achieved": d["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
                                    "frac": d["frac_of_hbm_peak"],
-                                   "kernel": "decode_split_mfma_kernel<128,4> + decode_merge_balanced_kernel"}
+                                   "kernel": f"decode_split_mfma_kernel<{args.head_dim},4> + decode_merge_balanced_kernel"}
         line["roofline_decode"]["traffic"], line["roofline_decode"]["traffic_source"] = (
-            measured_traffic("decode") if (args.decode_batch, args.decode_context) == (32, 65536)
+            measured_traffic("decode") if (args.decode_batch, args.decode_context, args.head_dim) == (32, 65536, 128)
             else (None, "not the profiled workload"))
     if "evict" in res:
         e = res["evict"]

@@ -128,8 +128,9 @@ int nats_prefill_tile_map(const uint8_t* roles, int64_t B, int64_t H_kv, int64_t
  *   that may overlap on the device need a workspace each.
  * D in {16, 32, 64, 128, 256} (the head dims of nats_flashattn_fwd.py:634); C > 0; W % C == 0;
  * H_q % H_kv == 0.
- * dtype bf16 with D 32, 64 or 128 runs QK^T and PV on bf16 MFMA with fp32 softmax state; dtype f32, and bf16 at the
- * other head dims, run an fp32 FMA kernel.
+ * dtype bf16 with D 32, 64, 128 or 256 runs QK^T and PV on bf16 MFMA with fp32 softmax state (D 256: a kernel of its
+ * own, four wavefronts with the whole register file; rows that are not 16-byte aligned go to the plain kernel);
+ * dtype f32, and bf16 at D 16, run an fp32 FMA kernel.
  */
 size_t nats_prefill_workspace_bytes(int64_t B, int64_t H_q, int64_t H_kv, int64_t L, int64_t D, int64_t C);
 
@@ -207,8 +208,8 @@ int nats_prefill_past_mask(const uint8_t* valid, const int64_t* size_global, con
  *           hold nothing valid (the cache's size_global_kv + size_local_kv and the start of the open chunk,
  *           components/cache/nats_chunk_layer_cache.py:644-656) and are skipped without reading valid
  *   workspace: nats_decode_workspace_bytes(...) bytes
- * D in {16, 32, 64, 128, 256}; H_q % H_kv == 0 (any group size); dtype bf16 (MFMA for D 32, 64 and 128) or f32 (fp32 FMA
- * kernel, which also takes bf16 at the other head dims and ignores the hint).
+ * D in {16, 32, 64, 128, 256}; H_q % H_kv == 0 (any group size); dtype bf16 (MFMA for D 32, 64, 128 and 256) or f32
+ * (fp32 FMA kernel, which also takes bf16 at D 16 and ignores the hint).
  * bf16: a batch of more than 1024 (b, kv head) streams is taken in groups of whole sequences, launched one after
  * the other on `stream`.
  */

@@ -471,7 +471,7 @@ __global__ void decode_merge_balanced_kernel(const float* __restrict__ ws_acc, c
   o[(int64_t)head * D + d] = f32_to_bf16_bits(lsum > 0.f ? sum / lsum : 0.f);
 }
 
-// T = float, or uint16_t for bf16 at the head dims the MFMA kernel does not take (16, 32, 256).
+// T = float, or uint16_t for bf16 at the head dim the MFMA kernel does not take (16).
 template <typename T>
 __device__ __forceinline__ float dec_load(const T* p);
 template <>
@@ -679,7 +679,7 @@ static int decode_fwd_impl(const void* q, const void* cache_k, const void* cache
                (long long)H_q, (long long)H_kv);
   NATS_REQUIRE(D == 16 || D == 32 || D == 64 || D == 128 || D == 256, NATS_ERR_UNSUPPORTED,
                "nats_decode_fwd: head_dim %lld (supported: 16, 32, 64, 128, 256)", (long long)D);
-  const bool mfma = dtype == NATS_DTYPE_BF16 && (D == 32 || D == 64 || D == 128);  // other bf16 head dims take the plain kernel
+  const bool mfma = dtype == NATS_DTYPE_BF16 && D >= 32;  // bf16 at head dim 16 takes the plain kernel
   NATS_REQUIRE(dtype == NATS_DTYPE_BF16 || dtype == NATS_DTYPE_F32, NATS_ERR_BAD_DTYPE, "nats_decode_fwd: dtype %d", dtype);
   NATS_REQUIRE(n_rows < (int64_t(1) << 30) && B * H_q <= (int64_t(1) << 30), NATS_ERR_BAD_SHAPE,
                "nats_decode_fwd: problem too large");
@@ -771,6 +771,9 @@ static int decode_fwd_impl(const void* q, const void* cache_k, const void* cache
     c.row_end = a.row_end ? a.row_end + b0 * H_kv : nullptr;
     c.o = static_cast<uint16_t*>(o) + b0 * H_q * D;
     c.n_wg = decode_balanced_workgroups(nb, H_kv, n_rows);
+    // (rows of 512 bytes: a workgroup's V buffers take 128 KB of LDS, so one workgroup fits a compute unit at a time; one
+    // round of workgroups with equal shares measures 1 % faster than two)
+    if (D == 256) c.n_wg = std::min(c.n_wg, compute_units_of_current_device());
     c.share_first = decode_share_first(c.n_wg, groups);
     c.head_table = static_cast<int2*>(workspace);
     c.ws_acc = reinterpret_cast<float*>(static_cast<char*>(workspace) + align256((size_t)(nb * H_kv) * sizeof(int2)));
@@ -782,6 +785,14 @@ static int decode_fwd_impl(const void* q, const void* cache_k, const void* cache
         case 4: rc = launch_mfma<128, 4>(c, groups, st); break;
         case 2: rc = launch_mfma<128, 2>(c, groups, st); break;
         default: rc = launch_mfma<128, 1>(c, groups, st); break;
+      }
+    } else if (D == 256) {
+      c.share_first = 128;
+      switch (nrep_k) {
+        case 8: rc = launch_mfma<256, 8>(c, groups, st); break;
+        case 4: rc = launch_mfma<256, 4>(c, groups, st); break;
+        case 2: rc = launch_mfma<256, 2>(c, groups, st); break;
+        default: rc = launch_mfma<256, 1>(c, groups, st); break;
       }
     } else if (D == 32) {
       switch (nrep_k) {

@@ -7,6 +7,8 @@
 //                              rows far behind a query plus granules near it (kMode 2); with n_split > 1 several
 //                              workgroups share one tile list and leave partial results
 //   prefill_split_merge_kernel combines those partial results
+//   prefill_mfma_wide_kernel   bf16 MFMA kernel for head dim 256: four wavefronts with the whole register file, whole
+//                              tiles masked row by row
 //   prefill_simple_kernel      fp32 (or bf16) FMA kernel, one query row per lane; the fp32 parity path
 //
 // Mask semantics (components/masks/utils.py:89-94, components/cache/nats_chunk_layer_cache.py:462-511, 603-616):
@@ -1185,6 +1187,411 @@ __global__ __launch_bounds__(256) void prefill_split_merge_kernel(PrefillArgs a)
   }
 }
 
+// ---------------------------------------------------------------------------------------------------
+// bf16 MFMA kernel for head dim 256.
+//
+// A wavefront's O accumulators (32 rows x 256 dims = 128 registers per lane) and Q fragments (64) leave no room for two
+// wavefronts per SIMD, and four K + four V tiles of 32 KB do not fit the LDS: this kernel runs four wavefronts per
+// workgroup, one per SIMD with the whole register file, over two K and two V tile buffers.  A wavefront owns 32 query
+// rows of one q head (hpw q heads of the kv head x 4 / hpw blocks of 32 rows per workgroup); all walk the same key
+// tiles: those whose largest row limit reaches the group's first query, found 64 tile summaries at a time with a
+// ballot.  Fragment layouts, swizzles, lazy rescaling and the fused step (scores of tile j + 1 under the exponentials
+// of tile j, then O += P V) are those of the kernel above.  With one wavefront per SIMD nothing else covers a wait, so
+// the tile transfers are issued from assembly -- the compiler, which cannot tell the buffers apart, would otherwise
+// wait for every transfer in flight before the first LDS read after it -- and the kernel orders them itself: a step
+// begins with a wait for everything in flight and a workgroup barrier, requests K of tile j + 2 and V of tile j + 1,
+// and reads K of tile j + 1 and V of tile j.  Chunks shorter than a tile are masked row by row (no packing).
+// ---------------------------------------------------------------------------------------------------
+struct WideSmem {
+  uint16_t k[2][kTile * 256];  // K of tile j in k[j & 1]
+  uint16_t v[2][kTile * 256];
+  int limk[4][kTile];          // row limits of tile j in limk[j & 3]
+};
+
+// One global -> LDS transfer: lane i moves kBytes from its own global address to LDS address (uniform) + i * kBytes.
+// Counted by vmcnt like any vector memory load.  (The host pass of the single-source compile never runs this.)
+template <int kBytes>
+__device__ __forceinline__ void lds_transfer(const void* gptr, const void* lds_ptr) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  const uint32_t lds_addr =
+      __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(const __attribute__((address_space(3))) unsigned char*)lds_ptr);
+  if (kBytes == 16) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(lds_addr) : "memory", "m0");
+  } else {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(gptr), "s"(lds_addr) : "memory", "m0");
+  }
+#endif
+}
+// The same with the address as a uniform base (scalar registers) plus a byte offset per lane: no 64-bit vector arithmetic.
+__device__ __forceinline__ void lds_transfer16_base(const void* base, uint32_t byte_off, const void* lds_ptr) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  const uint32_t lds_addr =
+      __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(const __attribute__((address_space(3))) unsigned char*)lds_ptr);
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(byte_off), "s"(base), "s"(lds_addr)
+               : "memory", "m0");
+#endif
+}
+__device__ __forceinline__ void wait_transfers() {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#endif
+}
+
+constexpr int kWideWaves = 4;
+
+__global__ __launch_bounds__(kWideWaves * kWave) void prefill_mfma_wide_kernel(PrefillArgs a) {
+  constexpr int D = 256;
+  constexpr int OCT = D / 8;
+  constexpr int N_INST = kTile * OCT / kWave;        // 1 KiB transfers per tile
+  constexpr int DMA_PER_WAVE = N_INST / kWideWaves;  // ... per wavefront and tensor
+  constexpr int DSTEPS = D / 16;
+  constexpr int DT = D / 32;
+  constexpr int kHalf = kTile / 2;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  WideSmem& sm = *reinterpret_cast<WideSmem*>(smem_raw);
+
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = tid & 63;
+  const int l32 = lane & 31;
+  const int hl = lane >> 5;
+
+  int ks, hg, rank;
+  map_workgroup(a, blockIdx.x, ks, hg, rank);
+  const int qg = a.n_qg - 1 - rank;  // heavy query groups first
+  const int b = ks / a.Hkv, hkv = ks % a.Hkv;
+  const int hq = hkv * a.n_rep + hg * a.hpw + (wave % a.hpw);
+  // (here qpw counts blocks of 32 query rows)
+  const int blk_first = a.r_begin / kHalf, blk_last = (a.r_end - 1) / kHalf;
+  const int blk_lo = blk_first + qg * a.qpw;
+  const int blk_hi = min(blk_lo + a.qpw - 1, blk_last);
+  const int my_blk = blk_lo + wave / a.hpw;
+  const bool wave_live = my_blk <= blk_hi;
+  const int q0 = my_blk * kHalf;  // region token of this wavefront's first row
+
+  const int2* tl = a.tile_lim + (int64_t)ks * a.Tk;
+  const int32_t* lim = a.tok_lim + (int64_t)ks * a.N;
+  const uint16_t* kp = static_cast<const uint16_t*>(a.k) + b * a.ks_b + hkv * a.ks_h;
+  const uint16_t* vp = static_cast<const uint16_t*>(a.v) + b * a.vs_b + hkv * a.vs_h;
+
+  const int r0_group = max(blk_lo * kHalf, a.r_begin);
+  const int rlast_group = min(blk_hi * kHalf + kHalf - 1, a.r_end - 1);
+  const int my_r0 = max(q0, a.r_begin);
+  const int my_rlast = min(q0 + kHalf - 1, a.r_end - 1);
+  const int kt_end_group = (a.base + rlast_group) / kTile;
+
+  // ---- Q fragments: B operand, lane (query l32, k-group hl) --------------------------------------
+  bf16x8 qreg[DSTEPS];
+  {
+    const uint16_t* qp = static_cast<const uint16_t*>(a.q) + b * a.qs_b + hq * a.qs_h;
+    int row = min(max(q0 + l32, a.r_begin), a.r_end - 1) - a.r_begin;
+    const uint4* rp = reinterpret_cast<const uint4*>(qp + (int64_t)row * a.qs_l + hl * 8);
+#pragma unroll
+    for (int s = 0; s < DSTEPS; ++s) qreg[s] = __builtin_bit_cast(bf16x8, rp[s * 2]);
+  }
+
+  f32x16 oacc[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) oacc[dt][i] = 0.f;
+  float m_run = -INFINITY;
+  float l_run = 0.f;
+  const float c = a.scale * 1.4426950408889634f;
+
+  // ---- the visited key tiles, in order: 64 summaries at a time (the same in every wavefront) --------
+  int kt0 = 0;
+  uint64_t vmask;
+  int cmin;  // lane i: smallest row limit of tile kt0 + i
+  auto refill = [&]() {
+    const int t = kt0 + lane;
+    const int2 val = tl[min(t, kt_end_group)];
+    cmin = val.y;
+    vmask = __ballot(t <= kt_end_group && val.x >= r0_group);
+  };
+  auto next_tile = [&](int& minlim) -> int {
+    while (vmask == 0) {
+      if (kt0 + kWave > kt_end_group) return -1;
+      kt0 += kWave;
+      refill();
+    }
+    const int i = __builtin_amdgcn_readfirstlane(__builtin_ctzll(vmask));
+    vmask &= vmask - 1;
+    minlim = __builtin_amdgcn_readlane(cmin, i);
+    return kt0 + i;
+  };
+  refill();
+
+  // ---- transfers ---------------------------------------------------------------------------------------
+  auto v_swizzle = [](int row) { return (row & 3) << 2; };
+  // Transfer j of this wavefront fills chunk slots [(wave * DMA_PER_WAVE + j) * 64, +64) of the LDS tile: rows
+  // wave * 16 + 2 j + hl, chunk l32 of each.  The row part of the address is uniform (scalar arithmetic); the lane adds
+  // hl rows and its swizzled chunk, which differs from transfer to transfer by an XOR with a constant: row % 32 =
+  // (wave & 1) * 16 + 2 j + hl has its three parts in separate bits, and so has (row & 3) << 2 = (j & 1) << 3 | hl << 2.
+  // Rows beyond N repeat row N-1 (they are later than every query, so the mask removes their scores).
+  const uint32_t k_lane = (uint32_t)(hl * a.ks_l * 2), v_lane = (uint32_t)(hl * a.vs_l * 2);  // bytes
+  const uint32_t k_chunk0 = (uint32_t)(l32 ^ (((wave & 1) << 4) | hl)), v_chunk0 = (uint32_t)(l32 ^ (hl << 2));
+  auto issue_rows = [&](const uint16_t* base, int64_t stride, uint16_t* dst, int kt, bool is_v) {
+    if (kt * kTile + kTile <= a.N) {
+      const uint16_t* tb = base + ((int64_t)kt * kTile + wave * (2 * DMA_PER_WAVE)) * stride;  // uniform
+#pragma unroll
+      for (int j = 0; j < DMA_PER_WAVE; ++j) {
+        const uint32_t off = is_v ? v_lane + ((v_chunk0 ^ (uint32_t)((j & 1) << 3)) << 4) : k_lane + ((k_chunk0 ^ (uint32_t)(2 * j)) << 4);
+        lds_transfer16_base(tb + (int64_t)(2 * j) * stride, off, dst + (wave * DMA_PER_WAVE + j) * kWave * 8);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < DMA_PER_WAVE; ++j) {
+        const int row = wave * (2 * DMA_PER_WAVE) + 2 * j + hl;
+        const int chunk = is_v ? l32 ^ v_swizzle(row) : l32 ^ (row % OCT);
+        const int n = min(kt * kTile + row, a.N - 1);
+        lds_transfer<16>(base + (int64_t)n * stride + chunk * 8, dst + (wave * DMA_PER_WAVE + j) * kWave * 8);
+      }
+    }
+  };
+  auto issue_lim = [&](int kt, int slot) {
+    if (wave == 0) lds_transfer<4>(lim + min(kt * kTile + lane, a.N - 1), &sm.limk[slot][0]);
+  };
+  auto issue_k = [&](int kt, int buf, int slot) {
+    issue_rows(kp, a.ks_l, sm.k[buf], kt, false);
+    issue_lim(kt, slot);
+  };
+  auto issue_v = [&](int kt, int buf) { issue_rows(vp, a.vs_l, sm.v[buf], kt, true); };
+
+  // ---- operand fragments -------------------------------------------------------------------------------
+  auto k_frag = [&](const uint16_t* Kt, int kb, int s) {
+    const int row = kb * 32 + l32;
+    const int chunk = (s * 2 + hl) ^ (row % OCT);
+    return *reinterpret_cast<const bf16x8*>(Kt + row * D + chunk * 8);
+  };
+  const int r16 = lane & 15;
+  const int dsel = (lane >> 4) & 1;
+  auto v_frag = [&](const uint16_t* Vt, int t, int dt) {
+    const int chunk0 = dt * 4 + dsel * 2 + ((r16 & 3) >> 1);
+    const int half4 = (r16 & 1) * 4;
+    const int row_lo = t * 16 + hl * 4 + (r16 >> 2);
+    const int row_hi = row_lo + 8;
+    const uint16_t* pl = Vt + row_lo * D + ((chunk0 ^ v_swizzle(row_lo)) * 8) + half4;
+    const uint16_t* ph = Vt + row_hi * D + ((chunk0 ^ v_swizzle(row_hi)) * 8) + half4;
+    bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((bf16x4 __attribute__((address_space(3)))*)pl);
+    bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((bf16x4 __attribute__((address_space(3)))*)ph);
+    bf16x8 va = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    return va;
+  };
+
+  // scores of the first tile: nothing to run under, the K fragments are requested eight ahead
+  auto qk_tile_first = [&](int buf, f32x16 (&sacc)[2]) {
+    const uint16_t* Kt = sm.k[buf];
+    constexpr int N_QK = 2 * DSTEPS;
+    constexpr int AHEAD = 8;
+    bf16x8 kf[AHEAD];
+#pragma unroll
+    for (int i = 0; i < AHEAD; ++i) kf[i] = k_frag(Kt, i & 1, i >> 1);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < N_QK; ++i) {
+      const int s = i >> 1, kb = i & 1;
+      if (s == 0) {
+        const f32x16 z = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i % AHEAD], qreg[s], z, 0, 0, 0);
+      } else {
+        sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i % AHEAD], qreg[s], sacc[kb], 0, 0, 0);
+      }
+      if (i + AHEAD < N_QK) kf[i % AHEAD] = k_frag(Kt, (i + AHEAD) & 1, (i + AHEAD) >> 1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  auto mask_scores = [&](int kt, int slot, f32x16 (&sv)[2]) {
+    const int qtok = q0 + l32;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+      for (int g4 = 0; g4 < 4; ++g4) {
+        int kk = kb * 32 + g4 * 8 + hl * 4;  // key offset in tile of accumulator 4*g4
+        int4 lm = *reinterpret_cast<const int4*>(&sm.limk[slot][kk]);
+        const int lv[4] = {lm.x, lm.y, lm.z, lm.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          int key = kt * kTile + kk + e - a.base;  // region token of the key row (negative: older row)
+          bool vis = key <= qtok && qtok <= lv[e];
+          if (!vis) sv[kb][g4 * 4 + e] = -INFINITY;
+        }
+      }
+    }
+  };
+  auto row_max = [&](const f32x16 (&sv)[2]) {
+    float m = -INFINITY;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) m = fmaxf(m, sv[kb][i]);
+    return half_swap_max(m) * c;
+  };
+  auto rescale = [&](float mx) {
+    float m_new = fmaxf(m_run, mx);
+    float alpha = m_run == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_run - m_new);
+    l_run *= alpha;
+    m_run = m_new;
+    // The accumulators live in the accumulation registers, which vector instructions reach only through moves.  The
+    // moves are written here, in this rarely taken branch: left to the compiler, all 128 are read into vector
+    // registers at the top of every step.  (The waits cover a matrix instruction that may still be writing.)
+#if defined(__HIP_DEVICE_COMPILE__)
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        float x = oacc[dt][i], tmp;
+        asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\tv_accvgpr_write_b32 %0, %1"
+                     : "+a"(x), "=&v"(tmp)
+                     : "v"(alpha));
+        oacc[dt][i] = x;
+      }
+    asm volatile("s_nop 4" ::: "memory");
+#endif
+  };
+  // n-th probability of the tile in the order the PV MFMAs consume them (16 keys per B operand)
+  auto prob = [&](const f32x16 (&sv)[2], int n, float m_use, float& rs, bf16x8 (&pb)[4]) {
+    const int t = n >> 3, i = n & 7;
+    float p = __builtin_amdgcn_exp2f(fmaf(sv[t >> 1][(t & 1) * 8 + i], c, -m_use));
+    rs += p;
+    pb[t][i] = (__bf16)p;
+  };
+  // scores of the next tile under the probabilities of keys 0..31 of this one, O += P V for keys 0..31 under the
+  // probabilities of keys 32..63, then O += P V for keys 32..63; LDS operands are fetched two slots ahead
+  auto fused_step = [&](int kbuf_next, int vbuf, const f32x16 (&sv)[2], f32x16 (&sacc)[2]) {
+    const uint16_t* Kt = sm.k[kbuf_next];
+    const uint16_t* Vt = sm.v[vbuf];
+    constexpr int N_QK = 2 * DSTEPS;  // score MFMAs
+    constexpr int N_PV = 4 * DT;      // PV MFMAs
+    const float m_use = m_run == -INFINITY ? 0.f : m_run;
+    float rs = 0.f;
+    bf16x8 pb[4];
+    int n = 0;
+    __builtin_amdgcn_sched_barrier(0);
+    auto k_at = [&](int i) { return k_frag(Kt, i & 1, i >> 1); };
+    auto v_at = [&](int i) { return v_frag(Vt, i / DT, i % DT); };
+    constexpr int R = 3;  // ring of operand fragments, fetched R - 1 slots ahead (deeper rings measure the same)
+    bf16x8 kf[R], vf[R];
+#pragma unroll
+    for (int i = 0; i < R - 1; ++i) kf[i] = k_at(i);
+#pragma unroll
+    for (int i = 0; i < N_QK; ++i) {
+      const int s = i >> 1, kb = i & 1;
+      if (i + R - 1 < N_QK) {
+        kf[(i + R - 1) % R] = k_at(i + R - 1);
+      } else {
+        vf[(i + R - 1 - N_QK) % R] = v_at(i + R - 1 - N_QK);
+      }
+      if (s == 0) {
+        const f32x16 z = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i % R], qreg[s], z, 0, 0, 0);
+      } else {
+        sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i % R], qreg[s], sacc[kb], 0, 0, 0);
+      }
+      if (n < 16) prob(sv, n++, m_use, rs, pb);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int i = 0; i < N_PV; ++i) {
+      const int t = i / DT, dt = i % DT;
+      if (i + R - 1 < N_PV) vf[(i + R - 1) % R] = v_at(i + R - 1);
+      oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[i % R], pb[t], oacc[dt], 0, 0, 0);
+      if (t < 2 && n < 32) prob(sv, n++, m_use, rs, pb);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    l_run += rs;
+  };
+
+  // ---- tile loop -----------------------------------------------------------------------------------------
+  int min_cur = 0, min_n1 = 0, min_n2 = 0;
+  int t_cur = next_tile(min_cur);
+  int t_n1 = t_cur >= 0 ? next_tile(min_n1) : -1;
+  int t_n2 = t_n1 >= 0 ? next_tile(min_n2) : -1;
+  f32x16 sacc[2];
+#pragma unroll
+  for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) sacc[kb][i] = 0.f;
+  if (t_cur >= 0) {
+    issue_k(t_cur, 0, 0);
+    issue_v(t_cur, 0);
+    if (t_n1 >= 0) issue_k(t_n1, 1, 1);
+    wait_transfers();
+    __syncthreads();
+    qk_tile_first(0, sacc);
+  }
+  for (int j = 0; t_cur >= 0; ++j) {
+    // everything requested has landed, and every wavefront is through step j - 1: K of tile j and V of tile j - 1
+    // have been read for the last time
+    wait_transfers();
+    __syncthreads();
+    if (t_n2 >= 0) issue_k(t_n2, j & 1, (j + 2) & 3);
+    if (t_n1 >= 0) issue_v(t_n1, (j + 1) & 1);
+    f32x16 sv[2] = {sacc[0], sacc[1]};
+    // no masked score: every key row is at or before the first query and visible to the last one
+    const bool full = t_cur * kTile + kTile - 1 - a.base <= my_r0 && min_cur >= my_rlast;
+    if (!full) mask_scores(t_cur, j & 3, sv);
+    const float mx = row_max(sv);
+    if (__builtin_expect(__ballot(mx > m_run + kRescaleSlack) != 0, 0)) rescale(mx);  // (rare: kept out of the way)
+    fused_step((j + 1) & 1, j & 1, sv, sacc);  // (after the last tile: scores of a stale tile that nobody reads)
+    t_cur = t_n1; min_cur = min_n1;
+    t_n1 = t_n2; min_n1 = min_n2;
+    t_n2 = t_n1 >= 0 ? next_tile(min_n2) : -1;
+  }
+  __syncthreads();  // the tile buffers are free
+
+  // ---- epilogue: O rows go through LDS so that every row leaves as whole 16-byte pieces ----------------
+  constexpr int kRowPitch = D * 2 + 16;  // bytes; the pad spreads the rows over the banks
+  static_assert(kWideWaves * kHalf * kRowPitch <= sizeof(WideSmem), "staging area fits the tile buffers");
+  unsigned char* stage = smem_raw + wave * (kHalf * kRowPitch);
+  {
+    const float l = half_swap_sum(l_run);
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+      for (int g4 = 0; g4 < 4; ++g4) {
+        int d = dt * 32 + g4 * 8 + hl * 4;
+        const bf16x4 ob = {(__bf16)(oacc[dt][g4 * 4 + 0] * inv), (__bf16)(oacc[dt][g4 * 4 + 1] * inv),
+                           (__bf16)(oacc[dt][g4 * 4 + 2] * inv), (__bf16)(oacc[dt][g4 * 4 + 3] * inv)};
+        *reinterpret_cast<uint2*>(stage + l32 * kRowPitch + d * 2) = __builtin_bit_cast(uint2, ob);
+      }
+    }
+  }
+  wave_lds_sync();
+  if (wave_live) {
+    uint16_t* op = static_cast<uint16_t*>(a.o) + b * a.os_b + hq * a.os_h;
+    constexpr int kPieces = kHalf * OCT / kWave;  // 16-byte pieces per lane
+#pragma unroll
+    for (int i = 0; i < kPieces; ++i) {
+      const int id = i * kWave + lane;
+      const int row = id / OCT, piece = id % OCT;
+      const int qtok = q0 + row;
+      if (qtok >= a.r_begin && qtok < a.r_end) {
+        const u32x4 val = *reinterpret_cast<const u32x4*>(stage + row * kRowPitch + piece * 16);
+        __builtin_nontemporal_store(val, reinterpret_cast<u32x4*>(op + (int64_t)(qtok - a.r_begin) * a.os_l + piece * 8));
+      }
+    }
+  }
+}
+
+static int launch_prefill_wide(const PrefillArgs& a, int64_t n_wg, hipStream_t st) {
+  static bool configured[kMaxDevices] = {};  // the attribute is set once per device
+  const size_t smem = sizeof(WideSmem);
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail(NATS_ERR_LAUNCH, "prefill: no current device");
+  if (!configured[dev]) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_mfma_wide_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) return fail(NATS_ERR_LAUNCH, "hipFuncSetAttribute(%zu bytes of LDS): %s", smem, hipGetErrorString(e));
+    configured[dev] = true;
+  }
+  hipLaunchKernelGGL(prefill_mfma_wide_kernel, dim3((unsigned)n_wg), dim3(kWideWaves * kWave), smem, st, a);
+  NATS_CHECK_LAUNCH("prefill_mfma_wide_kernel");
+  return NATS_OK;
+}
+
 template <int D, bool kUniform, int kMode = 0>
 static int launch_prefill_mfma(const PrefillArgs& a, int64_t n_wg, hipStream_t st) {
   static bool configured[kMaxDevices] = {};  // per instantiation; the attribute is set once per device
@@ -1307,7 +1714,28 @@ int launch_segment(const char* who, const SegmentShape& g, const void* q, const 
   a.scale = sm_scale;
   a.hpw = 1; a.qpw = 1; a.n_hg = 1; a.n_qg = (int)n_qt; a.xcd_mode = 0;
 
-  // fp32, and bf16 at the head dims the MFMA kernel does not take (16, 32, 256): the plain kernel
+  // bf16 at head dim 256 (rows that 16-byte transfers can take; other layouts go to the plain kernel)
+  if (dtype == NATS_DTYPE_BF16 && g.D == 256) {
+    bool rows16 = (reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
+                   reinterpret_cast<uintptr_t>(o)) % 16 == 0;
+    for (int i = 0; i < 3; ++i)
+      rows16 = rows16 && q_strides[i] % 8 == 0 && k_strides[i] % 8 == 0 && v_strides[i] % 8 == 0 && o_strides[i] % 8 == 0;
+    if (rows16) {
+      const int hpw = a.n_rep % 4 == 0 ? 4 : a.n_rep % 2 == 0 ? 2 : 1;
+      a.hpw = hpw;
+      a.qpw = kWideWaves / hpw;  // blocks of 32 query rows per workgroup
+      a.n_hg = a.n_rep / hpw;
+      const int64_t n_blk = (a.r_end - 1) / (kTile / 2) - a.r_begin / (kTile / 2) + 1;
+      a.n_qg = (int)((n_blk + a.qpw - 1) / a.qpw);
+      a.xcd_mode = ((g.B * g.H_kv) % 8 == 0) ? 1 : 0;
+      a.n_split = 1;
+      const int64_t n_wg = g.B * g.H_kv * a.n_hg * a.n_qg;
+      NATS_REQUIRE(n_wg < (int64_t(1) << 31), NATS_ERR_BAD_SHAPE, "%s: grid too large", who);
+      return launch_prefill_wide(a, n_wg, st);
+    }
+  }
+
+  // fp32, and bf16 at the head dim the MFMA kernels do not take (16): the plain kernel
   if (dtype == NATS_DTYPE_F32 || (g.D != 32 && g.D != 64 && g.D != 128)) {
     NATS_REQUIRE(g.B * g.H_q <= 65535, NATS_ERR_BAD_SHAPE, "%s: B*H_q too large for the plain kernel", who);
     dim3 grid((unsigned)n_qt, (unsigned)(g.B * g.H_q));

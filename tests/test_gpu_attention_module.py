@@ -212,3 +212,11 @@ def test_module_with_an_executor_under_a_side_stream():
 def test_module_with_other_head_dims(dim):
     """Head dims 16, 32 and 256 (the reference's kernel accepts them too): prefill, segments and one-token steps."""
     run_module([90, 1, 1, 40, 1, 1, 1, 17], 8, 16, dim=dim)
+
+
+@pytest.mark.parametrize("lens,C,W", [([300, 1, 1, 150, 70, 1, 200], 16, 64), ([130, 65, 1, 1, 1, 40, 260], 64, 128),
+                                      ([200] + [1] * 20 + [90, 33], 1, 16)])
+def test_module_at_head_dim_256_over_a_filled_cache(lens, C, W):
+    """Segments over the rows earlier segments left behind (ring, kept globals, locals up to the first global chunk)
+    on the head-dim-256 matrix kernels of both sides."""
+    run_module(lens, C, W, dim=2048)

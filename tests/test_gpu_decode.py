@@ -64,7 +64,7 @@ def run_case(B, Hq, Hkv, D, W, C, n_max_chunks, dtype, seed=0, frac=(0.1, 1.0), 
 
 
 @pytest.mark.parametrize("n_rep", [1, 2, 3, 4, 5, 6, 7, 8, 12, 16])
-@pytest.mark.parametrize("D", [32, 64, 128])
+@pytest.mark.parametrize("D", [32, 64, 128, 256])
 def test_bf16_group_sizes(n_rep, D):
     run_case(2, 2 * n_rep, 2, D, 128, 64, 20, torch.bfloat16, seed=n_rep + D)
 
@@ -118,6 +118,14 @@ def test_fp32(D):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_other_head_dims(D, dtype):
     run_case(2, 4, 2, D, 32, 8, 20, dtype, seed=D, fill=3)
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,chunks,fill,q_scale", [(1, 8, 2, 300, 13, 1.0), (4, 16, 4, 150, 0, 4.0),
+                                                           (40, 8, 8, 12, 37, 1.0)])
+def test_head_dim_256_on_the_matrix_kernel(B, Hq, Hkv, chunks, fill, q_scale):
+    """Rows of 512 bytes: a wavefront's two V tiles take 32 KB of LDS, one workgroup per compute unit.  A single long
+    sequence, peaked scores, more streams than workgroups."""
+    run_case(B, Hq, Hkv, 256, 256, 64, chunks, torch.bfloat16, seed=B + chunks, frac=(0.1, 1.0), fill=fill, q_scale=q_scale)
 
 
 def test_strided_cache_views():

@@ -70,11 +70,19 @@ def test_head_dim_32_on_the_matrix_kernels(Hq, Hkv, L, C, W):
     run_case(2, Hq, Hkv, L, 32, C, W, torch.bfloat16, seed=L + 32)
 
 
+@pytest.mark.parametrize("Hq,Hkv,L,C,W", [(8, 2, 1000, 64, 128), (8, 1, 777, 32, 64), (4, 4, 900, 16, 32), (4, 2, 650, 1, 16),
+                                          (6, 2, 2100, 128, 256), (2, 2, 31, 8, 8), (16, 8, 4100, 64, 256), (3, 1, 129, 3, 6)])
+def test_head_dim_256_on_the_matrix_kernel(Hq, Hkv, L, C, W):
+    """Rows of 512 bytes: four wavefronts per workgroup, one per SIMD, two K and two V tile buffers; groups of 1, 2, 3
+    and 8 q heads, chunks shorter than a tile masked row by row, lengths that end inside a block of 32 rows."""
+    run_case(2, Hq, Hkv, L, 256, C, W, torch.bfloat16, seed=L + 256)
+
+
 @pytest.mark.parametrize("D", [16, 32, 256])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_other_head_dims(D, dtype):
-    """The head dims the reference's kernel also accepts (models/transformer/triton/nats_flashattn_fwd.py:634) run
-    the plain kernel in both dtypes."""
+    """The other head dims the reference's kernel accepts (models/transformer/triton/nats_flashattn_fwd.py:634): the
+    plain kernel in fp32 and at 16, the matrix kernels in bf16 at 32 and 256."""
     run_case(2, 4, 2, 333, D, 8, 16, dtype, seed=D)
     run_case(1, 2, 2, 200, D, 64, 128, dtype, seed=D + 1)
 
@@ -404,6 +412,8 @@ def check_rising(B, Hq, Hkv, L, D, C, W, p, step_rows=48, step_nats=7.0, seed=0)
     (4, 2, 1200, 128, 8, 32, (0.3, 0.3, 0.4)),     # groups of two
     (6, 2, 900, 128, 64, 128, (0.4, 0.3, 0.3)),    # a group of three: the per-wavefront form
     (8, 2, 4500, 128, 64, 256, (1.0, 0.0, 0.0)),   # dense and long: lists of up to 71 tiles
+    (8, 2, 1500, 256, 64, 256, (1.0, 0.0, 0.0)),   # head_dim 256 (its own kernel), dense
+    (4, 2, 1300, 256, 16, 64, (0.3, 0.3, 0.4)),    # head_dim 256, short chunks, groups of two
 ])
 def test_rising_scores_rescale_the_accumulators(Hq, Hkv, L, D, C, W, p):
     say("prefill rising scores", Hq, Hkv, L, D, C, W, p)
