@@ -1223,10 +1223,16 @@ __device__ __forceinline__ void lds_transfer(const void* gptr, const void* lds_p
 #endif
 }
 // The same with the address as a uniform base (scalar registers) plus a byte offset per lane: no 64-bit vector arithmetic.
-__device__ __forceinline__ void lds_transfer16_base(const void* base, uint32_t byte_off, const void* lds_ptr) {
+// (the LDS address as a number: taken from a pointer once, it is plain scalar arithmetic from then on)
+__device__ __forceinline__ uint32_t lds_address(const void* lds_ptr) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  const uint32_t lds_addr =
-      __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(const __attribute__((address_space(3))) unsigned char*)lds_ptr);
+  return __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(const __attribute__((address_space(3))) unsigned char*)lds_ptr);
+#else
+  return 0;
+#endif
+}
+__device__ __forceinline__ void lds_transfer16_base(const void* base, uint32_t byte_off, uint32_t lds_addr) {
+#if defined(__HIP_DEVICE_COMPILE__)
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(byte_off), "s"(base), "s"(lds_addr)
                : "memory", "m0");
 #endif
@@ -1331,13 +1337,16 @@ __global__ __launch_bounds__(kWideWaves * kWave) void prefill_mfma_wide_kernel(P
   // Rows beyond N repeat row N-1 (they are later than every query, so the mask removes their scores).
   const uint32_t k_lane = (uint32_t)(hl * a.ks_l * 2), v_lane = (uint32_t)(hl * a.vs_l * 2);  // bytes
   const uint32_t k_chunk0 = (uint32_t)(l32 ^ (((wave & 1) << 4) | hl)), v_chunk0 = (uint32_t)(l32 ^ (hl << 2));
+  const uint32_t lds_k0 = lds_address(&sm.k[0][0]), lds_v0 = lds_address(&sm.v[0][0]);
   auto issue_rows = [&](const uint16_t* base, int64_t stride, uint16_t* dst, int kt, bool is_v) {
     if (kt * kTile + kTile <= a.N) {
       const uint16_t* tb = base + ((int64_t)kt * kTile + wave * (2 * DMA_PER_WAVE)) * stride;  // uniform
+      const uint32_t lds = (is_v ? lds_v0 + (uint32_t)((dst - &sm.v[0][0]) * 2) : lds_k0 + (uint32_t)((dst - &sm.k[0][0]) * 2)) +
+                           (uint32_t)(wave * DMA_PER_WAVE * kWave * 16);
 #pragma unroll
       for (int j = 0; j < DMA_PER_WAVE; ++j) {
         const uint32_t off = is_v ? v_lane + ((v_chunk0 ^ (uint32_t)((j & 1) << 3)) << 4) : k_lane + ((k_chunk0 ^ (uint32_t)(2 * j)) << 4);
-        lds_transfer16_base(tb + (int64_t)(2 * j) * stride, off, dst + (wave * DMA_PER_WAVE + j) * kWave * 8);
+        lds_transfer16_base(tb + (int64_t)(2 * j) * stride, off, lds + (uint32_t)(j * kWave * 16));
       }
     } else {
 #pragma unroll
