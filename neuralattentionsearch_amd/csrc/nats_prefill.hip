@@ -1222,8 +1222,7 @@ __device__ __forceinline__ void lds_transfer(const void* gptr, const void* lds_p
   }
 #endif
 }
-// The same with the address as a uniform base (scalar registers) plus a byte offset per lane: no 64-bit vector arithmetic.
-// (the LDS address as a number: taken from a pointer once, it is plain scalar arithmetic from then on)
+// The LDS address of an object as a number: taken from the pointer once, it is plain scalar arithmetic from then on.
 __device__ __forceinline__ uint32_t lds_address(const void* lds_ptr) {
 #if defined(__HIP_DEVICE_COMPILE__)
   return __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(const __attribute__((address_space(3))) unsigned char*)lds_ptr);
@@ -1231,6 +1230,8 @@ __device__ __forceinline__ uint32_t lds_address(const void* lds_ptr) {
   return 0;
 #endif
 }
+// A 16-byte transfer with the global address as a uniform base (scalar registers) plus a byte offset per lane (no 64-bit
+// vector arithmetic) and the LDS address as a number.
 __device__ __forceinline__ void lds_transfer16_base(const void* base, uint32_t byte_off, uint32_t lds_addr) {
 #if defined(__HIP_DEVICE_COMPILE__)
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(byte_off), "s"(base), "s"(lds_addr)
